@@ -1,0 +1,425 @@
+"""ctypes binding of the CPU oracle (oracle/mynn_oracle.c).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, __graft_entry__.smoke() and bench.py's
+cpu_baseline leg, as the checker or the timed CPU baseline.  The shipped package never
+imports this module.
+
+Arrays are numpy; 16-bit float tensors travel as uint16 bit patterns together with a dtype
+code (F32 = 0, BF16 = 1, F16 = 2).
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+F32, BF16, F16 = 0, 1, 2
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "_build", "libmynn_oracle.so")
+
+
+def build(force=False):
+    """Compiles the oracle with gcc (a few seconds)."""
+    if force and os.path.exists(_SO):
+        os.remove(_SO)
+    subprocess.check_call(["make", "-C", _HERE, "--no-print-directory"])
+    return _SO
+
+
+def _load():
+    if not os.path.exists(_SO):
+        build()
+    return C.CDLL(_SO)
+
+
+_lib = _load()
+_vp, _sz, _i, _ll, _f, _d = C.c_void_p, C.c_size_t, C.c_int, C.c_longlong, C.c_float, C.c_double
+
+
+def _sig(name, res, *args):
+    fn = getattr(_lib, name)
+    fn.restype = res
+    fn.argtypes = list(args)
+    return fn
+
+
+_sig("orc_set_lanes", None, _i)
+_sig("orc_get_lanes", _i)
+_sig("orc_set_threads", None, _i)
+_sig("orc_get_threads", _i)
+_sig("orc_f32_to_bf16", C.c_uint16, _f)
+_sig("orc_f32_to_f16", C.c_uint16, _f)
+_sig("orc_f16_to_f32", _f, C.c_uint16)
+_sig("orc_convert", None, _vp, _i, _vp, _i, _sz)
+_sig("orc_dequantize_linear", None, _vp, _vp, _vp, _sz, _sz, _i)
+_sig("orc_dequant_matmul", None, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _i, _i, _i)
+_sig("orc_quantized_matmul", None, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _i)
+_sig("orc_dynquant_i8", None, _vp, _vp, _vp, _sz, _sz, _i)
+_sig("orc_dynquant_i8_per_tensor", None, _vp, _vp, _vp, _sz, _i)
+_sig("orc_dynquant_u8_asym", None, _vp, _vp, _vp, _vp, _sz, _sz, _i)
+_sig("orc_attention", None, _vp, _vp, _vp, _vp, _vp, _vp, _ll, _sz, _sz, _sz, _sz, _sz, _sz, _i, _f, _i, _i)
+_sig("orc_attention_f64", None, _vp, _vp, _vp, _vp, _ll, _sz, _sz, _sz, _sz, _sz, _sz, _i, _d, _i)
+_sig("orc_kv_cache_update", None, _vp, _vp, _ll, _sz, _sz, _sz, _sz, _sz)
+_sig("orc_quantizing_kv_cache_update", None, _vp, _vp, _vp, _ll, _sz, _sz, _sz, _sz, _i)
+_sig("orc_rms_norm", None, _vp, _vp, _vp, _sz, _sz, _d, _i)
+_sig("orc_rope_table", None, _vp, _vp, _sz, _sz, _f, _i)
+_sig("orc_rope", None, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _i)
+_sig("orc_gather_rows", None, _vp, _vp, _vp, _sz, _sz, _sz)
+_sig("orc_swish", None, _vp, _vp, _sz, _i)
+_sig("orc_swiglu", None, _vp, _vp, _vp, _sz, _i)
+_sig("orc_add", None, _vp, _vp, _vp, _sz, _i)
+_sig("orc_argmax_last", C.c_int64, _vp, _sz, _i)
+_sig("orc_quantize_per_channel", None, _vp, _vp, _vp, _sz, _sz, _i)
+_sig("orc_ring_phys_index", _i, _i, _i, _i, _i)
+_sig("orc_streaming_kv_position", None, _vp, _sz, _sz, _sz, _sz)
+
+
+class ModelCfg(C.Structure):
+    _fields_ = [("n_layers", _i), ("hidden", _i), ("n_heads", _i), ("n_kv_heads", _i),
+                ("head_dim", _i), ("ffn", _i), ("vocab", _i), ("max_seq", _i),
+                ("eps", _d), ("rope_theta", _f), ("dtype", _i)]
+
+
+class Linear(C.Structure):
+    _fields_ = [("q", _vp), ("scale", _vp), ("w", _vp)]
+
+
+_sig("orc_model_create", _vp, C.POINTER(ModelCfg))
+_sig("orc_model_destroy", None, _vp)
+_sig("orc_model_set_embed", None, _vp, Linear)
+_sig("orc_model_set_lm_head", None, _vp, Linear)
+_sig("orc_model_set_final_norm", None, _vp, _vp)
+_sig("orc_model_set_linear", None, _vp, _i, _i, Linear)
+_sig("orc_model_set_norm", None, _vp, _i, _i, _vp)
+_sig("orc_model_reset", None, _vp)
+_sig("orc_model_past_len", _ll, _vp)
+_sig("orc_model_set_past_len", None, _vp, _ll)
+_sig("orc_model_forward", None, _vp, _vp, _vp, _sz, _ll, _ll, _i, _vp)
+_sig("orc_model_decode_step", C.c_int64, _vp, C.c_int64)
+_sig("orc_model_prefill", C.c_int64, _vp, _vp, _sz, _sz)
+_sig("orc_model_generate", _ll, _vp, _vp, _sz, _sz, _sz, C.c_int64, _vp)
+_sig("orc_model_k_cache", _vp, _vp, _i)
+_sig("orc_model_v_cache", _vp, _vp, _i)
+_sig("orc_model_last_hidden", _vp, _vp)
+
+
+# ------------------------------------------------------------------ helpers
+def np_dtype(dt):
+    return np.float32 if dt == F32 else np.uint16
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(_vp)
+
+
+def _c(a, dt=None):
+    a = np.ascontiguousarray(a)
+    if dt is not None and a.dtype != np.dtype(dt):
+        raise TypeError("expected %s, got %s" % (np.dtype(dt), a.dtype))
+    return a
+
+
+def set_lanes(n):
+    _lib.orc_set_lanes(int(n))
+
+
+def set_threads(n):
+    _lib.orc_set_threads(int(n))
+
+
+def get_threads():
+    return _lib.orc_get_threads()
+
+
+def to_storage(x, dt):
+    """float32 array -> storage array of type dt (RNE)."""
+    x = _c(np.asarray(x, dtype=np.float32))
+    if dt == F32:
+        return x.copy()
+    out = np.empty(x.shape, np.uint16)
+    _lib.orc_convert(_p(out), dt, _p(x), F32, x.size)
+    return out
+
+
+def to_f32(x, dt):
+    """storage array -> float32 (exact)."""
+    x = _c(x)
+    if dt == F32:
+        return x.astype(np.float32)
+    out = np.empty(x.shape, np.float32)
+    _lib.orc_convert(_p(out), F32, _p(x), dt, x.size)
+    return out
+
+
+def dequantize_linear(x_i8, scale, dt):
+    x_i8 = _c(x_i8, np.int8)
+    scale = _c(scale, np_dtype(dt))
+    rows = x_i8.shape[0]
+    cols = x_i8.size // rows
+    out = np.empty(x_i8.shape, np_dtype(dt))
+    _lib.orc_dequantize_linear(_p(out), _p(x_i8), _p(scale), rows, cols, dt)
+    return out
+
+
+def dequant_matmul(act, wq, scale, act_dt, out_dt, mode=-1):
+    act, wq, scale = _c(act, np_dtype(act_dt)), _c(wq, np.int8), _c(scale, np_dtype(out_dt))
+    N, K = wq.shape
+    M = act.size // K
+    out = np.empty(act.shape[:-1] + (N,), np_dtype(out_dt))
+    _lib.orc_dequant_matmul(_p(out), _p(act), _p(wq), _p(scale), M, N, K, act_dt, out_dt, mode)
+    return out
+
+
+def quantized_matmul(lhs, lhs_scale, rhs, rhs_scale, dt):
+    lhs, rhs = _c(lhs, np.int8), _c(rhs, np.int8)
+    lhs_scale, rhs_scale = _c(lhs_scale, np_dtype(dt)), _c(rhs_scale, np_dtype(dt))
+    M, K = lhs.shape
+    N = rhs.shape[0]
+    out = np.empty((M, N), np_dtype(dt))
+    acc = np.empty((M, N), np.int32)
+    _lib.orc_quantized_matmul(_p(out), _p(acc), _p(lhs), _p(lhs_scale), _p(rhs), _p(rhs_scale), M, N, K, dt)
+    return out, acc
+
+
+def dynquant_i8(x, dt):
+    x = _c(x, np_dtype(dt))
+    M, K = x.shape
+    y = np.empty((M, K), np.int8)
+    s = np.empty((M,), np_dtype(dt))
+    _lib.orc_dynquant_i8(_p(y), _p(s), _p(x), M, K, dt)
+    return y, s
+
+
+def dynquant_i8_per_tensor(x, dt):
+    x = _c(x, np_dtype(dt))
+    y = np.empty(x.shape, np.int8)
+    s = np.empty((1,), np_dtype(dt))
+    _lib.orc_dynquant_i8_per_tensor(_p(y), _p(s), _p(x), x.size, dt)
+    return y, s
+
+
+def dynquant_u8_asym(x, dt):
+    x = _c(x, np_dtype(dt))
+    M, K = x.shape
+    y = np.empty((M, K), np.uint8)
+    s = np.empty((M,), np_dtype(dt))
+    zp = np.empty((M,), np.uint8)
+    _lib.orc_dynquant_u8_asym(_p(y), _p(s), _p(zp), _p(x), M, K, dt)
+    return y, s, zp
+
+
+def attention(q, k, v, dt, scale, is_causal=False, active=-1, k_scale=None, v_scale=None):
+    kv_int8 = k.dtype == np.int8
+    q = _c(q, np_dtype(dt))
+    k = _c(k, np.int8 if kv_int8 else np_dtype(dt))
+    v = _c(v, np.int8 if kv_int8 else np_dtype(dt))
+    B, Hq, Sq, D = q.shape
+    Hkv, Sk = k.shape[1], k.shape[2]
+    out = np.empty(q.shape, np_dtype(dt))
+    ks = _c(k_scale, np_dtype(dt)) if kv_int8 else None
+    vs = _c(v_scale, np_dtype(dt)) if kv_int8 else None
+    _lib.orc_attention(_p(out), _p(q), _p(k), _p(v), _p(ks), _p(vs), int(active), B, Hq, Hkv, Sq, Sk, D,
+                       int(is_causal), float(scale), dt, int(kv_int8))
+    return out
+
+
+def attention_f64(q, k, v, dt, scale, is_causal=False, active=-1):
+    q, k, v = _c(q, np_dtype(dt)), _c(k, np_dtype(dt)), _c(v, np_dtype(dt))
+    B, Hq, Sq, D = q.shape
+    Hkv, Sk = k.shape[1], k.shape[2]
+    out = np.empty(q.shape, np.float64)
+    _lib.orc_attention_f64(_p(out), _p(q), _p(k), _p(v), int(active), B, Hq, Hkv, Sq, Sk, D,
+                           int(is_causal), float(scale), dt)
+    return out
+
+
+def kv_cache_update(cache, new_kv, offset):
+    """cache [B,H,max_seq,D] is updated in place (and returned)."""
+    assert cache.flags.c_contiguous
+    new_kv = _c(new_kv, cache.dtype)
+    B, H, max_seq, D = cache.shape
+    _lib.orc_kv_cache_update(_p(cache), _p(new_kv), int(offset), B * H, new_kv.shape[2], max_seq, D,
+                             cache.itemsize)
+    return cache
+
+
+def quantizing_kv_cache_update(cache, scale, new_kv, offset, dt):
+    assert cache.flags.c_contiguous and cache.dtype == np.int8 and scale.flags.c_contiguous
+    new_kv = _c(new_kv, np_dtype(dt))
+    B, H, max_seq, D = cache.shape
+    _lib.orc_quantizing_kv_cache_update(_p(cache), _p(scale), _p(new_kv), int(offset), B * H,
+                                        new_kv.shape[2], max_seq, D, dt)
+    return cache, scale
+
+
+def rms_norm(x, w, eps, dt):
+    x, w = _c(x, np_dtype(dt)), _c(w, np_dtype(dt))
+    dim = x.shape[-1]
+    out = np.empty(x.shape, np_dtype(dt))
+    _lib.orc_rms_norm(_p(out), _p(x), _p(w), x.size // dim, dim, float(eps), dt)
+    return out
+
+
+def rope_table(max_seq, D, base, dt):
+    cos = np.empty((max_seq, D), np_dtype(dt))
+    sin = np.empty((max_seq, D), np_dtype(dt))
+    _lib.orc_rope_table(_p(cos), _p(sin), max_seq, D, float(base), dt)
+    return cos, sin
+
+
+def rope(x, cos, sin, position, dt):
+    """x [..., S, D]; position [S] int64."""
+    x, cos, sin = _c(x, np_dtype(dt)), _c(cos, np_dtype(dt)), _c(sin, np_dtype(dt))
+    position = _c(np.asarray(position, np.int64))
+    S, D = x.shape[-2], x.shape[-1]
+    out = np.empty(x.shape, np_dtype(dt))
+    _lib.orc_rope(_p(out), _p(x), _p(cos), _p(sin), _p(position), x.size // (S * D), S, D, dt)
+    return out
+
+
+def gather_rows(data, idx):
+    data = _c(data)
+    idx = _c(np.asarray(idx, np.int64))
+    rows = data.shape[0]
+    row_bytes = data.nbytes // rows
+    out = np.empty(idx.shape + data.shape[1:], data.dtype)
+    _lib.orc_gather_rows(_p(out), _p(data), _p(idx), idx.size, rows, row_bytes)
+    return out
+
+
+def swish(x, dt):
+    x = _c(x, np_dtype(dt))
+    out = np.empty(x.shape, np_dtype(dt))
+    _lib.orc_swish(_p(out), _p(x), x.size, dt)
+    return out
+
+
+def swiglu(gate, up, dt):
+    gate, up = _c(gate, np_dtype(dt)), _c(up, np_dtype(dt))
+    out = np.empty(gate.shape, np_dtype(dt))
+    _lib.orc_swiglu(_p(out), _p(gate), _p(up), gate.size, dt)
+    return out
+
+
+def add(a, b, dt):
+    a, b = _c(a, np_dtype(dt)), _c(b, np_dtype(dt))
+    out = np.empty(a.shape, np_dtype(dt))
+    _lib.orc_add(_p(out), _p(a), _p(b), a.size, dt)
+    return out
+
+
+def argmax_last(logits, dt):
+    logits = _c(logits, np_dtype(dt))
+    return int(_lib.orc_argmax_last(_p(logits), logits.size, dt))
+
+
+def quantize_per_channel(w, scale_dt):
+    w = _c(np.asarray(w, np.float32))
+    rows = w.shape[0]
+    q = np.empty(w.shape, np.int8)
+    s = np.empty((rows,), np_dtype(scale_dt))
+    _lib.orc_quantize_per_channel(_p(q), _p(s), _p(w), rows, w.size // rows, scale_dt)
+    return q, s
+
+
+def ring_phys_index(rank, sink, window, start):
+    return _lib.orc_ring_phys_index(rank, sink, window, start)
+
+
+def streaming_kv_position(sink, window, stream_pos, max_seq):
+    out = np.empty((max_seq,), np.int64)
+    _lib.orc_streaming_kv_position(_p(out), sink, window, stream_pos, max_seq)
+    return out
+
+
+LIN_NAMES = ("q", "k", "v", "o", "gate", "up", "down")
+
+
+class Model:
+    """The decoder of crates/llm (decoder.rs build_decoder) plus the LlmSession loop.
+
+    weights: dict with
+      "embed", "lm_head", "layers.{i}.{q,k,v,o,gate,up,down}" -> (int8 [N,K], scale [N]) tuples for
+      quantised tensors or a single storage array [N,K] for plain ones;
+      "final_norm", "layers.{i}.norm1", "layers.{i}.norm2" -> storage arrays.
+    """
+
+    def __init__(self, cfg, weights):
+        self.cfg = ModelCfg(**cfg)
+        self.dt = cfg["dtype"]
+        self._keep = []
+        self._h = _lib.orc_model_create(C.byref(self.cfg))
+        _lib.orc_model_set_embed(self._h, self._lin(weights["embed"]))
+        _lib.orc_model_set_lm_head(self._h, self._lin(weights["lm_head"]))
+        _lib.orc_model_set_final_norm(self._h, _p(self._hold(weights["final_norm"])))
+        for l in range(cfg["n_layers"]):
+            for wi, nm in enumerate(LIN_NAMES):
+                _lib.orc_model_set_linear(self._h, l, wi, self._lin(weights["layers.%d.%s" % (l, nm)]))
+            _lib.orc_model_set_norm(self._h, l, 0, _p(self._hold(weights["layers.%d.norm1" % l])))
+            _lib.orc_model_set_norm(self._h, l, 1, _p(self._hold(weights["layers.%d.norm2" % l])))
+
+    def _hold(self, a):
+        a = np.ascontiguousarray(a)
+        self._keep.append(a)
+        return a
+
+    def _lin(self, w):
+        if isinstance(w, tuple):
+            q, s = self._hold(w[0]), self._hold(w[1])
+            assert q.dtype == np.int8
+            return Linear(q.ctypes.data, s.ctypes.data, None)
+        a = self._hold(w)
+        return Linear(None, None, a.ctypes.data)
+
+    def close(self):
+        if self._h:
+            _lib.orc_model_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        self.close()
+
+    def reset(self):
+        _lib.orc_model_reset(self._h)
+
+    @property
+    def past_len(self):
+        return _lib.orc_model_past_len(self._h)
+
+    @past_len.setter
+    def past_len(self, v):
+        _lib.orc_model_set_past_len(self._h, int(v))
+
+    def forward(self, ids, positions, past_len, active, is_causal):
+        ids = _c(np.asarray(ids, np.int64))
+        positions = _c(np.asarray(positions, np.int64))
+        S = ids.size
+        logits = np.empty((S, self.cfg.vocab), np_dtype(self.dt))
+        _lib.orc_model_forward(self._h, _p(ids), _p(positions), S, int(past_len), int(active),
+                               int(is_causal), _p(logits))
+        return logits
+
+    def decode_step(self, token):
+        return int(_lib.orc_model_decode_step(self._h, int(token)))
+
+    def prefill(self, ids, prefill_len):
+        ids = _c(np.asarray(ids, np.int64))
+        return int(_lib.orc_model_prefill(self._h, _p(ids), ids.size, prefill_len))
+
+    def generate(self, prompt, max_new, prefill_len=0, eos=-1):
+        prompt = _c(np.asarray(prompt, np.int64))
+        out = np.empty((max(max_new, 1),), np.int64)
+        n = _lib.orc_model_generate(self._h, _p(prompt), prompt.size, max_new, prefill_len, eos, _p(out))
+        if n < 0:
+            raise ValueError("PromptTooLong")
+        return [int(t) for t in out[:n]]
+
+    def kv_cache(self, layer):
+        n = self.cfg.n_kv_heads * self.cfg.max_seq * self.cfg.head_dim
+        shape = (self.cfg.n_kv_heads, self.cfg.max_seq, self.cfg.head_dim)
+        kp = _lib.orc_model_k_cache(self._h, layer)
+        vp = _lib.orc_model_v_cache(self._h, layer)
+        typ = C.c_float if self.dt == F32 else C.c_uint16
+        k = np.ctypeslib.as_array(C.cast(kp, C.POINTER(typ)), (n,)).reshape(shape).copy()
+        v = np.ctypeslib.as_array(C.cast(vp, C.POINTER(typ)), (n,)).reshape(shape).copy()
+        return k, v

@@ -1,0 +1,76 @@
+"""Whole-decoder pins for the oracle: the reference's exact greedy ids on its tiny random Llama
+(crates/llm/tests/tinyllama_random.rs:20-24) and the generate-loop bookkeeping."""
+import numpy as np
+import pytest
+
+import oracle as orc
+import llm_weights
+
+
+@pytest.mark.parametrize("dt", [orc.F32, orc.BF16, orc.F16])
+def test_tiny_llama_random_golden_ids(dt):
+    cfg, w, golden = llm_weights.tiny_llama_random(dt, max_seq=golden_max_seq())
+    m = orc.Model(cfg, w)
+    ids = m.generate(golden["prompt_ids"], len(golden["expected_new_ids"]))
+    assert ids == golden["expected_new_ids"]
+    # every prompt token and every generated token but the last is fed through one decode step
+    # (crates/llm/tests/mock_decode.rs:44-52: 3 prompt ids + 5 new -> past_len 7)
+    assert m.past_len == len(golden["prompt_ids"]) + len(ids) - 1
+    m.close()
+
+
+def golden_max_seq():
+    return 4 + 28  # STREAM_SINK + STREAM_WINDOW of the reference test
+
+
+@pytest.mark.parametrize("lanes", [1, 4, 64])
+def test_tiny_llama_random_ids_do_not_depend_on_summation_order(lanes):
+    orc.set_lanes(lanes)
+    try:
+        cfg, w, golden = llm_weights.tiny_llama_random(orc.BF16)
+        m = orc.Model(cfg, w)
+        assert m.generate(golden["prompt_ids"], 8) == golden["expected_new_ids"]
+    finally:
+        orc.set_lanes(16)
+
+
+def test_prefill_matches_decode_only():
+    """crates/llm/tests/tinyllama_random.rs cpu_multi_turn_prefill_matches_decode_only: a chunked,
+    zero-padded prefill gives the same ids as feeding the prompt token by token."""
+    cfg, w, golden = llm_weights.tiny_llama_random(orc.F32)
+    prompt = [15043, 29892, 590, 1024, 338, 29871, 13, 450, 4996, 17354, 1701]
+    a = orc.Model(cfg, w)
+    ids_decode = a.generate(prompt, 6)
+    b = orc.Model(cfg, w)
+    ids_prefill = b.generate(prompt, 6, prefill_len=4)
+    assert ids_decode == ids_prefill
+    assert a.past_len == b.past_len == len(prompt) + 6 - 1
+    # second turn on top of the kept KV cache
+    assert a.generate([3038, 25190], 3) == b.generate([3038, 25190], 3, prefill_len=4)
+
+
+def test_prompt_too_long_and_max_seq_stop():
+    cfg, w, _ = llm_weights.tiny_llama_random(orc.F32, max_seq=8)
+    m = orc.Model(cfg, w)
+    with pytest.raises(ValueError):
+        m.generate(list(range(9)), 1)
+    with pytest.raises(ValueError):  # 5 tokens padded to 2 chunks of 4 = 8 fits, 9 padded to 12 does not
+        m.generate(list(range(9)), 1, prefill_len=4)
+    m.reset()
+    ids = m.generate([1, 2, 3, 4, 5], 10)  # stops when past_len reaches max_seq
+    assert m.past_len == 8 and len(ids) == 4, (m.past_len, ids)
+    assert m.generate([], 5) == []
+
+
+def test_forward_rows_are_causal():
+    """Row s of a prefill run only sees tokens <= s: logits of a prefix do not change when the
+    suffix does."""
+    cfg, w, _ = llm_weights.tiny_llama_random(orc.F32)
+    m = orc.Model(cfg, w)
+    ids = np.array([5, 77, 3001, 12, 9], np.int64)
+    pos = np.arange(5)
+    a = m.forward(ids, pos, 0, 5, True)
+    ids2 = ids.copy()
+    ids2[3:] = [31999, 4]
+    b = m.forward(ids2, pos, 0, 5, True)
+    assert np.array_equal(a[:3], b[:3]) and not np.array_equal(a[3], b[3])
