@@ -1,0 +1,289 @@
+"""MI355X-native quantized-LLM hot path of my-nn-engine: ctypes binding of lib/libmynn_hip.so.
+
+The product is the C-ABI library (include/mynn_hip.h).  This module is plumbing for Python
+callers: it loads the library, checks return codes, and passes torch tensors' device pointers
+and the current HIP stream through.  There is no fallback: when the library is missing, or a
+kernel rejects its arguments, the call raises.
+
+The directory name carries a hyphen, so import it with
+    importlib.import_module("my-nn-engine_amd")
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libmynn_hip.so")
+CSRC = os.path.join(_HERE, "csrc")
+
+F32, BF16, F16 = 0, 1, 2
+
+
+class MynnError(RuntimeError):
+    pass
+
+
+def build(jobs=8):
+    """Compiles every HIP source for gfx950 (hipcc cross-compiles without a GPU)."""
+    import subprocess
+
+    subprocess.check_call(["make", "-C", CSRC, "-j%d" % jobs, "--no-print-directory"])
+    return LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise MynnError("HIP library not built: %s is missing (run __graft_entry__.build())" % LIB_PATH)
+        _lib = C.CDLL(LIB_PATH)
+        _declare(_lib)
+    return _lib
+
+
+_vp, _i, _sz, _f, _i64 = C.c_void_p, C.c_int, C.c_size_t, C.c_float, C.c_int64
+
+
+class ModelConfig(C.Structure):
+    _fields_ = [("n_layers", _i), ("hidden", _i), ("n_heads", _i), ("n_kv_heads", _i), ("head_dim", _i),
+                ("ffn", _i), ("vocab", _i), ("max_seq", _i), ("eps", _f), ("rope_theta", _f), ("dtype", _i),
+                ("seq_q", _i), ("batch", _i)]
+
+
+class KernelTime(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("ms", _f), ("bytes", C.c_double)]
+
+
+STEP_FN = C.CFUNCTYPE(_i64, _vp, _i64, _i64)
+
+# name -> (restype, argtypes): every symbol include/mynn_hip.h declares
+SIGNATURES = {
+    "mynn_last_error": (C.c_char_p, []),
+    "mynn_version": (_i, []),
+    "mynn_device_info": (_i, [C.POINTER(_i), C.POINTER(_i), C.POINTER(_i), C.c_char_p, _sz]),
+    "mynn_dequantize_linear": (_i, [_vp, _vp, _vp, _sz, _sz, _i, _vp]),
+    "mynn_dequant_gemv": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "mynn_dequant_matmul": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "mynn_quantized_matmul": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "mynn_dynamic_quantize_linear": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "mynn_attention": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "mynn_kvcache_update": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
+    "mynn_quantizing_kvcache_update": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
+    "mynn_rms_norm": (_i, [_vp, _vp, _vp, _i, _i, _f, _i, _vp]),
+    "mynn_rope": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "mynn_gather_rows": (_i, [_vp, _vp, _vp, _i, _i, _sz, _vp]),
+    "mynn_swiglu": (_i, [_vp, _vp, _vp, _sz, _i, _vp]),
+    "mynn_add": (_i, [_vp, _vp, _vp, _sz, _i, _vp]),
+    "mynn_argmax_last": (_i, [_vp, _vp, _i, _i, _vp]),
+    "mynn_model_configure": (_i, [C.POINTER(ModelConfig)]),
+    "model_init": (_vp, [C.POINTER(_vp), C.POINTER(_vp)]),
+    "model": (None, [_vp, C.POINTER(_vp), C.POINTER(_vp)]),
+    "model_destroy": (None, [_vp]),
+    "model_device_sync": (None, []),
+    "model_memcpy": (_i, [_vp, _vp, _sz, _i]),
+    "alloc_pinned": (_vp, [_sz]),
+    "free_pinned": (None, [_vp]),
+    "mynn_model_step": (_i, [_vp, _vp, _vp, _i64, _i64, _vp, _vp]),
+    "mynn_model_logits_device": (_vp, [_vp]),
+    "mynn_model_stats": (_i, [_vp, C.POINTER(_sz), C.POINTER(_i), C.POINTER(_i)]),
+    "mynn_model_decode_loop": (_i, [_vp, C.c_int32, _i64, _i, _vp]),
+    "mynn_model_profile_step": (_i, [_vp, C.c_int32, _i64, C.POINTER(KernelTime), _i]),
+    "mynn_quantize_per_channel": (_i, [_vp, _vp, _vp, _sz, _sz, _i]),
+    "mynn_rope_table": (_i, [_vp, _vp, _i, _i, _f, _i]),
+    "mynn_llm_create": (_vp, [_vp, _vp, _i, _i, _i64]),
+    "mynn_llm_destroy": (None, [_vp]),
+    "mynn_llm_reset": (None, [_vp]),
+    "mynn_llm_past_len": (_i64, [_vp]),
+    "mynn_llm_set_past_len": (None, [_vp, _i64]),
+    "mynn_llm_generate_ids": (_i, [_vp, _vp, _sz, _sz, _vp]),
+    "mynn_llm_create_with_step": (_vp, [STEP_FN, _vp, _i, _i64]),
+}
+
+
+def missing_symbols():
+    """Names declared in include/mynn_hip.h that the loaded library does not export."""
+    l = lib()
+    return [n for n in SIGNATURES if not hasattr(l, n)]
+
+
+def _declare(l):
+    for name, (res, args) in SIGNATURES.items():
+        try:
+            fn = getattr(l, name)
+        except AttributeError:
+            continue  # reported by missing_symbols(); calling it raises AttributeError
+        fn.restype = res
+        fn.argtypes = args
+
+
+def check(rc):
+    if rc != 0:
+        raise MynnError("mynn error %d: %s" % (rc, lib().mynn_last_error().decode()))
+
+
+# ------------------------------------------------------------------ torch plumbing
+def _dt(t):
+    import torch
+
+    return {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}[t.dtype]
+
+
+def _stream():
+    import torch
+
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    assert t.is_cuda and t.is_contiguous(), "device-resident contiguous tensors only"
+    return t.data_ptr()
+
+
+def device_info():
+    cu, wave, lds = _i(), _i(), _i()
+    arch = C.create_string_buffer(64)
+    check(lib().mynn_device_info(C.byref(cu), C.byref(wave), C.byref(lds), arch, 64))
+    return {"cu_count": cu.value, "wave_size": wave.value, "lds_bytes": lds.value, "arch": arch.value.decode()}
+
+
+def dequantize_linear(x_i8, scale):
+    import torch
+
+    out = torch.empty(x_i8.shape, dtype=scale.dtype, device=x_i8.device)
+    rows = x_i8.shape[0]
+    check(lib().mynn_dequantize_linear(_ptr(out), _ptr(x_i8), _ptr(scale), rows, x_i8.numel() // rows, _dt(scale),
+                                       _stream()))
+    return out
+
+
+def dequant_gemv(act, wq, scale):
+    import torch
+
+    N, K = wq.shape
+    out = torch.empty((N,), dtype=scale.dtype, device=wq.device)
+    check(lib().mynn_dequant_gemv(_ptr(out), _ptr(act), _ptr(wq), _ptr(scale), N, K, _dt(act), _dt(scale), _stream()))
+    return out
+
+
+def dequant_matmul(act, wq, scale):
+    import torch
+
+    N, K = wq.shape
+    M = act.numel() // K
+    out = torch.empty(tuple(act.shape[:-1]) + (N,), dtype=scale.dtype, device=wq.device)
+    check(lib().mynn_dequant_matmul(_ptr(out), _ptr(act), _ptr(wq), _ptr(scale), M, N, K, _dt(act), _dt(scale),
+                                    _stream()))
+    return out
+
+
+def quantized_matmul(lhs, lhs_scale, rhs, rhs_scale, want_acc=True):
+    import torch
+
+    M, K = lhs.shape
+    N = rhs.shape[0]
+    out = torch.empty((M, N), dtype=rhs_scale.dtype, device=lhs.device)
+    acc = torch.empty((M, N), dtype=torch.int32, device=lhs.device) if want_acc else None
+    check(lib().mynn_quantized_matmul(_ptr(out), _ptr(acc), _ptr(lhs), _ptr(lhs_scale), _ptr(rhs), _ptr(rhs_scale),
+                                      M, N, K, _dt(rhs_scale), _stream()))
+    return out, acc
+
+
+def dynamic_quantize_linear(x, symmetric=True):
+    import torch
+
+    rows = x.shape[0]
+    inner = x.numel() // rows
+    y = torch.empty(x.shape, dtype=torch.int8 if symmetric else torch.uint8, device=x.device)
+    s = torch.empty((rows,), dtype=x.dtype, device=x.device)
+    zp = torch.empty((rows,), dtype=y.dtype, device=x.device)
+    check(lib().mynn_dynamic_quantize_linear(_ptr(y), _ptr(s), _ptr(zp), _ptr(x), rows, inner, _dt(x),
+                                             int(symmetric), _stream()))
+    return y, s, zp
+
+
+def attention(q, k, v, scale, is_causal=False, active=None, d_active=None, q_pos_offset=None, k_scale=None,
+              v_scale=None):
+    import torch
+
+    B, Hq, Sq, D = q.shape
+    Hkv, cache_len = k.shape[1], k.shape[2]
+    if active is None:
+        active = cache_len
+    if q_pos_offset is None:
+        q_pos_offset = 0 if Sq == cache_len else active - Sq
+    out = torch.empty_like(q)
+    check(lib().mynn_attention(_ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(k_scale), _ptr(v_scale), float(scale),
+                               int(is_causal), B, Sq, int(active), _ptr(d_active), cache_len, int(q_pos_offset),
+                               Hq, Hkv, D, _dt(q), int(k.dtype == torch.int8), _stream()))
+    return out
+
+
+def kvcache_update(cache, new_kv, offset):
+    B, H, max_seq, D = cache.shape
+    check(lib().mynn_kvcache_update(_ptr(cache), _ptr(new_kv), int(offset), B * H, new_kv.shape[2], max_seq, D,
+                                    _dt(cache), _stream()))
+    return cache
+
+
+def quantizing_kvcache_update(cache, scale, new_kv, offset):
+    B, H, max_seq, D = cache.shape
+    check(lib().mynn_quantizing_kvcache_update(_ptr(cache), _ptr(scale), _ptr(new_kv), int(offset), B * H,
+                                               new_kv.shape[2], max_seq, D, _dt(new_kv), _stream()))
+    return cache, scale
+
+
+def rms_norm(x, w, eps):
+    import torch
+
+    out = torch.empty_like(x)
+    dim = x.shape[-1]
+    check(lib().mynn_rms_norm(_ptr(out), _ptr(x), _ptr(w), x.numel() // dim, dim, float(eps), _dt(x), _stream()))
+    return out
+
+
+def rope(x, cos_t, sin_t, position):
+    import torch
+
+    out = torch.empty_like(x)
+    S, D = x.shape[-2], x.shape[-1]
+    check(lib().mynn_rope(_ptr(out), _ptr(x), _ptr(cos_t), _ptr(sin_t), _ptr(position), x.numel() // (S * D), S, D,
+                          _dt(x), _stream()))
+    return out
+
+
+def gather_rows(data, idx):
+    import torch
+
+    rows = data.shape[0]
+    row_bytes = data.numel() // rows * data.element_size()
+    out = torch.empty(tuple(idx.shape) + tuple(data.shape[1:]), dtype=data.dtype, device=data.device)
+    check(lib().mynn_gather_rows(_ptr(out), _ptr(data), _ptr(idx), idx.numel(), rows, row_bytes, _stream()))
+    return out
+
+
+def swiglu(gate, up):
+    import torch
+
+    out = torch.empty_like(gate)
+    check(lib().mynn_swiglu(_ptr(out), _ptr(gate), _ptr(up), gate.numel(), _dt(gate), _stream()))
+    return out
+
+
+def add(a, b):
+    import torch
+
+    out = torch.empty_like(a)
+    check(lib().mynn_add(_ptr(out), _ptr(a), _ptr(b), a.numel(), _dt(a), _stream()))
+    return out
+
+
+def argmax_last(logits):
+    import torch
+
+    out = torch.empty((1,), dtype=torch.int32, device=logits.device)
+    check(lib().mynn_argmax_last(_ptr(out), _ptr(logits), logits.numel(), _dt(logits), _stream()))
+    return out

@@ -1,0 +1,290 @@
+// Int8 weight-dequant GEMV for gfx950 (wave64): out[m,n] = T(scale[n] * sum_k act[m,k] * wq[n,k]).
+//
+// Replaces the reference's dequant_gemv.cuh:12-59 (one 32-lane warp per row) and
+// dequant_matmul.cuh:12-51 (the scale-after-sum fallback for 1 < M < 16).
+//
+// Shape of the kernel: the weight matrix [N,K] int8 is streamed exactly once with 128-bit
+// loads (16 weights per lane per load); the activation row(s) are staged once per workgroup in
+// LDS as f32; each wave owns R consecutive rows so R independent 16-byte loads per lane are in
+// flight before the first FMA; dequantisation is an in-register int8->f32 convert; the f32
+// partial sums are combined with a wave64 xor butterfly; the scale is applied after the sum, as
+// the reference does.  Optional fused prologue/epilogues keep the decoder at five launches per
+// layer:
+//   NORM      RMSNorm of the activation row computed while it is staged (rms_norm.cuh:9-59
+//             semantics: y = (x * (1/sqrt(mean(x^2)+eps))) * w, rounded to T like the stored tensor)
+//   RESIDUAL  out = T(T(acc*scale) + residual[n])            (the Add that follows o/down proj)
+//   SWIGLU    rows interleaved gate,up: out[i] = T(silu(T(g)) * T(u))  (Swish+Mul group)
+#include "mynn_common.h"
+
+namespace mynn {
+
+enum { EPI_PLAIN = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
+
+struct GemvParams {
+    void *out;
+    const void *act;       // [MB, K]
+    const int8_t *wq;      // [N, K]
+    const void *scale;     // [N]
+    const void *residual;  // [MB, N_out] (EPI_RESIDUAL)
+    const void *norm_w;    // [K] (NORM)
+    float eps;
+    int N, K;
+    int act_stride;        // elements between activation rows
+    int out_stride;        // elements between output rows
+};
+
+constexpr int kGemvWaves = 4;
+constexpr int kGemvThreads = kGemvWaves * kWave;
+
+template <typename TA, typename TO, int R, int MB, int EPI, bool NORM>
+__global__ __launch_bounds__(kGemvThreads) void dequant_gemv_kernel(GemvParams p) {
+    extern __shared__ float act_lds[];  // [MB][K]
+    __shared__ float red[kGemvWaves];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int K = p.K, N = p.N;
+    const TA *act = (const TA *)p.act;
+
+    // ---- stage the activation row(s) in LDS as f32 (with the RMSNorm prologue when asked)
+    if constexpr (NORM) {
+        static_assert(!NORM || MB == 1, "norm prologue is a decode (one row) feature");
+        float ss = 0.f;
+        for (int k = tid; k < K; k += kGemvThreads) {
+            float v = Elem<TA>::ld(act, k);
+            act_lds[k] = v;
+            ss += v * v;
+        }
+        ss = wave_sum(ss);
+        if (lane == 0) red[wave] = ss;
+        __syncthreads();
+        float tot = 0.f;
+#pragma unroll
+        for (int w = 0; w < kGemvWaves; w++) tot += red[w];
+        const float inv = 1.0f / sqrtf(tot / (float)K + p.eps);
+        const TA *nw = (const TA *)p.norm_w;
+        for (int k = tid; k < K; k += kGemvThreads)
+            act_lds[k] = Elem<TA>::rnd((act_lds[k] * inv) * Elem<TA>::ld(nw, k));
+    } else {
+#pragma unroll
+        for (int m = 0; m < MB; m++)
+            for (int k = tid; k < K; k += kGemvThreads)
+                act_lds[m * K + k] = Elem<TA>::ld(act, (size_t)m * p.act_stride + k);
+    }
+    __syncthreads();
+
+    // ---- each wave: R rows
+    const int row0 = (blockIdx.x * kGemvWaves + wave) * R;
+    if (row0 >= N) return;
+    const U4 *wrow[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        int row = row0 + r < N ? row0 + r : N - 1;
+        wrow[r] = (const U4 *)(p.wq + (size_t)row * K);
+    }
+    float acc[R][MB];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int m = 0; m < MB; m++) acc[r][m] = 0.f;
+
+    const int nchunks = K >> 4;
+    for (int c = lane; c < nchunks; c += kWave) {
+        U4 w[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) w[r] = __builtin_nontemporal_load(&wrow[r][c]);
+        float a[MB][16];
+#pragma unroll
+        for (int m = 0; m < MB; m++) {
+            const float4 *ap = (const float4 *)(act_lds + m * K + c * 16);
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                float4 t = ap[q];
+                a[m][4 * q] = t.x; a[m][4 * q + 1] = t.y; a[m][4 * q + 2] = t.z; a[m][4 * q + 3] = t.w;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            float wf[16];
+            widen16_i8(w[r], wf);
+#pragma unroll
+            for (int m = 0; m < MB; m++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) acc[r][m] = fmaf(a[m][i], wf[i], acc[r][m]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int m = 0; m < MB; m++) acc[r][m] = wave_sum(acc[r][m]);
+
+    // ---- epilogue: lane r finishes row r
+    const TO *scale = (const TO *)p.scale;
+    TO *out = (TO *)p.out;
+    if constexpr (EPI == EPI_SWIGLU) {
+        static_assert(EPI != EPI_SWIGLU || (R % 2 == 0), "gate/up rows come in pairs");
+#pragma unroll
+        for (int r = 0; r < R; r += 2) {
+            if (lane == r && row0 + r + 1 < N) {
+#pragma unroll
+                for (int m = 0; m < MB; m++) {
+                    float g = Elem<TO>::rnd(acc[r][m] * Elem<TO>::ld(scale, row0 + r));
+                    float u = Elem<TO>::rnd(acc[r + 1][m] * Elem<TO>::ld(scale, row0 + r + 1));
+                    float sig = 1.0f / (1.0f + expf(-g));
+                    Elem<TO>::st(out, (size_t)m * p.out_stride + ((row0 + r) >> 1), (g * sig) * u);
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            if (lane == r && row0 + r < N) {
+#pragma unroll
+                for (int m = 0; m < MB; m++) {
+                    float y = acc[r][m] * Elem<TO>::ld(scale, row0 + r);
+                    size_t o = (size_t)m * p.out_stride + row0 + r;
+                    if constexpr (EPI == EPI_RESIDUAL)
+                        y = Elem<TO>::rnd(y) + Elem<TO>::ld((const TO *)p.residual, o);
+                    Elem<TO>::st(out, o, y);
+                }
+            }
+        }
+    }
+}
+
+template <typename TA, typename TO, int R, int MB, int EPI, bool NORM>
+static int launch_gemv(const GemvParams &p, hipStream_t s) {
+    const int rows_per_block = kGemvWaves * R;
+    dim3 grid((p.N + rows_per_block - 1) / rows_per_block);
+    size_t lds = (size_t)MB * p.K * sizeof(float);
+    hipLaunchKernelGGL((dequant_gemv_kernel<TA, TO, R, MB, EPI, NORM>), grid, dim3(kGemvThreads), lds, s, p);
+    return launch_status("dequant_gemv_kernel");
+}
+
+static int check_gemv(const GemvParams &p, int mb) {
+    MYNN_REQUIRE(p.out && p.act && p.wq && p.scale, MYNN_ERR_INVALID, "dequant_gemv: null operand");
+    MYNN_REQUIRE(p.N > 0 && p.K > 0, MYNN_ERR_INVALID, "dequant_gemv: N=%d K=%d", p.N, p.K);
+    MYNN_REQUIRE(p.K % 16 == 0, MYNN_ERR_UNSUPPORTED, "dequant_gemv: K=%d is not a multiple of 16", p.K);
+    MYNN_REQUIRE(aligned16(p.wq), MYNN_ERR_INVALID, "dequant_gemv: wq must be 16-byte aligned");
+    MYNN_REQUIRE((size_t)mb * p.K * sizeof(float) <= 64 * 1024, MYNN_ERR_UNSUPPORTED,
+                 "dequant_gemv: %d x K=%d activations do not fit the 64 KiB LDS stage", mb, p.K);
+    return 0;
+}
+
+// Picks rows-per-wave so that small matrices still spread over the chip: 4 rows per wave when
+// that leaves at least ~2 workgroups per CU, else 2.
+static int pick_r(int N) { return N >= 256 * 2 * kGemvWaves * 4 ? 4 : 2; }
+
+template <typename TA, typename TO, int MB>
+static int gemv_plain(const GemvParams &p, hipStream_t s) {
+    if (pick_r(p.N) == 4) return launch_gemv<TA, TO, 4, MB, EPI_PLAIN, false>(p, s);
+    return launch_gemv<TA, TO, 2, MB, EPI_PLAIN, false>(p, s);
+}
+
+// out [M,N]; M in 1..15 handled in row tiles of at most 4 activation rows
+template <typename TA, typename TO>
+static int gemv_small_m(GemvParams p, int M, hipStream_t s) {
+    const TA *act = (const TA *)p.act;
+    TO *out = (TO *)p.out;
+    int m = 0;
+    while (m < M) {
+        int mb = M - m >= 4 ? 4 : (M - m >= 2 ? 2 : 1);
+        GemvParams q = p;
+        q.act = act + (size_t)m * p.act_stride;
+        q.out = out + (size_t)m * p.out_stride;
+        int rc = check_gemv(q, mb);
+        if (rc) return rc;
+        rc = mb == 4 ? gemv_plain<TA, TO, 4>(q, s) : mb == 2 ? gemv_plain<TA, TO, 2>(q, s) : gemv_plain<TA, TO, 1>(q, s);
+        if (rc) return rc;
+        m += mb;
+    }
+    return 0;
+}
+
+// Fallback for shapes the streaming kernel does not take (K not a multiple of 16, unaligned
+// weights): one wave per output element, scalar loads -- the reference's dequant_matmul.cuh:12-51.
+template <typename TA, typename TO>
+__global__ __launch_bounds__(64) void dequant_matmul_naive_kernel(TO *out, const TA *act, const int8_t *wq,
+                                                                 const TO *scale, int N, int K) {
+    const int n = blockIdx.x, m = blockIdx.y, lane = threadIdx.x;
+    float acc = 0.f;
+    for (int k = lane; k < K; k += 64) acc = fmaf(Elem<TA>::ld(act, (size_t)m * K + k), (float)wq[(size_t)n * K + k], acc);
+    acc = wave_sum(acc);
+    if (lane == 0) Elem<TO>::st(out, (size_t)m * N + n, acc * Elem<TO>::ld(scale, n));
+}
+
+// scale-after-sum path for any act/out type pair the reference allows (f32 or 16-bit act;
+// out type = scale type)
+int dequant_gemv_dispatch(void *out, const void *act, const int8_t *wq, const void *scale, int M, int N,
+                          int K, int act_dtype, int out_dtype, hipStream_t s) {
+    GemvParams p{};
+    p.out = out; p.act = act; p.wq = wq; p.scale = scale; p.N = N; p.K = K; p.act_stride = K; p.out_stride = N;
+    MYNN_REQUIRE(M >= 1, MYNN_ERR_INVALID, "dequant_gemv: M=%d", M);
+    MYNN_REQUIRE(out && act && wq && scale && N > 0 && K > 0, MYNN_ERR_INVALID, "dequant_matmul: bad operand");
+    MYNN_REQUIRE(dtype_ok(act_dtype) && dtype_ok(out_dtype), MYNN_ERR_INVALID, "dequant_matmul: dtype");
+    const bool streaming = K % 16 == 0 && aligned16(wq) && M < 16 &&
+                           (size_t)(M < 4 ? M : 4) * K * sizeof(float) <= 64 * 1024;
+    return dispatch_dtype(act_dtype, [&](auto *ta) {
+        using TA = std::remove_pointer_t<decltype(ta)>;
+        return dispatch_dtype(out_dtype, [&](auto *to) {
+            using TO = std::remove_pointer_t<decltype(to)>;
+            if (streaming) return gemv_small_m<TA, TO>(p, M, s);
+            MYNN_REQUIRE(M <= 65535, MYNN_ERR_UNSUPPORTED, "dequant_matmul: M=%d too large for the plain kernel", M);
+            hipLaunchKernelGGL((dequant_matmul_naive_kernel<TA, TO>), dim3(N, M), dim3(64), 0, s, (TO *)out,
+                               (const TA *)act, wq, (const TO *)scale, N, K);
+            return launch_status("dequant_matmul_naive_kernel");
+        });
+    });
+}
+
+// ---- fused decode variants used by the decoder executor (one activation row, T in == T out)
+template <typename T>
+int gemv_norm(void *out, const void *x, const void *norm_w, float eps, const int8_t *wq, const void *scale,
+              int N, int K, hipStream_t s) {
+    GemvParams p{};
+    p.out = out; p.act = x; p.wq = wq; p.scale = scale; p.norm_w = norm_w; p.eps = eps; p.N = N; p.K = K;
+    p.act_stride = K; p.out_stride = N;
+    int rc = check_gemv(p, 1);
+    if (rc) return rc;
+    if (pick_r(N) == 4) return launch_gemv<T, T, 4, 1, EPI_PLAIN, true>(p, s);
+    return launch_gemv<T, T, 2, 1, EPI_PLAIN, true>(p, s);
+}
+template <typename T>
+int gemv_residual(void *out, const void *act, const int8_t *wq, const void *scale, const void *residual,
+                  int N, int K, hipStream_t s) {
+    GemvParams p{};
+    p.out = out; p.act = act; p.wq = wq; p.scale = scale; p.residual = residual; p.N = N; p.K = K;
+    p.act_stride = K; p.out_stride = N;
+    int rc = check_gemv(p, 1);
+    if (rc) return rc;
+    if (pick_r(N) == 4) return launch_gemv<T, T, 4, 1, EPI_RESIDUAL, false>(p, s);
+    return launch_gemv<T, T, 2, 1, EPI_RESIDUAL, false>(p, s);
+}
+// wq/scale hold gate and up rows interleaved (row 2i = gate_i, row 2i+1 = up_i); N = 2*ffn
+template <typename T>
+int gemv_norm_swiglu(void *out, const void *x, const void *norm_w, float eps, const int8_t *wq,
+                     const void *scale, int N, int K, hipStream_t s) {
+    GemvParams p{};
+    p.out = out; p.act = x; p.wq = wq; p.scale = scale; p.norm_w = norm_w; p.eps = eps; p.N = N; p.K = K;
+    p.act_stride = K; p.out_stride = N / 2;
+    MYNN_REQUIRE(N % 2 == 0, MYNN_ERR_INVALID, "gate/up rows must come in pairs (N=%d)", N);
+    int rc = check_gemv(p, 1);
+    if (rc) return rc;
+    if (pick_r(N) == 4) return launch_gemv<T, T, 4, 1, EPI_SWIGLU, true>(p, s);
+    return launch_gemv<T, T, 2, 1, EPI_SWIGLU, true>(p, s);
+}
+
+template int gemv_norm<bf16_t>(void *, const void *, const void *, float, const int8_t *, const void *, int, int, hipStream_t);
+template int gemv_norm<f16_t>(void *, const void *, const void *, float, const int8_t *, const void *, int, int, hipStream_t);
+template int gemv_residual<bf16_t>(void *, const void *, const int8_t *, const void *, const void *, int, int, hipStream_t);
+template int gemv_residual<f16_t>(void *, const void *, const int8_t *, const void *, const void *, int, int, hipStream_t);
+template int gemv_norm_swiglu<bf16_t>(void *, const void *, const void *, float, const int8_t *, const void *, int, int, hipStream_t);
+template int gemv_norm_swiglu<f16_t>(void *, const void *, const void *, float, const int8_t *, const void *, int, int, hipStream_t);
+
+}  // namespace mynn
+
+extern "C" int mynn_dequant_gemv(void *out, const void *act, const int8_t *wq, const void *scale, int N, int K,
+                                 int act_dtype, int out_dtype, mynn_stream s) {
+    MYNN_REQUIRE(K > 0 && K % 16 == 0, MYNN_ERR_UNSUPPORTED, "dequant_gemv: K=%d is not a multiple of 16", K);
+    MYNN_REQUIRE(mynn::aligned16(wq), MYNN_ERR_INVALID, "dequant_gemv: wq must be 16-byte aligned");
+    MYNN_REQUIRE((size_t)K * sizeof(float) <= 64 * 1024, MYNN_ERR_UNSUPPORTED, "dequant_gemv: K=%d exceeds the LDS stage", K);
+    return mynn::dequant_gemv_dispatch(out, act, wq, scale, 1, N, K, act_dtype, out_dtype, mynn::as_stream(s));
+}

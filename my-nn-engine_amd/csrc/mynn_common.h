@@ -1,0 +1,146 @@
+// Shared device/host helpers for the gfx950 kernel library: storage types, conversions with the
+// rounding the reference uses, wave64 reductions, launch-error plumbing.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/mynn_hip.h"
+
+namespace mynn {
+
+constexpr int kWave = 64;
+
+// ---- storage types -------------------------------------------------------------------------
+struct bf16_t { uint16_t bits; };
+using f16_t = _Float16;
+
+// f32 -> bf16, round to nearest even: (bits + 0x7fff + lsb) >> 16, NaN -> 0x7FC0
+// (reference: src/codegen/cpu/kernels/ftype.rs:41-50, crates/llm/src/quantize.rs:74-81)
+__host__ __device__ inline uint16_t f32_to_bf16_bits(float x) {
+    uint32_t u = __builtin_bit_cast(uint32_t, x);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return 0x7FC0;
+    return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+__host__ __device__ inline float bf16_bits_to_f32(uint16_t b) {
+    return __builtin_bit_cast(float, (uint32_t)b << 16);
+}
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+    static constexpr int code = MYNN_F32;
+    __host__ __device__ static float ld(const float *p, size_t i) { return p[i]; }
+    __host__ __device__ static void st(float *p, size_t i, float v) { p[i] = v; }
+    __host__ __device__ static float rnd(float v) { return v; }
+};
+template <> struct Elem<bf16_t> {
+    static constexpr int code = MYNN_BF16;
+    __host__ __device__ static float ld(const bf16_t *p, size_t i) { return bf16_bits_to_f32(p[i].bits); }
+    __host__ __device__ static void st(bf16_t *p, size_t i, float v) { p[i].bits = f32_to_bf16_bits(v); }
+    __host__ __device__ static float rnd(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
+};
+template <> struct Elem<f16_t> {
+    static constexpr int code = MYNN_F16;
+    __host__ __device__ static float ld(const f16_t *p, size_t i) { return (float)p[i]; }
+    __host__ __device__ static void st(f16_t *p, size_t i, float v) { p[i] = (f16_t)v; }  // RNE
+    __host__ __device__ static float rnd(float v) { return (float)(f16_t)v; }
+};
+
+inline size_t dtype_size(int dt) { return dt == MYNN_F32 ? 4 : 2; }
+inline bool dtype_ok(int dt) { return dt == MYNN_F32 || dt == MYNN_BF16 || dt == MYNN_F16; }
+
+// 8 consecutive 16-bit elements (one 128-bit load) widened to f32
+typedef uint32_t U4 __attribute__((ext_vector_type(4)));
+
+template <typename T> __device__ inline void widen8(const U4 &v, float *f);
+template <> __device__ inline void widen8<bf16_t>(const U4 &v, float *f) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        f[2 * i] = __builtin_bit_cast(float, w[i] << 16);
+        f[2 * i + 1] = __builtin_bit_cast(float, w[i] & 0xFFFF0000u);
+    }
+}
+template <> __device__ inline void widen8<f16_t>(const U4 &v, float *f) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        f[2 * i] = (float)__builtin_bit_cast(f16_t, (uint16_t)(w[i] & 0xFFFFu));
+        f[2 * i + 1] = (float)__builtin_bit_cast(f16_t, (uint16_t)(w[i] >> 16));
+    }
+}
+
+// 16 int8 (one 128-bit load) widened to f32
+__device__ inline void widen16_i8(const U4 &v, float *f) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        f[4 * i + 0] = (float)(int8_t)(w[i] & 0xFF);
+        f[4 * i + 1] = (float)(int8_t)((w[i] >> 8) & 0xFF);
+        f[4 * i + 2] = (float)(int8_t)((w[i] >> 16) & 0xFF);
+        f[4 * i + 3] = (float)(int8_t)(w[i] >> 24);
+    }
+}
+
+// ---- wave64 reductions ------------------------------------------------------------------------
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+__device__ inline float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+// sum over the lanes of an aligned group of `width` lanes (power of two <= 64)
+template <int width> __device__ inline float group_sum(float v) {
+#pragma unroll
+    for (int off = width / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// exp for softmax / SiLU: one definition for every kernel
+__device__ inline float fast_exp(float x) { return __expf(x); }
+
+// ---- errors ---------------------------------------------------------------------------------
+void set_error(const char *fmt, ...);
+int fail(int code, const char *fmt, ...);
+int hip_fail(hipError_t e, const char *what);
+
+#define MYNN_REQUIRE(cond, code, ...)                 \
+    do {                                              \
+        if (!(cond)) return ::mynn::fail((code), __VA_ARGS__); \
+    } while (0)
+
+#define MYNN_HIP(expr)                                          \
+    do {                                                        \
+        hipError_t e__ = (expr);                                \
+        if (e__ != hipSuccess) return ::mynn::hip_fail(e__, #expr); \
+    } while (0)
+
+inline int launch_status(const char *what) {
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : hip_fail(e, what);
+}
+
+inline hipStream_t as_stream(mynn_stream s) { return (hipStream_t)s; }
+inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+template <typename F> inline int dispatch_dtype(int dt, F &&f) {
+    switch (dt) {
+    case MYNN_F32: return f((float *)nullptr);
+    case MYNN_BF16: return f((bf16_t *)nullptr);
+    case MYNN_F16: return f((f16_t *)nullptr);
+    default: return fail(MYNN_ERR_INVALID, "unknown dtype %d", dt);
+    }
+}
+template <typename F> inline int dispatch_dtype16(int dt, F &&f) {
+    switch (dt) {
+    case MYNN_BF16: return f((bf16_t *)nullptr);
+    case MYNN_F16: return f((f16_t *)nullptr);
+    default: return fail(MYNN_ERR_UNSUPPORTED, "dtype %d: this kernel needs a 16-bit float type", dt);
+    }
+}
+
+}  // namespace mynn

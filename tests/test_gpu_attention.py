@@ -1,0 +1,157 @@
+"""GPU parity of the GQA attention kernels against the oracle, the reference's golden vectors
+and the f64 brute force of the reference's own state test (tests/session_state.rs:122-229)."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle as orc
+import pbreader
+from conftest import GOLDEN, close_either, max_abs_rel
+
+pytestmark = pytest.mark.gpu
+SO = os.path.join(GOLDEN, "single_op")
+
+
+@pytest.fixture(scope="module")
+def g():
+    import gpu_util
+
+    return gpu_util
+
+
+@pytest.mark.parametrize("name,causal,scale,active_slot", [
+    ("attention_decode", False, 8 ** -0.5, None),
+    ("attention_decode_gqa", False, 8 ** -0.5, None),
+    ("attention_decode_runtime_kv", False, 0.5, 3),
+    ("attention_causal", True, 8 ** -0.5, None),
+    ("attention_no_causal", False, 8 ** -0.5, None),
+])
+def test_attention_golden(g, name, causal, scale, active_slot):
+    ins, (o,) = pbreader.read_case(os.path.join(SO, name))
+    q, k, v = ins[0], ins[1], ins[2]
+    active = int(ins[active_slot].array) if active_slot is not None else None
+    got = g.to_host(g.mynn.attention(g.to_dev(q.array), g.to_dev(k.array), g.to_dev(v.array), scale, causal, active))
+    ok, md = close_either(got, o.array, 1e-4)
+    assert ok, md
+
+
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+@pytest.mark.parametrize("B,L", [(1, 512), (4, 2048), (16, 512), (2, 4096), (1, 37), (3, 1)])
+def test_decode_attention_vs_oracle_cfg2_shapes(g, dt, B, L):
+    """GQA decode attention op of the second benchmark config: 32 query heads, 4 KV heads,
+    head_dim 64, softmax scale 1/8, no mask beyond the cache length."""
+    rng = np.random.default_rng(B * 10007 + L)
+    Hq, Hkv, D = 32, 4, 64
+    q = orc.to_storage(rng.standard_normal((B, Hq, 1, D)), dt)
+    k = orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt)
+    v = orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt)
+    want = orc.attention(q, k, v, dt, 0.125)
+    got = g.to_host(g.mynn.attention(g.to_dev(q, dt), g.to_dev(k, dt), g.to_dev(v, dt), 0.125))
+    assert max_abs_rel(g.f32(got, dt), g.f32(want, dt)) <= 1e-2
+    exact = orc.attention_f64(q, k, v, dt, 0.125)
+    assert max_abs_rel(g.f32(got, dt), exact) <= 1e-2
+
+
+@pytest.mark.parametrize("dt", [orc.F32, orc.F16])
+@pytest.mark.parametrize("Hq,Hkv,D", [(8, 8, 128), (32, 8, 128), (4, 2, 8), (6, 3, 32), (4, 1, 16)])
+def test_decode_attention_head_shapes_and_active_length(g, dt, Hq, Hkv, D):
+    import torch
+
+    rng = np.random.default_rng(Hq * 100 + D)
+    B, L, active = 2, 300, 173
+    q = orc.to_storage(rng.standard_normal((B, Hq, 1, D)), dt)
+    k = orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt)
+    v = orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt)
+    want = orc.attention(q, k, v, dt, D ** -0.5, False, active)
+    tol = 1e-4 if dt == orc.F32 else 1e-2
+    got = g.to_host(g.mynn.attention(g.to_dev(q, dt), g.to_dev(k, dt), g.to_dev(v, dt), D ** -0.5, False, active))
+    assert max_abs_rel(g.f32(got, dt), g.f32(want, dt)) <= tol
+    # the same with the active length read on the device (what a captured graph replays)
+    d_active = torch.tensor([active], dtype=torch.int32, device="cuda")
+    got2 = g.to_host(g.mynn.attention(g.to_dev(q, dt), g.to_dev(k, dt), g.to_dev(v, dt), D ** -0.5, False,
+                                      active=L, d_active=d_active))
+    assert max_abs_rel(g.f32(got2, dt), g.f32(want, dt)) <= tol
+    # rows beyond `active` are never read: poison them
+    k2, v2 = k.copy(), v.copy()
+    k2[:, :, active:] = orc.to_storage(np.full((B, Hkv, L - active, D), np.nan), dt)
+    v2[:, :, active:] = orc.to_storage(np.full((B, Hkv, L - active, D), np.nan), dt)
+    got3 = g.to_host(g.mynn.attention(g.to_dev(q, dt), g.to_dev(k2, dt), g.to_dev(v2, dt), D ** -0.5, False, active))
+    assert np.array_equal(got3, got)
+
+
+@pytest.mark.parametrize("dt", [orc.F32, orc.F16, orc.BF16])
+def test_attention_invariants_on_gpu(g, dt):
+    rng = np.random.default_rng(11)
+    B, Hq, Hkv, L, D = 2, 8, 2, 200, 64
+    q = orc.to_storage(rng.standard_normal((B, Hq, 1, D)), dt)
+    k = orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt)
+    v = orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt)
+    dq, dk, dv = g.to_dev(q, dt), g.to_dev(k, dt), g.to_dev(v, dt)
+    # active = 1 -> exactly the first V row of the mapped kv head
+    out1 = g.to_host(g.mynn.attention(dq, dk, dv, 0.125, False, 1))
+    for h in range(Hq):
+        assert np.array_equal(out1[:, h, 0], v[:, h // (Hq // Hkv), 0])
+    # uniform keys -> mean of V
+    ku = np.repeat(k[:, :, :1], L, 2)
+    outu = g.f32(g.to_host(g.mynn.attention(dq, g.to_dev(ku, dt), dv, 0.125)), dt)
+    meanv = np.repeat(g.f32(v, dt).astype(np.float64).mean(2), Hq // Hkv, 1)
+    tol = 1e-5 if dt == orc.F32 else 1e-2
+    assert max_abs_rel(outu[:, :, 0], meanv) <= tol
+    # GQA == MHA with K/V heads repeated
+    kr, vr = np.repeat(k, Hq // Hkv, 1), np.repeat(v, Hq // Hkv, 1)
+    a = g.to_host(g.mynn.attention(dq, dk, dv, 0.125))
+    b = g.to_host(g.mynn.attention(dq, g.to_dev(kr, dt), g.to_dev(vr, dt), 0.125))
+    assert max_abs_rel(g.f32(a, dt), g.f32(b, dt)) <= tol
+
+
+@pytest.mark.parametrize("dt", [orc.F32, orc.F16])
+def test_causal_rows_plain_path(g, dt):
+    """Sq > 1 with a past: row sq sees keys [0, past + sq + 1)."""
+    rng = np.random.default_rng(12)
+    Hq, Hkv, S, D, past, L = 8, 2, 9, 64, 5, 32
+    q = orc.to_storage(rng.standard_normal((1, Hq, S, D)), dt)
+    k = orc.to_storage(rng.standard_normal((1, Hkv, L, D)), dt)
+    v = orc.to_storage(rng.standard_normal((1, Hkv, L, D)), dt)
+    want = orc.attention(q, k, v, dt, 0.125, True, past + S)
+    got = g.to_host(g.mynn.attention(g.to_dev(q, dt), g.to_dev(k, dt), g.to_dev(v, dt), 0.125, True, past + S))
+    assert max_abs_rel(g.f32(got, dt), g.f32(want, dt)) <= (1e-4 if dt == orc.F32 else 1e-2)
+
+
+def test_session_state_three_steps_on_gpu(g):
+    B, H, S_MAX, D = 1, 2, 8, 4
+    kc = g.to_dev(np.zeros((B, H, S_MAX, D), np.float32))
+    vc = g.to_dev(np.zeros((B, H, S_MAX, D), np.float32))
+    kh = np.zeros((B, H, S_MAX, D), np.float32)
+    vh = np.zeros((B, H, S_MAX, D), np.float32)
+
+    def data(step, kind):
+        i = np.arange(B * H * D, dtype=np.float64)
+        return np.clip(np.sin(i * 0.31 + step * 1.7 + kind * 2.4) * 0.5, -1, 1).astype(np.float32).reshape(B, H, 1, D)
+
+    for step in range(3):
+        q, sk, sv = data(step, 0), data(step, 1), data(step, 2)
+        g.mynn.kvcache_update(kc, g.to_dev(sk), step)
+        g.mynn.kvcache_update(vc, g.to_dev(sv), step)
+        kh[:, :, step], vh[:, :, step] = sk[:, :, 0], sv[:, :, 0]
+        got = g.to_host(g.mynn.attention(g.to_dev(q), kc, vc, 1 / np.sqrt(D), False, step + 1))
+        want = orc.attention_f64(q, kh, vh, orc.F32, 1 / np.sqrt(D), False, step + 1)
+        ok, md = close_either(got, want, 1e-4)
+        assert ok, (step, md)
+
+
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+def test_int8_kv_attention(g, dt):
+    rng = np.random.default_rng(13)
+    B, Hq, Hkv, L, D = 2, 32, 4, 257, 64
+    q = orc.to_storage(rng.standard_normal((B, Hq, 1, D)), dt)
+    kc = np.zeros((B, Hkv, L, D), np.int8)
+    vc = np.zeros((B, Hkv, L, D), np.int8)
+    ks = orc.to_storage(np.zeros((B, Hkv, L)), dt)
+    vs = orc.to_storage(np.zeros((B, Hkv, L)), dt)
+    orc.quantizing_kv_cache_update(kc, ks, orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt), 0, dt)
+    orc.quantizing_kv_cache_update(vc, vs, orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt), 0, dt)
+    want = orc.attention(q, kc, vc, dt, 0.125, False, 200, k_scale=ks, v_scale=vs)
+    got = g.to_host(g.mynn.attention(g.to_dev(q, dt), g.to_dev(kc), g.to_dev(vc), 0.125, False, 200,
+                                     k_scale=g.to_dev(ks, dt), v_scale=g.to_dev(vs, dt)))
+    assert max_abs_rel(g.f32(got, dt), g.f32(want, dt)) <= 1e-2
