@@ -38,6 +38,10 @@ def lib():
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise MynnError("HIP library not built: %s is missing (run __graft_entry__.build())" % LIB_PATH)
+        # torch ships its own libamdhip64.so.7; it has to be in the process before this library
+        # so that both share ONE HIP runtime (two runtimes in a process do not both see the GPU)
+        import torch  # noqa: F401
+
         _lib = C.CDLL(LIB_PATH)
         _declare(_lib)
     return _lib

@@ -43,9 +43,10 @@ __device__ inline void merge_state(float &m, float &l, float *o, int n, float m2
 
 template <typename T, int D, int G, bool KVI8>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p) {
-    constexpr int LPK = D / 8;        // lanes per key row
-    constexpr int KPW = 64 / LPK;     // keys per wave pass
-    static_assert(D % 8 == 0 && LPK <= 64 && (LPK & (LPK - 1)) == 0, "head_dim must be 8 * power of two");
+    constexpr int EPL = D >= 8 ? 8 : D;  // elements of a key row per lane
+    constexpr int LPK = D / EPL;         // lanes per key row
+    constexpr int KPW = 64 / LPK;        // keys per wave pass
+    static_assert(D % EPL == 0 && LPK <= 64 && (LPK & (LPK - 1)) == 0, "head_dim must be a power of two");
     __shared__ float sm_o[kAttnWaves][G][D];
     __shared__ float sm_ml[kAttnWaves][G][2];
     __shared__ int sm_last;
@@ -69,48 +70,57 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
     const int k1 = min(bound, k0 + chunk);
 
     const T *Q = (const T *)p.q;
-    float q[G][8];
+    float q[G][EPL];
 #pragma unroll
     for (int g = 0; g < G; g++) {
-        const size_t qo = ((size_t)(b * p.Hq + hkv * G + g) * Sq + sq) * D + dc * 8;
+        const size_t qo = ((size_t)(b * p.Hq + hkv * G + g) * Sq + sq) * D + dc * EPL;
 #pragma unroll
-        for (int i = 0; i < 8; i++) q[g][i] = Elem<T>::ld(Q, qo + i);
+        for (int i = 0; i < EPL; i++) q[g][i] = Elem<T>::ld(Q, qo + i);
     }
-    float m[G], l[G], o[G][8];
+    float m[G], l[G], o[G][EPL];
 #pragma unroll
     for (int g = 0; g < G; g++) {
         m[g] = -INFINITY;
         l[g] = 0.f;
 #pragma unroll
-        for (int i = 0; i < 8; i++) o[g][i] = 0.f;
+        for (int i = 0; i < EPL; i++) o[g][i] = 0.f;
     }
 
     const size_t kv_base = (size_t)bhkv * p.cache_len;
     for (int kk = k0 + wave * KPW + ks; kk < k1; kk += PASS) {
-        float kf[8], vf[8];
+        float kf[EPL], vf[EPL];
         float ksc = 1.f, vsc = 1.f;
+        const size_t ro = (kv_base + kk) * D + dc * EPL;
         if constexpr (KVI8) {
-            const uint2 kr = *(const uint2 *)((const int8_t *)p.k + (kv_base + kk) * D + dc * 8);
-            const uint2 vr = *(const uint2 *)((const int8_t *)p.v + (kv_base + kk) * D + dc * 8);
-            const uint32_t kw[2] = {kr.x, kr.y}, vw[2] = {vr.x, vr.y};
+            if constexpr (EPL == 8) {
+                const uint2 kr = *(const uint2 *)((const int8_t *)p.k + ro);
+                const uint2 vr = *(const uint2 *)((const int8_t *)p.v + ro);
+                const uint32_t kw[2] = {kr.x, kr.y}, vw[2] = {vr.x, vr.y};
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                kf[i] = (float)(int8_t)((kw[i >> 2] >> (8 * (i & 3))) & 0xFF);
-                vf[i] = (float)(int8_t)((vw[i >> 2] >> (8 * (i & 3))) & 0xFF);
+                for (int i = 0; i < 8; i++) {
+                    kf[i] = (float)(int8_t)((kw[i >> 2] >> (8 * (i & 3))) & 0xFF);
+                    vf[i] = (float)(int8_t)((vw[i >> 2] >> (8 * (i & 3))) & 0xFF);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < EPL; i++) {
+                    kf[i] = (float)((const int8_t *)p.k)[ro + i];
+                    vf[i] = (float)((const int8_t *)p.v)[ro + i];
+                }
             }
             ksc = Elem<T>::ld((const T *)p.k_scale, kv_base + kk);
             vsc = Elem<T>::ld((const T *)p.v_scale, kv_base + kk);
         } else {
-            if constexpr (sizeof(T) == 2) {
-                const U4 kr = *(const U4 *)((const T *)p.k + (kv_base + kk) * D + dc * 8);
-                const U4 vr = *(const U4 *)((const T *)p.v + (kv_base + kk) * D + dc * 8);
+            if constexpr (sizeof(T) == 2 && EPL == 8) {
+                const U4 kr = *(const U4 *)((const T *)p.k + ro);
+                const U4 vr = *(const U4 *)((const T *)p.v + ro);
                 widen8<T>(kr, kf);
                 widen8<T>(vr, vf);
             } else {
 #pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    kf[i] = Elem<T>::ld((const T *)p.k, (kv_base + kk) * D + dc * 8 + i);
-                    vf[i] = Elem<T>::ld((const T *)p.v, (kv_base + kk) * D + dc * 8 + i);
+                for (int i = 0; i < EPL; i++) {
+                    kf[i] = Elem<T>::ld((const T *)p.k, ro + i);
+                    vf[i] = Elem<T>::ld((const T *)p.v, ro + i);
                 }
             }
         }
@@ -118,17 +128,17 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
         for (int g = 0; g < G; g++) {
             float part = 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; i++) part = fmaf(q[g][i], kf[i], part);
+            for (int i = 0; i < EPL; i++) part = fmaf(q[g][i], kf[i], part);
             part = group_sum<LPK>(part);
             if constexpr (KVI8) part *= ksc;
             const float s = part * p.scale;
             const float mn = fmaxf(m[g], s);
             const float corr = fast_exp(m[g] - mn);  // exp(-inf) = 0 on the first key
             const float e = fast_exp(s - mn);
-            l[g] = l[g] * corr + e;
+            l[g] = fmaf(l[g], corr, e);
             const float ev = KVI8 ? e * vsc : e;
 #pragma unroll
-            for (int i = 0; i < 8; i++) o[g][i] = o[g][i] * corr + ev * vf[i];
+            for (int i = 0; i < EPL; i++) o[g][i] = fmaf(ev, vf[i], o[g][i] * corr);
             m[g] = mn;
         }
     }
@@ -139,17 +149,17 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
 #pragma unroll
         for (int g = 0; g < G; g++) {
             float m2 = __shfl_xor(m[g], off, 64), l2 = __shfl_xor(l[g], off, 64);
-            float o2[8];
+            float o2[EPL];
 #pragma unroll
-            for (int i = 0; i < 8; i++) o2[i] = __shfl_xor(o[g][i], off, 64);
-            merge_state(m[g], l[g], o[g], 8, m2, l2, o2);
+            for (int i = 0; i < EPL; i++) o2[i] = __shfl_xor(o[g][i], off, 64);
+            merge_state(m[g], l[g], o[g], EPL, m2, l2, o2);
         }
     }
     if (ks == 0) {
 #pragma unroll
         for (int g = 0; g < G; g++) {
 #pragma unroll
-            for (int i = 0; i < 8; i++) sm_o[wave][g][dc * 8 + i] = o[g][i];
+            for (int i = 0; i < EPL; i++) sm_o[wave][g][dc * EPL + i] = o[g][i];
             if (dc == 0) { sm_ml[wave][g][0] = m[g]; sm_ml[wave][g][1] = l[g]; }
         }
     }
@@ -230,12 +240,13 @@ static int launch_g(const AttnParams &p, hipStream_t s) {
 template <typename T, bool KVI8>
 static int launch_d(const AttnParams &p, int D, hipStream_t s) {
     switch (D) {
+    case 4: return launch_g<T, 4, KVI8>(p, s);
     case 8: return launch_g<T, 8, KVI8>(p, s);
     case 16: return launch_g<T, 16, KVI8>(p, s);
     case 32: return launch_g<T, 32, KVI8>(p, s);
     case 64: return launch_g<T, 64, KVI8>(p, s);
     case 128: return launch_g<T, 128, KVI8>(p, s);
-    default: return fail(MYNN_ERR_UNSUPPORTED, "attention: head_dim %d (supported: 8,16,32,64,128)", D);
+    default: return fail(MYNN_ERR_UNSUPPORTED, "attention: head_dim %d (supported: 4,8,16,32,64,128)", D);
     }
 }
 

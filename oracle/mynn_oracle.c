@@ -379,7 +379,9 @@ void orc_quantizing_kv_cache_update(int8_t *cache, void *scale, const void *new_
             float amax = 0.0f;
             for (size_t d = 0; d < D; d++) {
                 float x = ld(new_kv, src + d, dtype);
-                amax = fmaxf(amax, fmaxf(x, -x));
+                /* |x| as max(x, -x) in the reference; for x = +0 the sign of that maximum is
+                 * unspecified (maxnum), so the restatement takes fabsf and a zero row has scale +0 */
+                amax = fmaxf(amax, fabsf(x));
             }
             float s = amax * (1.0f / 127.0f);
             float inv = amax == 0.0f ? 0.0f : 127.0f / amax;
