@@ -53,7 +53,7 @@ _vp, _i, _sz, _f, _i64 = C.c_void_p, C.c_int, C.c_size_t, C.c_float, C.c_int64
 class ModelConfig(C.Structure):
     _fields_ = [("n_layers", _i), ("hidden", _i), ("n_heads", _i), ("n_kv_heads", _i), ("head_dim", _i),
                 ("ffn", _i), ("vocab", _i), ("max_seq", _i), ("eps", _f), ("rope_theta", _f), ("dtype", _i),
-                ("seq_q", _i), ("batch", _i)]
+                ("seq_q", _i), ("batch", _i), ("weights_int8", _i)]
 
 
 class KernelTime(C.Structure):
@@ -90,6 +90,7 @@ SIGNATURES = {
     "alloc_pinned": (_vp, [_sz]),
     "free_pinned": (None, [_vp]),
     "mynn_model_step": (_i, [_vp, _vp, _vp, _i64, _i64, _vp, _vp]),
+    "mynn_model_argmax_row": (_i, [_vp, _i, C.POINTER(C.c_int32)]),
     "mynn_model_logits_device": (_vp, [_vp]),
     "mynn_model_stats": (_i, [_vp, C.POINTER(_sz), C.POINTER(_i), C.POINTER(_i)]),
     "mynn_model_decode_loop": (_i, [_vp, C.c_int32, _i64, _i, _vp]),
@@ -291,3 +292,183 @@ def argmax_last(logits):
     out = torch.empty((1,), dtype=torch.int32, device=logits.device)
     check(lib().mynn_argmax_last(_ptr(out), _ptr(logits), logits.numel(), _dt(logits), _stream()))
     return out
+
+
+# ------------------------------------------------------------------ decoder executor (seam 1)
+LIN_NAMES = ("q", "k", "v", "o", "gate", "up", "down")
+
+
+class Decoder:
+    """Thin holder around model_init / model_step / model_destroy.
+
+    weights: dict of cuda tensors keyed like the oracle's Model:
+      "embed", "lm_head", "layers.{i}.{q,k,v,o,gate,up,down}" -> (int8 [N,K], scale [N]) or a
+      single float tensor [N,K]; "final_norm", "layers.{i}.norm1|norm2".
+    kv: optional list of (k_cache, v_cache) cuda tensors [batch,Hkv,max_seq,D] per layer, so a
+      prefill and a decode model can share them (PersistentBuffers in the reference).
+    """
+
+    def __init__(self, cfg, weights, seq_q=1, batch=1, kv=None):
+        import torch
+
+        tdt = {F16: torch.float16, BF16: torch.bfloat16}[cfg["dtype"]]
+        quant = isinstance(weights["embed"], tuple)
+        self.cfg = ModelConfig(cfg["n_layers"], cfg["hidden"], cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"],
+                               cfg["ffn"], cfg["vocab"], cfg["max_seq"], float(cfg["eps"]), float(cfg["rope_theta"]),
+                               cfg["dtype"], seq_q, batch, int(quant))
+        self.weights = weights  # keep the tensors alive
+        if kv is None:
+            shape = (batch, cfg["n_kv_heads"], cfg["max_seq"], cfg["head_dim"])
+            kv = [(torch.zeros(shape, dtype=tdt, device="cuda"), torch.zeros(shape, dtype=tdt, device="cuda"))
+                  for _ in range(cfg["n_layers"])]
+        self.kv = kv
+        init = []
+
+        def lin(w):
+            if quant:
+                init.extend([_ptr(w[0]), _ptr(w[1])])
+            else:
+                init.extend([_ptr(w), None])
+
+        lin(weights["embed"])
+        for l in range(cfg["n_layers"]):
+            init.append(_ptr(weights["layers.%d.norm1" % l]))
+            for nm in ("q", "k", "v", "o"):
+                lin(weights["layers.%d.%s" % (l, nm)])
+            init.append(_ptr(weights["layers.%d.norm2" % l]))
+            for nm in ("gate", "up", "down"):
+                lin(weights["layers.%d.%s" % (l, nm)])
+        init.append(_ptr(weights["final_norm"]))
+        lin(weights["lm_head"])
+        state = []
+        for k, v in kv:
+            state.extend([_ptr(k), _ptr(v)])
+        self._init = (_vp * len(init))(*init)
+        self._state = (_vp * len(state))(*state)
+        check(lib().mynn_model_configure(C.byref(self.cfg)))
+        torch.cuda.synchronize()
+        self.handle = lib().model_init(self._init, self._state)
+        if not self.handle:
+            raise MynnError("model_init failed: %s" % lib().mynn_last_error().decode())
+
+    def close(self):
+        if getattr(self, "handle", None):
+            lib().model_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        self.close()
+
+    def step(self, ids, positions, past_len, active, want_logits=False):
+        """One graph run; returns (next tokens per sequence, logits numpy or None)."""
+        import numpy as np
+
+        ids = np.ascontiguousarray(np.asarray(ids, np.int64).ravel())
+        positions = np.ascontiguousarray(np.asarray(positions, np.int64).ravel())
+        assert ids.size == self.cfg.batch * self.cfg.seq_q and positions.size == self.cfg.seq_q
+        nxt = (C.c_int32 * self.cfg.batch)()
+        logits = None
+        lp = None
+        if want_logits:
+            npdt = np.uint16
+            logits = np.empty((self.cfg.batch * self.cfg.seq_q, self.cfg.vocab), npdt)
+            lp = logits.ctypes.data_as(_vp)
+        check(lib().mynn_model_step(self.handle, ids.ctypes.data_as(_vp), positions.ctypes.data_as(_vp),
+                                    int(past_len), int(active), nxt, lp))
+        return list(nxt), logits
+
+    def model(self, ids, positions, past_len, active):
+        """The reference ABI call `model(state, output, input)` with host pointers."""
+        import numpy as np
+
+        ids = np.ascontiguousarray(np.asarray(ids, np.int64).ravel())
+        positions = np.ascontiguousarray(np.asarray(positions, np.int64).ravel())
+        pl = np.array([past_len], np.int64)
+        ac = np.array([active], np.int64)
+        logits = np.empty((self.cfg.batch * self.cfg.seq_q, self.cfg.vocab), np.uint16)
+        inp = (_vp * 4)(ids.ctypes.data, positions.ctypes.data, pl.ctypes.data, ac.ctypes.data)
+        out = (_vp * 1)(logits.ctypes.data)
+        lib().model(self.handle, out, inp)
+        return logits
+
+    def decode_loop(self, token, past_len, n_steps):
+        out = (C.c_int32 * n_steps)()
+        check(lib().mynn_model_decode_loop(self.handle, int(token), int(past_len), n_steps, out))
+        return list(out)
+
+    def profile_step(self, token, past_len, cap=1024):
+        arr = (KernelTime * cap)()
+        n = lib().mynn_model_profile_step(self.handle, int(token), int(past_len), arr, cap)
+        if n < 0:
+            check(n)
+        return [(arr[i].name.decode(), arr[i].ms, arr[i].bytes) for i in range(n)]
+
+    def stats(self):
+        a, n, g = _sz(), _i(), _i()
+        check(lib().mynn_model_stats(self.handle, C.byref(a), C.byref(n), C.byref(g)))
+        return {"arena_bytes": a.value, "launches_per_step": n.value, "graph": bool(g.value)}
+
+
+class LlmSession:
+    """crates/llm LlmSession: decode model + optional prefill model over shared weights and KV."""
+
+    def __init__(self, decoder, prefill=None, eos=-1):
+        self.decoder, self.prefill = decoder, prefill
+        pl = prefill.cfg.seq_q if prefill is not None else 0
+        self.handle = lib().mynn_llm_create(decoder.handle, prefill.handle if prefill is not None else None, pl,
+                                            decoder.cfg.max_seq, int(eos))
+        if not self.handle:
+            raise MynnError(lib().mynn_last_error().decode())
+
+    def close(self):
+        if getattr(self, "handle", None):
+            lib().mynn_llm_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        self.close()
+
+    def reset(self):
+        lib().mynn_llm_reset(self.handle)
+
+    @property
+    def past_len(self):
+        return lib().mynn_llm_past_len(self.handle)
+
+    @past_len.setter
+    def past_len(self, v):
+        lib().mynn_llm_set_past_len(self.handle, int(v))
+
+    def generate_ids(self, prompt_ids, max_new_tokens):
+        import numpy as np
+
+        p = np.ascontiguousarray(np.asarray(prompt_ids, np.int64))
+        out = np.empty((max(max_new_tokens, 1),), np.int64)
+        n = lib().mynn_llm_generate_ids(self.handle, p.ctypes.data_as(_vp), p.size, max_new_tokens,
+                                        out.ctypes.data_as(_vp))
+        if n < 0:
+            raise MynnError("generate_ids error %d: %s" % (n, lib().mynn_last_error().decode()))
+        return [int(t) for t in out[:n]]
+
+
+def quantize_per_channel(w_f32, scale_dt):
+    """Host quantiser of the library (numpy in, numpy out)."""
+    import numpy as np
+
+    w = np.ascontiguousarray(np.asarray(w_f32, np.float32))
+    rows = w.shape[0]
+    q = np.empty(w.shape, np.int8)
+    s = np.empty((rows,), np.float32 if scale_dt == F32 else np.uint16)
+    check(lib().mynn_quantize_per_channel(q.ctypes.data_as(_vp), s.ctypes.data_as(_vp), w.ctypes.data_as(_vp), rows,
+                                          w.size // rows, scale_dt))
+    return q, s
+
+
+def rope_table(max_seq, head_dim, base, dt):
+    import numpy as np
+
+    npdt = np.float32 if dt == F32 else np.uint16
+    cos = np.empty((max_seq, head_dim), npdt)
+    sin = np.empty((max_seq, head_dim), npdt)
+    check(lib().mynn_rope_table(cos.ctypes.data_as(_vp), sin.ctypes.data_as(_vp), max_seq, head_dim, float(base), dt))
+    return cos, sin

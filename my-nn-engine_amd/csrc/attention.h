@@ -1,0 +1,43 @@
+// Launch parameters shared by the attention kernels and their callers.
+#pragma once
+#include "mynn_common.h"
+
+namespace mynn {
+
+struct AttnParams {
+    void *out;
+    const void *q, *k, *v, *k_scale, *v_scale;
+    float scale;
+    int is_causal;
+    int B, Sq, Hq, Hkv, cache_len;
+    int active;               // host value, used when d_active == nullptr
+    const int32_t *d_active;  // device value (graph replay)
+    int q_pos_offset;         // host value, used when d_active == nullptr
+    int nsplit;
+    float *part_o;            // [B*Hq*Sq, nsplit, D]
+    float *part_ml;           // [B*Hq*Sq, nsplit, 2]
+    unsigned *counters;       // [B*Hkv*Sq], zero between launches
+    // element strides of Q and out: batch, head, row.  Reference layout [B,Hq,Sq,D] is
+    // (Hq*Sq*D, Sq*D, D); token-major [B,Sq,Hq*D] is (Sq*Hq*D, D, Hq*D).
+    long q_bs, q_hs, q_rs, o_bs, o_hs, o_rs;
+};
+
+inline void attn_reference_layout(AttnParams &p, int D) {
+    p.q_bs = p.o_bs = (long)p.Hq * p.Sq * D;
+    p.q_hs = p.o_hs = (long)p.Sq * D;
+    p.q_rs = p.o_rs = D;
+}
+inline void attn_token_major_layout(AttnParams &p, int D) {
+    p.q_bs = p.o_bs = (long)p.Sq * p.Hq * D;
+    p.q_hs = p.o_hs = D;
+    p.q_rs = p.o_rs = (long)p.Hq * D;
+}
+
+int attn_pick_nsplit(int B, int Hkv, int Sq, int kv_len);
+size_t attn_scratch_bytes(int B, int Hq, int Sq, int D, int nsplit);
+size_t attn_counter_bytes(int B, int Hkv, int Sq);
+int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *scratch, void *counters, hipStream_t s);
+int attention_prefill_launch(const AttnParams &p, int D, int dtype, hipStream_t s);
+bool attention_prefill_supported(const AttnParams &p, int D, int dtype, int kv_int8);
+
+}  // namespace mynn

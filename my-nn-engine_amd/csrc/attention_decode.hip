@@ -10,24 +10,10 @@
 //
 // The same kernel with gridDim.z = Sq is the correct-but-plain path for Sq > 1 (causal rows get
 // their own key bound); the matrix-core prefill kernel lives in attention_prefill.hip.
-#include "mynn_common.h"
+#include "attention.h"
 
 namespace mynn {
 
-struct AttnParams {
-    void *out;
-    const void *q, *k, *v, *k_scale, *v_scale;
-    float scale;
-    int is_causal;
-    int B, Sq, Hq, Hkv, cache_len;
-    int active;               // host value, used when d_active == nullptr
-    const int32_t *d_active;  // device value (graph replay)
-    int q_pos_offset;         // host value, used when d_active == nullptr
-    int nsplit;
-    float *part_o;            // [B*Hq*Sq, nsplit, D]
-    float *part_ml;           // [B*Hq*Sq, nsplit, 2]
-    unsigned *counters;       // [B*Hkv*Sq], zero between launches
-};
 
 constexpr int kAttnThreads = 256;
 constexpr int kAttnWaves = 4;
@@ -73,7 +59,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
     float q[G][EPL];
 #pragma unroll
     for (int g = 0; g < G; g++) {
-        const size_t qo = ((size_t)(b * p.Hq + hkv * G + g) * Sq + sq) * D + dc * EPL;
+        const size_t qo = (size_t)b * p.q_bs + (size_t)(hkv * G + g) * p.q_hs + (size_t)sq * p.q_rs + dc * EPL;
 #pragma unroll
         for (int i = 0; i < EPL; i++) q[g][i] = Elem<T>::ld(Q, qo + i);
     }
@@ -182,8 +168,9 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
             ot += sm_o[w][g][d] * c;
         }
         const size_t row = row_base + (size_t)g * Sq;
+        const size_t oo = (size_t)b * p.o_bs + (size_t)(hkv * G + g) * p.o_hs + (size_t)sq * p.o_rs + d;
         if (p.nsplit == 1) {
-            Elem<T>::st(out, row * D + d, ot / lt);
+            Elem<T>::st(out, oo, ot / lt);
         } else {
             p.part_o[(row * p.nsplit + split) * D + d] = ot;
             if (d == 0) {
@@ -218,7 +205,8 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
             lt += __builtin_nontemporal_load(&ml[2 * s + 1]) * c;
             ot += __builtin_nontemporal_load(&po[s * D + d]) * c;
         }
-        Elem<T>::st(out, row * D + d, ot / lt);
+        const size_t oo = (size_t)b * p.o_bs + (size_t)(hkv * G + g) * p.o_hs + (size_t)sq * p.o_rs + d;
+        Elem<T>::st(out, oo, ot / lt);
     }
     if (threadIdx.x == 0) p.counters[(size_t)bhkv * Sq + sq] = 0;  // ready for the next launch
 }
@@ -306,8 +294,6 @@ static int ensure(Grown &g, size_t bytes, bool zero, hipStream_t s) {
     return 0;
 }
 
-int attention_prefill_launch(const AttnParams &p, int D, int dtype, hipStream_t s);  // attention_prefill.hip
-bool attention_prefill_supported(const AttnParams &p, int D, int dtype, int kv_int8);
 
 }  // namespace mynn
 
@@ -329,6 +315,7 @@ extern "C" int mynn_attention(void *out, const void *Q, const void *K, const voi
     p.out = out; p.q = Q; p.k = K; p.v = V; p.k_scale = k_scale; p.v_scale = v_scale; p.scale = scale;
     p.is_causal = is_causal; p.B = B; p.Sq = Sq; p.Hq = num_q_heads; p.Hkv = num_kv_heads;
     p.cache_len = cache_seq_len; p.active = active_seq_kv; p.d_active = d_active; p.q_pos_offset = q_pos_offset;
+    attn_reference_layout(p, head_dim);
     hipStream_t st = as_stream(s);
     if (Sq > 1 && attention_prefill_supported(p, head_dim, dtype, kv_int8))
         return attention_prefill_launch(p, head_dim, dtype, st);

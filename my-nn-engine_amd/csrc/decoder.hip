@@ -1,0 +1,599 @@
+// Static Llama decoder executor behind the reference's per-session model ABI
+// (model_init / model / model_destroy, src/codegen/cuda.rs:2727-2825).
+//
+// The reference generates one libmodel.so per graph whose model() launches ~30 kernels per layer
+// over up to 16 streams, reading `past_len` / `active_seq_kv` on the host at launch time.  Here the
+// op sequence of crates/llm/src/decoder.rs:222-391,780-865 is fixed code:
+//   decode (seq_q == 1, int8 weights): 6 launches per layer, all scalars (token, position,
+//     past_len, active length) live in device memory, the whole step is captured once into a
+//     hipGraph and replayed; a decode loop can run many steps without a host round trip.
+//   everything else (prefill rows, un-quantised checkpoints): op-by-op launches in the
+//     reference's order, with the reference's kernel choice per op.
+// One stream, one arena allocated at init; weights and KV buffers stay caller-owned.
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <vector>
+
+#include "attention.h"
+#include "kernels.h"
+
+namespace mynn {
+
+// ---- plain (un-quantised) linear: out[m,n] = T(sum_k act[m,k] * w[n,k]), one wave per element.
+// Serves the reference's float checkpoints (its cuBLAS Gemm path); not a tuned kernel.
+template <typename T>
+__global__ __launch_bounds__(64) void dense_linear_kernel(T *out, const T *act, const T *w, int N, int K,
+                                                         int out_stride) {
+    const int n = blockIdx.x, m = blockIdx.y, lane = threadIdx.x;
+    float acc = 0.f;
+    for (int k = lane; k < K; k += 64) acc = fmaf(Elem<T>::ld(act, (size_t)m * K + k), Elem<T>::ld(w, (size_t)n * K + k), acc);
+    acc = wave_sum(acc);
+    if (lane == 0) Elem<T>::st(out, (size_t)m * out_stride + n, acc);
+}
+
+template <typename T>
+__global__ void swiglu_rows_kernel(T *out, const T *gate, const T *up, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float g = Elem<T>::ld(gate, i);
+    float sig = 1.0f / (1.0f + expf(-g));
+    Elem<T>::st(out, i, (g * sig) * Elem<T>::ld(up, i));
+}
+
+// device-side bookkeeping between two replayed decode steps: the greedy token becomes the next
+// input, position / past_len / active length move on by one
+__global__ void advance_kernel(int64_t *ids, int64_t *pos, int32_t *past, int32_t *active, const int32_t *next,
+                               int32_t *tokens, int32_t *step, int cap) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    int t = next[0];
+    int i = *step;
+    if (i < cap) tokens[i] = t;
+    *step = i + 1;
+    ids[0] = t;
+    pos[0] += 1;
+    *past += 1;
+    *active += 1;
+}
+
+struct Lin {
+    const void *w = nullptr;      // int8 [N,K] when scale != nullptr, else T [N,K]
+    const void *scale = nullptr;  // T [N]
+    int N = 0, K = 0;
+};
+
+struct Layer {
+    const void *norm1 = nullptr, *norm2 = nullptr;
+    Lin qkv, o, gate, up, gu, down;  // qkv = rows of q,k,v concatenated; gu = gate/up rows interleaved
+    void *k_cache = nullptr, *v_cache = nullptr;
+    void *own_qkv_w = nullptr, *own_qkv_s = nullptr, *own_gu_w = nullptr, *own_gu_s = nullptr;
+};
+
+struct Launch {
+    const char *name;
+    double bytes;
+};
+
+struct Model {
+    mynn_model_config cfg{};
+    bool quant = true;
+    Lin embed, lm_head;
+    const void *final_norm = nullptr;
+    std::vector<Layer> layers;
+    void *cos_t = nullptr, *sin_t = nullptr;
+    // arena
+    char *arena = nullptr;
+    size_t arena_bytes = 0;
+    void *x = nullptr, *x2 = nullptr, *nrm = nullptr, *qkv = nullptr, *q = nullptr, *attn = nullptr, *g = nullptr,
+         *u = nullptr, *hmid = nullptr, *proj = nullptr, *logits = nullptr;
+    int64_t *d_ids = nullptr, *d_pos = nullptr;
+    int32_t *d_past = nullptr, *d_active = nullptr, *d_next = nullptr, *d_tokens = nullptr, *d_step = nullptr;
+    void *attn_scratch = nullptr, *attn_counters = nullptr;
+    int nsplit = 1;
+    int token_cap = 0;
+    // host staging (pinned)
+    char *h_stage = nullptr;
+    size_t stage_bytes = 0;
+    hipStream_t stream = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t graph_exec = nullptr;
+    bool use_graph = false;
+    int launches = 0;
+    // per-launch record of the last enqueue (names + algorithmic bytes), events when profiling
+    std::vector<Launch> record;
+    bool profiling = false;
+    std::vector<hipEvent_t> events;
+};
+
+static mynn_model_config g_cfg{};
+static bool g_cfg_set = false;
+static int g_weights_quantized = 1;
+static std::mutex g_mu;
+
+static size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+struct ArenaPlan {
+    size_t off = 0;
+    size_t take(size_t bytes) {
+        size_t o = off;
+        off = align_up(off + bytes, 256);
+        return o;
+    }
+};
+
+static void note(Model &m, const char *name, double bytes) {
+    if (m.profiling) {
+        hipEvent_t e;
+        hipEventCreate(&e);
+        hipEventRecord(e, m.stream);
+        m.events.push_back(e);
+    }
+    m.record.push_back({name, bytes});
+}
+
+template <typename T>
+static int linear_rows(Model &m, void *out, const void *act, const Lin &l, int M, const char *name) {
+    const double eb = sizeof(T);
+    if (l.scale) {
+        note(m, name, (double)l.N * l.K + l.N * eb + (double)M * l.K * eb + (double)M * l.N * eb);
+        if (M >= 16 && l.K % 32 == 0)
+            return dequant_gemm_mfma(out, act, (const int8_t *)l.w, l.scale, M, l.N, l.K, m.cfg.dtype, m.stream);
+        return dequant_gemv_dispatch(out, act, (const int8_t *)l.w, l.scale, M, l.N, l.K, m.cfg.dtype, m.cfg.dtype,
+                                     m.stream);
+    }
+    note(m, name, ((double)l.N * l.K + (double)M * l.K + (double)M * l.N) * eb);
+    hipLaunchKernelGGL(dense_linear_kernel<T>, dim3(l.N, M), dim3(64), 0, m.stream, (T *)out, (const T *)act,
+                       (const T *)l.w, l.N, l.K, l.N);
+    return launch_status("dense_linear_kernel");
+}
+
+#define TRY(expr)            \
+    do {                     \
+        int rc__ = (expr);   \
+        if (rc__) return rc__; \
+    } while (0)
+
+template <typename T>
+static int enqueue_step(Model &m) {
+    const mynn_model_config &c = m.cfg;
+    const int S = c.seq_q, B = c.batch, rows = B * S;
+    const int H = c.hidden, Hq = c.n_heads, Hkv = c.n_kv_heads, D = c.head_dim, F = c.ffn, V = c.vocab;
+    const int QD = Hq * D, KD = Hkv * D;
+    const double eb = sizeof(T);
+    const bool fused = m.quant && rows == 1;
+    hipStream_t s = m.stream;
+    m.record.clear();
+    for (hipEvent_t e : m.events) hipEventDestroy(e);
+    m.events.clear();
+
+    // embed: DequantizeLinear(table) -> Gather(ids), one row per token
+    if (m.quant) {
+        note(m, "embed_dequant", (double)rows * (H + eb + H * eb));
+        TRY(embed_dequant<T>(m.x, (const int8_t *)m.embed.w, m.embed.scale, m.d_ids, rows, V, H, s));
+    } else {
+        note(m, "embed_gather", (double)rows * 2 * H * eb);
+        TRY(mynn_gather_rows(m.x, m.embed.w, m.d_ids, rows, V, (size_t)H * sizeof(T), s));
+    }
+    const float softmax_scale = 1.0f / sqrtf((float)D);
+    for (Layer &L : m.layers) {
+        // ---- attention block
+        if (fused) {
+            note(m, "gemv_norm_qkv", (double)L.qkv.N * H + L.qkv.N * eb + 2 * H * eb + L.qkv.N * eb);
+            TRY(gemv_norm<T>(m.qkv, m.x, L.norm1, c.eps, (const int8_t *)L.qkv.w, L.qkv.scale, L.qkv.N, H, s));
+        } else {
+            note(m, "rms_norm", 2.0 * rows * H * eb + H * eb);
+            TRY(mynn_rms_norm(m.nrm, m.x, L.norm1, rows, H, c.eps, c.dtype, s));
+            TRY(linear_rows<T>(m, m.qkv, m.nrm, L.qkv, rows, "linear_qkv"));
+        }
+        note(m, "rope_kv_append", (double)rows * (QD + 2 * KD) * 2 * eb);
+        TRY(rope_kv_append<T>(m.q, L.k_cache, L.v_cache, m.qkv, m.cos_t, m.sin_t, m.d_pos, m.d_past, 0, B, S, Hq, Hkv,
+                              D, c.max_seq, s));
+        {
+            AttnParams p{};
+            p.out = m.attn; p.q = m.q; p.k = L.k_cache; p.v = L.v_cache; p.scale = softmax_scale;
+            p.is_causal = S > 1; p.B = B; p.Sq = S; p.Hq = Hq; p.Hkv = Hkv; p.cache_len = c.max_seq;
+            p.d_active = m.d_active; p.nsplit = m.nsplit;
+            attn_token_major_layout(p, D);
+            // bytes: K and V rows of the active prefix (upper bound max_seq is not known on the host
+            // under replay; the caller scales by the real context when it reports)
+            note(m, "attention", (double)B * (2.0 * QD * eb * S));
+            if (S > 1 && attention_prefill_supported(p, D, c.dtype, 0)) TRY(attention_prefill_launch(p, D, c.dtype, s));
+            else TRY(attention_decode_launch(p, D, c.dtype, 0, m.attn_scratch, m.attn_counters, s));
+        }
+        if (fused) {
+            note(m, "gemv_o_residual", (double)H * QD + H * eb + QD * eb + 2 * H * eb);
+            TRY(gemv_residual<T>(m.x2, m.attn, (const int8_t *)L.o.w, L.o.scale, m.x, H, QD, s));
+            note(m, "gemv_norm_gateup_swiglu", (double)L.gu.N * H + L.gu.N * eb + 2 * H * eb + F * eb);
+            TRY(gemv_norm_swiglu<T>(m.hmid, m.x2, L.norm2, c.eps, (const int8_t *)L.gu.w, L.gu.scale, L.gu.N, H, s));
+            note(m, "gemv_down_residual", (double)H * F + H * eb + F * eb + 2 * H * eb);
+            TRY(gemv_residual<T>(m.x, m.hmid, (const int8_t *)L.down.w, L.down.scale, m.x2, H, F, s));
+        } else {
+            TRY(linear_rows<T>(m, m.proj, m.attn, L.o, rows, "linear_o"));
+            note(m, "add", 3.0 * rows * H * eb);
+            TRY(mynn_add(m.x2, m.x, m.proj, (size_t)rows * H, c.dtype, s));
+            note(m, "rms_norm", 2.0 * rows * H * eb + H * eb);
+            TRY(mynn_rms_norm(m.nrm, m.x2, L.norm2, rows, H, c.eps, c.dtype, s));
+            TRY(linear_rows<T>(m, m.g, m.nrm, L.gate, rows, "linear_gate"));
+            TRY(linear_rows<T>(m, m.u, m.nrm, L.up, rows, "linear_up"));
+            note(m, "swiglu", 3.0 * rows * F * eb);
+            TRY(mynn_swiglu(m.hmid, m.g, m.u, (size_t)rows * F, c.dtype, s));
+            TRY(linear_rows<T>(m, m.proj, m.hmid, L.down, rows, "linear_down"));
+            note(m, "add", 3.0 * rows * H * eb);
+            TRY(mynn_add(m.x, m.x2, m.proj, (size_t)rows * H, c.dtype, s));
+        }
+    }
+    if (fused) {
+        note(m, "gemv_norm_lm_head", (double)V * H + V * eb + 2 * H * eb + V * eb);
+        TRY(gemv_norm<T>(m.logits, m.x, m.final_norm, c.eps, (const int8_t *)m.lm_head.w, m.lm_head.scale, V, H, s));
+    } else {
+        note(m, "rms_norm", 2.0 * rows * H * eb + H * eb);
+        TRY(mynn_rms_norm(m.nrm, m.x, m.final_norm, rows, H, c.eps, c.dtype, s));
+        TRY(linear_rows<T>(m, m.logits, m.nrm, m.lm_head, rows, "linear_lm_head"));
+    }
+    // greedy token of the last row of each sequence
+    note(m, "argmax_last", (double)B * V * eb);
+    for (int b = 0; b < B; b++)
+        TRY(argmax_rows<T>(m.d_next + b, (const T *)m.logits + ((size_t)b * S + (S - 1)) * V, 1, V, s));
+    if (rows == 1) {
+        note(m, "advance", 64);
+        hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(64), 0, s, m.d_ids, m.d_pos, m.d_past, m.d_active, m.d_next,
+                           m.d_tokens, m.d_step, m.token_cap);
+        TRY(launch_status("advance_kernel"));
+    }
+    if (m.profiling) {
+        hipEvent_t e;
+        hipEventCreate(&e);
+        hipEventRecord(e, s);
+        m.events.push_back(e);
+    }
+    m.launches = (int)m.record.size();
+    return 0;
+}
+
+static int enqueue(Model &m) {
+    return dispatch_dtype16(m.cfg.dtype, [&](auto *t) {
+        using T = std::remove_pointer_t<decltype(t)>;
+        return enqueue_step<T>(m);
+    });
+}
+
+// ---- weight repacking (explicit, at init, into library-owned buffers) --------------------------
+static int concat_rows(void **out, const void *const *parts, const size_t *bytes, int n) {
+    size_t total = 0;
+    for (int i = 0; i < n; i++) total += bytes[i];
+    MYNN_HIP(hipMalloc(out, total));
+    size_t off = 0;
+    for (int i = 0; i < n; i++) {
+        MYNN_HIP(hipMemcpy((char *)*out + off, parts[i], bytes[i], hipMemcpyDeviceToDevice));
+        off += bytes[i];
+    }
+    return 0;
+}
+static int interleave_rows(void **out, const void *a, const void *b, size_t rows, size_t row_bytes) {
+    MYNN_HIP(hipMalloc(out, 2 * rows * row_bytes));
+    MYNN_HIP(hipMemcpy2D(*out, 2 * row_bytes, a, row_bytes, row_bytes, rows, hipMemcpyDeviceToDevice));
+    MYNN_HIP(hipMemcpy2D((char *)*out + row_bytes, 2 * row_bytes, b, row_bytes, row_bytes, rows, hipMemcpyDeviceToDevice));
+    return 0;
+}
+
+static int host_rope_tables(Model &m);
+
+static int build(Model &m, void **init, void **state) {
+    const mynn_model_config &c = m.cfg;
+    const size_t eb = dtype_size(c.dtype);
+    const int H = c.hidden, QD = c.n_heads * c.head_dim, KD = c.n_kv_heads * c.head_dim, F = c.ffn, V = c.vocab;
+    const size_t wb = m.quant ? 1 : eb;  // bytes per weight element
+    int i = 0;
+    auto lin = [&](Lin &l, int N, int K) {
+        l.w = init[i++];
+        l.scale = m.quant ? init[i++] : (i++, nullptr);
+        l.N = N;
+        l.K = K;
+    };
+    lin(m.embed, V, H);
+    m.layers.resize(c.n_layers);
+    for (int li = 0; li < c.n_layers; li++) {
+        Layer &L = m.layers[li];
+        L.norm1 = init[i++];
+        Lin q, k, v;
+        lin(q, QD, H); lin(k, KD, H); lin(v, KD, H);
+        lin(L.o, H, QD);
+        L.norm2 = init[i++];
+        lin(L.gate, F, H); lin(L.up, F, H); lin(L.down, H, F);
+        MYNN_REQUIRE(L.norm1 && L.norm2 && q.w && k.w && v.w && L.o.w && L.gate.w && L.up.w && L.down.w,
+                     MYNN_ERR_INVALID, "model_init: null weight in layer %d", li);
+        MYNN_REQUIRE(!m.quant || (q.scale && k.scale && v.scale && L.o.scale && L.gate.scale && L.up.scale && L.down.scale),
+                     MYNN_ERR_INVALID, "model_init: null scale in layer %d", li);
+        const void *parts[3] = {q.w, k.w, v.w};
+        const size_t pb[3] = {(size_t)QD * H * wb, (size_t)KD * H * wb, (size_t)KD * H * wb};
+        TRY(concat_rows(&L.own_qkv_w, parts, pb, 3));
+        L.qkv.w = L.own_qkv_w; L.qkv.N = QD + 2 * KD; L.qkv.K = H;
+        if (m.quant) {
+            const void *sp[3] = {q.scale, k.scale, v.scale};
+            const size_t sb[3] = {(size_t)QD * eb, (size_t)KD * eb, (size_t)KD * eb};
+            TRY(concat_rows(&L.own_qkv_s, sp, sb, 3));
+            L.qkv.scale = L.own_qkv_s;
+            TRY(interleave_rows(&L.own_gu_w, L.gate.w, L.up.w, F, (size_t)H));
+            TRY(interleave_rows(&L.own_gu_s, L.gate.scale, L.up.scale, F, eb));
+            L.gu.w = L.own_gu_w; L.gu.scale = L.own_gu_s; L.gu.N = 2 * F; L.gu.K = H;
+        }
+        L.k_cache = state[2 * li];
+        L.v_cache = state[2 * li + 1];
+        MYNN_REQUIRE(L.k_cache && L.v_cache, MYNN_ERR_INVALID, "model_init: null KV buffer in layer %d", li);
+    }
+    m.final_norm = init[i++];
+    lin(m.lm_head, V, H);
+    MYNN_REQUIRE(m.embed.w && m.final_norm && m.lm_head.w, MYNN_ERR_INVALID, "model_init: null embed/norm/lm_head");
+
+    MYNN_HIP(hipStreamCreateWithFlags(&m.stream, hipStreamNonBlocking));
+    TRY(host_rope_tables(m));
+
+    // ---- arena: every activation of one step, the device scalars, attention split scratch
+    const int rows = c.batch * c.seq_q;
+    m.nsplit = attn_pick_nsplit(c.batch, c.n_kv_heads, c.seq_q, c.max_seq);
+    m.token_cap = c.max_seq + 8;
+    ArenaPlan plan;
+    size_t o_x = plan.take((size_t)rows * H * eb), o_x2 = plan.take((size_t)rows * H * eb);
+    size_t o_n = plan.take((size_t)rows * H * eb), o_qkv = plan.take((size_t)rows * (QD + 2 * KD) * eb);
+    size_t o_q = plan.take((size_t)rows * QD * eb), o_attn = plan.take((size_t)rows * QD * eb);
+    size_t o_g = plan.take((size_t)rows * F * eb), o_u = plan.take((size_t)rows * F * eb);
+    size_t o_h = plan.take((size_t)rows * F * eb), o_p = plan.take((size_t)rows * H * eb);
+    size_t o_l = plan.take((size_t)rows * V * eb);
+    size_t o_ids = plan.take((size_t)rows * 8), o_pos = plan.take((size_t)c.seq_q * 8);
+    size_t o_sc = plan.take(256), o_tok = plan.take((size_t)m.token_cap * 4);
+    size_t o_as = plan.take(attn_scratch_bytes(c.batch, c.n_heads, c.seq_q, c.head_dim, m.nsplit));
+    size_t o_ac = plan.take(attn_counter_bytes(c.batch, c.n_kv_heads, c.seq_q));
+    m.arena_bytes = plan.off;
+    MYNN_HIP(hipMalloc((void **)&m.arena, m.arena_bytes));
+    MYNN_HIP(hipMemset(m.arena, 0, m.arena_bytes));
+    m.x = m.arena + o_x; m.x2 = m.arena + o_x2; m.nrm = m.arena + o_n; m.qkv = m.arena + o_qkv; m.q = m.arena + o_q;
+    m.attn = m.arena + o_attn; m.g = m.arena + o_g; m.u = m.arena + o_u; m.hmid = m.arena + o_h; m.proj = m.arena + o_p;
+    m.logits = m.arena + o_l;
+    m.d_ids = (int64_t *)(m.arena + o_ids); m.d_pos = (int64_t *)(m.arena + o_pos);
+    m.d_past = (int32_t *)(m.arena + o_sc); m.d_active = m.d_past + 1; m.d_step = m.d_past + 2;
+    m.d_next = m.d_past + 8;  // up to 56 sequences' tokens after the scalars
+    MYNN_REQUIRE(c.batch <= 56, MYNN_ERR_UNSUPPORTED, "batch %d > 56", c.batch);
+    m.d_tokens = (int32_t *)(m.arena + o_tok);
+    m.attn_scratch = m.arena + o_as; m.attn_counters = m.arena + o_ac;
+    m.stage_bytes = align_up((size_t)rows * 8 + (size_t)c.seq_q * 8 + 64 + (size_t)m.token_cap * 4, 256) + 512;
+    MYNN_HIP(hipHostMalloc((void **)&m.h_stage, m.stage_bytes, hipHostMallocDefault));
+    MYNN_HIP(hipDeviceSynchronize());
+
+    // ---- capture the decode step once
+    if (rows == 1) {
+        hipError_t e = hipStreamBeginCapture(m.stream, hipStreamCaptureModeThreadLocal);
+        if (e == hipSuccess) {
+            int rc = enqueue(m);
+            hipError_t e2 = hipStreamEndCapture(m.stream, &m.graph);
+            if (rc == 0 && e2 == hipSuccess && hipGraphInstantiate(&m.graph_exec, m.graph, nullptr, nullptr, 0) == hipSuccess)
+                m.use_graph = true;
+            else {
+                (void)hipGetLastError();
+                if (rc) return rc;
+            }
+        } else (void)hipGetLastError();
+    }
+    return 0;
+}
+
+static int host_rope_tables(Model &m) {
+    const mynn_model_config &c = m.cfg;
+    const size_t eb = dtype_size(c.dtype), n = (size_t)c.max_seq * c.head_dim;
+    std::vector<char> hc(n * eb), hs(n * eb);
+    TRY(mynn_rope_table(hc.data(), hs.data(), c.max_seq, c.head_dim, c.rope_theta, c.dtype));
+    MYNN_HIP(hipMalloc(&m.cos_t, n * eb));
+    MYNN_HIP(hipMalloc(&m.sin_t, n * eb));
+    MYNN_HIP(hipMemcpy(m.cos_t, hc.data(), n * eb, hipMemcpyHostToDevice));
+    MYNN_HIP(hipMemcpy(m.sin_t, hs.data(), n * eb, hipMemcpyHostToDevice));
+    return 0;
+}
+
+static void destroy(Model *m) {
+    if (!m) return;
+    if (m->stream) hipStreamSynchronize(m->stream);
+    for (hipEvent_t e : m->events) hipEventDestroy(e);
+    if (m->graph_exec) hipGraphExecDestroy(m->graph_exec);
+    if (m->graph) hipGraphDestroy(m->graph);
+    for (Layer &L : m->layers) {
+        if (L.own_qkv_w) hipFree(L.own_qkv_w);
+        if (L.own_qkv_s) hipFree(L.own_qkv_s);
+        if (L.own_gu_w) hipFree(L.own_gu_w);
+        if (L.own_gu_s) hipFree(L.own_gu_s);
+    }
+    if (m->cos_t) hipFree(m->cos_t);
+    if (m->sin_t) hipFree(m->sin_t);
+    if (m->arena) hipFree(m->arena);
+    if (m->h_stage) hipHostFree(m->h_stage);
+    if (m->stream) hipStreamDestroy(m->stream);
+    delete m;
+}
+
+// H2D of one step's inputs (ids, positions, past_len, active, step counter = 0) in one copy
+static int upload_inputs(Model &m, const int64_t *ids, const int64_t *pos, int64_t past, int64_t active) {
+    const mynn_model_config &c = m.cfg;
+    const int rows = c.batch * c.seq_q;
+    MYNN_REQUIRE(past >= 0 && past + c.seq_q <= c.max_seq, MYNN_ERR_TOO_LONG,
+                 "past_len %lld + %d rows exceeds max_seq %d", (long long)past, c.seq_q, c.max_seq);
+    MYNN_REQUIRE(active >= 1 && active <= c.max_seq, MYNN_ERR_INVALID, "active_seq_kv %lld out of range", (long long)active);
+    for (int s = 0; s < c.seq_q; s++)
+        MYNN_REQUIRE(pos[s] >= 0 && pos[s] < c.max_seq, MYNN_ERR_INVALID, "position_id[%d]=%lld outside the RoPE table", s,
+                     (long long)pos[s]);
+    for (int r = 0; r < rows; r++)
+        MYNN_REQUIRE(ids[r] >= -c.vocab && ids[r] < c.vocab, MYNN_ERR_INVALID, "input_ids[%d]=%lld outside the vocabulary", r,
+                     (long long)ids[r]);
+    int64_t *h_ids = (int64_t *)m.h_stage;
+    int64_t *h_pos = h_ids + rows;
+    int32_t *h_sc = (int32_t *)(h_pos + c.seq_q);
+    memcpy(h_ids, ids, (size_t)rows * 8);
+    memcpy(h_pos, pos, (size_t)c.seq_q * 8);
+    h_sc[0] = (int32_t)past; h_sc[1] = (int32_t)active; h_sc[2] = 0;
+    MYNN_HIP(hipMemcpyAsync(m.d_ids, h_ids, (size_t)rows * 8, hipMemcpyHostToDevice, m.stream));
+    MYNN_HIP(hipMemcpyAsync(m.d_pos, h_pos, (size_t)c.seq_q * 8, hipMemcpyHostToDevice, m.stream));
+    MYNN_HIP(hipMemcpyAsync(m.d_past, h_sc, 12, hipMemcpyHostToDevice, m.stream));
+    return 0;
+}
+
+static int run_once(Model &m) {
+    if (m.use_graph && !m.profiling) {
+        MYNN_HIP(hipGraphLaunch(m.graph_exec, m.stream));
+        return 0;
+    }
+    return enqueue(m);
+}
+
+}  // namespace mynn
+
+using namespace mynn;
+
+extern "C" int mynn_model_configure(const mynn_model_config *cfg) {
+    MYNN_REQUIRE(cfg, MYNN_ERR_INVALID, "model_configure: null config");
+    MYNN_REQUIRE(cfg->n_layers > 0 && cfg->hidden > 0 && cfg->n_heads > 0 && cfg->n_kv_heads > 0 && cfg->head_dim > 0 &&
+                     cfg->ffn > 0 && cfg->vocab > 0 && cfg->max_seq > 0 && cfg->seq_q > 0 && cfg->batch > 0,
+                 MYNN_ERR_INVALID, "model_configure: non-positive dimension");
+    MYNN_REQUIRE(cfg->hidden == cfg->n_heads * cfg->head_dim, MYNN_ERR_INVALID,
+                 "model_configure: hidden %d != n_heads %d * head_dim %d", cfg->hidden, cfg->n_heads, cfg->head_dim);
+    MYNN_REQUIRE(cfg->n_heads % cfg->n_kv_heads == 0, MYNN_ERR_INVALID, "model_configure: heads not a multiple of kv heads");
+    MYNN_REQUIRE(cfg->dtype == MYNN_F16 || cfg->dtype == MYNN_BF16, MYNN_ERR_UNSUPPORTED,
+                 "model_configure: dtype %d (fp16 or bf16 only)", cfg->dtype);
+    MYNN_REQUIRE(cfg->seq_q <= cfg->max_seq, MYNN_ERR_INVALID, "model_configure: prefill_len %d > max_seq %d", cfg->seq_q,
+                 cfg->max_seq);
+    std::lock_guard<std::mutex> lk(g_mu);
+    g_cfg = *cfg;
+    g_cfg_set = true;
+    g_weights_quantized = cfg->weights_int8;
+    return 0;
+}
+
+extern "C" void *model_init(void **initializer, void **session_state) {
+    mynn_model_config cfg;
+    int quant;
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        if (!g_cfg_set) {
+            fail(MYNN_ERR_STATE, "model_init: call mynn_model_configure first");
+            return nullptr;
+        }
+        cfg = g_cfg;
+        quant = g_weights_quantized;
+    }
+    if (!initializer || !session_state) {
+        fail(MYNN_ERR_INVALID, "model_init: null initializer / session_state array");
+        return nullptr;
+    }
+    Model *m = new Model;
+    m->cfg = cfg;
+    m->quant = quant != 0;
+    int rc = build(*m, initializer, session_state);
+    if (rc) {
+        destroy(m);
+        return nullptr;
+    }
+    return m;
+}
+
+extern "C" void model_destroy(void *state) { destroy((Model *)state); }
+extern "C" void model_device_sync(void) { (void)hipDeviceSynchronize(); }
+extern "C" int model_memcpy(void *dst, const void *src, size_t n, int kind) {
+    return (int)hipMemcpy(dst, src, n, (hipMemcpyKind)kind);
+}
+extern "C" void *alloc_pinned(size_t n) {
+    void *p = nullptr;
+    if (hipHostMalloc(&p, n, hipHostMallocDefault) != hipSuccess) return nullptr;
+    return p;
+}
+extern "C" void free_pinned(void *p) {
+    if (p) (void)hipHostFree(p);
+}
+
+extern "C" int mynn_model_step(void *state, const int64_t *input_ids, const int64_t *position_id, int64_t past_len,
+                               int64_t active_seq_kv, int32_t *next_token, void *logits_host) {
+    MYNN_REQUIRE(state && input_ids && position_id, MYNN_ERR_INVALID, "model_step: null argument");
+    Model &m = *(Model *)state;
+    TRY(upload_inputs(m, input_ids, position_id, past_len, active_seq_kv));
+    TRY(run_once(m));
+    const mynn_model_config &c = m.cfg;
+    if (next_token) MYNN_HIP(hipMemcpyAsync(m.h_stage + m.stage_bytes - 256, m.d_next, (size_t)c.batch * 4, hipMemcpyDeviceToHost, m.stream));
+    if (logits_host)
+        MYNN_HIP(hipMemcpyAsync(logits_host, m.logits, (size_t)c.batch * c.seq_q * c.vocab * dtype_size(c.dtype),
+                                hipMemcpyDeviceToHost, m.stream));
+    MYNN_HIP(hipStreamSynchronize(m.stream));
+    if (next_token) memcpy(next_token, m.h_stage + m.stage_bytes - 256, (size_t)c.batch * 4);
+    return 0;
+}
+
+// Reference ABI: void, host pointers, synchronous.  A failure is reported on stderr and through
+// mynn_last_error(); it never exits the process.
+extern "C" void model(void *state, void **output, void **input) {
+    if (!state || !output || !input) {
+        fail(MYNN_ERR_INVALID, "model: null argument");
+        fprintf(stderr, "mynn model(): %s\n", mynn_last_error());
+        return;
+    }
+    int rc = mynn_model_step(state, (const int64_t *)input[0], (const int64_t *)input[1], *(const int64_t *)input[2],
+                             *(const int64_t *)input[3], nullptr, output[0]);
+    if (rc) fprintf(stderr, "mynn model(): error %d: %s\n", rc, mynn_last_error());
+}
+
+extern "C" int mynn_model_argmax_row(void *state, int row, int32_t *token) {
+    MYNN_REQUIRE(state && token, MYNN_ERR_INVALID, "model_argmax_row: null argument");
+    Model &m = *(Model *)state;
+    const mynn_model_config &c = m.cfg;
+    MYNN_REQUIRE(row >= 0 && row < c.batch * c.seq_q, MYNN_ERR_INVALID, "model_argmax_row: row %d", row);
+    const char *l = (const char *)m.logits + (size_t)row * c.vocab * dtype_size(c.dtype);
+    TRY(mynn_argmax_last(m.d_next, l, c.vocab, c.dtype, m.stream));
+    MYNN_HIP(hipMemcpyAsync(m.h_stage, m.d_next, 4, hipMemcpyDeviceToHost, m.stream));
+    MYNN_HIP(hipStreamSynchronize(m.stream));
+    memcpy(token, m.h_stage, 4);
+    return 0;
+}
+
+extern "C" const void *mynn_model_logits_device(void *state) { return state ? ((Model *)state)->logits : nullptr; }
+
+extern "C" int mynn_model_stats(void *state, size_t *arena_bytes, int *launches_per_step, int *graph) {
+    MYNN_REQUIRE(state, MYNN_ERR_INVALID, "model_stats: null state");
+    Model &m = *(Model *)state;
+    if (arena_bytes) *arena_bytes = m.arena_bytes;
+    if (launches_per_step) *launches_per_step = m.launches;
+    if (graph) *graph = m.use_graph ? 1 : 0;
+    return 0;
+}
+
+extern "C" int mynn_model_decode_loop(void *state, int32_t token, int64_t past_len, int n_steps, int32_t *out_tokens) {
+    MYNN_REQUIRE(state && out_tokens && n_steps > 0, MYNN_ERR_INVALID, "decode_loop: bad argument");
+    Model &m = *(Model *)state;
+    const mynn_model_config &c = m.cfg;
+    MYNN_REQUIRE(c.batch * c.seq_q == 1, MYNN_ERR_STATE, "decode_loop: needs a batch-1 decode model");
+    MYNN_REQUIRE(past_len + n_steps <= c.max_seq && n_steps <= m.token_cap, MYNN_ERR_TOO_LONG,
+                 "decode_loop: past_len %lld + %d steps exceeds max_seq %d", (long long)past_len, n_steps, c.max_seq);
+    int64_t id = token, pos = past_len;
+    TRY(upload_inputs(m, &id, &pos, past_len, past_len + 1));
+    for (int i = 0; i < n_steps; i++) TRY(run_once(m));
+    MYNN_HIP(hipMemcpyAsync(m.h_stage, m.d_tokens, (size_t)n_steps * 4, hipMemcpyDeviceToHost, m.stream));
+    MYNN_HIP(hipStreamSynchronize(m.stream));
+    memcpy(out_tokens, m.h_stage, (size_t)n_steps * 4);
+    return 0;
+}
+
+extern "C" int mynn_model_profile_step(void *state, int32_t token, int64_t past_len, mynn_kernel_time *out, int cap) {
+    MYNN_REQUIRE(state && out && cap > 0, MYNN_ERR_INVALID, "profile_step: bad argument");
+    Model &m = *(Model *)state;
+    const mynn_model_config &c = m.cfg;
+    MYNN_REQUIRE(c.batch * c.seq_q == 1, MYNN_ERR_STATE, "profile_step: needs a batch-1 decode model");
+    int64_t id = token, pos = past_len;
+    TRY(upload_inputs(m, &id, &pos, past_len, past_len + 1));
+    m.profiling = true;
+    int rc = enqueue(m);
+    m.profiling = false;
+    if (rc) return rc;
+    MYNN_HIP(hipStreamSynchronize(m.stream));
+    int n = (int)m.record.size();
+    for (int i = 0; i < n && i < cap; i++) {
+        float ms = 0.f;
+        MYNN_HIP(hipEventElapsedTime(&ms, m.events[i], m.events[i + 1]));
+        out[i].name = m.record[i].name;
+        out[i].ms = ms;
+        out[i].bytes = m.record[i].bytes;
+    }
+    return n < cap ? n : cap;
+}

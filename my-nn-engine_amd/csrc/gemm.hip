@@ -15,3 +15,9 @@ extern "C" int mynn_dequant_matmul(void *out, const void *act, const int8_t *wq,
         return fail(MYNN_ERR_UNSUPPORTED, "dequant_matmul: matrix-core GEMM not built yet");
     return dequant_gemv_dispatch(out, act, wq, scale, M, N, K, act_dtype, out_dtype, as_stream(s));
 }
+
+namespace mynn {
+int dequant_gemm_mfma(void *, const void *, const int8_t *, const void *, int, int, int, int, hipStream_t) {
+    return fail(MYNN_ERR_UNSUPPORTED, "dequant_matmul: matrix-core GEMM not built yet");
+}
+}  // namespace mynn

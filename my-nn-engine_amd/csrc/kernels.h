@@ -1,0 +1,40 @@
+// Internal launchers shared between translation units (the C ABI wraps some of them; the decoder
+// executor calls them directly).
+#pragma once
+#include "mynn_common.h"
+
+namespace mynn {
+
+// gemv.hip -- one activation row, T in == T out
+template <typename T>
+int gemv_norm(void *out, const void *x, const void *norm_w, float eps, const int8_t *wq, const void *scale,
+              int N, int K, hipStream_t s);
+template <typename T>
+int gemv_residual(void *out, const void *act, const int8_t *wq, const void *scale, const void *residual,
+                  int N, int K, hipStream_t s);
+template <typename T>
+int gemv_norm_swiglu(void *out, const void *x, const void *norm_w, float eps, const int8_t *wq,
+                     const void *scale, int N, int K, hipStream_t s);
+int dequant_gemv_dispatch(void *out, const void *act, const int8_t *wq, const void *scale, int M, int N, int K,
+                          int act_dtype, int out_dtype, hipStream_t s);
+
+// gemm.hip -- matrix-core DequantMatMul, M >= 16, 16-bit types
+int dequant_gemm_mfma(void *out, const void *act, const int8_t *wq, const void *scale, int M, int N, int K,
+                      int dtype, hipStream_t s);
+
+// elementwise.hip
+template <typename T> int argmax_rows(int32_t *out, const void *logits, int rows, int n, hipStream_t s);
+template <typename T>
+int embed_dequant(void *out, const int8_t *table, const void *scale, const int64_t *ids, int n_ids, int vocab,
+                  int hidden, hipStream_t s);
+
+// rope_kv.hip -- RoPE of q and k plus the KV-cache append, from the fused qkv projection output.
+// qkv [B*S, (Hq+2*Hkv)*D] token-major; q_out [B*S, Hq*D]; caches [B,Hkv,max_seq,D];
+// position[S] selects the table row; rows land at cache positions past+s where past is *d_past
+// when d_past != nullptr, else past_host.
+template <typename T>
+int rope_kv_append(void *q_out, void *k_cache, void *v_cache, const void *qkv, const void *cos_t, const void *sin_t,
+                   const int64_t *position, const int32_t *d_past, int past_host, int B, int S, int Hq, int Hkv, int D,
+                   int max_seq, hipStream_t s);
+
+}  // namespace mynn

@@ -38,6 +38,15 @@ def max_abs_rel(got, want):
     return float(np.max(np.abs(got - want) / np.maximum(np.abs(want), floor)))
 
 
+def max_err_rel_to_max(got, want):
+    """max|x-y| / max|y|: the error relative to the tensor's magnitude.  Used for results that
+    pass through many 16-bit roundings (whole-decoder logits), where elements near zero carry an
+    absolute error set by the large ones."""
+    got = np.asarray(got, np.float64).ravel()
+    want = np.asarray(want, np.float64).ravel()
+    return float(np.max(np.abs(got - want)) / max(float(np.max(np.abs(want))), 1e-30))
+
+
 @pytest.fixture(scope="session")
 def golden_dir():
     return GOLDEN

@@ -41,3 +41,32 @@ def to_host(t):
 
 def f32(a, dt):
     return orc.to_f32(a, dt)
+
+
+def greedy_compare(ref, dec, prompt, n_new, dt):
+    """Runs the GPU decoder greedily (prompt fed token by token, as LlmSession does without a
+    prefill session) and the oracle on the SAME token stream (teacher-forced with the GPU's
+    choices, so both always see the same context).  Returns (gpu_ids, oracle_ids, near_ties):
+    oracle_ids[i] is the oracle's greedy choice at step i; near_ties lists the steps where the two
+    differ together with the oracle's logit gap between its choice and the GPU's, in units of the
+    16-bit spacing at the top logit."""
+    ulp = {orc.F32: 2.0 ** -23, orc.BF16: 2.0 ** -8, orc.F16: 2.0 ** -11}[dt]
+    gpu_ids, ref_ids, near = [], [], []
+    stream = list(prompt)
+    pos = 0
+    tok_gpu = None
+    while len(gpu_ids) < n_new:
+        t = stream[pos]
+        logits = ref.forward([t], [pos], pos, pos + 1, False)[0]
+        nxt, _ = dec.step([t], [pos], pos, pos + 1)
+        pos += 1
+        if pos >= len(prompt):
+            lf = orc.to_f32(logits, dt)
+            r = orc.argmax_last(logits, dt)
+            gpu_ids.append(nxt[0])
+            ref_ids.append(r)
+            if r != nxt[0]:
+                gap = float(lf[r] - lf[nxt[0]])
+                near.append((len(gpu_ids) - 1, gap / (ulp * max(abs(float(lf[r])), 1e-30))))
+            stream.append(nxt[0])
+    return gpu_ids, ref_ids, near

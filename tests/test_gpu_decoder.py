@@ -1,0 +1,148 @@
+"""End-to-end parity of the decoder executor (model_init / model / LlmSession) against the
+oracle and the reference's own known answer on its tiny random Llama."""
+import numpy as np
+import pytest
+
+import oracle as orc
+import llm_weights
+from conftest import max_abs_rel, max_err_rel_to_max
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def g():
+    import gpu_util
+
+    return gpu_util
+
+
+def dev_weights(g, w, dt):
+    out = {}
+    for k, v in w.items():
+        out[k] = (g.to_dev(v[0]), g.to_dev(v[1], dt)) if isinstance(v, tuple) else g.to_dev(v, dt)
+    return out
+
+
+SMALL = dict(n_layers=3, hidden=256, n_heads=8, n_kv_heads=2, head_dim=32, ffn=704, vocab=1000, max_seq=96,
+             eps=1e-5, rope_theta=10000.0)
+
+
+@pytest.mark.parametrize("dt", [orc.BF16, orc.F16])
+def test_tiny_llama_random_golden_ids_on_gpu(g, dt):
+    """crates/llm/tests/tinyllama_random.rs:20-24: prompt "Hello" -> 8 exact ids (un-quantised
+    checkpoint, narrowed to the 16-bit type)."""
+    cfg, w, golden = llm_weights.tiny_llama_random(dt)
+    dec = g.mynn.Decoder(cfg, dev_weights(g, w, dt))
+    llm = g.mynn.LlmSession(dec, eos=1)
+    ids = llm.generate_ids(golden["prompt_ids"], len(golden["expected_new_ids"]))
+    assert ids == golden["expected_new_ids"]
+    assert llm.past_len == len(golden["prompt_ids"]) + len(ids) - 1
+    llm.close(), dec.close()
+
+
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+def test_int8_decoder_step_logits_and_kv_vs_oracle(g, dt):
+    cfg, w = llm_weights.synthetic_int8(SMALL, dt, seed=7)
+    ref = orc.Model(cfg, w)
+    dec = g.mynn.Decoder(cfg, dev_weights(g, w, dt))
+    st = dec.stats()
+    assert st["graph"], "the decode step must replay a captured hipGraph"
+    assert st["launches_per_step"] <= 2 + 6 * cfg["n_layers"] + 3
+    toks = [5, 999, 123, 0, 77]
+    for i, t in enumerate(toks):
+        want = ref.forward([t], [i], i, i + 1, False)
+        nxt, got = dec.step([t], [i], i, i + 1, want_logits=True)
+        assert max_err_rel_to_max(g.f32(got, dt), g.f32(want, dt)) <= 1e-2, i
+        assert nxt[0] == orc.argmax_last(got[0], dt)
+    # KV rows written by the fused RoPE + append kernel
+    for l in range(cfg["n_layers"]):
+        k_ref, v_ref = ref.kv_cache(l)
+        k_gpu, v_gpu = g.to_host(dec.kv[l][0])[0], g.to_host(dec.kv[l][1])[0]
+        n = len(toks)
+        assert max_err_rel_to_max(g.f32(k_gpu[:, :n], dt), g.f32(k_ref[:, :n], dt)) <= 1e-2
+        assert max_err_rel_to_max(g.f32(v_gpu[:, :n], dt), g.f32(v_ref[:, :n], dt)) <= 1e-2
+        assert not k_gpu[:, n:].any() and not v_gpu[:, n:].any()
+    # the reference ABI entry point returns the same logits
+    l2 = dec.model([3], [5], 5, 6)
+    _, l3 = dec.step([3], [5], 5, 6, want_logits=True)
+    assert np.array_equal(l2, l3)
+    dec.close()
+
+
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+def test_int8_greedy_tokens_vs_oracle_small(g, dt):
+    """Greedy ids of the HIP path against the oracle on a small int8 model.  The oracle is
+    teacher-forced with the GPU's tokens; any step where the two disagree must be a tie at
+    16-bit resolution in the ORACLE's own logits (a few spacings of the storage type), which is
+    the only way two f32-summation orders can pick different tokens."""
+    cfg, w = llm_weights.synthetic_int8(SMALL, dt, seed=11)
+    ref = orc.Model(cfg, w)
+    rng = np.random.default_rng(5)
+    prompt = rng.integers(0, cfg["vocab"], 24).tolist()
+    dec = g.mynn.Decoder(cfg, dev_weights(g, w, dt))
+    got, want, near = g.greedy_compare(ref, dec, prompt, 48, dt)
+    assert all(abs(gap) <= 8.0 for _, gap in near), near
+    assert len(near) <= 4, near
+    # LlmSession drives the same steps; the device-resident decode loop repeats them
+    llm = g.mynn.LlmSession(dec)
+    assert llm.generate_ids(prompt, 48) == got
+    assert llm.past_len == len(prompt) + 48 - 1
+    first = None
+    for i, t in enumerate(prompt):
+        first, _ = dec.step([t], [i], i, i + 1)
+    loop = dec.decode_loop(first[0], len(prompt), 47)
+    assert [first[0]] + loop == got
+    llm.close(), dec.close()
+
+
+def test_generate_bookkeeping_and_errors(g):
+    dt = orc.F16
+    cfg, w = llm_weights.synthetic_int8(dict(SMALL, max_seq=16), dt, seed=3)
+    dec = g.mynn.Decoder(cfg, dev_weights(g, w, dt))
+    llm = g.mynn.LlmSession(dec)
+    with pytest.raises(g.mynn.MynnError):  # PromptTooLong
+        llm.generate_ids(list(range(17)), 1)
+    assert llm.generate_ids([], 4) == []
+    ids = llm.generate_ids([1, 2, 3, 4, 5], 100)  # stops when the cache is full
+    assert llm.past_len == 16 and len(ids) == 12
+    llm.reset()
+    assert llm.past_len == 0
+    with pytest.raises(g.mynn.MynnError):
+        dec.step([cfg["vocab"]], [0], 0, 1)  # token outside the vocabulary
+    with pytest.raises(g.mynn.MynnError):
+        dec.step([1], [16], 0, 1)  # position outside the RoPE table
+    llm.close(), dec.close()
+
+
+def test_mock_step_session_follows_logit_table(g):
+    """crates/llm/tests/mock_decode.rs: a 6-token logit table, prompt [0,1,2] -> [3,4,5,0,1];
+    past_len counts every decode step; a stop rewinds it."""
+    import ctypes as C
+    import json
+    import os
+
+    from conftest import GOLDEN
+
+    table = json.load(open(os.path.join(GOLDEN, "mock_decode", "expected_sequence.json")))
+    vocab = table["vocab"]
+    calls = []
+
+    def step(user, token, past_len):
+        calls.append((token, past_len))
+        return (token + 1) % vocab
+
+    cb = g.mynn.STEP_FN(step)
+    h = g.mynn.lib().mynn_llm_create_with_step(cb, None, 16, 999)
+    prompt = np.array([0, 1, 2], np.int64)
+    out = np.empty(5, np.int64)
+    n = g.mynn.lib().mynn_llm_generate_ids(h, prompt.ctypes.data_as(C.c_void_p), 3, 5, out.ctypes.data_as(C.c_void_p))
+    assert n == 5 and out.tolist() == [3, 4, 5, 0, 1]
+    assert out.tolist() == table["sequence"][2:7]
+    assert g.mynn.lib().mynn_llm_past_len(h) == 7  # 3 prompt steps + 4 fed-back tokens
+    assert [c[1] for c in calls] == list(range(7))
+    g.mynn.lib().mynn_llm_set_past_len(h, 5)  # stop-string rewind
+    assert g.mynn.lib().mynn_llm_past_len(h) == 5
+    g.mynn.lib().mynn_llm_reset(h)
+    assert g.mynn.lib().mynn_llm_past_len(h) == 0
+    g.mynn.lib().mynn_llm_destroy(h)
