@@ -1,0 +1,199 @@
+#!/usr/bin/env python3
+"""Headline benchmark: batch-1 greedy decode of a TinyLlama-1.1B-shape int8 model on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one decode step (one token) through the HIP decoder executor; the K timed steps are
+replays of the captured hipGraph with inputs, weights and KV cache resident in HBM.  Prints ONE
+JSON line: decode tok/s, the roofline of the dominant kernel (HIP-event timing of the same
+launches), and a CPU baseline (the oracle, a port of the reference CPU backend) timed on the
+host cores of the same box.
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+TINYLLAMA = dict(n_layers=22, hidden=2048, n_heads=32, n_kv_heads=4, head_dim=64, ffn=5632, vocab=32000,
+                 max_seq=384, eps=1e-5, rope_theta=10000.0)
+PROMPT_LEN = 128
+
+
+def make_weights(cfg, dt, seed):
+    """Seeded random-init weights generated on the device: f32 ~ N(0, 0.02), quantised per output
+    channel with the reference rule (crates/llm/src/quantize.rs:124-169: scale = amax/127,
+    q = clamp(round_half_away(w/scale), -128, 127)); norm weights 1."""
+    import torch
+
+    tdt = {1: torch.bfloat16, 2: torch.float16}[dt]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed)
+    H, F, V = cfg["hidden"], cfg["ffn"], cfg["vocab"]
+    QD, KD = cfg["n_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
+
+    def lin(n, k):
+        w = torch.randn((n, k), generator=gen, device="cuda", dtype=torch.float32) * 0.02
+        amax = w.abs().amax(dim=1, keepdim=True)
+        scale = torch.where(amax == 0, torch.ones_like(amax), amax / 127.0)
+        r = w / scale
+        q = (torch.sign(r) * torch.floor(r.abs() + 0.5)).clamp_(-128, 127).to(torch.int8)
+        return q.contiguous(), scale.reshape(-1).to(tdt).contiguous()
+
+    ones = torch.ones((H,), dtype=tdt, device="cuda")
+    w = {"embed": lin(V, H), "lm_head": lin(V, H), "final_norm": ones}
+    shapes = {"q": (QD, H), "k": (KD, H), "v": (KD, H), "o": (H, QD), "gate": (F, H), "up": (F, H), "down": (H, F)}
+    for l in range(cfg["n_layers"]):
+        for k, (n, kk) in shapes.items():
+            w["layers.%d.%s" % (l, k)] = lin(n, kk)
+        w["layers.%d.norm1" % l] = ones
+        w["layers.%d.norm2" % l] = ones
+    return w
+
+
+def to_host_weights(w):
+    import numpy as np
+    import torch
+
+    def h(t):
+        if t.dtype in (torch.float16, torch.bfloat16):
+            return t.view(torch.int16).cpu().numpy().view(np.uint16)
+        return t.cpu().numpy()
+
+    return {k: (h(v[0]), h(v[1])) if isinstance(v, tuple) else h(v) for k, v in w.items()}
+
+
+def algorithmic_bytes_per_token(cfg, eb, context):
+    """int8 weights + scales of every linear, embedding row, KV rows read at `context` and the
+    row written."""
+    H, F, V = cfg["hidden"], cfg["ffn"], cfg["vocab"]
+    QD, KD = cfg["n_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
+    per_layer_w = QD * H + 2 * KD * H + H * QD + 2 * F * H + H * F
+    per_layer_s = (QD + 2 * KD + H + 2 * F + H) * eb
+    w = cfg["n_layers"] * (per_layer_w + per_layer_s) + V * H + V * eb
+    kv = cfg["n_layers"] * 2 * KD * eb * (context + 1)
+    return w + kv + H + eb
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--dtype", choices=["f16", "bf16"], default="f16")
+    ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-steps", type=int, default=96)
+    ap.add_argument("--check-tokens", type=int, default=0,
+                    help="also compare the first N greedy tokens with the oracle (slow: CPU decode)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives are built)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    mynn = importlib.import_module("my-nn-engine_amd")
+    dt = {"f16": mynn.F16, "bf16": mynn.BF16}[args.dtype]
+    eb = 2
+    cfg = dict(TINYLLAMA, dtype=dt)
+    K, W = args.steps, args.warmup
+    assert PROMPT_LEN + max(K, W) <= cfg["max_seq"], "steps/warmup do not fit max_seq %d" % cfg["max_seq"]
+
+    weights = make_weights(cfg, dt, args.seed)
+    torch.cuda.synchronize()
+    dec = mynn.Decoder(cfg, weights)
+    stats = dec.stats()
+    rng = np.random.default_rng(args.seed)
+    prompt = rng.integers(0, cfg["vocab"], PROMPT_LEN).tolist()
+
+    # prompt through the decode path, token by token (the reference's path without a prefill session)
+    first = None
+    for i, t in enumerate(prompt):
+        first, _ = dec.step([t], [i], i, i + 1)
+    first = first[0]
+
+    if W > 0:
+        dec.decode_loop(first, PROMPT_LEN, W)  # untimed; its KV rows are overwritten below
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    toks = dec.decode_loop(first, PROMPT_LEN, K)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    generated = [first] + toks[:-1]
+    ms_per_step = elapsed * 1e3 / K
+    tok_s = K / elapsed
+
+    # ---- roofline of the dominant kernel: HIP events around every launch of eager steps at
+    # contexts spread over the timed range, on the executor's own stream
+    agg = {}
+    n_prof = 8
+    for j in range(n_prof):
+        past = PROMPT_LEN + (j * (K - 1)) // max(n_prof - 1, 1)
+        for name, ms, nbytes in dec.profile_step(generated[min(past - PROMPT_LEN, K - 1)], past):
+            a = agg.setdefault(name, [0, 0.0, 0.0])
+            a[0] += 1
+            a[1] += ms
+            a[2] += nbytes
+    gemv = {k: v for k, v in agg.items() if k.startswith("gemv_")}
+    dom = max(gemv, key=lambda k: gemv[k][1])
+    calls, ms_tot, bytes_tot = gemv[dom]
+    achieved = bytes_tot / (ms_tot * 1e-3) / 1e9
+    all_gemv_gbs = sum(v[2] for v in gemv.values()) / (sum(v[1] for v in gemv.values()) * 1e-3) / 1e9
+    step_bytes = algorithmic_bytes_per_token(cfg, eb, PROMPT_LEN + K // 2)
+
+    out = {
+        "metric": "decode tok/s bs1 TinyLlama-shape int8; dequant-GEMV HBM GB/s vs peak",
+        "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32 accumulate over int8 weights, %s activations/KV" % args.dtype, "data": "synthetic",
+        "config": {"workload": "configs[2]: TinyLlama-1.1B-shape int8 decoder, batch 1 greedy decode, 128 prompt tokens "
+                               "fed through the decode path then %d generated (timed: the generated tokens)" % K,
+                   "prompt_len": PROMPT_LEN, "max_seq": cfg["max_seq"], "launches_per_step": stats["launches_per_step"],
+                   "hipgraph": stats["graph"], "seed": args.seed,
+                   "step_algorithmic_bytes": step_bytes,
+                   "step_hbm_frac": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "bytes_per_launch": bytes_tot / calls, "avg_launch_us": round(ms_tot / calls * 1e3, 3),
+                     "all_gemv_GBs": round(all_gemv_gbs, 1)},
+    }
+
+    if not args.no_cpu_baseline:
+        import oracle as orc
+
+        hw = to_host_weights(weights)
+        ref = orc.Model(dict(cfg), hw)
+        n_cpu = args.cpu_steps
+        ref.past_len = 0
+        stream = prompt + generated
+        # bounded sample: the first n_cpu decode steps of the same token stream
+        t0 = time.perf_counter()
+        last = None
+        for i in range(n_cpu):
+            last = ref.decode_step(stream[i])
+        cpu_elapsed = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": round(n_cpu / cpu_elapsed, 3), "unit": "tok/s", "cores": orc.get_threads(),
+                               "kind": "port",
+                               "sample": "first %d decode steps (contexts 0..%d) of the same model and token stream, "
+                                         "C port of the reference CPU backend, OpenMP over N" % (n_cpu, n_cpu - 1)}
+        if args.check_tokens:
+            n = min(args.check_tokens, K)
+            ref2 = orc.Model(dict(cfg), hw)
+            want = ref2.generate(prompt, n)
+            out["config"]["tokens_identical_to_oracle"] = (want == generated[:n])
+            out["config"]["tokens_checked"] = n
+    dec.close()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

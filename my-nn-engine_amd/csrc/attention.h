@@ -14,6 +14,11 @@ struct AttnParams {
     const int32_t *d_active;  // device value (graph replay)
     int q_pos_offset;         // host value, used when d_active == nullptr
     int nsplit;
+    int slice;                // key rows per slice (gridDim.y slices cover the cache)
+    // fused decode form: raw qkv projection row(s) [B, (Hq+2*Hkv)*D], RoPE tables, device position;
+    // K and V then are the caches the new row is appended to
+    const void *qkv, *cos_t, *sin_t;
+    const int64_t *d_pos;
     float *part_o;            // [B*Hq*Sq, nsplit, D]
     float *part_ml;           // [B*Hq*Sq, nsplit, 2]
     unsigned *counters;       // [B*Hkv*Sq], zero between launches
@@ -33,7 +38,8 @@ inline void attn_token_major_layout(AttnParams &p, int D) {
     p.q_rs = p.o_rs = (long)p.Hq * D;
 }
 
-int attn_pick_nsplit(int B, int Hkv, int Sq, int kv_len);
+void attn_plan(int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, int *slice, int *nsplit);
+bool attention_fused_supported(int D, int G);
 size_t attn_scratch_bytes(int B, int Hq, int Sq, int D, int nsplit);
 size_t attn_counter_bytes(int B, int Hkv, int Sq);
 int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *scratch, void *counters, hipStream_t s);

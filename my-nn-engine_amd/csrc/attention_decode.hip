@@ -2,174 +2,246 @@
 //
 // Replaces the reference's attention_decode (attention.cuh:495-606), which walks the cache rows
 // serially with two block barriers per key and re-reads K/V once per query head.  Here one
-// workgroup serves ALL query heads of a KV head (so K/V are read once per group), the cache
-// length is split over gridDim.y workgroups, every lane streams 16-byte pieces of K and V rows,
-// and the online-softmax states (m, l, o) are merged lane-group -> wave -> workgroup -> split.
-// The last workgroup of a (batch, kv head, row) to finish merges the splits (a counter in
-// device memory; nobody spins).
+// workgroup of 512 threads serves ALL query heads of a KV head over one slice of the cache:
+//   1. every lane issues all of its 16-byte K and V loads for the slice at once (one HBM latency),
+//   2. K stays in registers: a group of D/8 lanes owns a key, dots its piece with all G query
+//      heads and reduces inside the group; scores go to LDS,
+//   3. V is parked in LDS; one wave per query head does max / exp / sum over the slice,
+//   4. thread (head, d) accumulates sum_k p[head,k] * V[k,d] from LDS -- no cross-lane merging.
+// Longer caches are cut into slices over gridDim.y; the last workgroup of a (batch, kv head, row)
+// to finish merges the slices (a counter in device memory; nobody spins).
 //
-// The same kernel with gridDim.z = Sq is the correct-but-plain path for Sq > 1 (causal rows get
-// their own key bound); the matrix-core prefill kernel lives in attention_prefill.hip.
+// FUSE form (decoder executor, one new token): the kernel also applies RoPE to q and to the new
+// k row, appends k/v to the cache and attends to the new row from registers -- the reference's
+// ~16 launches for Slice/Neg/Concat/Mul/Add RoPE (crates/llm/src/builder.rs:402-438), the
+// transposes and the two kvcache_update launches (kvcache_update.cuh:6-26) disappear.
+//
+// The same kernel with gridDim.z = Sq is the plain path for Sq > 1 (each causal row gets its own
+// key bound); the matrix-core prefill kernel lives in attention_prefill.hip.
+#include <type_traits>
+
 #include "attention.h"
 
 namespace mynn {
 
+constexpr int kAttnThreads = 512;
+constexpr int kAttnWaves = kAttnThreads / 64;
+constexpr int kAttnNI = 8;  // key rows per lane group and slice, at most
 
-constexpr int kAttnThreads = 256;
-constexpr int kAttnWaves = 4;
+template <typename TKV, int EPL> struct ChunkOf { using type = uint32_t; static constexpr bool vec = false; };
+template <> struct ChunkOf<bf16_t, 8> { using type = U4; static constexpr bool vec = true; };
+template <> struct ChunkOf<f16_t, 8> { using type = U4; static constexpr bool vec = true; };
+template <> struct ChunkOf<int8_t, 8> { using type = uint2; static constexpr bool vec = true; };
 
-__device__ inline void merge_state(float &m, float &l, float *o, int n, float m2, float l2, const float *o2) {
-    float mn = fmaxf(m, m2);
-    float c1 = (m == -INFINITY) ? 0.f : fast_exp(m - mn);
-    float c2 = (m2 == -INFINITY) ? 0.f : fast_exp(m2 - mn);
-    l = l * c1 + l2 * c2;
-    for (int i = 0; i < n; i++) o[i] = o[i] * c1 + o2[i] * c2;
-    m = mn;
-}
-
-template <typename T, int D, int G, bool KVI8>
+template <typename T, int D, int G, bool KVI8, bool FUSE>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p) {
-    constexpr int EPL = D >= 8 ? 8 : D;  // elements of a key row per lane
-    constexpr int LPK = D / EPL;         // lanes per key row
-    constexpr int KPW = 64 / LPK;        // keys per wave pass
-    static_assert(D % EPL == 0 && LPK <= 64 && (LPK & (LPK - 1)) == 0, "head_dim must be a power of two");
-    __shared__ float sm_o[kAttnWaves][G][D];
-    __shared__ float sm_ml[kAttnWaves][G][2];
+    constexpr int EPL = D >= 8 ? 8 : D;      // elements of a key row per lane
+    constexpr int LPK = D / EPL;             // lanes per key row
+    constexpr int GPB = kAttnThreads / LPK;  // key rows per pass of the workgroup
+    static_assert(D % EPL == 0 && (LPK & (LPK - 1)) == 0 && LPK <= 64, "head_dim must be a power of two");
+    using TKV = typename std::conditional<KVI8, int8_t, T>::type;
+    using Chunk = typename ChunkOf<TKV, EPL>::type;
+    constexpr bool kVec = ChunkOf<TKV, EPL>::vec;
+
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ float q_s[G][D];
+    __shared__ float new_s[2][D];  // FUSE: rotated k row and v row of the new token (values rounded to T)
+    __shared__ float ml_s[G][2];
     __shared__ int sm_last;
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int ks = lane / LPK, dc = lane % LPK;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int grp = tid / LPK, dc = tid % LPK;
     const int bhkv = blockIdx.x, split = blockIdx.y, sq = blockIdx.z;
     const int b = bhkv / p.Hkv, hkv = bhkv % p.Hkv;
     const int Sq = p.Sq;
 
-    int active = p.d_active ? *p.d_active : p.active;
-    int qoff = p.d_active ? active - Sq : p.q_pos_offset;
+    const int active = p.d_active ? *p.d_active : p.active;
+    const int qoff = p.d_active ? active - Sq : p.q_pos_offset;
     int bound = active;
     if (p.is_causal) bound = min(bound, qoff + sq + 1);
     bound = min(bound, p.cache_len);
-    // key range of this split: equal chunks, rounded up to whole workgroup passes
-    constexpr int PASS = kAttnWaves * KPW;
-    int chunk = (bound + p.nsplit - 1) / p.nsplit;
-    chunk = (chunk + PASS - 1) / PASS * PASS;
-    const int k0 = split * chunk;
-    const int k1 = min(bound, k0 + chunk);
+    const int nmax = p.slice;  // key rows per slice (multiple of GPB, <= GPB * kAttnNI)
+    const int k0 = split * nmax;
+    const int k1 = min(bound, k0 + nmax);
+    const int n = max(k1 - k0, 0);
+    const int new_row = FUSE ? active - 1 : -1;  // cache row of the token being decoded
 
-    const T *Q = (const T *)p.q;
-    float q[G][EPL];
-#pragma unroll
-    for (int g = 0; g < G; g++) {
-        const size_t qo = (size_t)b * p.q_bs + (size_t)(hkv * G + g) * p.q_hs + (size_t)sq * p.q_rs + dc * EPL;
-#pragma unroll
-        for (int i = 0; i < EPL; i++) q[g][i] = Elem<T>::ld(Q, qo + i);
-    }
-    float m[G], l[G], o[G][EPL];
-#pragma unroll
-    for (int g = 0; g < G; g++) {
-        m[g] = -INFINITY;
-        l[g] = 0.f;
-#pragma unroll
-        for (int i = 0; i < EPL; i++) o[g][i] = 0.f;
-    }
+    TKV *v_s = (TKV *)smem;                                        // [nmax][D]
+    float *sc = (float *)(smem + (size_t)nmax * D * sizeof(TKV));  // [G][nmax]
+    float *vsc_s = sc + (size_t)G * nmax;                          // [nmax] (int8 KV: per-token v scale)
 
+    // ---- 1. all K / V loads of the slice
     const size_t kv_base = (size_t)bhkv * p.cache_len;
-    for (int kk = k0 + wave * KPW + ks; kk < k1; kk += PASS) {
-        float kf[EPL], vf[EPL];
-        float ksc = 1.f, vsc = 1.f;
-        const size_t ro = (kv_base + kk) * D + dc * EPL;
-        if constexpr (KVI8) {
-            if constexpr (EPL == 8) {
-                const uint2 kr = *(const uint2 *)((const int8_t *)p.k + ro);
-                const uint2 vr = *(const uint2 *)((const int8_t *)p.v + ro);
-                const uint32_t kw[2] = {kr.x, kr.y}, vw[2] = {vr.x, vr.y};
+    Chunk kreg[kAttnNI], vreg[kAttnNI];
+    float kfl[kVec ? 1 : kAttnNI][kVec ? 1 : EPL], vfl[kVec ? 1 : kAttnNI][kVec ? 1 : EPL];
 #pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    kf[i] = (float)(int8_t)((kw[i >> 2] >> (8 * (i & 3))) & 0xFF);
-                    vf[i] = (float)(int8_t)((vw[i >> 2] >> (8 * (i & 3))) & 0xFF);
-                }
+    for (int i = 0; i < kAttnNI; i++) {
+        const int key = k0 + grp + i * GPB;
+        if (key < k1 && key != new_row) {
+            const size_t ro = (kv_base + key) * D + dc * EPL;
+            if constexpr (kVec) {
+                kreg[i] = *(const Chunk *)((const TKV *)p.k + ro);
+                vreg[i] = *(const Chunk *)((const TKV *)p.v + ro);
             } else {
 #pragma unroll
-                for (int i = 0; i < EPL; i++) {
-                    kf[i] = (float)((const int8_t *)p.k)[ro + i];
-                    vf[i] = (float)((const int8_t *)p.v)[ro + i];
+                for (int e = 0; e < EPL; e++) {
+                    if constexpr (KVI8) {
+                        kfl[i][e] = (float)((const int8_t *)p.k)[ro + e];
+                        vfl[i][e] = (float)((const int8_t *)p.v)[ro + e];
+                    } else {
+                        kfl[i][e] = Elem<T>::ld((const T *)p.k, ro + e);
+                        vfl[i][e] = Elem<T>::ld((const T *)p.v, ro + e);
+                    }
                 }
             }
-            ksc = Elem<T>::ld((const T *)p.k_scale, kv_base + kk);
-            vsc = Elem<T>::ld((const T *)p.v_scale, kv_base + kk);
-        } else {
-            if constexpr (sizeof(T) == 2 && EPL == 8) {
-                const U4 kr = *(const U4 *)((const T *)p.k + ro);
-                const U4 vr = *(const U4 *)((const T *)p.v + ro);
-                widen8<T>(kr, kf);
-                widen8<T>(vr, vf);
-            } else {
-#pragma unroll
-                for (int i = 0; i < EPL; i++) {
-                    kf[i] = Elem<T>::ld((const T *)p.k, ro + i);
-                    vf[i] = Elem<T>::ld((const T *)p.v, ro + i);
-                }
-            }
-        }
-#pragma unroll
-        for (int g = 0; g < G; g++) {
-            float part = 0.f;
-#pragma unroll
-            for (int i = 0; i < EPL; i++) part = fmaf(q[g][i], kf[i], part);
-            part = group_sum<LPK>(part);
-            if constexpr (KVI8) part *= ksc;
-            const float s = part * p.scale;
-            const float mn = fmaxf(m[g], s);
-            const float corr = fast_exp(m[g] - mn);  // exp(-inf) = 0 on the first key
-            const float e = fast_exp(s - mn);
-            l[g] = fmaf(l[g], corr, e);
-            const float ev = KVI8 ? e * vsc : e;
-#pragma unroll
-            for (int i = 0; i < EPL; i++) o[g][i] = fmaf(ev, vf[i], o[g][i] * corr);
-            m[g] = mn;
         }
     }
 
-    // ---- merge the KPW key slots of the wave (lanes that share dc)
-#pragma unroll
-    for (int off = LPK; off < 64; off <<= 1) {
-#pragma unroll
-        for (int g = 0; g < G; g++) {
-            float m2 = __shfl_xor(m[g], off, 64), l2 = __shfl_xor(l[g], off, 64);
-            float o2[EPL];
-#pragma unroll
-            for (int i = 0; i < EPL; i++) o2[i] = __shfl_xor(o[g][i], off, 64);
-            merge_state(m[g], l[g], o[g], EPL, m2, l2, o2);
+    // ---- 0. query rows (and, FUSE, the new k/v rows) into LDS while the loads fly
+    if constexpr (FUSE) {
+        const int half = D / 2;
+        const int width = (p.Hq + 2 * p.Hkv) * D;
+        const T *row = (const T *)p.qkv + (size_t)b * width;
+        const size_t tab = (size_t)(*p.d_pos) * D;
+        const T *cos_t = (const T *)p.cos_t, *sin_t = (const T *)p.sin_t;
+        // G query heads + 1 key head to rotate: (G+1) * D/2 pairs; then D values of v to copy
+        for (int idx = tid; idx < (G + 1) * half; idx += kAttnThreads) {
+            const int h = idx / half, j = idx % half;
+            const T *src = h < G ? row + (size_t)(hkv * G + h) * D : row + (size_t)(p.Hq + hkv) * D;
+            const float xl = Elem<T>::ld(src, j), xh = Elem<T>::ld(src, j + half);
+            const float cl = Elem<T>::ld(cos_t, tab + j), ch = Elem<T>::ld(cos_t, tab + j + half);
+            const float sl = Elem<T>::ld(sin_t, tab + j), sh = Elem<T>::ld(sin_t, tab + j + half);
+            const float lo = Elem<T>::rnd(xl * cl - xh * sl), hi = Elem<T>::rnd(xh * ch + xl * sh);
+            if (h < G) {
+                q_s[h][j] = lo;
+                q_s[h][j + half] = hi;
+            } else {
+                new_s[0][j] = lo;
+                new_s[0][j + half] = hi;
+                if (split == 0) {  // one workgroup appends the row
+                    T *kc = (T *)p.k + (kv_base + new_row) * D;
+                    Elem<T>::st(kc, j, lo);
+                    Elem<T>::st(kc, j + half, hi);
+                }
+            }
         }
-    }
-    if (ks == 0) {
-#pragma unroll
-        for (int g = 0; g < G; g++) {
-#pragma unroll
-            for (int i = 0; i < EPL; i++) sm_o[wave][g][dc * EPL + i] = o[g][i];
-            if (dc == 0) { sm_ml[wave][g][0] = m[g]; sm_ml[wave][g][1] = l[g]; }
+        for (int d = tid; d < D; d += kAttnThreads) {
+            const T *src = row + (size_t)(p.Hq + p.Hkv + hkv) * D;
+            new_s[1][d] = Elem<T>::ld(src, d);
+            if (split == 0) ((T *)p.v)[(kv_base + new_row) * D + d] = src[d];
+        }
+    } else {
+        for (int idx = tid; idx < G * D; idx += kAttnThreads) {
+            const int g = idx / D, d = idx % D;
+            const size_t qo = (size_t)b * p.q_bs + (size_t)(hkv * G + g) * p.q_hs + (size_t)sq * p.q_rs + d;
+            q_s[g][d] = Elem<T>::ld((const T *)p.q, qo);
         }
     }
     __syncthreads();
 
-    // ---- merge the waves; thread handles (g, d) pairs
+    // ---- 2. scores: group of LPK lanes per key, all G heads
+    float q[G][EPL];
+#pragma unroll
+    for (int g = 0; g < G; g++)
+#pragma unroll
+        for (int e = 0; e < EPL; e++) q[g][e] = q_s[g][dc * EPL + e];
+#pragma unroll
+    for (int i = 0; i < kAttnNI; i++) {
+        const int key = k0 + grp + i * GPB;
+        if (key < k1) {
+            float kf[EPL], vf[EPL];
+            if (FUSE && key == new_row) {
+#pragma unroll
+                for (int e = 0; e < EPL; e++) {
+                    kf[e] = new_s[0][dc * EPL + e];
+                    vf[e] = new_s[1][dc * EPL + e];
+                }
+            } else if constexpr (kVec && !KVI8) {
+                widen8<T>(kreg[i], kf);
+                widen8<T>(vreg[i], vf);
+            } else if constexpr (kVec && KVI8) {
+                const uint32_t kw[2] = {kreg[i].x, kreg[i].y}, vw[2] = {vreg[i].x, vreg[i].y};
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    kf[e] = (float)(int8_t)((kw[e >> 2] >> (8 * (e & 3))) & 0xFF);
+                    vf[e] = (float)(int8_t)((vw[e >> 2] >> (8 * (e & 3))) & 0xFF);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < EPL; e++) {
+                    kf[e] = kfl[kVec ? 0 : i][kVec ? 0 : e];
+                    vf[e] = vfl[kVec ? 0 : i][kVec ? 0 : e];
+                }
+            }
+            // park V (storage type) for phase 4
+            TKV *vrow = v_s + (size_t)(key - k0) * D + dc * EPL;
+#pragma unroll
+            for (int e = 0; e < EPL; e++) {
+                if constexpr (KVI8) vrow[e] = (int8_t)vf[e];
+                else Elem<T>::st((T *)vrow, e, vf[e]);
+            }
+            float ksc = 1.f;
+            if constexpr (KVI8) {
+                ksc = Elem<T>::ld((const T *)p.k_scale, kv_base + key);
+                if (dc == 0) vsc_s[key - k0] = Elem<T>::ld((const T *)p.v_scale, kv_base + key);
+            }
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                float part = 0.f;
+#pragma unroll
+                for (int e = 0; e < EPL; e++) part = fmaf(q[g][e], kf[e], part);
+                part = group_sum<LPK>(part);
+                if constexpr (KVI8) part *= ksc;
+                if (dc == g % LPK) sc[(size_t)g * nmax + (key - k0)] = part * p.scale;
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- 3. softmax statistics: one wave per head
+    for (int g = wave; g < G; g += kAttnWaves) {
+        float *row = sc + (size_t)g * nmax;
+        float m = -INFINITY;
+        for (int k = lane; k < n; k += 64) m = fmaxf(m, row[k]);
+        m = wave_max(m);
+        float l = 0.f;
+        for (int k = lane; k < n; k += 64) {
+            const float e = fast_exp(row[k] - m);
+            l += e;
+            row[k] = KVI8 ? e * vsc_s[k] : e;
+        }
+        l = wave_sum(l);
+        if (lane == 0) {
+            ml_s[g][0] = m;
+            ml_s[g][1] = l;
+        }
+    }
+    __syncthreads();
+
+    // ---- 4. o[g,d] = sum_k p[g,k] * V[k,d]; thread owns (g,d)
     T *out = (T *)p.out;
     const size_t row_base = (size_t)(b * p.Hq + hkv * G) * Sq + sq;  // + g*Sq
-    for (int idx = threadIdx.x; idx < G * D; idx += kAttnThreads) {
+    for (int idx = tid; idx < G * D; idx += kAttnThreads) {
         const int g = idx / D, d = idx % D;
-        float mt = -INFINITY;
-#pragma unroll
-        for (int w = 0; w < kAttnWaves; w++) mt = fmaxf(mt, sm_ml[w][g][0]);
-        float lt = 0.f, ot = 0.f;
-#pragma unroll
-        for (int w = 0; w < kAttnWaves; w++) {
-            float mw = sm_ml[w][g][0];
-            float c = (mw == -INFINITY) ? 0.f : fast_exp(mw - mt);
-            lt += sm_ml[w][g][1] * c;
-            ot += sm_o[w][g][d] * c;
+        const float *pr = sc + (size_t)g * nmax;
+        auto vld = [&](int k) -> float {
+            if constexpr (KVI8) return (float)((const int8_t *)v_s)[(size_t)k * D + d];
+            else return Elem<T>::ld((const T *)v_s, (size_t)k * D + d);
+        };
+        float acc0 = 0.f, acc1 = 0.f, acc2 = 0.f, acc3 = 0.f;
+        int k = 0;
+        for (; k + 3 < n; k += 4) {
+            acc0 = fmaf(pr[k], vld(k), acc0);
+            acc1 = fmaf(pr[k + 1], vld(k + 1), acc1);
+            acc2 = fmaf(pr[k + 2], vld(k + 2), acc2);
+            acc3 = fmaf(pr[k + 3], vld(k + 3), acc3);
         }
+        for (; k < n; k++) acc0 = fmaf(pr[k], vld(k), acc0);
+        const float ot = (acc0 + acc1) + (acc2 + acc3);
+        const float mt = ml_s[g][0], lt = ml_s[g][1];
         const size_t row = row_base + (size_t)g * Sq;
-        const size_t oo = (size_t)b * p.o_bs + (size_t)(hkv * G + g) * p.o_hs + (size_t)sq * p.o_rs + d;
         if (p.nsplit == 1) {
+            const size_t oo = (size_t)b * p.o_bs + (size_t)(hkv * G + g) * p.o_hs + (size_t)sq * p.o_rs + d;
             Elem<T>::st(out, oo, ot / lt);
         } else {
             p.part_o[(row * p.nsplit + split) * D + d] = ot;
@@ -181,17 +253,17 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
     }
     if (p.nsplit == 1) return;
 
-    // ---- last workgroup of this (batch, kv head, row) merges the splits
+    // ---- 5. last workgroup of this (batch, kv head, row) merges the slices
     __threadfence();
     __syncthreads();
-    if (threadIdx.x == 0) {
+    if (tid == 0) {
         unsigned prev = atomicAdd(&p.counters[(size_t)bhkv * Sq + sq], 1u);
         sm_last = (prev == (unsigned)p.nsplit - 1);
     }
     __syncthreads();
     if (!sm_last) return;
     __threadfence();
-    for (int idx = threadIdx.x; idx < G * D; idx += kAttnThreads) {
+    for (int idx = tid; idx < G * D; idx += kAttnThreads) {
         const int g = idx / D, d = idx % D;
         const size_t row = row_base + (size_t)g * Sq;
         const float *ml = p.part_ml + row * p.nsplit * 2;
@@ -200,54 +272,91 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
         for (int s = 0; s < p.nsplit; s++) mt = fmaxf(mt, __builtin_nontemporal_load(&ml[2 * s]));
         float lt = 0.f, ot = 0.f;
         for (int s = 0; s < p.nsplit; s++) {
-            float ms = __builtin_nontemporal_load(&ml[2 * s]);
-            float c = (ms == -INFINITY) ? 0.f : fast_exp(ms - mt);
-            lt += __builtin_nontemporal_load(&ml[2 * s + 1]) * c;
-            ot += __builtin_nontemporal_load(&po[s * D + d]) * c;
+            const float ms = __builtin_nontemporal_load(&ml[2 * s]);
+            const float c = (ms == -INFINITY) ? 0.f : fast_exp(ms - mt);
+            lt = fmaf(__builtin_nontemporal_load(&ml[2 * s + 1]), c, lt);
+            ot = fmaf(__builtin_nontemporal_load(&po[s * D + d]), c, ot);
         }
         const size_t oo = (size_t)b * p.o_bs + (size_t)(hkv * G + g) * p.o_hs + (size_t)sq * p.o_rs + d;
         Elem<T>::st(out, oo, ot / lt);
     }
-    if (threadIdx.x == 0) p.counters[(size_t)bhkv * Sq + sq] = 0;  // ready for the next launch
+    if (tid == 0) p.counters[(size_t)bhkv * Sq + sq] = 0;  // ready for the next launch
 }
 
-template <typename T, int D, bool KVI8>
-static int launch_g(const AttnParams &p, hipStream_t s) {
-    dim3 grid(p.B * p.Hkv, p.nsplit, p.Sq), block(kAttnThreads);
-    const int G = p.Hq / p.Hkv;
-    switch (G) {
-    case 1: hipLaunchKernelGGL((attn_decode_kernel<T, D, 1, KVI8>), grid, block, 0, s, p); break;
-    case 2: hipLaunchKernelGGL((attn_decode_kernel<T, D, 2, KVI8>), grid, block, 0, s, p); break;
-    case 4: hipLaunchKernelGGL((attn_decode_kernel<T, D, 4, KVI8>), grid, block, 0, s, p); break;
-    case 8: hipLaunchKernelGGL((attn_decode_kernel<T, D, 8, KVI8>), grid, block, 0, s, p); break;
-    default: return fail(MYNN_ERR_UNSUPPORTED, "attention: %d query heads per kv head (supported: 1,2,4,8)", G);
+// LDS the kernel may use per workgroup for the V slice, the scores and the v scales
+constexpr size_t kAttnLdsBudget = 96 * 1024;
+
+static int slice_rows(int D, int G, size_t kv_elem) {
+    const int EPL = D >= 8 ? 8 : D, LPK = D / EPL, GPB = kAttnThreads / LPK;
+    size_t per_row = (size_t)D * kv_elem + (size_t)G * 4 + 4;
+    int rows = (int)(kAttnLdsBudget / per_row);
+    rows = rows / GPB * GPB;
+    if (rows > GPB * kAttnNI) rows = GPB * kAttnNI;
+    if (rows < GPB) rows = GPB;
+    return rows;
+}
+static size_t slice_lds_bytes(int rows, int D, int G, size_t kv_elem) {
+    return (size_t)rows * D * kv_elem + (size_t)G * rows * 4 + (size_t)rows * 4;
+}
+
+template <typename T, int D, int G, bool KVI8, bool FUSE>
+static int launch_one(const AttnParams &p, hipStream_t s) {
+    const size_t kv_elem = KVI8 ? 1 : sizeof(T);
+    const size_t lds = slice_lds_bytes(p.slice, D, G, kv_elem);
+    static bool attr_set = false;
+    if (!attr_set) {
+        MYNN_HIP(hipFuncSetAttribute((const void *)attn_decode_kernel<T, D, G, KVI8, FUSE>,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kAttnLdsBudget + 16384)));
+        attr_set = true;
     }
+    dim3 grid(p.B * p.Hkv, p.nsplit, p.Sq), block(kAttnThreads);
+    hipLaunchKernelGGL((attn_decode_kernel<T, D, G, KVI8, FUSE>), grid, block, lds, s, p);
     return launch_status("attn_decode_kernel");
 }
 
-template <typename T, bool KVI8>
-static int launch_d(const AttnParams &p, int D, hipStream_t s) {
-    switch (D) {
-    case 4: return launch_g<T, 4, KVI8>(p, s);
-    case 8: return launch_g<T, 8, KVI8>(p, s);
-    case 16: return launch_g<T, 16, KVI8>(p, s);
-    case 32: return launch_g<T, 32, KVI8>(p, s);
-    case 64: return launch_g<T, 64, KVI8>(p, s);
-    case 128: return launch_g<T, 128, KVI8>(p, s);
-    default: return fail(MYNN_ERR_UNSUPPORTED, "attention: head_dim %d (supported: 4,8,16,32,64,128)", D);
+template <typename T, int D, bool KVI8, bool FUSE>
+static int launch_g(const AttnParams &p, hipStream_t s) {
+    switch (p.Hq / p.Hkv) {
+    case 1: return launch_one<T, D, 1, KVI8, FUSE>(p, s);
+    case 2: return launch_one<T, D, 2, KVI8, FUSE>(p, s);
+    case 4: return launch_one<T, D, 4, KVI8, FUSE>(p, s);
+    case 8: return launch_one<T, D, 8, KVI8, FUSE>(p, s);
+    default:
+        return fail(MYNN_ERR_UNSUPPORTED, "attention: %d query heads per kv head (supported: 1,2,4,8)", p.Hq / p.Hkv);
     }
 }
 
-// number of key-range splits for a launch: enough workgroups to cover the chip, at least 64
-// keys each, at most 64 splits
-int attn_pick_nsplit(int B, int Hkv, int Sq, int kv_len) {
-    int groups = B * Hkv * Sq;
-    int want = (512 + groups - 1) / groups;
-    int by_len = (kv_len + 63) / 64;
-    int n = want < by_len ? want : by_len;
+template <typename T, bool KVI8, bool FUSE>
+static int launch_d(const AttnParams &p, int D, hipStream_t s) {
+    if constexpr (!FUSE) {
+        switch (D) {
+        case 4: return launch_g<T, 4, KVI8, FUSE>(p, s);
+        case 8: return launch_g<T, 8, KVI8, FUSE>(p, s);
+        case 16: return launch_g<T, 16, KVI8, FUSE>(p, s);
+        default: break;
+        }
+    }
+    switch (D) {
+    case 32: return launch_g<T, 32, KVI8, FUSE>(p, s);
+    case 64: return launch_g<T, 64, KVI8, FUSE>(p, s);
+    case 128: return launch_g<T, 128, KVI8, FUSE>(p, s);
+    default: break;
+    }
+    return fail(MYNN_ERR_UNSUPPORTED, "attention: head_dim %d (supported: 4,8,16,32,64,128; fused decode: 32,64,128)", D);
+}
+
+bool attention_fused_supported(int D, int G) {
+    return (D == 32 || D == 64 || D == 128) && (G == 1 || G == 2 || G == 4 || G == 8);
+}
+
+// Slice length and number of slices for a launch.  kv_len = longest key range any row can have.
+void attn_plan(int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, int *slice, int *nsplit) {
+    const size_t kv_elem = kv_int8 ? 1 : dtype_size(dtype);
+    const int rows = slice_rows(D, Hq / Hkv, kv_elem);
+    int n = (kv_len + rows - 1) / rows;
     if (n < 1) n = 1;
-    if (n > 64) n = 64;
-    return n;
+    *slice = rows;
+    *nsplit = n;
 }
 size_t attn_scratch_bytes(int B, int Hq, int Sq, int D, int nsplit) {
     size_t rows = (size_t)B * Hq * Sq;
@@ -268,9 +377,18 @@ int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *s
         p.part_ml = p.part_o + rows * p.nsplit * D;
         p.counters = (unsigned *)counters;
     }
+    const bool fuse = p.qkv != nullptr;
     return dispatch_dtype(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
-        return kv_int8 ? launch_d<T, true>(p, D, s) : launch_d<T, false>(p, D, s);
+        if constexpr (sizeof(T) == 2) {
+            if (fuse) {
+                if (kv_int8) return fail(MYNN_ERR_UNSUPPORTED, "fused decode attention: int8 KV");
+                return launch_d<T, false, true>(p, D, s);
+            }
+        } else {
+            if (fuse) return fail(MYNN_ERR_UNSUPPORTED, "fused decode attention needs a 16-bit type");
+        }
+        return kv_int8 ? launch_d<T, true, false>(p, D, s) : launch_d<T, false, false>(p, D, s);
     });
 }
 
@@ -294,7 +412,6 @@ static int ensure(Grown &g, size_t bytes, bool zero, hipStream_t s) {
     return 0;
 }
 
-
 }  // namespace mynn
 
 using namespace mynn;
@@ -311,6 +428,8 @@ extern "C" int mynn_attention(void *out, const void *Q, const void *K, const voi
     MYNN_REQUIRE(!kv_int8 || (k_scale && v_scale), MYNN_ERR_INVALID, "attention: int8 KV needs k_scale and v_scale");
     MYNN_REQUIRE(d_active || (active_seq_kv >= 1), MYNN_ERR_INVALID, "attention: active_seq_kv=%d", active_seq_kv);
     MYNN_REQUIRE(aligned16(K) && aligned16(V), MYNN_ERR_INVALID, "attention: K and V must be 16-byte aligned");
+    MYNN_REQUIRE(dtype_ok(dtype), MYNN_ERR_INVALID, "attention: dtype %d", dtype);
+    MYNN_REQUIRE(Sq <= 65535, MYNN_ERR_UNSUPPORTED, "attention: Sq=%d too large for the per-row kernel", Sq);
     AttnParams p{};
     p.out = out; p.q = Q; p.k = K; p.v = V; p.k_scale = k_scale; p.v_scale = v_scale; p.scale = scale;
     p.is_causal = is_causal; p.B = B; p.Sq = Sq; p.Hq = num_q_heads; p.Hkv = num_kv_heads;
@@ -320,7 +439,8 @@ extern "C" int mynn_attention(void *out, const void *Q, const void *K, const voi
     if (Sq > 1 && attention_prefill_supported(p, head_dim, dtype, kv_int8))
         return attention_prefill_launch(p, head_dim, dtype, st);
     int kv_len = d_active ? cache_seq_len : (active_seq_kv < cache_seq_len ? active_seq_kv : cache_seq_len);
-    p.nsplit = attn_pick_nsplit(B, num_kv_heads, Sq, kv_len);
+    attn_plan(num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, kv_len, &p.slice, &p.nsplit);
+    MYNN_REQUIRE(p.nsplit <= 65535, MYNN_ERR_UNSUPPORTED, "attention: cache of %d rows needs too many slices", kv_len);
     if (p.nsplit > 1) {
         int rc = ensure(g_scratch, attn_scratch_bytes(B, num_q_heads, Sq, head_dim, p.nsplit), false, st);
         if (rc) return rc;

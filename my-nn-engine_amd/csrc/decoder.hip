@@ -42,21 +42,6 @@ __global__ void swiglu_rows_kernel(T *out, const T *gate, const T *up, size_t n)
     Elem<T>::st(out, i, (g * sig) * Elem<T>::ld(up, i));
 }
 
-// device-side bookkeeping between two replayed decode steps: the greedy token becomes the next
-// input, position / past_len / active length move on by one
-__global__ void advance_kernel(int64_t *ids, int64_t *pos, int32_t *past, int32_t *active, const int32_t *next,
-                               int32_t *tokens, int32_t *step, int cap) {
-    if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    int t = next[0];
-    int i = *step;
-    if (i < cap) tokens[i] = t;
-    *step = i + 1;
-    ids[0] = t;
-    pos[0] += 1;
-    *past += 1;
-    *active += 1;
-}
-
 struct Lin {
     const void *w = nullptr;      // int8 [N,K] when scale != nullptr, else T [N,K]
     const void *scale = nullptr;  // T [N]
@@ -90,7 +75,7 @@ struct Model {
     int64_t *d_ids = nullptr, *d_pos = nullptr;
     int32_t *d_past = nullptr, *d_active = nullptr, *d_next = nullptr, *d_tokens = nullptr, *d_step = nullptr;
     void *attn_scratch = nullptr, *attn_counters = nullptr;
-    int nsplit = 1;
+    int nsplit = 1, slice = 0;
     int token_cap = 0;
     // host staging (pinned)
     char *h_stage = nullptr;
@@ -137,7 +122,7 @@ static int linear_rows(Model &m, void *out, const void *act, const Lin &l, int M
     const double eb = sizeof(T);
     if (l.scale) {
         note(m, name, (double)l.N * l.K + l.N * eb + (double)M * l.K * eb + (double)M * l.N * eb);
-        if (M >= 16 && l.K % 32 == 0)
+        if (M >= 16 && l.K % 8 == 0)
             return dequant_gemm_mfma(out, act, (const int8_t *)l.w, l.scale, M, l.N, l.K, m.cfg.dtype, m.stream);
         return dequant_gemv_dispatch(out, act, (const int8_t *)l.w, l.scale, M, l.N, l.K, m.cfg.dtype, m.cfg.dtype,
                                      m.stream);
@@ -186,20 +171,28 @@ static int enqueue_step(Model &m) {
             TRY(mynn_rms_norm(m.nrm, m.x, L.norm1, rows, H, c.eps, c.dtype, s));
             TRY(linear_rows<T>(m, m.qkv, m.nrm, L.qkv, rows, "linear_qkv"));
         }
-        note(m, "rope_kv_append", (double)rows * (QD + 2 * KD) * 2 * eb);
-        TRY(rope_kv_append<T>(m.q, L.k_cache, L.v_cache, m.qkv, m.cos_t, m.sin_t, m.d_pos, m.d_past, 0, B, S, Hq, Hkv,
-                              D, c.max_seq, s));
         {
             AttnParams p{};
             p.out = m.attn; p.q = m.q; p.k = L.k_cache; p.v = L.v_cache; p.scale = softmax_scale;
             p.is_causal = S > 1; p.B = B; p.Sq = S; p.Hq = Hq; p.Hkv = Hkv; p.cache_len = c.max_seq;
-            p.d_active = m.d_active; p.nsplit = m.nsplit;
+            p.d_active = m.d_active; p.nsplit = m.nsplit; p.slice = m.slice;
             attn_token_major_layout(p, D);
-            // bytes: K and V rows of the active prefix (upper bound max_seq is not known on the host
-            // under replay; the caller scales by the real context when it reports)
-            note(m, "attention", (double)B * (2.0 * QD * eb * S));
-            if (S > 1 && attention_prefill_supported(p, D, c.dtype, 0)) TRY(attention_prefill_launch(p, D, c.dtype, s));
-            else TRY(attention_decode_launch(p, D, c.dtype, 0, m.attn_scratch, m.attn_counters, s));
+            const bool fuse_attn = fused && attention_fused_supported(D, Hq / Hkv);
+            if (fuse_attn) {
+                // RoPE(q), RoPE(k), both cache appends and the attention in one launch
+                p.qkv = m.qkv; p.cos_t = m.cos_t; p.sin_t = m.sin_t; p.d_pos = m.d_pos;
+                note(m, "attention_rope_append", (double)(QD + 2 * KD) * eb + 2.0 * KD * eb + QD * eb);
+                TRY(attention_decode_launch(p, D, c.dtype, 0, m.attn_scratch, m.attn_counters, s));
+            } else {
+                note(m, "rope_kv_append", (double)rows * (QD + 2 * KD) * 2 * eb);
+                TRY(rope_kv_append<T>(m.q, L.k_cache, L.v_cache, m.qkv, m.cos_t, m.sin_t, m.d_pos, m.d_past, 0, B, S,
+                                      Hq, Hkv, D, c.max_seq, s));
+                // bytes: q in, out; the K/V rows read depend on the context, which the host does not
+                // know under replay -- callers add 2*KD*eb per cached row when they report
+                note(m, "attention", (double)rows * 2.0 * QD * eb);
+                if (S > 1 && attention_prefill_supported(p, D, c.dtype, 0)) TRY(attention_prefill_launch(p, D, c.dtype, s));
+                else TRY(attention_decode_launch(p, D, c.dtype, 0, m.attn_scratch, m.attn_counters, s));
+            }
         }
         if (fused) {
             note(m, "gemv_o_residual", (double)H * QD + H * eb + QD * eb + 2 * H * eb);
@@ -231,15 +224,13 @@ static int enqueue_step(Model &m) {
         TRY(mynn_rms_norm(m.nrm, m.x, m.final_norm, rows, H, c.eps, c.dtype, s));
         TRY(linear_rows<T>(m, m.logits, m.nrm, m.lm_head, rows, "linear_lm_head"));
     }
-    // greedy token of the last row of each sequence
-    note(m, "argmax_last", (double)B * V * eb);
-    for (int b = 0; b < B; b++)
-        TRY(argmax_rows<T>(m.d_next + b, (const T *)m.logits + ((size_t)b * S + (S - 1)) * V, 1, V, s));
-    if (rows == 1) {
-        note(m, "advance", 64);
-        hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(64), 0, s, m.d_ids, m.d_pos, m.d_past, m.d_active, m.d_next,
-                           m.d_tokens, m.d_step, m.token_cap);
-        TRY(launch_status("advance_kernel"));
+    // greedy token of the last row of each sequence; for a batch-1 decode step the same launch
+    // moves the device-side loop state on (token -> next input, position / past / active + 1)
+    note(m, rows == 1 ? "argmax_advance" : "argmax_last", (double)B * V * eb);
+    for (int b = 0; b < B; b++) {
+        AdvanceState adv{};
+        if (rows == 1) adv = AdvanceState{m.d_ids, m.d_pos, m.d_past, m.d_active, m.d_tokens, m.d_step, m.token_cap};
+        TRY(argmax_rows<T>(m.d_next + b, (const T *)m.logits + ((size_t)b * S + (S - 1)) * V, 1, V, adv, s));
     }
     if (m.profiling) {
         hipEvent_t e;
@@ -331,7 +322,7 @@ static int build(Model &m, void **init, void **state) {
 
     // ---- arena: every activation of one step, the device scalars, attention split scratch
     const int rows = c.batch * c.seq_q;
-    m.nsplit = attn_pick_nsplit(c.batch, c.n_kv_heads, c.seq_q, c.max_seq);
+    attn_plan(c.n_heads, c.n_kv_heads, c.head_dim, c.dtype, 0, c.max_seq, &m.slice, &m.nsplit);
     m.token_cap = c.max_seq + 8;
     ArenaPlan plan;
     size_t o_x = plan.take((size_t)rows * H * eb), o_x2 = plan.take((size_t)rows * H * eb);

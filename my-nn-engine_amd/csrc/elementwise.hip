@@ -1,7 +1,7 @@
 // The small memory-bound operators of the decoder: RMSNorm, RoPE, KV-cache updates (plain and
 // quantizing), DequantizeLinear, row gather, SwiGLU / Add groups, dynamic activation
 // quantisation and the greedy argmax.  All compute in f32 and round once at the store.
-#include "mynn_common.h"
+#include "kernels.h"
 
 namespace mynn {
 
@@ -202,47 +202,62 @@ __global__ __launch_bounds__(kEwThreads) void dynquant_kernel(void *y_, T *y_sca
 }
 
 // ---- greedy argmax, last maximum wins (reference crates/llm/src/session.rs:683-690) -----------
-// one workgroup of 1024 threads; (value, index) pairs ordered by value then by index
-__device__ inline void argmax_merge(float &v, int &i, float ov, int oi) {
-    if (ov > v || (ov == v && oi > i)) { v = ov; i = oi; }
+// one workgroup of 1024 threads per row, 16-byte loads; (value, index) ordered by value, then index
+__device__ inline void argmax_take(float &bv, int &bi, float v, int i) {
+    if (bi < 0 || v > bv || (v == bv && i > bi)) { bv = v; bi = i; }
 }
 template <typename T>
-__global__ __launch_bounds__(1024) void argmax_last_kernel(int32_t *out, const T *logits, int n) {
+__global__ __launch_bounds__(1024) void argmax_last_kernel(int32_t *out, const T *logits, int n, AdvanceState adv) {
     __shared__ float sv[16];
     __shared__ int si[16];
+    const T *row = logits + (size_t)blockIdx.x * n;
     float bv = -INFINITY;
     int bi = -1;
-    for (int i = threadIdx.x; i < n; i += 1024) {
-        float v = Elem<T>::ld(logits, i);
-        if (v >= bv || bi < 0) { bv = v; bi = i; }  // ascending i: >= keeps the last
+    if constexpr (sizeof(T) == 2) {
+        const int nvec = (((uintptr_t)row & 15) == 0) ? n / 8 : 0;
+        for (int c = threadIdx.x; c < nvec; c += 1024) {
+            float f[8];
+            widen8<T>(((const U4 *)row)[c], f);
+#pragma unroll
+            for (int e = 0; e < 8; e++) argmax_take(bv, bi, f[e], c * 8 + e);
+        }
+        for (int i = nvec * 8 + threadIdx.x; i < n; i += 1024) argmax_take(bv, bi, Elem<T>::ld(row, i), i);
+    } else {
+        for (int i = threadIdx.x; i < n; i += 1024) argmax_take(bv, bi, Elem<T>::ld(row, i), i);
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
         float ov = __shfl_xor(bv, off, 64);
         int oi = __shfl_xor(bi, off, 64);
-        if (oi >= 0 && (bi < 0 || ov > bv || (ov == bv && oi > bi))) { bv = ov; bi = oi; }
+        if (oi >= 0) argmax_take(bv, bi, ov, oi);
     }
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
     __syncthreads();
     if (threadIdx.x == 0) {
         for (int w = 1; w < 16; w++)
-            if (si[w] >= 0 && (bi < 0 || sv[w] > bv || (sv[w] == bv && si[w] > bi))) { bv = sv[w]; bi = si[w]; }
+            if (si[w] >= 0) argmax_take(bv, bi, sv[w], si[w]);
         out[blockIdx.x] = bi;
+        if (adv.ids) {
+            const int i = *adv.step;
+            if (i < adv.cap) adv.tokens[i] = bi;
+            *adv.step = i + 1;
+            adv.ids[0] = bi;
+            adv.pos[0] += 1;
+            *adv.past += 1;
+            *adv.active += 1;
+        }
     }
 }
 
-template <typename T> int argmax_rows(int32_t *out, const void *logits, int rows, int n, hipStream_t s) {
-    // one workgroup per row
-    const T *l = (const T *)logits;
-    for (int r = 0; r < rows; r++) {
-        hipLaunchKernelGGL(argmax_last_kernel<T>, dim3(1), dim3(1024), 0, s, out + r, l + (size_t)r * n, n);
-    }
+template <typename T>
+int argmax_rows(int32_t *out, const void *logits, int rows, int n, AdvanceState adv, hipStream_t s) {
+    hipLaunchKernelGGL(argmax_last_kernel<T>, dim3(rows), dim3(1024), 0, s, out, (const T *)logits, n, adv);
     return launch_status("argmax_last_kernel");
 }
-template int argmax_rows<bf16_t>(int32_t *, const void *, int, int, hipStream_t);
-template int argmax_rows<f16_t>(int32_t *, const void *, int, int, hipStream_t);
-template int argmax_rows<float>(int32_t *, const void *, int, int, hipStream_t);
+template int argmax_rows<bf16_t>(int32_t *, const void *, int, int, AdvanceState, hipStream_t);
+template int argmax_rows<f16_t>(int32_t *, const void *, int, int, AdvanceState, hipStream_t);
+template int argmax_rows<float>(int32_t *, const void *, int, int, AdvanceState, hipStream_t);
 
 template <typename T>
 int embed_dequant(void *out, const int8_t *table, const void *scale, const int64_t *ids, int n_ids, int vocab,
@@ -380,6 +395,6 @@ extern "C" int mynn_argmax_last(int32_t *out_index, const void *logits, int n, i
     MYNN_REQUIRE(out_index && logits && n > 0, MYNN_ERR_INVALID, "argmax_last: bad operand");
     return dispatch_dtype(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
-        return argmax_rows<T>(out_index, logits, 1, n, as_stream(s));
+        return argmax_rows<T>(out_index, logits, 1, n, AdvanceState{}, as_stream(s));
     });
 }

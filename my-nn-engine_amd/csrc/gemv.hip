@@ -150,6 +150,114 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv_kernel(GemvParams p
     }
 }
 
+// Decode form (one activation row): every lane issues ALL of its weight loads -- R rows x NC
+// 16-byte chunks -- before anything else, so a whole per-CU slice of the matrix is in flight at
+// once and the RMSNorm / activation staging runs under the HBM latency.  NC = ceil(K / 1024).
+template <typename T, int R, int NC, int EPI, bool NORM>
+__global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(GemvParams p) {
+    extern __shared__ float act_lds[];  // [K]
+    __shared__ float red[kGemvWaves];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int K = p.K, N = p.N;
+    const int nchunks = K >> 4;
+    const int row0 = (blockIdx.x * kGemvWaves + wave) * R;
+
+    U4 w[R][NC];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int row = row0 + r < N ? row0 + r : N - 1;
+        const U4 *wrow = (const U4 *)(p.wq + (size_t)row * K);
+#pragma unroll
+        for (int j = 0; j < NC; j++) {
+            const int c = lane + j * kWave;
+            if (c < nchunks) w[r][j] = __builtin_nontemporal_load(&wrow[c]);
+            else w[r][j] = U4{0u, 0u, 0u, 0u};
+        }
+    }
+
+    const T *act = (const T *)p.act;
+    if constexpr (NORM) {
+        float ss = 0.f;
+        for (int k = tid; k < K; k += kGemvThreads) {
+            float v = Elem<T>::ld(act, k);
+            act_lds[k] = v;
+            ss = fmaf(v, v, ss);
+        }
+        ss = wave_sum(ss);
+        if (lane == 0) red[wave] = ss;
+        __syncthreads();
+        float tot = 0.f;
+#pragma unroll
+        for (int i = 0; i < kGemvWaves; i++) tot += red[i];
+        const float inv = 1.0f / sqrtf(tot / (float)K + p.eps);
+        const T *nw = (const T *)p.norm_w;
+        for (int k = tid; k < K; k += kGemvThreads)
+            act_lds[k] = Elem<T>::rnd((act_lds[k] * inv) * Elem<T>::ld(nw, k));
+    } else {
+        for (int k = tid; k < K; k += kGemvThreads) act_lds[k] = Elem<T>::ld(act, k);
+    }
+    __syncthreads();
+    if (row0 >= N) return;
+
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.f;
+#pragma unroll
+    for (int j = 0; j < NC; j++) {
+        const int c = lane + j * kWave;
+        if (c < nchunks) {
+            float a[16];
+            const float4 *ap = (const float4 *)(act_lds + c * 16);
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                float4 t = ap[q];
+                a[4 * q] = t.x; a[4 * q + 1] = t.y; a[4 * q + 2] = t.z; a[4 * q + 3] = t.w;
+            }
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                float wf[16];
+                widen16_i8(w[r][j], wf);
+#pragma unroll
+                for (int i = 0; i < 16; i++) acc[r] = fmaf(a[i], wf[i], acc[r]);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = wave_sum(acc[r]);
+
+    const T *scale = (const T *)p.scale;
+    T *out = (T *)p.out;
+    if constexpr (EPI == EPI_SWIGLU) {
+#pragma unroll
+        for (int r = 0; r < R; r += 2) {
+            if (lane == r && row0 + r + 1 < N) {
+                float g = Elem<T>::rnd(acc[r] * Elem<T>::ld(scale, row0 + r));
+                float u = Elem<T>::rnd(acc[r + 1] * Elem<T>::ld(scale, row0 + r + 1));
+                float sig = 1.0f / (1.0f + expf(-g));
+                Elem<T>::st(out, (size_t)((row0 + r) >> 1), (g * sig) * u);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            if (lane == r && row0 + r < N) {
+                float y = acc[r] * Elem<T>::ld(scale, row0 + r);
+                if constexpr (EPI == EPI_RESIDUAL) y = Elem<T>::rnd(y) + Elem<T>::ld((const T *)p.residual, row0 + r);
+                Elem<T>::st(out, row0 + r, y);
+            }
+        }
+    }
+}
+
+template <typename T, int R, int NC, int EPI, bool NORM>
+static int launch_gemv1(const GemvParams &p, hipStream_t s) {
+    const int rows_per_block = kGemvWaves * R;
+    dim3 grid((p.N + rows_per_block - 1) / rows_per_block);
+    hipLaunchKernelGGL((dequant_gemv1_kernel<T, R, NC, EPI, NORM>), grid, dim3(kGemvThreads),
+                       (size_t)p.K * sizeof(float), s, p);
+    return launch_status("dequant_gemv1_kernel");
+}
+
 template <typename TA, typename TO, int R, int MB, int EPI, bool NORM>
 static int launch_gemv(const GemvParams &p, hipStream_t s) {
     const int rows_per_block = kGemvWaves * R;
@@ -211,6 +319,9 @@ __global__ __launch_bounds__(64) void dequant_matmul_naive_kernel(TO *out, const
     if (lane == 0) Elem<TO>::st(out, (size_t)m * N + n, acc * Elem<TO>::ld(scale, n));
 }
 
+template <typename T, int EPI, bool NORM>
+static int gemv1_dispatch(const GemvParams &p, hipStream_t s);
+
 // scale-after-sum path for any act/out type pair the reference allows (f32 or 16-bit act;
 // out type = scale type)
 int dequant_gemv_dispatch(void *out, const void *act, const int8_t *wq, const void *scale, int M, int N,
@@ -226,6 +337,9 @@ int dequant_gemv_dispatch(void *out, const void *act, const int8_t *wq, const vo
         using TA = std::remove_pointer_t<decltype(ta)>;
         return dispatch_dtype(out_dtype, [&](auto *to) {
             using TO = std::remove_pointer_t<decltype(to)>;
+            if constexpr (std::is_same<TA, TO>::value && sizeof(TA) == 2) {
+                if (streaming && M == 1) return gemv1_dispatch<TA, EPI_PLAIN, false>(p, s);
+            }
             if (streaming) return gemv_small_m<TA, TO>(p, M, s);
             MYNN_REQUIRE(M <= 65535, MYNN_ERR_UNSUPPORTED, "dequant_matmul: M=%d too large for the plain kernel", M);
             hipLaunchKernelGGL((dequant_matmul_naive_kernel<TA, TO>), dim3(N, M), dim3(64), 0, s, (TO *)out,
@@ -236,6 +350,25 @@ int dequant_gemv_dispatch(void *out, const void *act, const int8_t *wq, const vo
 }
 
 // ---- fused decode variants used by the decoder executor (one activation row, T in == T out)
+// rows per wave: 4 for wide matrices, 2 otherwise (more workgroups for the narrow ones)
+template <typename T, int EPI, bool NORM>
+static int gemv1_dispatch(const GemvParams &p, hipStream_t s) {
+    const int nc = (p.K + 1023) / 1024;
+    const bool wide = pick_r(p.N) == 4;
+#define MYNN_GEMV1(NC_)                                                   \
+    return wide ? launch_gemv1<T, 4, NC_, EPI, NORM>(p, s) : launch_gemv1<T, 2, NC_, EPI, NORM>(p, s)
+    if (nc <= 1) { MYNN_GEMV1(1); }
+    if (nc <= 2) { MYNN_GEMV1(2); }
+    if (nc <= 4) { MYNN_GEMV1(4); }
+    if (nc <= 6) { MYNN_GEMV1(6); }
+    if (nc <= 8) { MYNN_GEMV1(8); }
+    if (nc <= 14) { MYNN_GEMV1(14); }
+#undef MYNN_GEMV1
+    // longer rows: the looping kernel
+    if (wide) return launch_gemv<T, T, 4, 1, EPI, NORM>(p, s);
+    return launch_gemv<T, T, 2, 1, EPI, NORM>(p, s);
+}
+
 template <typename T>
 int gemv_norm(void *out, const void *x, const void *norm_w, float eps, const int8_t *wq, const void *scale,
               int N, int K, hipStream_t s) {
@@ -244,8 +377,7 @@ int gemv_norm(void *out, const void *x, const void *norm_w, float eps, const int
     p.act_stride = K; p.out_stride = N;
     int rc = check_gemv(p, 1);
     if (rc) return rc;
-    if (pick_r(N) == 4) return launch_gemv<T, T, 4, 1, EPI_PLAIN, true>(p, s);
-    return launch_gemv<T, T, 2, 1, EPI_PLAIN, true>(p, s);
+    return gemv1_dispatch<T, EPI_PLAIN, true>(p, s);
 }
 template <typename T>
 int gemv_residual(void *out, const void *act, const int8_t *wq, const void *scale, const void *residual,
@@ -255,8 +387,7 @@ int gemv_residual(void *out, const void *act, const int8_t *wq, const void *scal
     p.act_stride = K; p.out_stride = N;
     int rc = check_gemv(p, 1);
     if (rc) return rc;
-    if (pick_r(N) == 4) return launch_gemv<T, T, 4, 1, EPI_RESIDUAL, false>(p, s);
-    return launch_gemv<T, T, 2, 1, EPI_RESIDUAL, false>(p, s);
+    return gemv1_dispatch<T, EPI_RESIDUAL, false>(p, s);
 }
 // wq/scale hold gate and up rows interleaved (row 2i = gate_i, row 2i+1 = up_i); N = 2*ffn
 template <typename T>
@@ -268,8 +399,7 @@ int gemv_norm_swiglu(void *out, const void *x, const void *norm_w, float eps, co
     MYNN_REQUIRE(N % 2 == 0, MYNN_ERR_INVALID, "gate/up rows must come in pairs (N=%d)", N);
     int rc = check_gemv(p, 1);
     if (rc) return rc;
-    if (pick_r(N) == 4) return launch_gemv<T, T, 4, 1, EPI_SWIGLU, true>(p, s);
-    return launch_gemv<T, T, 2, 1, EPI_SWIGLU, true>(p, s);
+    return gemv1_dispatch<T, EPI_SWIGLU, true>(p, s);
 }
 
 template int gemv_norm<bf16_t>(void *, const void *, const void *, float, const int8_t *, const void *, int, int, hipStream_t);

@@ -23,7 +23,16 @@ int dequant_gemm_mfma(void *out, const void *act, const int8_t *wq, const void *
                       int dtype, hipStream_t s);
 
 // elementwise.hip
-template <typename T> int argmax_rows(int32_t *out, const void *logits, int rows, int n, hipStream_t s);
+// device-side loop state of a batch-1 decode model; a null `ids` means "no bookkeeping"
+struct AdvanceState {
+    int64_t *ids, *pos;
+    int32_t *past, *active, *tokens, *step;
+    int cap;
+};
+// out[r] = index of the LAST maximum of logits row r; when adv.ids != nullptr the launch also
+// records the token and moves the decode loop on by one position
+template <typename T>
+int argmax_rows(int32_t *out, const void *logits, int rows, int n, AdvanceState adv, hipStream_t s);
 template <typename T>
 int embed_dequant(void *out, const int8_t *table, const void *scale, const int64_t *ids, int n_ids, int vocab,
                   int hidden, hipStream_t s);

@@ -39,11 +39,21 @@ template <> struct Elem<bf16_t> {
     __host__ __device__ static void st(bf16_t *p, size_t i, float v) { p[i].bits = f32_to_bf16_bits(v); }
     __host__ __device__ static float rnd(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
 };
+// f32 -> f16, round to nearest even, of a value that has ALREADY been rounded to f32.  The empty
+// asm keeps the compiler from folding the producing multiply into v_fma_mixlo_f16, which rounds
+// the exact product straight to f16 (one rounding) and so differs from "f32 result, then narrow"
+// (two roundings, what the reference's kernels do) whenever the f32 result is a tie.
+__host__ __device__ inline f16_t f32_to_f16(float v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("" : "+v"(v));
+#endif
+    return (f16_t)v;
+}
 template <> struct Elem<f16_t> {
     static constexpr int code = MYNN_F16;
     __host__ __device__ static float ld(const f16_t *p, size_t i) { return (float)p[i]; }
-    __host__ __device__ static void st(f16_t *p, size_t i, float v) { p[i] = (f16_t)v; }  // RNE
-    __host__ __device__ static float rnd(float v) { return (float)(f16_t)v; }
+    __host__ __device__ static void st(f16_t *p, size_t i, float v) { p[i] = f32_to_f16(v); }
+    __host__ __device__ static float rnd(float v) { return (float)f32_to_f16(v); }
 };
 
 inline size_t dtype_size(int dt) { return dt == MYNN_F32 ? 4 : 2; }
