@@ -92,6 +92,7 @@ _sig("orc_model_set_final_norm", None, _vp, _vp)
 _sig("orc_model_set_linear", None, _vp, _i, _i, Linear)
 _sig("orc_model_set_norm", None, _vp, _i, _i, _vp)
 _sig("orc_model_reset", None, _vp)
+_sig("orc_model_set_gemm_mode", None, _vp, _i)
 _sig("orc_model_past_len", _ll, _vp)
 _sig("orc_model_set_past_len", None, _vp, _ll)
 _sig("orc_model_forward", None, _vp, _vp, _vp, _sz, _ll, _ll, _i, _vp)
@@ -381,6 +382,10 @@ class Model:
 
     def reset(self):
         _lib.orc_model_reset(self._h)
+
+    def set_gemm_mode(self, mode):
+        """-1: CPU backend's kernel choice (default); 2: CUDA backend's."""
+        _lib.orc_model_set_gemm_mode(self._h, int(mode))
 
     @property
     def past_len(self):

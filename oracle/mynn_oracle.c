@@ -543,6 +543,7 @@ struct orc_model {
     struct orc_layer *layers;
     void *cos_t, *sin_t;
     long long past_len;
+    int gemm_mode; /* -1: CPU backend's dispatch; 2: CUDA backend's (M >= 16 -> W rounded first) */
     void *last_hidden;
     size_t last_S;
 };
@@ -550,6 +551,7 @@ struct orc_model {
 orc_model *orc_model_create(const orc_model_cfg *cfg) {
     orc_model *m = (orc_model *)calloc(1, sizeof(orc_model));
     m->cfg = *cfg;
+    m->gemm_mode = -1;
     size_t eb = esize(cfg->dtype);
     m->layers = (struct orc_layer *)calloc((size_t)cfg->n_layers, sizeof(struct orc_layer));
     size_t kvn = (size_t)cfg->n_kv_heads * (size_t)cfg->max_seq * (size_t)cfg->head_dim;
@@ -575,6 +577,7 @@ void orc_model_set_final_norm(orc_model *m, const void *w) { m->final_norm = w; 
 void orc_model_set_linear(orc_model *m, int layer, int which, orc_linear w) { m->layers[layer].lin[which] = w; }
 void orc_model_set_norm(orc_model *m, int layer, int which, const void *w) { m->layers[layer].norm[which] = w; }
 void orc_model_reset(orc_model *m) { m->past_len = 0; }
+void orc_model_set_gemm_mode(orc_model *m, int mode) { m->gemm_mode = mode; }
 long long orc_model_past_len(const orc_model *m) { return m->past_len; }
 void orc_model_set_past_len(orc_model *m, long long p) { m->past_len = p; }
 const void *orc_model_k_cache(const orc_model *m, int layer) { return m->layers[layer].k_cache; }
@@ -587,7 +590,11 @@ static void linear(const orc_model *m, void *out, const void *x, const orc_linea
                    size_t N, size_t K) {
     int dt = m->cfg.dtype;
     if (w->q) {
-        orc_dequant_matmul(out, x, w->q, w->scale, S, N, K, dt, dt, -1);
+        /* kernel choice per backend: CPU (translator.rs:3002-3115) M==1 fused decode else
+         * dequantise+sgemm; CUDA (cuda.rs:1518-1652) M>=16 && K%8==0 tensor cores else
+         * scale-after-sum */
+        int mode = m->gemm_mode == 2 ? ((S >= 16 && K % 8 == 0 && dt != ORC_F32) ? 2 : 0) : -1;
+        orc_dequant_matmul(out, x, w->q, w->scale, S, N, K, dt, dt, mode);
     } else {
         float *a = widen(x, S * K, dt);
         int nt = nthreads_for(N);

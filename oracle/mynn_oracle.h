@@ -164,6 +164,9 @@ void orc_model_set_linear(orc_model *m, int layer, int which, orc_linear w);
 /* which: 0 input_layernorm, 1 post_attention_layernorm */
 void orc_model_set_norm(orc_model *m, int layer, int which, const void *w);
 void orc_model_reset(orc_model *m);                 /* past_len = 0 (session.rs:303-305) */
+/* which backend's DequantMatMul kernel choice the linears follow: -1 the CPU backend's (default),
+ * 2 the CUDA backend's (rows >= 16: weight rounded to the 16-bit type before the product) */
+void orc_model_set_gemm_mode(orc_model *m, int mode);
 long long orc_model_past_len(const orc_model *m);
 void orc_model_set_past_len(orc_model *m, long long p);
 /* One graph run with S tokens: positions[s], writes KV rows past_len..past_len+S-1, attends
