@@ -1,11 +1,205 @@
-// Causal prefill attention on the matrix cores (replaces the reference's attention_tc,
-// attention.cuh:45-314).  Until that kernel is in, every Sq > 1 call takes the per-row
-// flash-decode path of attention_decode.hip.
+// Causal / full prefill attention on the matrix cores (flash-attention form), replacing the
+// reference's attention_tc (attention.cuh:45-314: mma.m16n8k16, S and P round-tripping through
+// shared memory, 16 lanes doing the softmax serially).
+//
+// One workgroup = 4 waves = 128 query rows of one (batch, query head); each wave owns 32 rows.
+// Per 32-key tile (staged once in LDS for the four waves, K row-major, V transposed):
+//   S^T = K . Q^T      v_mfma_f32_32x32x16: A = K rows from LDS, B = Q kept in registers
+//   softmax            each lane owns ONE query column and 16 of the 32 keys of the tile, so the
+//                      row max / sum are in-lane plus a single exchange with lane ^ 32
+//   O^T += V^T . P^T   the D-layout of S^T is already the B-operand layout of P^T (keys are
+//                      contracted in the permuted order 4g+0..3, 8+4g+0..3), so P never leaves
+//                      registers; A = V^T read from LDS with two 8-byte reads
+// The rescale factor of the online softmax is a per-lane scalar because O^T keeps the same query
+// column per lane.  Key tiles past a wave's last causal position are skipped.
 #include "attention.h"
+#include "mfma.h"
 
 namespace mynn {
-bool attention_prefill_supported(const AttnParams &, int, int, int) { return false; }
-int attention_prefill_launch(const AttnParams &, int, int, hipStream_t) {
-    return fail(MYNN_ERR_UNSUPPORTED, "attention: matrix-core prefill kernel not built");
+
+constexpr int kPfThreads = 256, kPfRows = 128, kPfKeys = 32;
+
+template <typename T, int D>
+__global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(AttnParams p) {
+    constexpr int LDK = D + 8;          // K tile row stride (elements): conflict-free 16-byte reads
+    constexpr int LDV = kPfKeys + 4;    // V^T tile row stride
+    constexpr int KS = D / 16;          // k-steps of the S^T product
+    constexpr int DT = D / 32;          // 32-row tiles of O^T
+    constexpr int CH = (kPfKeys * D / 8) / kPfThreads;  // 16-byte chunks per thread and tile (1 or 2)
+    static_assert(CH >= 1, "tile smaller than the workgroup");
+    __shared__ __align__(16) uint16_t Ks[2][kPfKeys * LDK];
+    __shared__ __align__(16) uint16_t Vt[2][D * LDV];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, g = lane >> 5;
+    const int bh = blockIdx.y, b = bh / p.Hq, h = bh % p.Hq;
+    const int G = p.Hq / p.Hkv, hkv = h / G;
+    const int Sq = p.Sq;
+    const int active = p.d_active ? *p.d_active : p.active;
+    const int qoff = p.d_active ? active - Sq : p.q_pos_offset;
+    const int kv_bound = min(active, p.cache_len);
+
+    const int q_blk = blockIdx.x * kPfRows;
+    const int qrow = q_blk + wave * 32 + col;           // this lane's query row
+    const int qrow_c = min(qrow, Sq - 1);
+    // keys this lane's query may see, and the furthest any row of the wave / workgroup may see
+    const int my_bound = p.is_causal ? min(kv_bound, qoff + qrow_c + 1) : kv_bound;
+    const int wave_last = min(q_blk + wave * 32 + 31, Sq - 1);
+    const int wave_bound = p.is_causal ? min(kv_bound, qoff + wave_last + 1) : kv_bound;
+    const int blk_last = min(q_blk + kPfRows - 1, Sq - 1);
+    const int blk_bound = p.is_causal ? min(kv_bound, qoff + blk_last + 1) : kv_bound;
+    const int ntiles = (blk_bound + kPfKeys - 1) / kPfKeys;
+
+    // Q^T fragments: B operand, lane (query col, g): d = 16*ks + 8*g .. +7
+    const T *Q = (const T *)p.q + (size_t)b * p.q_bs + (size_t)h * p.q_hs + (size_t)qrow_c * p.q_rs;
+    U4 qf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) qf[ks] = *(const U4 *)(Q + 16 * ks + 8 * g);
+
+    const T *Kg = (const T *)p.k + (size_t)(b * p.Hkv + hkv) * p.cache_len * D;
+    const T *Vg = (const T *)p.v + (size_t)(b * p.Hkv + hkv) * p.cache_len * D;
+    U4 rk[CH], rv[CH];
+    auto load_tile = [&](int t) {
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int chunk = tid + c * kPfThreads;
+            const int key = t * kPfKeys + chunk / (D / 8), dd = (chunk % (D / 8)) * 8;
+            if (key < blk_bound) {
+                rk[c] = *(const U4 *)(Kg + (size_t)key * D + dd);
+                rv[c] = *(const U4 *)(Vg + (size_t)key * D + dd);
+            } else {
+                rk[c] = U4{0u, 0u, 0u, 0u};
+                rv[c] = U4{0u, 0u, 0u, 0u};
+            }
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int chunk = tid + c * kPfThreads;
+            const int kk = chunk / (D / 8), dd = (chunk % (D / 8)) * 8;
+            *(U4 *)&Ks[buf][kk * LDK + dd] = rk[c];
+            const uint32_t w[4] = {rv[c].x, rv[c].y, rv[c].z, rv[c].w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                Vt[buf][(dd + 2 * i) * LDV + kk] = (uint16_t)(w[i] & 0xFFFFu);
+                Vt[buf][(dd + 2 * i + 1) * LDV + kk] = (uint16_t)(w[i] >> 16);
+            }
+        }
+    };
+
+    f16x_t o[DT];
+#pragma unroll
+    for (int t = 0; t < DT; t++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) o[t][e] = 0.f;
+    float m = -INFINITY, l = 0.f;
+
+    if (ntiles > 0) {
+        load_tile(0);
+        store_tile(0);
+    }
+    __syncthreads();
+    for (int t = 0; t < ntiles; t++) {
+        const int buf = t & 1;
+        if (t + 1 < ntiles) load_tile(t + 1);
+        const int k0 = t * kPfKeys;
+        if (k0 < wave_bound) {
+            // ---- S^T tile: rows = keys, cols = queries
+            f16x_t s;
+#pragma unroll
+            for (int e = 0; e < 16; e++) s[e] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                const U4 a = *(const U4 *)&Ks[buf][col * LDK + 16 * ks + 8 * g];
+                s = Mfma<T>::run(a, qf[ks], s);
+            }
+            // ---- online softmax for this lane's query over its 16 keys (+ partner lane's 16)
+            float mloc = -INFINITY;
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int key = k0 + 8 * (e >> 2) + 4 * g + (e & 3);
+                s[e] = key < my_bound ? s[e] * p.scale : -INFINITY;
+                mloc = fmaxf(mloc, s[e]);
+            }
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+            const float mn = fmaxf(m, mloc);
+            float corr = 1.f;
+            float pe[16];
+            if (mn == -INFINITY) {
+#pragma unroll
+                for (int e = 0; e < 16; e++) pe[e] = 0.f;
+            } else {
+                corr = fast_exp(m - mn);
+                float ls = 0.f;
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    pe[e] = fast_exp(s[e] - mn);
+                    ls += pe[e];
+                }
+                l = fmaf(l, corr, ls);
+                m = mn;
+            }
+#pragma unroll
+            for (int t2 = 0; t2 < DT; t2++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) o[t2][e] *= corr;
+            // ---- O^T += V^T . P^T, keys contracted in the order the D-layout delivers them
+#pragma unroll
+            for (int st = 0; st < 2; st++) {
+                const U4 pf = U4{pack2<T>(pe[8 * st + 0], pe[8 * st + 1]), pack2<T>(pe[8 * st + 2], pe[8 * st + 3]),
+                                 pack2<T>(pe[8 * st + 4], pe[8 * st + 5]), pack2<T>(pe[8 * st + 6], pe[8 * st + 7])};
+#pragma unroll
+                for (int t2 = 0; t2 < DT; t2++) {
+                    const uint16_t *vr = &Vt[buf][(32 * t2 + col) * LDV + 16 * st + 4 * g];
+                    const uint2 lo = *(const uint2 *)vr, hi = *(const uint2 *)(vr + 8);
+                    o[t2] = Mfma<T>::run(U4{lo.x, lo.y, hi.x, hi.y}, pf, o[t2]);
+                }
+            }
+        }
+        if (t + 1 < ntiles) {
+            store_tile(buf ^ 1);
+            __syncthreads();
+        }
+    }
+
+    // ---- out[query, d] = O^T[d, query] / l
+    l += __shfl_xor(l, 32, 64);
+    if (qrow < Sq) {
+        T *out = (T *)p.out + (size_t)b * p.o_bs + (size_t)h * p.o_hs + (size_t)qrow * p.o_rs;
+        const float inv = 1.0f / l;
+#pragma unroll
+        for (int t2 = 0; t2 < DT; t2++)
+#pragma unroll
+            for (int e4 = 0; e4 < 4; e4++) {
+                const int d = 32 * t2 + 8 * e4 + 4 * g;
+                uint2 w;
+                w.x = pack2<T>(o[t2][4 * e4 + 0] * inv, o[t2][4 * e4 + 1] * inv);
+                w.y = pack2<T>(o[t2][4 * e4 + 2] * inv, o[t2][4 * e4 + 3] * inv);
+                *(uint2 *)(out + d) = w;
+            }
+    }
 }
+
+bool attention_prefill_supported(const AttnParams &p, int D, int dtype, int kv_int8) {
+    if (kv_int8 || (dtype != MYNN_F16 && dtype != MYNN_BF16)) return false;
+    if (D != 64 && D != 128) return false;
+    if (p.Sq < 16) return false;  // a handful of rows: the per-row kernel wastes less
+    // 16-byte loads of Q rows and 8-byte stores of out rows
+    if ((p.q_rs % 8) || (p.q_hs % 8) || (p.q_bs % 8) || (p.o_rs % 4) || (p.o_hs % 4) || (p.o_bs % 4)) return false;
+    if (((uintptr_t)p.q & 15) || ((uintptr_t)p.out & 7) || ((uintptr_t)p.k & 15) || ((uintptr_t)p.v & 15)) return false;
+    return true;
+}
+
+int attention_prefill_launch(const AttnParams &p, int D, int dtype, hipStream_t s) {
+    MYNN_REQUIRE(p.B * p.Hq <= 65535, MYNN_ERR_UNSUPPORTED, "attention: batch*heads = %d exceeds the grid", p.B * p.Hq);
+    dim3 grid((p.Sq + kPfRows - 1) / kPfRows, p.B * p.Hq);
+    return dispatch_dtype16(dtype, [&](auto *t) {
+        using T = std::remove_pointer_t<decltype(t)>;
+        if (D == 64) hipLaunchKernelGGL((attn_prefill_kernel<T, 64>), grid, dim3(kPfThreads), 0, s, p);
+        else hipLaunchKernelGGL((attn_prefill_kernel<T, 128>), grid, dim3(kPfThreads), 0, s, p);
+        return launch_status("attn_prefill_kernel");
+    });
+}
+
 }  // namespace mynn

@@ -12,24 +12,9 @@
 // operands staged through padded LDS tiles (conflict-free 128-bit reads), next tile prefetched
 // into registers while the current one is multiplied.
 #include "kernels.h"
+#include "mfma.h"
 
 namespace mynn {
-
-typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
-typedef __bf16 b8_t __attribute__((ext_vector_type(8)));
-typedef float f16x_t __attribute__((ext_vector_type(16)));
-
-template <typename T> struct Mfma;
-template <> struct Mfma<f16_t> {
-    __device__ static f16x_t run(const U4 &a, const U4 &b, f16x_t c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8_t, a), __builtin_bit_cast(h8_t, b), c, 0, 0, 0);
-    }
-};
-template <> struct Mfma<bf16_t> {
-    __device__ static f16x_t run(const U4 &a, const U4 &b, f16x_t c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(b8_t, a), __builtin_bit_cast(b8_t, b), c, 0, 0, 0);
-    }
-};
 
 // ---- (1) dequantise: 8 weights per thread; rows are written with stride Kp (K rounded up to the
 // GEMM's K step) and zero padding

@@ -7,7 +7,7 @@ import pytest
 
 import oracle as orc
 import pbreader
-from conftest import GOLDEN, close_either, max_abs_rel
+from conftest import GOLDEN, close_either, max_abs_rel, max_err_rel_to_max
 
 pytestmark = pytest.mark.gpu
 SO = os.path.join(GOLDEN, "single_op")
@@ -155,3 +155,54 @@ def test_int8_kv_attention(g, dt):
     got = g.to_host(g.mynn.attention(g.to_dev(q, dt), g.to_dev(kc), g.to_dev(vc), 0.125, False, 200,
                                      k_scale=g.to_dev(ks, dt), v_scale=g.to_dev(vs, dt)))
     assert max_abs_rel(g.f32(got, dt), g.f32(want, dt)) <= 1e-2
+
+
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+@pytest.mark.parametrize("B,Hq,Hkv,S,D,past,causal", [
+    (1, 8, 2, 128, 64, 0, True),
+    (2, 4, 4, 100, 64, 0, True),      # ragged: rows past the last 128-row block, MHA
+    (1, 32, 4, 257, 64, 31, True),    # TinyLlama heads, a past, odd length
+    (1, 8, 8, 64, 128, 0, True),      # head_dim 128
+    (2, 16, 2, 96, 128, 40, True),    # 8 query heads per kv head, D=128
+    (1, 4, 2, 130, 64, 0, False),     # full (non-causal) attention
+    (1, 2, 1, 16, 64, 5, True),       # the smallest shape the matrix-core kernel takes
+])
+def test_prefill_attention_matrix_cores_vs_oracle(g, dt, B, Hq, Hkv, S, D, past, causal):
+    rng = np.random.default_rng(S * 131 + D + past)
+    L = past + S + 7  # cache longer than the active prefix
+    q = orc.to_storage(rng.standard_normal((B, Hq, S, D)), dt)
+    k = orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt)
+    v = orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt)
+    # rows beyond the active prefix must never be read
+    k[:, :, past + S:] = orc.to_storage(np.full((B, Hkv, L - past - S, D), np.nan), dt)
+    v[:, :, past + S:] = orc.to_storage(np.full((B, Hkv, L - past - S, D), np.nan), dt)
+    scale = D ** -0.5
+    want = orc.attention_f64(q, k, v, dt, scale, causal, past + S)
+    got = g.to_host(g.mynn.attention(g.to_dev(q, dt), g.to_dev(k, dt), g.to_dev(v, dt), scale, causal, past + S))
+    assert not np.isnan(g.f32(got, dt)).any()
+    # The probabilities enter the second product in the 16-bit type (as in the reference's
+    # tensor-core kernel, attention.cuh:45-314), so the error is set by the tensor's scale, not by
+    # each element's: an output near zero that is the sum of +-v terms carries the same absolute
+    # error as a large one.  Bound: error / max|out| <= 1e-2 (measured: ~1e-3 bf16, ~1e-4 f16).
+    assert max_err_rel_to_max(g.f32(got, dt), want) <= (3e-3 if dt == orc.BF16 else 5e-4)
+    ref = orc.attention(q, k, v, dt, scale, causal, past + S)
+    assert max_err_rel_to_max(g.f32(got, dt), g.f32(ref, dt)) <= 1e-2
+    if dt == orc.F16:
+        assert max_abs_rel(g.f32(got, dt), want) <= 1e-2  # elementwise too at fp16 resolution
+
+
+def test_prefill_attention_rows_equal_decode_rows(g):
+    """Size-independent property at the full prefill length (1024 rows, TinyLlama heads): each
+    causal row equals a decode call with that row's prefix."""
+    dt = orc.F16
+    rng = np.random.default_rng(77)
+    Hq, Hkv, S, D = 32, 4, 1024, 64
+    q = orc.to_storage(rng.standard_normal((1, Hq, S, D)), dt)
+    k = orc.to_storage(rng.standard_normal((1, Hkv, S, D)), dt)
+    v = orc.to_storage(rng.standard_normal((1, Hkv, S, D)), dt)
+    dq, dk, dv = g.to_dev(q, dt), g.to_dev(k, dt), g.to_dev(v, dt)
+    full = g.f32(g.to_host(g.mynn.attention(dq, dk, dv, 0.125, True, S)), dt)
+    for row in (0, 1, 31, 32, 500, 1023):
+        one = g.mynn.attention(dq[:, :, row:row + 1].contiguous(), dk, dv, 0.125, False, row + 1)
+        assert max_err_rel_to_max(full[:, :, row], g.f32(g.to_host(one), dt)[:, :, 0]) <= 2e-3, row
+    assert np.array_equal(full[:, :, 0], np.repeat(g.f32(v, dt)[:, :, 0], Hq // Hkv, 1))  # first row sees one key
