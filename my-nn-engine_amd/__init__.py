@@ -352,12 +352,15 @@ class Decoder:
             raise MynnError("model_init failed: %s" % lib().mynn_last_error().decode())
 
     def close(self):
-        if getattr(self, "handle", None):
-            lib().model_destroy(self.handle)
+        if getattr(self, "handle", None) and _lib is not None:
+            _lib.model_destroy(self.handle)
             self.handle = None
 
     def __del__(self):
-        self.close()
+        try:
+            self.close()
+        except Exception:  # interpreter shutdown
+            pass
 
     def step(self, ids, positions, past_len, active, want_logits=False):
         """One graph run; returns (next tokens per sequence, logits numpy or None)."""
@@ -421,12 +424,15 @@ class LlmSession:
             raise MynnError(lib().mynn_last_error().decode())
 
     def close(self):
-        if getattr(self, "handle", None):
-            lib().mynn_llm_destroy(self.handle)
+        if getattr(self, "handle", None) and _lib is not None:
+            _lib.mynn_llm_destroy(self.handle)
             self.handle = None
 
     def __del__(self):
-        self.close()
+        try:
+            self.close()
+        except Exception:  # interpreter shutdown
+            pass
 
     def reset(self):
         lib().mynn_llm_reset(self.handle)

@@ -115,39 +115,6 @@ def test_generate_bookkeeping_and_errors(g):
     llm.close(), dec.close()
 
 
-def test_mock_step_session_follows_logit_table(g):
-    """crates/llm/tests/mock_decode.rs: a 6-token logit table, prompt [0,1,2] -> [3,4,5,0,1];
-    past_len counts every decode step; a stop rewinds it."""
-    import ctypes as C
-    import json
-    import os
-
-    from conftest import GOLDEN
-
-    table = json.load(open(os.path.join(GOLDEN, "mock_decode", "expected_sequence.json")))
-    vocab = table["vocab"]
-    calls = []
-
-    def step(user, token, past_len):
-        calls.append((token, past_len))
-        return (token + 1) % vocab
-
-    cb = g.mynn.STEP_FN(step)
-    h = g.mynn.lib().mynn_llm_create_with_step(cb, None, 16, 999)
-    prompt = np.array([0, 1, 2], np.int64)
-    out = np.empty(5, np.int64)
-    n = g.mynn.lib().mynn_llm_generate_ids(h, prompt.ctypes.data_as(C.c_void_p), 3, 5, out.ctypes.data_as(C.c_void_p))
-    assert n == 5 and out.tolist() == [3, 4, 5, 0, 1]
-    assert out.tolist() == table["sequence"][2:7]
-    assert g.mynn.lib().mynn_llm_past_len(h) == 7  # 3 prompt steps + 4 fed-back tokens
-    assert [c[1] for c in calls] == list(range(7))
-    g.mynn.lib().mynn_llm_set_past_len(h, 5)  # stop-string rewind
-    assert g.mynn.lib().mynn_llm_past_len(h) == 5
-    g.mynn.lib().mynn_llm_reset(h)
-    assert g.mynn.lib().mynn_llm_past_len(h) == 0
-    g.mynn.lib().mynn_llm_destroy(h)
-
-
 @pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
 @pytest.mark.parametrize("P", [4, 32])
 def test_prefill_model_logits_and_kv_vs_oracle(g, dt, P):
