@@ -150,111 +150,150 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv_kernel(GemvParams p
     }
 }
 
-// Decode form (one activation row): every lane issues ALL of its weight loads -- R rows x NC
-// 16-byte chunks -- before anything else, so a whole per-CU slice of the matrix is in flight at
-// once and the RMSNorm / activation staging runs under the HBM latency.  NC = ceil(K / 1024).
+// Decode form (one activation row, 16-bit types).  A workgroup stages the activation row ONCE
+// in LDS as f32 (128-bit global loads; with NORM the RMSNorm statistics come from the same
+// registers: one butterfly + one cross-wave step), then its waves walk row groups of R rows
+// (group g, g + total_waves, ...).  For a group every lane issues all R x NC 16-byte weight loads
+// before the first multiply, dequantises in registers (int8 -> f32 convert + FMA) and the partial
+// sums meet in a wave64 butterfly; the scale is applied after the sum.  NC = ceil(K / 1024).
 template <typename T, int R, int NC, int EPI, bool NORM>
-__global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(GemvParams p) {
+__global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(GemvParams p, int groups, int total_waves) {
     extern __shared__ float act_lds[];  // [K]
     __shared__ float red[kGemvWaves];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int K = p.K, N = p.N;
     const int nchunks = K >> 4;
-    const int row0 = (blockIdx.x * kGemvWaves + wave) * R;
+    int g = blockIdx.x * kGemvWaves + wave;
 
     U4 w[R][NC];
+    auto load_group = [&](int gg) {
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-        const int row = row0 + r < N ? row0 + r : N - 1;
-        const U4 *wrow = (const U4 *)(p.wq + (size_t)row * K);
+        for (int r = 0; r < R; r++) {
+            const int row = gg * R + r < N ? gg * R + r : N - 1;
+            const U4 *wrow = (const U4 *)(p.wq + (size_t)row * K);
 #pragma unroll
-        for (int j = 0; j < NC; j++) {
-            const int c = lane + j * kWave;
-            if (c < nchunks) w[r][j] = __builtin_nontemporal_load(&wrow[c]);
-            else w[r][j] = U4{0u, 0u, 0u, 0u};
+            for (int j = 0; j < NC; j++) {
+                const int c = lane + j * kWave;
+                if (c < nchunks) w[r][j] = __builtin_nontemporal_load(&wrow[c]);
+                else w[r][j] = U4{0u, 0u, 0u, 0u};
+            }
         }
-    }
+    };
+    if (g < groups) load_group(g);  // in flight while the activation is staged
 
-    const T *act = (const T *)p.act;
-    if constexpr (NORM) {
+    // ---- stage: thread t owns the 8-element pieces t, t + 256, ... of the row
+    {
+        const U4 *ap = (const U4 *)p.act;
+        const int npieces = K >> 3;
+        constexpr int PMAX = (NC * 1024 / 8 + kGemvThreads - 1) / kGemvThreads;  // pieces per thread
+        float f[PMAX][8];
         float ss = 0.f;
-        for (int k = tid; k < K; k += kGemvThreads) {
-            float v = Elem<T>::ld(act, k);
-            act_lds[k] = v;
-            ss = fmaf(v, v, ss);
-        }
-        ss = wave_sum(ss);
-        if (lane == 0) red[wave] = ss;
-        __syncthreads();
-        float tot = 0.f;
 #pragma unroll
-        for (int i = 0; i < kGemvWaves; i++) tot += red[i];
-        const float inv = 1.0f / sqrtf(tot / (float)K + p.eps);
-        const T *nw = (const T *)p.norm_w;
-        for (int k = tid; k < K; k += kGemvThreads)
-            act_lds[k] = Elem<T>::rnd((act_lds[k] * inv) * Elem<T>::ld(nw, k));
-    } else {
-        for (int k = tid; k < K; k += kGemvThreads) act_lds[k] = Elem<T>::ld(act, k);
+        for (int q = 0; q < PMAX; q++) {
+            const int pc = tid + q * kGemvThreads;
+            if (pc < npieces) {
+                widen8<T>(ap[pc], f[q]);
+                if constexpr (NORM) {
+#pragma unroll
+                    for (int i = 0; i < 8; i++) ss = fmaf(f[q][i], f[q][i], ss);
+                }
+            }
+        }
+        float inv = 1.f;
+        if constexpr (NORM) {
+            ss = wave_sum(ss);
+            if (lane == 0) red[wave] = ss;
+            __syncthreads();
+            float tot = 0.f;
+#pragma unroll
+            for (int i = 0; i < kGemvWaves; i++) tot += red[i];
+            inv = 1.0f / sqrtf(tot / (float)K + p.eps);
+        }
+#pragma unroll
+        for (int q = 0; q < PMAX; q++) {
+            const int pc = tid + q * kGemvThreads;
+            if (pc < npieces) {
+                if constexpr (NORM) {
+                    float nw[8];
+                    widen8<T>(((const U4 *)p.norm_w)[pc], nw);
+#pragma unroll
+                    for (int i = 0; i < 8; i++) f[q][i] = Elem<T>::rnd((f[q][i] * inv) * nw[i]);
+                }
+                float4 *dst = (float4 *)(act_lds + pc * 8);
+                dst[0] = float4{f[q][0], f[q][1], f[q][2], f[q][3]};
+                dst[1] = float4{f[q][4], f[q][5], f[q][6], f[q][7]};
+            }
+        }
     }
     __syncthreads();
-    if (row0 >= N) return;
-
-    float acc[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) acc[r] = 0.f;
-#pragma unroll
-    for (int j = 0; j < NC; j++) {
-        const int c = lane + j * kWave;
-        if (c < nchunks) {
-            float a[16];
-            const float4 *ap = (const float4 *)(act_lds + c * 16);
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                float4 t = ap[q];
-                a[4 * q] = t.x; a[4 * q + 1] = t.y; a[4 * q + 2] = t.z; a[4 * q + 3] = t.w;
-            }
-#pragma unroll
-            for (int r = 0; r < R; r++) {
-                float wf[16];
-                widen16_i8(w[r][j], wf);
-#pragma unroll
-                for (int i = 0; i < 16; i++) acc[r] = fmaf(a[i], wf[i], acc[r]);
-            }
-        }
-    }
-#pragma unroll
-    for (int r = 0; r < R; r++) acc[r] = wave_sum(acc[r]);
 
     const T *scale = (const T *)p.scale;
     T *out = (T *)p.out;
-    if constexpr (EPI == EPI_SWIGLU) {
+    bool loaded = true;
+    for (; g < groups; g += total_waves) {
+        if (!loaded) load_group(g);
+        loaded = false;
+        float acc[R];
 #pragma unroll
-        for (int r = 0; r < R; r += 2) {
-            if (lane == r && row0 + r + 1 < N) {
-                float g = Elem<T>::rnd(acc[r] * Elem<T>::ld(scale, row0 + r));
-                float u = Elem<T>::rnd(acc[r + 1] * Elem<T>::ld(scale, row0 + r + 1));
-                float sig = 1.0f / (1.0f + expf(-g));
-                Elem<T>::st(out, (size_t)((row0 + r) >> 1), (g * sig) * u);
+        for (int r = 0; r < R; r++) acc[r] = 0.f;
+#pragma unroll
+        for (int j = 0; j < NC; j++) {
+            const int c = lane + j * kWave;
+            if (c < nchunks) {
+                float a[16];
+                const float4 *ap = (const float4 *)(act_lds + c * 16);
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    float4 t = ap[q];
+                    a[4 * q] = t.x; a[4 * q + 1] = t.y; a[4 * q + 2] = t.z; a[4 * q + 3] = t.w;
+                }
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    float wf[16];
+                    pin(w[r][j]);
+                    widen16_i8(w[r][j], wf);
+#pragma unroll
+                    for (int i = 0; i < 16; i++) acc[r] = fmaf(a[i], wf[i], acc[r]);
+                }
             }
         }
-    } else {
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            if (lane == r && row0 + r < N) {
-                float y = acc[r] * Elem<T>::ld(scale, row0 + r);
-                if constexpr (EPI == EPI_RESIDUAL) y = Elem<T>::rnd(y) + Elem<T>::ld((const T *)p.residual, row0 + r);
-                Elem<T>::st(out, row0 + r, y);
+        for (int r = 0; r < R; r++) acc[r] = wave_sum(acc[r]);
+        const int row0 = g * R;
+        if constexpr (EPI == EPI_SWIGLU) {
+#pragma unroll
+            for (int r = 0; r < R; r += 2) {
+                if (lane == r && row0 + r + 1 < N) {
+                    float gt = Elem<T>::rnd(acc[r] * Elem<T>::ld(scale, row0 + r));
+                    float up = Elem<T>::rnd(acc[r + 1] * Elem<T>::ld(scale, row0 + r + 1));
+                    float sig = 1.0f / (1.0f + expf(-gt));
+                    Elem<T>::st(out, (size_t)((row0 + r) >> 1), (gt * sig) * up);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                if (lane == r && row0 + r < N) {
+                    float y = acc[r] * Elem<T>::ld(scale, row0 + r);
+                    if constexpr (EPI == EPI_RESIDUAL) y = Elem<T>::rnd(y) + Elem<T>::ld((const T *)p.residual, row0 + r);
+                    Elem<T>::st(out, row0 + r, y);
+                }
             }
         }
     }
 }
 
+// waves are spread so that every wave gets the same number of row groups (no tail wave)
 template <typename T, int R, int NC, int EPI, bool NORM>
 static int launch_gemv1(const GemvParams &p, hipStream_t s) {
-    const int rows_per_block = kGemvWaves * R;
-    dim3 grid((p.N + rows_per_block - 1) / rows_per_block);
-    hipLaunchKernelGGL((dequant_gemv1_kernel<T, R, NC, EPI, NORM>), grid, dim3(kGemvThreads),
-                       (size_t)p.K * sizeof(float), s, p);
+    const int groups = (p.N + R - 1) / R;
+    const int max_waves = 256 * 16;  // four resident waves per SIMD (measured best of 8/16/32)
+    const int passes = (groups + max_waves - 1) / max_waves;
+    int waves = (groups + passes - 1) / passes;
+    const int blocks = (waves + kGemvWaves - 1) / kGemvWaves;
+    waves = blocks * kGemvWaves;
+    hipLaunchKernelGGL((dequant_gemv1_kernel<T, R, NC, EPI, NORM>), dim3(blocks), dim3(kGemvThreads),
+                       (size_t)p.K * sizeof(float), s, p, groups, waves);
     return launch_status("dequant_gemv1_kernel");
 }
 
@@ -350,11 +389,14 @@ int dequant_gemv_dispatch(void *out, const void *act, const int8_t *wq, const vo
 }
 
 // ---- fused decode variants used by the decoder executor (one activation row, T in == T out)
-// rows per wave: 4 for wide matrices, 2 otherwise (more workgroups for the narrow ones)
 template <typename T, int EPI, bool NORM>
 static int gemv1_dispatch(const GemvParams &p, hipStream_t s) {
     const int nc = (p.K + 1023) / 1024;
-    const bool wide = pick_r(p.N) == 4;
+    const bool wide = false;  // two rows per wave measured as fast or faster than four at every shape
+    if (!aligned16(p.act) || (NORM && !aligned16(p.norm_w)) || p.K % 8 != 0 || nc > 14) {
+        if (wide) return launch_gemv<T, T, 4, 1, EPI, NORM>(p, s);  // the looping kernel
+        return launch_gemv<T, T, 2, 1, EPI, NORM>(p, s);
+    }
 #define MYNN_GEMV1(NC_)                                                   \
     return wide ? launch_gemv1<T, 4, NC_, EPI, NORM>(p, s) : launch_gemv1<T, 2, NC_, EPI, NORM>(p, s)
     if (nc <= 1) { MYNN_GEMV1(1); }

@@ -80,6 +80,13 @@ template <> __device__ inline void widen8<f16_t>(const U4 &v, float *f) {
     }
 }
 
+// Pins a 128-bit register value at this point of the instruction stream: nothing computed from
+// it can be scheduled earlier.  Used to keep int8 -> f32 converts next to their FMAs (left alone,
+// the compiler converts every loaded chunk up front and quadruples the register count).
+__device__ inline void pin(U4 &v) {
+    asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w));
+}
+
 // 16 int8 (one 128-bit load) widened to f32
 __device__ inline void widen16_i8(const U4 &v, float *f) {
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
