@@ -15,6 +15,7 @@ struct AttnParams {
     int q_pos_offset;         // host value, used when d_active == nullptr
     int nsplit;
     int slice;                // key rows per slice (gridDim.y slices cover the cache)
+    int heads_per_wg;         // query heads one workgroup serves (divides Hq/Hkv)
     // fused decode form: raw qkv projection row(s) [B, (Hq+2*Hkv)*D], RoPE tables, device position;
     // K and V then are the caches the new row is appended to
     const void *qkv, *cos_t, *sin_t;
@@ -38,10 +39,11 @@ inline void attn_token_major_layout(AttnParams &p, int D) {
     p.q_rs = p.o_rs = (long)p.Hq * D;
 }
 
-void attn_plan(int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, int *slice, int *nsplit);
+void attn_plan(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, int *slice, int *nsplit,
+               int *heads_per_wg);
 bool attention_fused_supported(int D, int G);
 size_t attn_scratch_bytes(int B, int Hq, int Sq, int D, int nsplit);
-size_t attn_counter_bytes(int B, int Hkv, int Sq);
+size_t attn_counter_bytes(int B, int Hq, int Sq);
 int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *scratch, void *counters, hipStream_t s);
 int attention_prefill_launch(const AttnParams &p, int D, int dtype, hipStream_t s);
 bool attention_prefill_supported(const AttnParams &p, int D, int dtype, int kv_int8);

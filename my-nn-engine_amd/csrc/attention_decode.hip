@@ -33,6 +33,8 @@ template <> struct ChunkOf<bf16_t, 8> { using type = U4; static constexpr bool v
 template <> struct ChunkOf<f16_t, 8> { using type = U4; static constexpr bool vec = true; };
 template <> struct ChunkOf<int8_t, 8> { using type = uint2; static constexpr bool vec = true; };
 
+// G = query heads served by one workgroup: all heads of the kv head, or a part of them when there
+// are too few (batch, kv head) pairs to fill the chip (K/V are then read once per part, from L2).
 template <typename T, int D, int G, bool KVI8, bool FUSE>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p) {
     constexpr int EPL = D >= 8 ? 8 : D;      // elements of a key row per lane
@@ -51,8 +53,11 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int grp = tid / LPK, dc = tid % LPK;
-    const int bhkv = blockIdx.x, split = blockIdx.y, sq = blockIdx.z;
+    const int Gt = p.Hq / p.Hkv, nparts = Gt / G;  // heads per kv head, parts per kv head
+    const int bhkv = blockIdx.x / nparts, part = blockIdx.x % nparts;
+    const int split = blockIdx.y, sq = blockIdx.z;
     const int b = bhkv / p.Hkv, hkv = bhkv % p.Hkv;
+    const int head0 = hkv * Gt + part * G;  // first query head of this workgroup
     const int Sq = p.Sq;
 
     const int active = p.d_active ? *p.d_active : p.active;
@@ -107,7 +112,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
         // G query heads + 1 key head to rotate: (G+1) * D/2 pairs; then D values of v to copy
         for (int idx = tid; idx < (G + 1) * half; idx += kAttnThreads) {
             const int h = idx / half, j = idx % half;
-            const T *src = h < G ? row + (size_t)(hkv * G + h) * D : row + (size_t)(p.Hq + hkv) * D;
+            const T *src = h < G ? row + (size_t)(head0 + h) * D : row + (size_t)(p.Hq + hkv) * D;
             const float xl = Elem<T>::ld(src, j), xh = Elem<T>::ld(src, j + half);
             const float cl = Elem<T>::ld(cos_t, tab + j), ch = Elem<T>::ld(cos_t, tab + j + half);
             const float sl = Elem<T>::ld(sin_t, tab + j), sh = Elem<T>::ld(sin_t, tab + j + half);
@@ -118,7 +123,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
             } else {
                 new_s[0][j] = lo;
                 new_s[0][j + half] = hi;
-                if (split == 0) {  // one workgroup appends the row
+                if (split == 0 && part == 0) {  // one workgroup appends the row
                     T *kc = (T *)p.k + (kv_base + new_row) * D;
                     Elem<T>::st(kc, j, lo);
                     Elem<T>::st(kc, j + half, hi);
@@ -128,12 +133,12 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
         for (int d = tid; d < D; d += kAttnThreads) {
             const T *src = row + (size_t)(p.Hq + p.Hkv + hkv) * D;
             new_s[1][d] = Elem<T>::ld(src, d);
-            if (split == 0) ((T *)p.v)[(kv_base + new_row) * D + d] = src[d];
+            if (split == 0 && part == 0) ((T *)p.v)[(kv_base + new_row) * D + d] = src[d];
         }
     } else {
         for (int idx = tid; idx < G * D; idx += kAttnThreads) {
             const int g = idx / D, d = idx % D;
-            const size_t qo = (size_t)b * p.q_bs + (size_t)(hkv * G + g) * p.q_hs + (size_t)sq * p.q_rs + d;
+            const size_t qo = (size_t)b * p.q_bs + (size_t)(head0 + g) * p.q_hs + (size_t)sq * p.q_rs + d;
             q_s[g][d] = Elem<T>::ld((const T *)p.q, qo);
         }
     }
@@ -218,30 +223,42 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
     }
     __syncthreads();
 
-    // ---- 4. o[g,d] = sum_k p[g,k] * V[k,d]; thread owns (g,d)
+    // ---- 4. o[g,d] = sum_k p[g,k] * V[k,d]; thread owns (g, d) and one of KP interleaved key
+    // subsets; the KP partial sums meet in LDS
+    constexpr int KP = (G * D >= kAttnThreads) ? 1 : kAttnThreads / (G * D);
     T *out = (T *)p.out;
-    const size_t row_base = (size_t)(b * p.Hq + hkv * G) * Sq + sq;  // + g*Sq
-    for (int idx = tid; idx < G * D; idx += kAttnThreads) {
-        const int g = idx / D, d = idx % D;
+    const size_t row_base = (size_t)(b * p.Hq + head0) * Sq + sq;  // + g*Sq
+    float *part_s = vsc_s + nmax;  // [KP][G*D] (KP > 1 only)
+    for (int idx0 = 0; idx0 < G * D * KP; idx0 += kAttnThreads) {
+        const int idx = idx0 + tid;
+        const int kp = idx / (G * D), gd = idx % (G * D);
+        const int g = gd / D, d = gd % D;
         const float *pr = sc + (size_t)g * nmax;
         auto vld = [&](int k) -> float {
             if constexpr (KVI8) return (float)((const int8_t *)v_s)[(size_t)k * D + d];
             else return Elem<T>::ld((const T *)v_s, (size_t)k * D + d);
         };
         float acc0 = 0.f, acc1 = 0.f, acc2 = 0.f, acc3 = 0.f;
-        int k = 0;
-        for (; k + 3 < n; k += 4) {
+        int k = kp;
+        for (; k + 3 * KP < n; k += 4 * KP) {
             acc0 = fmaf(pr[k], vld(k), acc0);
-            acc1 = fmaf(pr[k + 1], vld(k + 1), acc1);
-            acc2 = fmaf(pr[k + 2], vld(k + 2), acc2);
-            acc3 = fmaf(pr[k + 3], vld(k + 3), acc3);
+            acc1 = fmaf(pr[k + KP], vld(k + KP), acc1);
+            acc2 = fmaf(pr[k + 2 * KP], vld(k + 2 * KP), acc2);
+            acc3 = fmaf(pr[k + 3 * KP], vld(k + 3 * KP), acc3);
         }
-        for (; k < n; k++) acc0 = fmaf(pr[k], vld(k), acc0);
-        const float ot = (acc0 + acc1) + (acc2 + acc3);
+        for (; k < n; k += KP) acc0 = fmaf(pr[k], vld(k), acc0);
+        float ot = (acc0 + acc1) + (acc2 + acc3);
+        if constexpr (KP > 1) {
+            part_s[kp * (G * D) + gd] = ot;
+            __syncthreads();
+            if (kp != 0) continue;
+#pragma unroll
+            for (int q = 1; q < KP; q++) ot += part_s[q * (G * D) + gd];
+        }
         const float mt = ml_s[g][0], lt = ml_s[g][1];
         const size_t row = row_base + (size_t)g * Sq;
         if (p.nsplit == 1) {
-            const size_t oo = (size_t)b * p.o_bs + (size_t)(hkv * G + g) * p.o_hs + (size_t)sq * p.o_rs + d;
+            const size_t oo = (size_t)b * p.o_bs + (size_t)(head0 + g) * p.o_hs + (size_t)sq * p.o_rs + d;
             Elem<T>::st(out, oo, ot / lt);
         } else {
             p.part_o[(row * p.nsplit + split) * D + d] = ot;
@@ -257,7 +274,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
     __threadfence();
     __syncthreads();
     if (tid == 0) {
-        unsigned prev = atomicAdd(&p.counters[(size_t)bhkv * Sq + sq], 1u);
+        unsigned prev = atomicAdd(&p.counters[(size_t)blockIdx.x * Sq + sq], 1u);
         sm_last = (prev == (unsigned)p.nsplit - 1);
     }
     __syncthreads();
@@ -277,10 +294,10 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
             lt = fmaf(__builtin_nontemporal_load(&ml[2 * s + 1]), c, lt);
             ot = fmaf(__builtin_nontemporal_load(&po[s * D + d]), c, ot);
         }
-        const size_t oo = (size_t)b * p.o_bs + (size_t)(hkv * G + g) * p.o_hs + (size_t)sq * p.o_rs + d;
+        const size_t oo = (size_t)b * p.o_bs + (size_t)(head0 + g) * p.o_hs + (size_t)sq * p.o_rs + d;
         Elem<T>::st(out, oo, ot / lt);
     }
-    if (tid == 0) p.counters[(size_t)bhkv * Sq + sq] = 0;  // ready for the next launch
+    if (tid == 0) p.counters[(size_t)blockIdx.x * Sq + sq] = 0;  // ready for the next launch
 }
 
 // LDS the kernel may use per workgroup for the V slice, the scores and the v scales
@@ -296,7 +313,8 @@ static int slice_rows(int D, int G, size_t kv_elem) {
     return rows;
 }
 static size_t slice_lds_bytes(int rows, int D, int G, size_t kv_elem) {
-    return (size_t)rows * D * kv_elem + (size_t)G * rows * 4 + (size_t)rows * 4;
+    // V slice | scores | v scales | key-subset partials (at most one value per thread)
+    return (size_t)rows * D * kv_elem + (size_t)G * rows * 4 + (size_t)rows * 4 + (size_t)kAttnThreads * 4;
 }
 
 template <typename T, int D, int G, bool KVI8, bool FUSE>
@@ -309,14 +327,14 @@ static int launch_one(const AttnParams &p, hipStream_t s) {
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kAttnLdsBudget + 16384)));
         attr_set = true;
     }
-    dim3 grid(p.B * p.Hkv, p.nsplit, p.Sq), block(kAttnThreads);
+    dim3 grid(p.B * p.Hkv * ((p.Hq / p.Hkv) / G), p.nsplit, p.Sq), block(kAttnThreads);
     hipLaunchKernelGGL((attn_decode_kernel<T, D, G, KVI8, FUSE>), grid, block, lds, s, p);
     return launch_status("attn_decode_kernel");
 }
 
 template <typename T, int D, bool KVI8, bool FUSE>
 static int launch_g(const AttnParams &p, hipStream_t s) {
-    switch (p.Hq / p.Hkv) {
+    switch (p.heads_per_wg) {
     case 1: return launch_one<T, D, 1, KVI8, FUSE>(p, s);
     case 2: return launch_one<T, D, 2, KVI8, FUSE>(p, s);
     case 4: return launch_one<T, D, 4, KVI8, FUSE>(p, s);
@@ -349,22 +367,30 @@ bool attention_fused_supported(int D, int G) {
     return (D == 32 || D == 64 || D == 128) && (G == 1 || G == 2 || G == 4 || G == 8);
 }
 
-// Slice length and number of slices for a launch.  kv_len = longest key range any row can have.
-void attn_plan(int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, int *slice, int *nsplit) {
+// Slice length, number of slices and query heads per workgroup for a launch.  kv_len = longest key
+// range any row can have.  All heads of a kv head share one workgroup (one K/V read) unless that
+// leaves fewer than ~64 workgroups; then the heads are divided, halving until there are enough.
+void attn_plan(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, int *slice, int *nsplit,
+               int *heads_per_wg) {
     const size_t kv_elem = kv_int8 ? 1 : dtype_size(dtype);
-    const int rows = slice_rows(D, Hq / Hkv, kv_elem);
+    const int Gt = Hq / Hkv;
+    const int rows = slice_rows(D, Gt, kv_elem);
     int n = (kv_len + rows - 1) / rows;
     if (n < 1) n = 1;
+    int hb = Gt;
+    while (hb > 1 && hb % 2 == 0 && (long)B * Hkv * Sq * n * (Gt / hb) < 64) hb /= 2;
     *slice = rows;
     *nsplit = n;
+    *heads_per_wg = hb;
 }
 size_t attn_scratch_bytes(int B, int Hq, int Sq, int D, int nsplit) {
     size_t rows = (size_t)B * Hq * Sq;
     size_t bytes = rows * nsplit * (D + 2) * sizeof(float);
     return (bytes + 255) / 256 * 256;
 }
-size_t attn_counter_bytes(int B, int Hkv, int Sq) {
-    return ((size_t)B * Hkv * Sq * sizeof(unsigned) + 255) / 256 * 256;
+size_t attn_counter_bytes(int B, int Hq, int Sq) {
+    // one per (batch, kv head, part, row); at most one part per query head
+    return ((size_t)B * Hq * Sq * sizeof(unsigned) + 255) / 256 * 256;
 }
 
 // scratch = [part_o | part_ml] (contents need not survive); counters = one unsigned per
@@ -439,12 +465,12 @@ extern "C" int mynn_attention(void *out, const void *Q, const void *K, const voi
     if (Sq > 1 && attention_prefill_supported(p, head_dim, dtype, kv_int8))
         return attention_prefill_launch(p, head_dim, dtype, st);
     int kv_len = d_active ? cache_seq_len : (active_seq_kv < cache_seq_len ? active_seq_kv : cache_seq_len);
-    attn_plan(num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, kv_len, &p.slice, &p.nsplit);
+    attn_plan(B, Sq, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, kv_len, &p.slice, &p.nsplit, &p.heads_per_wg);
     MYNN_REQUIRE(p.nsplit <= 65535, MYNN_ERR_UNSUPPORTED, "attention: cache of %d rows needs too many slices", kv_len);
     if (p.nsplit > 1) {
         int rc = ensure(g_scratch, attn_scratch_bytes(B, num_q_heads, Sq, head_dim, p.nsplit), false, st);
         if (rc) return rc;
-        rc = ensure(g_counters, attn_counter_bytes(B, num_kv_heads, Sq), true, st);
+        rc = ensure(g_counters, attn_counter_bytes(B, num_q_heads, Sq), true, st);
         if (rc) return rc;
     }
     return attention_decode_launch(p, head_dim, dtype, kv_int8, g_scratch.ptr, g_counters.ptr, st);

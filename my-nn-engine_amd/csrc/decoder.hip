@@ -75,7 +75,7 @@ struct Model {
     int64_t *d_ids = nullptr, *d_pos = nullptr;
     int32_t *d_past = nullptr, *d_active = nullptr, *d_next = nullptr, *d_tokens = nullptr, *d_step = nullptr;
     void *attn_scratch = nullptr, *attn_counters = nullptr;
-    int nsplit = 1, slice = 0;
+    int nsplit = 1, slice = 0, heads_per_wg = 1;
     int token_cap = 0;
     // host staging (pinned)
     char *h_stage = nullptr;
@@ -175,7 +175,7 @@ static int enqueue_step(Model &m) {
             AttnParams p{};
             p.out = m.attn; p.q = m.q; p.k = L.k_cache; p.v = L.v_cache; p.scale = softmax_scale;
             p.is_causal = S > 1; p.B = B; p.Sq = S; p.Hq = Hq; p.Hkv = Hkv; p.cache_len = c.max_seq;
-            p.d_active = m.d_active; p.nsplit = m.nsplit; p.slice = m.slice;
+            p.d_active = m.d_active; p.nsplit = m.nsplit; p.slice = m.slice; p.heads_per_wg = m.heads_per_wg;
             attn_token_major_layout(p, D);
             const bool fuse_attn = fused && attention_fused_supported(D, Hq / Hkv);
             if (fuse_attn) {
@@ -322,7 +322,7 @@ static int build(Model &m, void **init, void **state) {
 
     // ---- arena: every activation of one step, the device scalars, attention split scratch
     const int rows = c.batch * c.seq_q;
-    attn_plan(c.n_heads, c.n_kv_heads, c.head_dim, c.dtype, 0, c.max_seq, &m.slice, &m.nsplit);
+    attn_plan(c.batch, c.seq_q, c.n_heads, c.n_kv_heads, c.head_dim, c.dtype, 0, c.max_seq, &m.slice, &m.nsplit, &m.heads_per_wg);
     m.token_cap = c.max_seq + 8;
     ArenaPlan plan;
     size_t o_x = plan.take((size_t)rows * H * eb), o_x2 = plan.take((size_t)rows * H * eb);
@@ -334,7 +334,7 @@ static int build(Model &m, void **init, void **state) {
     size_t o_ids = plan.take((size_t)rows * 8), o_pos = plan.take((size_t)c.seq_q * 8);
     size_t o_sc = plan.take(256), o_tok = plan.take((size_t)m.token_cap * 4);
     size_t o_as = plan.take(attn_scratch_bytes(c.batch, c.n_heads, c.seq_q, c.head_dim, m.nsplit));
-    size_t o_ac = plan.take(attn_counter_bytes(c.batch, c.n_kv_heads, c.seq_q));
+    size_t o_ac = plan.take(attn_counter_bytes(c.batch, c.n_heads, c.seq_q));
     m.arena_bytes = plan.off;
     MYNN_HIP(hipMalloc((void **)&m.arena, m.arena_bytes));
     MYNN_HIP(hipMemset(m.arena, 0, m.arena_bytes));
