@@ -44,40 +44,61 @@ __global__ void dequant_rows_kernel(T *out, const int8_t *wq, const T *scale, in
 }
 
 // ---- (2) C[M,N] = A[M,K] . B[N,K]^T, f32 accumulate, one rounding at the store
-constexpr int BM = 128, BN = 128, BK = 32, LDT = BK + 8;  // LDS row stride in elements (80 B)
-constexpr int kGemmThreads = 256;
+// 256 x 128 output tile per workgroup of 8 waves (4 x 2, 64 x 64 per wave = 2 x 2 MFMA tiles),
+// K step 32, two LDS buffers, next tile prefetched into registers during the multiply.
+constexpr int BM = 256, BN = 128, BK = 32, LDT = BK + 8;  // LDS row stride in elements (80 B)
+constexpr int kGemmThreads = 512;
 
-template <typename T>
-__global__ __launch_bounds__(kGemmThreads) void gemm_nt_mfma_kernel(T *C, const T *A, const T *B, int M, int N, int K,
+// Workgroup -> output tile.  Hardware deals consecutive workgroup ids round-robin over the 8 XCDs
+// (each with its own L2), so id b is first turned into a per-XCD contiguous index; inside an XCD
+// tiles are walked in bands of 8 tile-rows so that the A rows and the B rows being multiplied at
+// one time stay L2-resident.
+__device__ inline void tile_of(int b, int nblocks, int tiles_m, int tiles_n, int &tm, int &tn) {
+    constexpr int XCD = 8, BAND = 8;
+    int l = b;
+    if (nblocks % XCD == 0) l = (b % XCD) * (nblocks / XCD) + b / XCD;
+    const int band_tiles = BAND * tiles_n;
+    const int band = l / band_tiles, in_band = l % band_tiles;
+    const int rows_here = min(BAND, tiles_m - band * BAND);
+    tm = band * BAND + in_band % rows_here;
+    tn = in_band / rows_here;
+}
+
+// KTAIL: K is not a multiple of 2*BK, so the last steps mask the columns of A past K.
+template <typename T, bool KTAIL>
+__global__ __launch_bounds__(kGemmThreads, 2) void gemm_nt_mfma_kernel(T *C, const T *A, const T *B, int M, int N, int K,
                                                                     int Kp) {
     __shared__ __align__(16) uint16_t As[2][BM * LDT];
     __shared__ __align__(16) uint16_t Bs[2][BN * LDT];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;  // wave tile origin: (64*wm, 64*wn)
-    // workgroup -> tile: consecutive workgroups walk M first so that neighbours share the B tile
-    const int tiles_m = (M + BM - 1) / BM;
-    const int tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m;
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    int tm, tn;
+    tile_of(blockIdx.x, gridDim.x, tiles_m, tiles_n, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
 
-    // global -> register staging: a tile is 128 rows x 32 elements = 512 chunks of 8; 2 per thread
-    const int lr = tid >> 2, lc = (tid & 3) * 8;  // row (0..63) and element offset within BK
-    U4 ra[2], rb[2];
-    auto load_tiles = [&](int k0) {
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const int r = lr + 64 * h;
-            const int gm = m0 + r, gn = n0 + r;
-            ra[h] = (gm < M && k0 + lc < K) ? *(const U4 *)(A + (size_t)gm * K + k0 + lc) : U4{0u, 0u, 0u, 0u};
-            rb[h] = gn < N ? *(const U4 *)(B + (size_t)gn * Kp + k0 + lc) : U4{0u, 0u, 0u, 0u};
-        }
+    // global -> register staging: A tile 256 x 32 = 1024 chunks of 8 (2 per thread), B tile 512 (1 per
+    // thread).  Two register sets: tile kt+1 waits in one while tile kt+2 is still in flight in the
+    // other, so a load has two multiply phases of every resident wave to complete.
+    const int lr = tid >> 2, lc = (tid & 3) * 8;  // row (0..127) and element offset within BK
+    struct Stage { U4 a0, a1, b; uint32_t mask; };
+    // Branch-free: rows past M / N re-read the last row (their products land in rows that are never
+    // stored), columns past K are masked to zero.  No branch means the compiler can wait for exactly
+    // the older register set (vmcnt(3)) instead of for everything in flight.
+    const T *a0p = A + (size_t)min(m0 + lr, M - 1) * K;
+    const T *a1p = A + (size_t)min(m0 + lr + 128, M - 1) * K;
+    const T *bp = B + (size_t)min(n0 + lr, N - 1) * Kp;
+    auto load_tiles = [&](Stage &r, int k0) {
+        const int ka = min(k0 + lc, K - 8);
+        if (KTAIL) r.mask = k0 + lc < K ? 0xFFFFFFFFu : 0u;  // applied when the registers are consumed
+        r.a0 = *(const U4 *)(a0p + ka);
+        r.a1 = *(const U4 *)(a1p + ka);
+        r.b = *(const U4 *)(bp + k0 + lc);
     };
-    auto store_tiles = [&](int buf) {
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const int r = lr + 64 * h;
-            *(U4 *)&As[buf][r * LDT + lc] = ra[h];
-            *(U4 *)&Bs[buf][r * LDT + lc] = rb[h];
-        }
+    auto store_tiles = [&](int buf, const Stage &r) {
+        *(U4 *)&As[buf][lr * LDT + lc] = KTAIL ? r.a0 & r.mask : r.a0;
+        *(U4 *)&As[buf][(lr + 128) * LDT + lc] = KTAIL ? r.a1 & r.mask : r.a1;
+        *(U4 *)&Bs[buf][lr * LDT + lc] = r.b;
     };
 
     f16x_t acc[2][2];
@@ -89,13 +110,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_mfma_kernel(T *C, const 
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
     const int fr = lane & 31, fk = (lane >> 5) * 8;  // fragment row within a 32-row tile, k offset
-    load_tiles(0);
-    store_tiles(0);
-    __syncthreads();
-    const int nk = Kp / BK;
-    for (int kt = 0; kt < nk; kt++) {
-        const int buf = kt & 1;
-        if (kt + 1 < nk) load_tiles((kt + 1) * BK);
+    auto multiply = [&](int buf) {
 #pragma unroll
         for (int ks = 0; ks < BK; ks += 16) {
             U4 fa[2], fb[2];
@@ -108,10 +123,24 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_mfma_kernel(T *C, const 
 #pragma unroll
                 for (int j = 0; j < 2; j++) acc[i][j] = Mfma<T>::run(fa[i], fb[j], acc[i][j]);
         }
-        if (kt + 1 < nk) {
-            store_tiles(buf ^ 1);
-            __syncthreads();
-        }
+    };
+
+    const int nk = Kp / BK;  // even: Kp is a multiple of 2*BK
+    Stage rA, rB;
+    load_tiles(rA, 0);
+    store_tiles(0, rA);
+    load_tiles(rA, BK);
+    load_tiles(rB, min(2, nk - 1) * BK);
+    __syncthreads();
+    for (int kt = 0; kt < nk; kt += 2) {
+        multiply(0);                                   // tile kt
+        store_tiles(1, rA);                            // tile kt+1
+        load_tiles(rA, min(kt + 3, nk - 1) * BK);      // (a repeat of the last tile near the end; unused)
+        __syncthreads();
+        multiply(1);                                   // tile kt+1
+        store_tiles(0, rB);                            // tile kt+2
+        load_tiles(rB, min(kt + 4, nk - 1) * BK);
+        __syncthreads();
     }
 
     // epilogue: D[i][j] of a 32x32 tile sits in lane (j + 32*((i/4)%2)), element 4*(i/8) + i%4
@@ -135,7 +164,7 @@ static size_t g_ws_bytes = 0;
 template <typename T>
 static int gemm_launch(void *out, const void *act, const int8_t *wq, const void *scale, int M, int N, int K,
                        hipStream_t s) {
-    const int Kp = (K + BK - 1) / BK * BK;
+    const int Kp = (K + 2 * BK - 1) / (2 * BK) * (2 * BK);  // the GEMM walks K in pairs of steps
     const size_t need = (size_t)N * Kp * sizeof(T);
     if (need > g_ws_bytes) {
         MYNN_HIP(hipStreamSynchronize(s));
@@ -151,8 +180,12 @@ static int gemm_launch(void *out, const void *act, const int8_t *wq, const void 
     int rc = launch_status("dequant_rows_kernel");
     if (rc) return rc;
     const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-    hipLaunchKernelGGL(gemm_nt_mfma_kernel<T>, dim3(tiles), dim3(kGemmThreads), 0, s, (T *)out, (const T *)act,
-                       (const T *)g_ws, M, N, K, Kp);
+    if (K == Kp)
+        hipLaunchKernelGGL((gemm_nt_mfma_kernel<T, false>), dim3(tiles), dim3(kGemmThreads), 0, s, (T *)out,
+                           (const T *)act, (const T *)g_ws, M, N, K, Kp);
+    else
+        hipLaunchKernelGGL((gemm_nt_mfma_kernel<T, true>), dim3(tiles), dim3(kGemmThreads), 0, s, (T *)out,
+                           (const T *)act, (const T *)g_ws, M, N, K, Kp);
     return launch_status("gemm_nt_mfma_kernel");
 }
 
