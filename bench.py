@@ -1,7 +1,10 @@
 #!/usr/bin/env python3
 """Headline benchmark: batch-1 greedy decode of a TinyLlama-1.1B-shape int8 model on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode|prefill]
+
+`--workload prefill` times the matrix-core side of the same path instead: one step = one prefill
+pass of 8 prompts x 1024 tokens through the decoder executor (roofline bound: MFMA).
 
 One step = one decode step (one token) through the HIP decoder executor; the K timed steps are
 replays of the captured hipGraph with inputs, weights and KV cache resident in HBM.  Prints ONE
@@ -20,6 +23,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16/fp16 matrix rate
+PREFILL_BATCH, PREFILL_LEN = 8, 1024
 
 TINYLLAMA = dict(n_layers=22, hidden=2048, n_heads=32, n_kv_heads=4, head_dim=64, ffn=5632, vocab=32000,
                  max_seq=384, eps=1e-5, rope_theta=10000.0)
@@ -81,11 +86,86 @@ def algorithmic_bytes_per_token(cfg, eb, context):
     return w + kv + H + eb
 
 
+def prefill_main(args, mynn, cfg):
+    """8 x 1024 prompt tokens through the prefill executor: every linear on the matrix cores, causal
+    flash attention, logits for every row (the reference computes [1, S, vocab])."""
+    import numpy as np
+    import torch
+
+    B, S = PREFILL_BATCH, PREFILL_LEN
+    K = 5 if args.steps is None else args.steps
+    W = 2 if args.warmup is None else args.warmup
+    cfg = dict(cfg, max_seq=S)
+    weights = make_weights(cfg, cfg["dtype"], args.seed)
+    torch.cuda.synchronize()
+    dec = mynn.Decoder(cfg, weights, seq_q=S, batch=B)
+    rng = np.random.default_rng(args.seed)
+    ids = rng.integers(0, cfg["vocab"], B * S)
+    pos = np.arange(S)
+    for _ in range(W):
+        dec.step(ids, pos, 0, S)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(K):
+        dec.step(ids, pos, 0, S)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / K
+
+    agg = {}
+    for _ in range(2):
+        for name, ms, nbytes, flops in dec.profile(ids, pos, 0, S):
+            a = agg.setdefault(name, [0, 0.0, 0.0, 0.0])
+            a[0] += 1
+            a[1] += ms
+            a[2] += nbytes
+            a[3] += flops
+    mm = {k: v for k, v in agg.items() if v[3] > 0}
+    dom = max(mm, key=lambda k: mm[k][1])
+    calls, ms_tot, _, fl_tot = mm[dom]
+    achieved = fl_tot / (ms_tot * 1e-3) / 1e12
+    step_flops = sum(v[3] for v in agg.values()) / 2
+    lin = {k: v for k, v in mm.items() if k.startswith("linear_")}
+    lin_tflops = sum(v[3] for v in lin.values()) / (sum(v[1] for v in lin.values()) * 1e-3) / 1e12
+    out = {
+        "metric": "prefill tok/s 8x1024 TinyLlama-shape int8; MFMA utilisation",
+        "value": round(B * S * K / elapsed, 1), "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32 accumulate over %s (int8 weights dequantised to %s)" % (args.dtype, args.dtype),
+        "data": "synthetic",
+        "config": {"workload": "configs[3]: TinyLlama-1.1B-shape int8 decoder, prefill of 8 prompts x 1024 tokens, "
+                               "KV cache filled, logits for every row",
+                   "batch": B, "seq": S, "launches_per_step": dec.stats()["launches_per_step"], "seed": args.seed,
+                   "step_flops": step_flops,
+                   "step_mfma_frac": round(step_flops / (ms_per_step * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4),
+                   "per_kernel_ms": {k: round(v[1] / 2, 3) for k, v in sorted(agg.items(), key=lambda kv: -kv[1][1])}},
+        "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 1), "peak": MFMA_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                     "flops_per_launch": fl_tot / calls, "avg_launch_us": round(ms_tot / calls * 1e3, 2),
+                     "all_linear_TFLOPs": round(lin_tflops, 1)},
+    }
+    if not args.no_cpu_baseline:
+        import oracle as orc
+
+        ref = orc.Model(dict(cfg), to_host_weights(weights))
+        n_cpu = 256  # bounded sample: the first rows of the first prompt
+        t0 = time.perf_counter()
+        ref.forward(ids[:n_cpu], pos[:n_cpu], 0, n_cpu, True)
+        cpu_elapsed = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": round(n_cpu / cpu_elapsed, 2), "unit": "tok/s", "cores": orc.get_threads(),
+                               "kind": "port",
+                               "sample": "one causal prefill pass over the first %d tokens of the first prompt, C port "
+                                         "of the reference CPU backend (dequantise + blocked f32 GEMM, OpenMP)" % n_cpu}
+    dec.close()
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=256)
-    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--workload", choices=["decode", "prefill"], default="decode")
+    ap.add_argument("--steps", type=int, default=None, help="default 256 (decode) / 5 (prefill)")
+    ap.add_argument("--warmup", type=int, default=None, help="default 16 (decode) / 2 (prefill)")
     ap.add_argument("--dtype", choices=["f16", "bf16"], default="f16")
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -105,7 +185,10 @@ def main():
     dt = {"f16": mynn.F16, "bf16": mynn.BF16}[args.dtype]
     eb = 2
     cfg = dict(TINYLLAMA, dtype=dt)
-    K, W = args.steps, args.warmup
+    if args.workload == "prefill":
+        return prefill_main(args, mynn, cfg)
+    K = 256 if args.steps is None else args.steps
+    W = 16 if args.warmup is None else args.warmup
     assert PROMPT_LEN + max(K, W) <= cfg["max_seq"], "steps/warmup do not fit max_seq %d" % cfg["max_seq"]
 
     weights = make_weights(cfg, dt, args.seed)
@@ -138,7 +221,7 @@ def main():
     n_prof = 8
     for j in range(n_prof):
         past = PROMPT_LEN + (j * (K - 1)) // max(n_prof - 1, 1)
-        for name, ms, nbytes in dec.profile_step(generated[min(past - PROMPT_LEN, K - 1)], past):
+        for name, ms, nbytes, _ in dec.profile_step(generated[min(past - PROMPT_LEN, K - 1)], past):
             a = agg.setdefault(name, [0, 0.0, 0.0])
             a[0] += 1
             a[1] += ms

@@ -57,7 +57,7 @@ class ModelConfig(C.Structure):
 
 
 class KernelTime(C.Structure):
-    _fields_ = [("name", C.c_char_p), ("ms", _f), ("bytes", C.c_double)]
+    _fields_ = [("name", C.c_char_p), ("ms", _f), ("bytes", C.c_double), ("flops", C.c_double)]
 
 
 STEP_FN = C.CFUNCTYPE(_i64, _vp, _i64, _i64)
@@ -70,6 +70,7 @@ SIGNATURES = {
     "mynn_dequantize_linear": (_i, [_vp, _vp, _vp, _sz, _sz, _i, _vp]),
     "mynn_dequant_gemv": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mynn_dequant_matmul": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "mynn_set_gemm_tile": (_i, [_i]),
     "mynn_quantized_matmul": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mynn_dynamic_quantize_linear": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mynn_attention": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
@@ -95,6 +96,7 @@ SIGNATURES = {
     "mynn_model_stats": (_i, [_vp, C.POINTER(_sz), C.POINTER(_i), C.POINTER(_i)]),
     "mynn_model_decode_loop": (_i, [_vp, C.c_int32, _i64, _i, _vp]),
     "mynn_model_profile_step": (_i, [_vp, C.c_int32, _i64, C.POINTER(KernelTime), _i]),
+    "mynn_model_profile": (_i, [_vp, _vp, _vp, _i64, _i64, C.POINTER(KernelTime), _i]),
     "mynn_quantize_per_channel": (_i, [_vp, _vp, _vp, _sz, _sz, _i]),
     "mynn_rope_table": (_i, [_vp, _vp, _i, _i, _f, _i]),
     "mynn_llm_create": (_vp, [_vp, _vp, _i, _i, _i64]),
@@ -400,11 +402,26 @@ class Decoder:
         return list(out)
 
     def profile_step(self, token, past_len, cap=1024):
+        """[(name, ms, algorithmic bytes, flops)] of one eager batch-1 decode step."""
         arr = (KernelTime * cap)()
         n = lib().mynn_model_profile_step(self.handle, int(token), int(past_len), arr, cap)
         if n < 0:
             check(n)
-        return [(arr[i].name.decode(), arr[i].ms, arr[i].bytes) for i in range(n)]
+        return [(arr[i].name.decode(), arr[i].ms, arr[i].bytes, arr[i].flops) for i in range(n)]
+
+    def profile(self, ids, positions, past_len, active, cap=2048):
+        """Same for any model shape; operands as in step()."""
+        import numpy as np
+
+        ids = np.ascontiguousarray(np.asarray(ids, np.int64).ravel())
+        positions = np.ascontiguousarray(np.asarray(positions, np.int64).ravel())
+        assert ids.size == self.cfg.batch * self.cfg.seq_q and positions.size == self.cfg.seq_q
+        arr = (KernelTime * cap)()
+        n = lib().mynn_model_profile(self.handle, ids.ctypes.data_as(_vp), positions.ctypes.data_as(_vp),
+                                     int(past_len), int(active), arr, cap)
+        if n < 0:
+            check(n)
+        return [(arr[i].name.decode(), arr[i].ms, arr[i].bytes, arr[i].flops) for i in range(n)]
 
     def stats(self):
         a, n, g = _sz(), _i(), _i()
@@ -455,6 +472,11 @@ class LlmSession:
         if n < 0:
             raise MynnError("generate_ids error %d: %s" % (n, lib().mynn_last_error().decode()))
         return [int(t) for t in out[:n]]
+
+
+def set_gemm_tile(which):
+    """0 = per-shape choice, 1 = 256x128, 2 = 256x256 workgroup tile of the matrix-core GEMM."""
+    check(lib().mynn_set_gemm_tile(int(which)))
 
 
 def quantize_per_channel(w_f32, scale_dt):

@@ -53,11 +53,14 @@ struct Layer {
     Lin qkv, o, gate, up, gu, down;  // qkv = rows of q,k,v concatenated; gu = gate/up rows interleaved
     void *k_cache = nullptr, *v_cache = nullptr;
     void *own_qkv_w = nullptr, *own_qkv_s = nullptr, *own_gu_w = nullptr, *own_gu_s = nullptr;
+    // prefill executors: weights dequantised once to the 16-bit type, [N, Kp] (wt_gu: gate/up in groups of 32)
+    void *wt_qkv = nullptr, *wt_o = nullptr, *wt_gu = nullptr, *wt_down = nullptr;
 };
 
 struct Launch {
     const char *name;
     double bytes;
+    double flops;
 };
 
 struct Model {
@@ -66,6 +69,8 @@ struct Model {
     Lin embed, lm_head;
     const void *final_norm = nullptr;
     std::vector<Layer> layers;
+    void *wt_lm_head = nullptr;
+    bool resident16 = false;  // the wt_* copies exist and the matrix-core path with fused stores is used
     void *cos_t = nullptr, *sin_t = nullptr;
     // arena
     char *arena = nullptr;
@@ -107,30 +112,14 @@ struct ArenaPlan {
     }
 };
 
-static void note(Model &m, const char *name, double bytes) {
+static void note(Model &m, const char *name, double bytes, double flops = 0.0) {
     if (m.profiling) {
         hipEvent_t e;
         hipEventCreate(&e);
         hipEventRecord(e, m.stream);
         m.events.push_back(e);
     }
-    m.record.push_back({name, bytes});
-}
-
-template <typename T>
-static int linear_rows(Model &m, void *out, const void *act, const Lin &l, int M, const char *name) {
-    const double eb = sizeof(T);
-    if (l.scale) {
-        note(m, name, (double)l.N * l.K + l.N * eb + (double)M * l.K * eb + (double)M * l.N * eb);
-        if (M >= 16 && l.K % 8 == 0)
-            return dequant_gemm_mfma(out, act, (const int8_t *)l.w, l.scale, M, l.N, l.K, m.cfg.dtype, m.stream);
-        return dequant_gemv_dispatch(out, act, (const int8_t *)l.w, l.scale, M, l.N, l.K, m.cfg.dtype, m.cfg.dtype,
-                                     m.stream);
-    }
-    note(m, name, ((double)l.N * l.K + (double)M * l.K + (double)M * l.N) * eb);
-    hipLaunchKernelGGL(dense_linear_kernel<T>, dim3(l.N, M), dim3(64), 0, m.stream, (T *)out, (const T *)act,
-                       (const T *)l.w, l.N, l.K, l.N);
-    return launch_status("dense_linear_kernel");
+    m.record.push_back({name, bytes, flops});
 }
 
 #define TRY(expr)            \
@@ -138,6 +127,35 @@ static int linear_rows(Model &m, void *out, const void *act, const Lin &l, int M
         int rc__ = (expr);   \
         if (rc__) return rc__; \
     } while (0)
+
+// one matrix-core GEMM against a resident dequantised weight
+static int gemm_rows(Model &m, void *out, const void *act, const void *wt, const void *res, int M, int N, int K, int epi,
+                     const char *name) {
+    const double eb = 2.0, n_out = epi == GEMM_SWIGLU ? N / 2 : N;
+    note(m, name, ((double)N * K + (double)M * K + (double)M * n_out * (epi == GEMM_RESIDUAL ? 2 : 1)) * eb, 2.0 * M * N * K);
+    return gemm_nt_mfma(out, act, wt, res, M, N, K, m.cfg.dtype, epi, m.stream);
+}
+
+template <typename T>
+static int linear_rows(Model &m, void *out, const void *act, const Lin &l, int M, const char *name) {
+    const double eb = sizeof(T);
+    if (l.scale) {
+        if (M >= 16 && l.K % 8 == 0) {
+            // W_T = T(wq * scale) into the workspace, then the matrix-core product (two launches, two records)
+            note(m, "dequant_weight", (double)l.N * l.K * (1 + eb) + l.N * eb);
+            TRY(dequant_weight_to_workspace((const int8_t *)l.w, l.scale, l.N, l.K, m.cfg.dtype, m.stream));
+            note(m, name, ((double)l.N * l.K + (double)M * l.K + (double)M * l.N) * eb, 2.0 * M * l.N * l.K);
+            return gemm_from_workspace(out, act, M, l.N, l.K, m.cfg.dtype, m.stream);
+        }
+        note(m, name, (double)l.N * l.K + l.N * eb + (double)M * l.K * eb + (double)M * l.N * eb, 2.0 * M * l.N * l.K);
+        return dequant_gemv_dispatch(out, act, (const int8_t *)l.w, l.scale, M, l.N, l.K, m.cfg.dtype, m.cfg.dtype,
+                                     m.stream);
+    }
+    note(m, name, ((double)l.N * l.K + (double)M * l.K + (double)M * l.N) * eb, 2.0 * M * l.N * l.K);
+    hipLaunchKernelGGL(dense_linear_kernel<T>, dim3(l.N, M), dim3(64), 0, m.stream, (T *)out, (const T *)act,
+                       (const T *)l.w, l.N, l.K, l.N);
+    return launch_status("dense_linear_kernel");
+}
 
 template <typename T>
 static int enqueue_step(Model &m) {
@@ -169,7 +187,8 @@ static int enqueue_step(Model &m) {
         } else {
             note(m, "rms_norm", 2.0 * rows * H * eb + H * eb);
             TRY(mynn_rms_norm(m.nrm, m.x, L.norm1, rows, H, c.eps, c.dtype, s));
-            TRY(linear_rows<T>(m, m.qkv, m.nrm, L.qkv, rows, "linear_qkv"));
+            if (m.resident16) TRY(gemm_rows(m, m.qkv, m.nrm, L.wt_qkv, nullptr, rows, L.qkv.N, H, GEMM_PLAIN, "linear_qkv"));
+            else TRY(linear_rows<T>(m, m.qkv, m.nrm, L.qkv, rows, "linear_qkv"));
         }
         {
             AttnParams p{};
@@ -189,7 +208,8 @@ static int enqueue_step(Model &m) {
                                       Hq, Hkv, D, c.max_seq, s));
                 // bytes: q in, out; the K/V rows read depend on the context, which the host does not
                 // know under replay -- callers add 2*KD*eb per cached row when they report
-                note(m, "attention", (double)rows * 2.0 * QD * eb);
+                // flops: the causal half of QK^T and PV over the new rows alone (exact when past_len is 0)
+                note(m, "attention", (double)rows * 2.0 * QD * eb, S > 1 ? 2.0 * B * Hq * D * (double)S * (S + 1) : 0.0);
                 if (S > 1 && attention_prefill_supported(p, D, c.dtype, 0)) TRY(attention_prefill_launch(p, D, c.dtype, s));
                 else TRY(attention_decode_launch(p, D, c.dtype, 0, m.attn_scratch, m.attn_counters, s));
             }
@@ -201,6 +221,13 @@ static int enqueue_step(Model &m) {
             TRY(gemv_norm_swiglu<T>(m.hmid, m.x2, L.norm2, c.eps, (const int8_t *)L.gu.w, L.gu.scale, L.gu.N, H, s));
             note(m, "gemv_down_residual", (double)H * F + H * eb + F * eb + 2 * H * eb);
             TRY(gemv_residual<T>(m.x, m.hmid, (const int8_t *)L.down.w, L.down.scale, m.x2, H, F, s));
+        } else if (m.resident16) {
+            // residual adds and SwiGLU ride on the GEMM stores
+            TRY(gemm_rows(m, m.x2, m.attn, L.wt_o, m.x, rows, H, QD, GEMM_RESIDUAL, "linear_o_residual"));
+            note(m, "rms_norm", 2.0 * rows * H * eb + H * eb);
+            TRY(mynn_rms_norm(m.nrm, m.x2, L.norm2, rows, H, c.eps, c.dtype, s));
+            TRY(gemm_rows(m, m.hmid, m.nrm, L.wt_gu, nullptr, rows, 2 * F, H, GEMM_SWIGLU, "linear_gateup_swiglu"));
+            TRY(gemm_rows(m, m.x, m.hmid, L.wt_down, m.x2, rows, H, F, GEMM_RESIDUAL, "linear_down_residual"));
         } else {
             TRY(linear_rows<T>(m, m.proj, m.attn, L.o, rows, "linear_o"));
             note(m, "add", 3.0 * rows * H * eb);
@@ -222,7 +249,8 @@ static int enqueue_step(Model &m) {
     } else {
         note(m, "rms_norm", 2.0 * rows * H * eb + H * eb);
         TRY(mynn_rms_norm(m.nrm, m.x, m.final_norm, rows, H, c.eps, c.dtype, s));
-        TRY(linear_rows<T>(m, m.logits, m.nrm, m.lm_head, rows, "linear_lm_head"));
+        if (m.resident16) TRY(gemm_rows(m, m.logits, m.nrm, m.wt_lm_head, nullptr, rows, V, H, GEMM_PLAIN, "linear_lm_head"));
+        else TRY(linear_rows<T>(m, m.logits, m.nrm, m.lm_head, rows, "linear_lm_head"));
     }
     // greedy token of the last row of each sequence; for a batch-1 decode step the same launch
     // moves the device-side loop state on (token -> next input, position / past / active + 1)
@@ -320,6 +348,27 @@ static int build(Model &m, void **init, void **state) {
     MYNN_HIP(hipStreamCreateWithFlags(&m.stream, hipStreamNonBlocking));
     TRY(host_rope_tables(m));
 
+    // ---- prefill executors keep every linear weight dequantised to the 16-bit type (2 bytes per weight
+    // on top of the int8 originals): the matrix-core GEMM reads them directly, and the values are
+    // those of the per-call dequantisation, T(wq * scale)
+    if (m.quant && c.batch * c.seq_q >= 16 && H % 8 == 0 && QD % 8 == 0 && F % 32 == 0) {
+        auto resident = [&](void **dst, const Lin &l) {
+            MYNN_HIP(hipMalloc(dst, gemm_weight_bytes(l.N, l.K)));
+            return dequant_weight_rows(*dst, (const int8_t *)l.w, l.scale, l.N, l.K, c.dtype, 0, 0, m.stream);
+        };
+        for (Layer &L : m.layers) {
+            TRY(resident(&L.wt_qkv, L.qkv));
+            TRY(resident(&L.wt_o, L.o));
+            TRY(resident(&L.wt_down, L.down));
+            MYNN_HIP(hipMalloc(&L.wt_gu, gemm_weight_bytes(2 * F, H)));
+            TRY(dequant_weight_rows(L.wt_gu, (const int8_t *)L.gate.w, L.gate.scale, F, H, c.dtype, 32, 0, m.stream));
+            TRY(dequant_weight_rows(L.wt_gu, (const int8_t *)L.up.w, L.up.scale, F, H, c.dtype, 32, 1, m.stream));
+        }
+        TRY(resident(&m.wt_lm_head, m.lm_head));
+        MYNN_HIP(hipStreamSynchronize(m.stream));
+        m.resident16 = true;
+    }
+
     // ---- arena: every activation of one step, the device scalars, attention split scratch
     const int rows = c.batch * c.seq_q;
     attn_plan(c.batch, c.seq_q, c.n_heads, c.n_kv_heads, c.head_dim, c.dtype, 0, c.max_seq, &m.slice, &m.nsplit, &m.heads_per_wg);
@@ -391,7 +440,12 @@ static void destroy(Model *m) {
         if (L.own_qkv_s) hipFree(L.own_qkv_s);
         if (L.own_gu_w) hipFree(L.own_gu_w);
         if (L.own_gu_s) hipFree(L.own_gu_s);
+        if (L.wt_qkv) hipFree(L.wt_qkv);
+        if (L.wt_o) hipFree(L.wt_o);
+        if (L.wt_gu) hipFree(L.wt_gu);
+        if (L.wt_down) hipFree(L.wt_down);
     }
+    if (m->wt_lm_head) hipFree(m->wt_lm_head);
     if (m->cos_t) hipFree(m->cos_t);
     if (m->sin_t) hipFree(m->sin_t);
     if (m->arena) hipFree(m->arena);
@@ -566,13 +620,7 @@ extern "C" int mynn_model_decode_loop(void *state, int32_t token, int64_t past_l
     return 0;
 }
 
-extern "C" int mynn_model_profile_step(void *state, int32_t token, int64_t past_len, mynn_kernel_time *out, int cap) {
-    MYNN_REQUIRE(state && out && cap > 0, MYNN_ERR_INVALID, "profile_step: bad argument");
-    Model &m = *(Model *)state;
-    const mynn_model_config &c = m.cfg;
-    MYNN_REQUIRE(c.batch * c.seq_q == 1, MYNN_ERR_STATE, "profile_step: needs a batch-1 decode model");
-    int64_t id = token, pos = past_len;
-    TRY(upload_inputs(m, &id, &pos, past_len, past_len + 1));
+static int profile_enqueue(Model &m, mynn_kernel_time *out, int cap) {
     m.profiling = true;
     int rc = enqueue(m);
     m.profiling = false;
@@ -585,6 +633,25 @@ extern "C" int mynn_model_profile_step(void *state, int32_t token, int64_t past_
         out[i].name = m.record[i].name;
         out[i].ms = ms;
         out[i].bytes = m.record[i].bytes;
+        out[i].flops = m.record[i].flops;
     }
     return n < cap ? n : cap;
+}
+
+extern "C" int mynn_model_profile_step(void *state, int32_t token, int64_t past_len, mynn_kernel_time *out, int cap) {
+    MYNN_REQUIRE(state && out && cap > 0, MYNN_ERR_INVALID, "profile_step: bad argument");
+    Model &m = *(Model *)state;
+    const mynn_model_config &c = m.cfg;
+    MYNN_REQUIRE(c.batch * c.seq_q == 1, MYNN_ERR_STATE, "profile_step: needs a batch-1 decode model");
+    int64_t id = token, pos = past_len;
+    TRY(upload_inputs(m, &id, &pos, past_len, past_len + 1));
+    return profile_enqueue(m, out, cap);
+}
+
+extern "C" int mynn_model_profile(void *state, const int64_t *input_ids, const int64_t *position_id, int64_t past_len,
+                                  int64_t active_seq_kv, mynn_kernel_time *out, int cap) {
+    MYNN_REQUIRE(state && input_ids && position_id && out && cap > 0, MYNN_ERR_INVALID, "profile: bad argument");
+    Model &m = *(Model *)state;
+    TRY(upload_inputs(m, input_ids, position_id, past_len, active_seq_kv));
+    return profile_enqueue(m, out, cap);
 }

@@ -2,6 +2,7 @@
 // quantizing), DequantizeLinear, row gather, SwiGLU / Add groups, dynamic activation
 // quantisation and the greedy argmax.  All compute in f32 and round once at the store.
 #include "kernels.h"
+#include "mfma.h"
 
 namespace mynn {
 
@@ -44,6 +45,45 @@ __global__ __launch_bounds__(kEwThreads) void rms_norm_kernel(T *out, const T *x
     const float inv = 1.0f / sqrtf(tot / (float)dim + eps);
     for (int i = threadIdx.x; i < dim; i += kEwThreads)
         Elem<T>::st(out, base + i, (Elem<T>::ld(x, base + i) * inv) * Elem<T>::ld(w, i));
+}
+
+// Rows of 16-bit values whose length is a multiple of 8 and at most 8 * 4 * kEwThreads: 128-bit
+// loads, the row read once and kept in registers between the two passes.
+template <typename T>
+__global__ __launch_bounds__(kEwThreads) void rms_norm_vec_kernel(T *out, const T *x, const T *w, int dim, float eps) {
+    __shared__ float red[4];
+    const size_t base = (size_t)blockIdx.x * dim;
+    const int chunks = dim >> 3;
+    U4 v[4];
+    float ss = 0.f;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int c = threadIdx.x + q * kEwThreads;
+        if (c < chunks) {
+            v[q] = *(const U4 *)(x + base + (size_t)c * 8);
+            float f[8];
+            widen8<T>(v[q], f);
+#pragma unroll
+            for (int i = 0; i < 8; i++) ss += f[i] * f[i];
+        }
+    }
+    const float tot = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(tot / (float)dim + eps);
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int c = threadIdx.x + q * kEwThreads;
+        if (c < chunks) {
+            float f[8], g[8];
+            widen8<T>(v[q], f);
+            widen8<T>(*(const U4 *)(w + (size_t)c * 8), g);
+            U4 o;
+            o.x = pack2<T>((f[0] * inv) * g[0], (f[1] * inv) * g[1]);
+            o.y = pack2<T>((f[2] * inv) * g[2], (f[3] * inv) * g[3]);
+            o.z = pack2<T>((f[4] * inv) * g[4], (f[5] * inv) * g[5]);
+            o.w = pack2<T>((f[6] * inv) * g[6], (f[7] * inv) * g[7]);
+            *(U4 *)(out + base + (size_t)c * 8) = o;
+        }
+    }
 }
 
 // ---- Rope (reference rope.cuh:18-46): one thread per (row, j < D/2) --------------------------
@@ -280,6 +320,13 @@ extern "C" int mynn_rms_norm(void *out, const void *x, const void *w, int rows, 
     MYNN_REQUIRE(out && x && w && rows > 0 && dim > 0, MYNN_ERR_INVALID, "rms_norm: bad operand");
     return dispatch_dtype(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
+        if constexpr (sizeof(T) == 2) {
+            if (dim % 8 == 0 && dim <= 8 * 4 * kEwThreads && aligned16(out) && aligned16(x) && aligned16(w)) {
+                hipLaunchKernelGGL(rms_norm_vec_kernel<T>, dim3(rows), dim3(kEwThreads), 0, as_stream(s), (T *)out,
+                                   (const T *)x, (const T *)w, dim, eps);
+                return launch_status("rms_norm_vec_kernel");
+            }
+        }
         hipLaunchKernelGGL(rms_norm_kernel<T>, dim3(rows), dim3(kEwThreads), 0, as_stream(s), (T *)out, (const T *)x,
                            (const T *)w, dim, eps);
         return launch_status("rms_norm_kernel");

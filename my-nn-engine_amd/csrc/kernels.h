@@ -19,6 +19,19 @@ int dequant_gemv_dispatch(void *out, const void *act, const int8_t *wq, const vo
                           int act_dtype, int out_dtype, hipStream_t s);
 
 // gemm.hip -- matrix-core DequantMatMul, M >= 16, 16-bit types
+// matrix-core GEMM pieces.  A dequantised weight is [N, Kp] of the 16-bit type, Kp = K rounded up to 64,
+// zero padded (gemm_weight_bytes); dequant_weight_rows writes one (group/which: see gemm.hip), and
+// gemm_nt_mfma multiplies by it: out = store(act . wt^T) with the store one of GEMM_*.
+enum { GEMM_PLAIN = 0, GEMM_RESIDUAL = 1, GEMM_SWIGLU = 2 };
+size_t gemm_weight_bytes(int N, int K);
+int dequant_weight_rows(void *dst, const int8_t *wq, const void *scale, int N, int K, int dtype, int group, int which,
+                        hipStream_t s);
+void gemm_set_tile(int which);  // 0 heuristic, 1 = 256x128, 2 = 256x256 workgroup tile
+int gemm_nt_mfma(void *out, const void *act, const void *wt, const void *res, int M, int N, int K, int dtype, int epi,
+                 hipStream_t s);
+// the two halves of dequant_gemm_mfma: W_T = T(wq * scale) into the library workspace, then out = act . W_T^T
+int dequant_weight_to_workspace(const int8_t *wq, const void *scale, int N, int K, int dtype, hipStream_t s);
+int gemm_from_workspace(void *out, const void *act, int M, int N, int K, int dtype, hipStream_t s);
 int dequant_gemm_mfma(void *out, const void *act, const int8_t *wq, const void *scale, int M, int N, int K,
                       int dtype, hipStream_t s);
 

@@ -6,6 +6,7 @@
 // Arithmetic is unchanged: lo' = lo*cos[p,j] - hi*sin[p,j], hi' = hi*cos[p,j+D/2] + lo*sin[p,j+D/2]
 // with separate products and one rounding; v is copied.
 #include "kernels.h"
+#include "mfma.h"
 
 namespace mynn {
 
@@ -36,11 +37,64 @@ __global__ void rope_kv_append_kernel(T *q_out, T *k_cache, T *v_cache, const T 
     }
 }
 
+// Same work for head_dim % 16 == 0, 128 bits per access: one workgroup per token row, one thread per
+// (head, 8 rotation pairs) -- it loads the 8 low and the 8 high elements and the matching table
+// entries, and writes both halves; v heads copy two chunks.
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kv_append_vec_kernel(T *q_out, T *k_cache, T *v_cache, const T *qkv,
+                                                                 const T *cos_t, const T *sin_t, const int64_t *position,
+                                                                 const int32_t *d_past, int past_host, int S, int Hq,
+                                                                 int Hkv, int D, int max_seq) {
+    const int s = blockIdx.x, b = blockIdx.y;
+    const int half = D / 2, upc = half / 8;  // units per head
+    const int past = d_past ? *d_past : past_host;
+    const size_t row = (size_t)b * S + s;
+    const int heads = Hq + 2 * Hkv;
+    const T *src_row = qkv + row * (size_t)heads * D;
+    const size_t tab = (size_t)position[s] * D;
+    for (int u = threadIdx.x; u < heads * upc; u += blockDim.x) {
+        const int head = u / upc, j = (u % upc) * 8;
+        const T *src = src_row + (size_t)head * D;
+        const U4 lo = *(const U4 *)(src + j), hi = *(const U4 *)(src + j + half);
+        if (head >= Hq + Hkv) {
+            T *dst = v_cache + (((size_t)b * Hkv + (head - Hq - Hkv)) * max_seq + past + s) * D;
+            *(U4 *)(dst + j) = lo;
+            *(U4 *)(dst + j + half) = hi;
+            continue;
+        }
+        T *dst = head < Hq ? q_out + row * (size_t)Hq * D + (size_t)head * D
+                           : k_cache + (((size_t)b * Hkv + (head - Hq)) * max_seq + past + s) * D;
+        float xl[8], xh[8], cl[8], ch[8], sl[8], sh[8], ol[8], oh[8];
+        widen8<T>(lo, xl);
+        widen8<T>(hi, xh);
+        widen8<T>(*(const U4 *)(cos_t + tab + j), cl);
+        widen8<T>(*(const U4 *)(cos_t + tab + j + half), ch);
+        widen8<T>(*(const U4 *)(sin_t + tab + j), sl);
+        widen8<T>(*(const U4 *)(sin_t + tab + j + half), sh);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            ol[i] = xl[i] * cl[i] - xh[i] * sl[i];
+            oh[i] = xh[i] * ch[i] + xl[i] * sh[i];
+        }
+        *(U4 *)(dst + j) = U4{pack2<T>(ol[0], ol[1]), pack2<T>(ol[2], ol[3]), pack2<T>(ol[4], ol[5]), pack2<T>(ol[6], ol[7])};
+        *(U4 *)(dst + j + half) = U4{pack2<T>(oh[0], oh[1]), pack2<T>(oh[2], oh[3]), pack2<T>(oh[4], oh[5]), pack2<T>(oh[6], oh[7])};
+    }
+}
+
 template <typename T>
 int rope_kv_append(void *q_out, void *k_cache, void *v_cache, const void *qkv, const void *cos_t, const void *sin_t,
                    const int64_t *position, const int32_t *d_past, int past_host, int B, int S, int Hq, int Hkv, int D,
                    int max_seq, hipStream_t s) {
     MYNN_REQUIRE(S <= 65535 * 32 && Hq + 2 * Hkv <= 65535 && B <= 65535, MYNN_ERR_UNSUPPORTED, "rope_kv_append: grid");
+    if (D % 16 == 0 && S <= 65535 * 32 && aligned16(q_out) && aligned16(k_cache) && aligned16(v_cache) && aligned16(qkv) &&
+        aligned16(cos_t) && aligned16(sin_t)) {
+        const int units = (Hq + 2 * Hkv) * (D / 16);
+        const int threads = units >= 256 ? 256 : (units + 63) / 64 * 64;
+        hipLaunchKernelGGL(rope_kv_append_vec_kernel<T>, dim3(S, B), dim3(threads), 0, s, (T *)q_out, (T *)k_cache,
+                           (T *)v_cache, (const T *)qkv, (const T *)cos_t, (const T *)sin_t, position, d_past, past_host,
+                           S, Hq, Hkv, D, max_seq);
+        return launch_status("rope_kv_append_vec_kernel");
+    }
     int threads = D / 2 >= 64 ? 64 : 32;
     hipLaunchKernelGGL(rope_kv_append_kernel<T>, dim3(S, Hq + 2 * Hkv, B), dim3(threads), 0, s, (T *)q_out,
                        (T *)k_cache, (T *)v_cache, (const T *)qkv, (const T *)cos_t, (const T *)sin_t, position, d_past,

@@ -115,9 +115,16 @@ def test_generate_bookkeeping_and_errors(g):
     llm.close(), dec.close()
 
 
+@pytest.fixture(params=[0, 1, 2], ids=["tile_auto", "tile_256x128", "tile_256x256"])
+def gemm_tile(g, request):
+    g.mynn.set_gemm_tile(request.param)
+    yield request.param
+    g.mynn.set_gemm_tile(0)
+
+
 @pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
 @pytest.mark.parametrize("P", [4, 32])
-def test_prefill_model_logits_and_kv_vs_oracle(g, dt, P):
+def test_prefill_model_logits_and_kv_vs_oracle(g, dt, P, gemm_tile):
     """Mode::Prefill{len}: one graph run over P tokens writes P cache rows and returns [P, vocab]
     logits; rows < 16 take the scale-after-sum kernels, rows >= 16 the matrix cores, exactly as
     the reference dispatches (src/codegen/cuda.rs:1518-1652)."""

@@ -40,7 +40,8 @@ def test_dequant_matmul_goldens(g, name):
 
 
 @pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
-@pytest.mark.parametrize("M,N,K", [(16, 128, 32), (200, 300, 512), (129, 127, 40), (515, 385, 96), (128, 2560, 2048), (64, 2048, 5632)])
+@pytest.mark.parametrize("M,N,K", [(16, 128, 32), (200, 300, 512), (129, 127, 40), (515, 385, 96), (128, 2560, 2048), (64, 2048, 5632),
+                                   (4096, 4096, 64), (4000, 4090, 72)])
 def test_dequant_matmul_mfma_vs_oracle(g, dt, M, N, K):
     rng = np.random.default_rng(M * 7 + N * 3 + K)
     act = orc.to_storage(rng.standard_normal((M, K)), dt)
