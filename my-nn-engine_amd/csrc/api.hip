@@ -22,6 +22,11 @@ int fail(int code, const char *fmt, ...) {
     va_end(ap);
     return code;
 }
+LaunchTimer &launch_timer() {
+    static thread_local LaunchTimer t;
+    return t;
+}
+
 int hip_fail(hipError_t e, const char *what) {
     snprintf(g_err, sizeof g_err, "%s: %s (%d)", what, hipGetErrorString(e), (int)e);
     return (int)e;

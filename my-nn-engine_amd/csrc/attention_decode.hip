@@ -328,7 +328,7 @@ static int launch_one(const AttnParams &p, hipStream_t s) {
         attr_set = true;
     }
     dim3 grid(p.B * p.Hkv * ((p.Hq / p.Hkv) / G), p.nsplit, p.Sq), block(kAttnThreads);
-    hipLaunchKernelGGL((attn_decode_kernel<T, D, G, KVI8, FUSE>), grid, block, lds, s, p);
+    MYNN_LAUNCH((attn_decode_kernel<T, D, G, KVI8, FUSE>), grid, block, lds, s, p);
     return launch_status("attn_decode_kernel");
 }
 

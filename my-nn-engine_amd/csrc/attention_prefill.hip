@@ -196,8 +196,8 @@ int attention_prefill_launch(const AttnParams &p, int D, int dtype, hipStream_t 
     dim3 grid((p.Sq + kPfRows - 1) / kPfRows, p.B * p.Hq);
     return dispatch_dtype16(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
-        if (D == 64) hipLaunchKernelGGL((attn_prefill_kernel<T, 64>), grid, dim3(kPfThreads), 0, s, p);
-        else hipLaunchKernelGGL((attn_prefill_kernel<T, 128>), grid, dim3(kPfThreads), 0, s, p);
+        if (D == 64) MYNN_LAUNCH((attn_prefill_kernel<T, 64>), grid, dim3(kPfThreads), 0, s, p);
+        else MYNN_LAUNCH((attn_prefill_kernel<T, 128>), grid, dim3(kPfThreads), 0, s, p);
         return launch_status("attn_prefill_kernel");
     });
 }

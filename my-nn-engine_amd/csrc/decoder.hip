@@ -114,10 +114,13 @@ struct ArenaPlan {
 
 static void note(Model &m, const char *name, double bytes, double flops = 0.0) {
     if (m.profiling) {
-        hipEvent_t e;
-        hipEventCreate(&e);
-        hipEventRecord(e, m.stream);
-        m.events.push_back(e);
+        // the launch that follows stamps these two with its own start and end
+        hipEvent_t a, b;
+        hipEventCreate(&a);
+        hipEventCreate(&b);
+        m.events.push_back(a);
+        m.events.push_back(b);
+        launch_timer() = LaunchTimer{a, b};
     }
     m.record.push_back({name, bytes, flops});
 }
@@ -152,7 +155,7 @@ static int linear_rows(Model &m, void *out, const void *act, const Lin &l, int M
                                      m.stream);
     }
     note(m, name, ((double)l.N * l.K + (double)M * l.K + (double)M * l.N) * eb, 2.0 * M * l.N * l.K);
-    hipLaunchKernelGGL(dense_linear_kernel<T>, dim3(l.N, M), dim3(64), 0, m.stream, (T *)out, (const T *)act,
+    MYNN_LAUNCH(dense_linear_kernel<T>, dim3(l.N, M), dim3(64), 0, m.stream, (T *)out, (const T *)act,
                        (const T *)l.w, l.N, l.K, l.N);
     return launch_status("dense_linear_kernel");
 }
@@ -260,12 +263,7 @@ static int enqueue_step(Model &m) {
         if (rows == 1) adv = AdvanceState{m.d_ids, m.d_pos, m.d_past, m.d_active, m.d_tokens, m.d_step, m.token_cap};
         TRY(argmax_rows<T>(m.d_next + b, (const T *)m.logits + ((size_t)b * S + (S - 1)) * V, 1, V, adv, s));
     }
-    if (m.profiling) {
-        hipEvent_t e;
-        hipEventCreate(&e);
-        hipEventRecord(e, s);
-        m.events.push_back(e);
-    }
+    launch_timer() = LaunchTimer{};
     m.launches = (int)m.record.size();
     return 0;
 }
@@ -621,15 +619,22 @@ extern "C" int mynn_model_decode_loop(void *state, int32_t token, int64_t past_l
 }
 
 static int profile_enqueue(Model &m, mynn_kernel_time *out, int cap) {
+    for (hipEvent_t e : m.events) hipEventDestroy(e);
+    m.events.clear();
     m.profiling = true;
     int rc = enqueue(m);
     m.profiling = false;
+    launch_timer() = LaunchTimer{};
     if (rc) return rc;
     MYNN_HIP(hipStreamSynchronize(m.stream));
     int n = (int)m.record.size();
     for (int i = 0; i < n && i < cap; i++) {
         float ms = 0.f;
-        MYNN_HIP(hipEventElapsedTime(&ms, m.events[i], m.events[i + 1]));
+        // a record whose launch did not take the pair (or that made none) reports 0
+        if (hipEventElapsedTime(&ms, m.events[2 * i], m.events[2 * i + 1]) != hipSuccess) {
+            (void)hipGetLastError();
+            ms = 0.f;
+        }
         out[i].name = m.record[i].name;
         out[i].ms = ms;
         out[i].bytes = m.record[i].bytes;

@@ -292,7 +292,7 @@ __global__ __launch_bounds__(1024) void argmax_last_kernel(int32_t *out, const T
 
 template <typename T>
 int argmax_rows(int32_t *out, const void *logits, int rows, int n, AdvanceState adv, hipStream_t s) {
-    hipLaunchKernelGGL(argmax_last_kernel<T>, dim3(rows), dim3(1024), 0, s, out, (const T *)logits, n, adv);
+    MYNN_LAUNCH(argmax_last_kernel<T>, dim3(rows), dim3(1024), 0, s, out, (const T *)logits, n, adv);
     return launch_status("argmax_last_kernel");
 }
 template int argmax_rows<bf16_t>(int32_t *, const void *, int, int, AdvanceState, hipStream_t);
@@ -302,7 +302,7 @@ template int argmax_rows<float>(int32_t *, const void *, int, int, AdvanceState,
 template <typename T>
 int embed_dequant(void *out, const int8_t *table, const void *scale, const int64_t *ids, int n_ids, int vocab,
                   int hidden, hipStream_t s) {
-    hipLaunchKernelGGL(embed_dequant_kernel<T>, dim3(n_ids), dim3(256), 0, s, (T *)out, table, (const T *)scale, ids,
+    MYNN_LAUNCH(embed_dequant_kernel<T>, dim3(n_ids), dim3(256), 0, s, (T *)out, table, (const T *)scale, ids,
                        vocab, hidden);
     return launch_status("embed_dequant_kernel");
 }
@@ -322,12 +322,12 @@ extern "C" int mynn_rms_norm(void *out, const void *x, const void *w, int rows, 
         using T = std::remove_pointer_t<decltype(t)>;
         if constexpr (sizeof(T) == 2) {
             if (dim % 8 == 0 && dim <= 8 * 4 * kEwThreads && aligned16(out) && aligned16(x) && aligned16(w)) {
-                hipLaunchKernelGGL(rms_norm_vec_kernel<T>, dim3(rows), dim3(kEwThreads), 0, as_stream(s), (T *)out,
+                MYNN_LAUNCH(rms_norm_vec_kernel<T>, dim3(rows), dim3(kEwThreads), 0, as_stream(s), (T *)out,
                                    (const T *)x, (const T *)w, dim, eps);
                 return launch_status("rms_norm_vec_kernel");
             }
         }
-        hipLaunchKernelGGL(rms_norm_kernel<T>, dim3(rows), dim3(kEwThreads), 0, as_stream(s), (T *)out, (const T *)x,
+        MYNN_LAUNCH(rms_norm_kernel<T>, dim3(rows), dim3(kEwThreads), 0, as_stream(s), (T *)out, (const T *)x,
                            (const T *)w, dim, eps);
         return launch_status("rms_norm_kernel");
     });
@@ -340,7 +340,7 @@ extern "C" int mynn_rope(void *out, const void *x, const void *cos_t, const void
     size_t pairs = (size_t)outer * S * (D / 2);
     return dispatch_dtype(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
-        hipLaunchKernelGGL(rope_kernel<T>, dim3(nblocks(pairs, 256)), dim3(256), 0, as_stream(s), (T *)out,
+        MYNN_LAUNCH(rope_kernel<T>, dim3(nblocks(pairs, 256)), dim3(256), 0, as_stream(s), (T *)out,
                            (const T *)x, (const T *)cos_t, (const T *)sin_t, position, S, D, pairs);
         return launch_status("rope_kernel");
     });
@@ -357,11 +357,11 @@ extern "C" int mynn_kvcache_update(void *cache, const void *new_kv, int offset, 
     if (row_bytes % 4 == 0) {
         int dw = (int)(row_bytes / 4);
         size_t total = (size_t)BH * S_new * dw;
-        hipLaunchKernelGGL(kvcache_update_kernel<uint32_t>, dim3(nblocks(total, 256)), dim3(256), 0, as_stream(s),
+        MYNN_LAUNCH(kvcache_update_kernel<uint32_t>, dim3(nblocks(total, 256)), dim3(256), 0, as_stream(s),
                            (uint32_t *)cache, (const uint32_t *)new_kv, offset, S_new, max_seq, dw, total);
     } else {
         size_t total = (size_t)BH * S_new * D;
-        hipLaunchKernelGGL(kvcache_update_kernel<uint16_t>, dim3(nblocks(total, 256)), dim3(256), 0, as_stream(s),
+        MYNN_LAUNCH(kvcache_update_kernel<uint16_t>, dim3(nblocks(total, 256)), dim3(256), 0, as_stream(s),
                            (uint16_t *)cache, (const uint16_t *)new_kv, offset, S_new, max_seq, D, total);
     }
     return launch_status("kvcache_update_kernel");
@@ -374,7 +374,7 @@ extern "C" int mynn_quantizing_kvcache_update(int8_t *cache, void *scale, const 
                  "quantizing_kvcache_update: offset %d + %d rows exceeds max_seq %d", offset, S_new, max_seq);
     return dispatch_dtype(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
-        hipLaunchKernelGGL(quantizing_kvcache_update_kernel<T>, dim3(BH * S_new), dim3(64), 0, as_stream(s), cache,
+        MYNN_LAUNCH(quantizing_kvcache_update_kernel<T>, dim3(BH * S_new), dim3(64), 0, as_stream(s), cache,
                            (T *)scale, (const T *)new_kv, offset, S_new, max_seq, D);
         return launch_status("quantizing_kvcache_update_kernel");
     });
@@ -386,7 +386,7 @@ extern "C" int mynn_dequantize_linear(void *out, const int8_t *x, const void *sc
     size_t total = rows * cols;
     return dispatch_dtype(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
-        hipLaunchKernelGGL(dequantize_linear_kernel<T>, dim3(nblocks(total, 256)), dim3(256), 0, as_stream(s),
+        MYNN_LAUNCH(dequantize_linear_kernel<T>, dim3(nblocks(total, 256)), dim3(256), 0, as_stream(s),
                            (T *)out, x, (const T *)scale, cols, total);
         return launch_status("dequantize_linear_kernel");
     });
@@ -396,7 +396,7 @@ extern "C" int mynn_gather_rows(void *out, const void *data, const int64_t *idx,
                                 mynn_stream s) {
     MYNN_REQUIRE(out && data && idx && n_idx > 0 && rows > 0 && row_bytes > 0, MYNN_ERR_INVALID,
                  "gather_rows: bad operand");
-    hipLaunchKernelGGL(gather_rows_kernel, dim3(n_idx), dim3(256), 0, as_stream(s), (uint8_t *)out,
+    MYNN_LAUNCH(gather_rows_kernel, dim3(n_idx), dim3(256), 0, as_stream(s), (uint8_t *)out,
                        (const uint8_t *)data, idx, rows, row_bytes);
     return launch_status("gather_rows_kernel");
 }
@@ -405,7 +405,7 @@ extern "C" int mynn_swiglu(void *out, const void *gate, const void *up, size_t n
     MYNN_REQUIRE(out && gate && up && n > 0, MYNN_ERR_INVALID, "swiglu: bad operand");
     return dispatch_dtype(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
-        hipLaunchKernelGGL(swiglu_kernel<T>, dim3(nblocks(n, 256)), dim3(256), 0, as_stream(s), (T *)out,
+        MYNN_LAUNCH(swiglu_kernel<T>, dim3(nblocks(n, 256)), dim3(256), 0, as_stream(s), (T *)out,
                            (const T *)gate, (const T *)up, n);
         return launch_status("swiglu_kernel");
     });
@@ -415,7 +415,7 @@ extern "C" int mynn_add(void *out, const void *a, const void *b, size_t n, int d
     MYNN_REQUIRE(out && a && b && n > 0, MYNN_ERR_INVALID, "add: bad operand");
     return dispatch_dtype(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
-        hipLaunchKernelGGL(add_kernel<T>, dim3(nblocks(n, 256)), dim3(256), 0, as_stream(s), (T *)out, (const T *)a,
+        MYNN_LAUNCH(add_kernel<T>, dim3(nblocks(n, 256)), dim3(256), 0, as_stream(s), (T *)out, (const T *)a,
                            (const T *)b, n);
         return launch_status("add_kernel");
     });
@@ -429,10 +429,10 @@ extern "C" int mynn_dynamic_quantize_linear(void *y, void *y_scale, void *y_zero
     return dispatch_dtype(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
         if (symmetric)
-            hipLaunchKernelGGL((dynquant_kernel<T, true>), dim3(axis_dim), dim3(kEwThreads), 0, as_stream(s), y,
+            MYNN_LAUNCH((dynquant_kernel<T, true>), dim3(axis_dim), dim3(kEwThreads), 0, as_stream(s), y,
                                (T *)y_scale, y_zero_point, (const T *)x, inner_size);
         else
-            hipLaunchKernelGGL((dynquant_kernel<T, false>), dim3(axis_dim), dim3(kEwThreads), 0, as_stream(s), y,
+            MYNN_LAUNCH((dynquant_kernel<T, false>), dim3(axis_dim), dim3(kEwThreads), 0, as_stream(s), y,
                                (T *)y_scale, y_zero_point, (const T *)x, inner_size);
         return launch_status("dynquant_kernel");
     });

@@ -247,7 +247,7 @@ int dequant_weight_rows(void *dst, const int8_t *wq, const void *scale, int N, i
     const size_t chunks = (size_t)N * Kp / 8;
     return dispatch_dtype16(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
-        hipLaunchKernelGGL(dequant_rows_kernel<T>, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, s, (T *)dst, wq,
+        MYNN_LAUNCH(dequant_rows_kernel<T>, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, s, (T *)dst, wq,
                            (const T *)scale, K, Kp, chunks, group, which);
         return launch_status("dequant_rows_kernel");
     });
@@ -267,10 +267,10 @@ static int gemm_launch_tile(void *out, const void *act, const void *wt, const vo
         lds_set = true;
     }
     if (K == Kp)
-        hipLaunchKernelGGL((gemm_nt_mfma_kernel<T, G, false, EPI>), dim3(tiles), dim3(G::THREADS), G::LDS, s, (T *)out,
+        MYNN_LAUNCH((gemm_nt_mfma_kernel<T, G, false, EPI>), dim3(tiles), dim3(G::THREADS), G::LDS, s, (T *)out,
                            (const T *)act, (const T *)wt, (const T *)res, M, N, K, Kp);
     else
-        hipLaunchKernelGGL((gemm_nt_mfma_kernel<T, G, true, EPI>), dim3(tiles), dim3(G::THREADS), G::LDS, s, (T *)out,
+        MYNN_LAUNCH((gemm_nt_mfma_kernel<T, G, true, EPI>), dim3(tiles), dim3(G::THREADS), G::LDS, s, (T *)out,
                            (const T *)act, (const T *)wt, (const T *)res, M, N, K, Kp);
     return launch_status("gemm_nt_mfma_kernel");
 }

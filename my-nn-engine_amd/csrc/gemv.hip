@@ -292,7 +292,7 @@ static int launch_gemv1(const GemvParams &p, hipStream_t s) {
     int waves = (groups + passes - 1) / passes;
     const int blocks = (waves + kGemvWaves - 1) / kGemvWaves;
     waves = blocks * kGemvWaves;
-    hipLaunchKernelGGL((dequant_gemv1_kernel<T, R, NC, EPI, NORM>), dim3(blocks), dim3(kGemvThreads),
+    MYNN_LAUNCH((dequant_gemv1_kernel<T, R, NC, EPI, NORM>), dim3(blocks), dim3(kGemvThreads),
                        (size_t)p.K * sizeof(float), s, p, groups, waves);
     return launch_status("dequant_gemv1_kernel");
 }
@@ -302,7 +302,7 @@ static int launch_gemv(const GemvParams &p, hipStream_t s) {
     const int rows_per_block = kGemvWaves * R;
     dim3 grid((p.N + rows_per_block - 1) / rows_per_block);
     size_t lds = (size_t)MB * p.K * sizeof(float);
-    hipLaunchKernelGGL((dequant_gemv_kernel<TA, TO, R, MB, EPI, NORM>), grid, dim3(kGemvThreads), lds, s, p);
+    MYNN_LAUNCH((dequant_gemv_kernel<TA, TO, R, MB, EPI, NORM>), grid, dim3(kGemvThreads), lds, s, p);
     return launch_status("dequant_gemv_kernel");
 }
 
@@ -381,7 +381,7 @@ int dequant_gemv_dispatch(void *out, const void *act, const int8_t *wq, const vo
             }
             if (streaming) return gemv_small_m<TA, TO>(p, M, s);
             MYNN_REQUIRE(M <= 65535, MYNN_ERR_UNSUPPORTED, "dequant_matmul: M=%d too large for the plain kernel", M);
-            hipLaunchKernelGGL((dequant_matmul_naive_kernel<TA, TO>), dim3(N, M), dim3(64), 0, s, (TO *)out,
+            MYNN_LAUNCH((dequant_matmul_naive_kernel<TA, TO>), dim3(N, M), dim3(64), 0, s, (TO *)out,
                                (const TA *)act, wq, (const TO *)scale, N, K);
             return launch_status("dequant_matmul_naive_kernel");
         });

@@ -3,6 +3,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 #include "../../include/mynn_hip.h"
@@ -134,6 +135,25 @@ int hip_fail(hipError_t e, const char *what);
     do {                                                        \
         hipError_t e__ = (expr);                                \
         if (e__ != hipSuccess) return ::mynn::hip_fail(e__, #expr); \
+    } while (0)
+
+// A pair of events that the NEXT kernel launch made by this thread ties to its own start and end
+// timestamps (hipExtLaunchKernelGGL); that launch consumes the pair.  The executor's per-launch
+// profile sets it; everywhere else it is empty and launches are ordinary.
+struct LaunchTimer {
+    hipEvent_t start = nullptr, stop = nullptr;
+};
+LaunchTimer &launch_timer();
+
+#define MYNN_LAUNCH(kernel, grid, block, shmem, stream, ...)                                                       \
+    do {                                                                                                           \
+        mynn::LaunchTimer &lt_ = mynn::launch_timer();                                                             \
+        if (lt_.start) {                                                                                           \
+            hipExtLaunchKernelGGL(kernel, grid, block, shmem, stream, lt_.start, lt_.stop, 0, __VA_ARGS__);        \
+            lt_.start = lt_.stop = nullptr;                                                                        \
+        } else {                                                                                                   \
+            hipLaunchKernelGGL(kernel, grid, block, shmem, stream, __VA_ARGS__);                                   \
+        }                                                                                                          \
     } while (0)
 
 inline int launch_status(const char *what) {

@@ -146,7 +146,7 @@ static int qmatmul_launch(void *out, int32_t *acc_out, const int8_t *lhs, const 
                           const void *rs, int M, int N, int K, hipStream_t s) {
     if (M >= 16) {
         const int tiles = ((M + QBM - 1) / QBM) * ((N + QBN - 1) / QBN);
-        hipLaunchKernelGGL(qgemm_i8_mfma_kernel<T>, dim3(tiles), dim3(256), 0, s, (T *)out, acc_out, lhs, (const T *)ls, rhs,
+        MYNN_LAUNCH(qgemm_i8_mfma_kernel<T>, dim3(tiles), dim3(256), 0, s, (T *)out, acc_out, lhs, (const T *)ls, rhs,
                            (const T *)rs, M, N, K);
         return launch_status("qgemm_i8_mfma_kernel");
     }
@@ -156,13 +156,13 @@ static int qmatmul_launch(void *out, int32_t *acc_out, const int8_t *lhs, const 
     while (m < M) {
         const int mb = M - m >= 4 ? 4 : (M - m >= 2 ? 2 : 1);
         if (mb == 4)
-            hipLaunchKernelGGL((qgemv_i8_kernel<T, R, 4>), grid, dim3(256), 0, s, (T *)out, acc_out, lhs, (const T *)ls, rhs,
+            MYNN_LAUNCH((qgemv_i8_kernel<T, R, 4>), grid, dim3(256), 0, s, (T *)out, acc_out, lhs, (const T *)ls, rhs,
                                (const T *)rs, m, N, K);
         else if (mb == 2)
-            hipLaunchKernelGGL((qgemv_i8_kernel<T, R, 2>), grid, dim3(256), 0, s, (T *)out, acc_out, lhs, (const T *)ls, rhs,
+            MYNN_LAUNCH((qgemv_i8_kernel<T, R, 2>), grid, dim3(256), 0, s, (T *)out, acc_out, lhs, (const T *)ls, rhs,
                                (const T *)rs, m, N, K);
         else
-            hipLaunchKernelGGL((qgemv_i8_kernel<T, R, 1>), grid, dim3(256), 0, s, (T *)out, acc_out, lhs, (const T *)ls, rhs,
+            MYNN_LAUNCH((qgemv_i8_kernel<T, R, 1>), grid, dim3(256), 0, s, (T *)out, acc_out, lhs, (const T *)ls, rhs,
                                (const T *)rs, m, N, K);
         int rc = launch_status("qgemv_i8_kernel");
         if (rc) return rc;

@@ -90,13 +90,13 @@ int rope_kv_append(void *q_out, void *k_cache, void *v_cache, const void *qkv, c
         aligned16(cos_t) && aligned16(sin_t)) {
         const int units = (Hq + 2 * Hkv) * (D / 16);
         const int threads = units >= 256 ? 256 : (units + 63) / 64 * 64;
-        hipLaunchKernelGGL(rope_kv_append_vec_kernel<T>, dim3(S, B), dim3(threads), 0, s, (T *)q_out, (T *)k_cache,
+        MYNN_LAUNCH(rope_kv_append_vec_kernel<T>, dim3(S, B), dim3(threads), 0, s, (T *)q_out, (T *)k_cache,
                            (T *)v_cache, (const T *)qkv, (const T *)cos_t, (const T *)sin_t, position, d_past, past_host,
                            S, Hq, Hkv, D, max_seq);
         return launch_status("rope_kv_append_vec_kernel");
     }
     int threads = D / 2 >= 64 ? 64 : 32;
-    hipLaunchKernelGGL(rope_kv_append_kernel<T>, dim3(S, Hq + 2 * Hkv, B), dim3(threads), 0, s, (T *)q_out,
+    MYNN_LAUNCH(rope_kv_append_kernel<T>, dim3(S, Hq + 2 * Hkv, B), dim3(threads), 0, s, (T *)q_out,
                        (T *)k_cache, (T *)v_cache, (const T *)qkv, (const T *)cos_t, (const T *)sin_t, position, d_past,
                        past_host, S, Hq, Hkv, D, max_seq);
     return launch_status("rope_kv_append_kernel");
