@@ -15,8 +15,23 @@
  * order instead: ORC_LANES interleaved partial sums (element i goes to lane i % lanes), lanes
  * combined by a fixed pairwise tree.  orc_set_lanes(1) gives the plain sequential order.
  *
- * Pin status of each function (which golden vector / closed form checks it) is listed in
- * oracle/README.md and exercised by tests/test_oracle_*.py.
+ * Pin status (what checks each function besides its own formula; all in tests/test_oracle_*.py):
+ *   orc_dequant_matmul        10 dequant_matmul* fixtures of tests/single_op.rs (mode 2 bit-exact), f64 closed form
+ *   orc_quantized_matmul      5 quantized_matmul* fixtures (int32 part exact), integer brute force
+ *   orc_dynquant_*            4 dyn_quantize_linear* fixtures, round-trip bound
+ *   orc_dequantize_linear     dequantize_linear fixture
+ *   orc_attention             5 attention* fixtures, f64 brute force of tests/session_state.rs, softmax invariants
+ *   orc_kv_cache_update       kv_cache_update fixture + 3-step persistence
+ *   orc_quantizing_kv_update  quantizing_kvcache_update fixture
+ *   orc_rms_norm, orc_rope, orc_rope_table, orc_swish   closed forms of crates/llm/tests/builder_ops.rs, swish fixture
+ *   orc_gather_rows           2 gather* fixtures
+ *   orc_quantize_per_channel  known answers of crates/llm/tests/quantize.rs:106-159
+ *   orc_f32_to_f16 / bf16     exhaustive against numpy
+ *   orc_model_* (decoder executor and generate loop)   the reference's exact ids on its tiny random Llama
+ *                             (crates/llm/tests/tinyllama_random.rs:20-24) in f32/bf16/f16 and three summation orders;
+ *                             mock_decode expectations (crates/llm/tests/mock_decode.rs:30-87)
+ * Parity unpinned: none.  What no offline check fixes bit for bit is the reference's own f32 summation
+ * order (LLVM fast-math vectorisation, BLAS sgemm) and libm expf; those are covered by tolerance.
  */
 #ifndef MYNN_ORACLE_H_
 #define MYNN_ORACLE_H_
