@@ -23,6 +23,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+# HBM bytes per launch of the gate/up GEMV (TinyLlama shape, 16-bit activations) from rocprofv3
+# --pmc FETCH_SIZE (x2.000, scaled by a 256 MiB copy) + WRITE_SIZE (x1.000): 11430.0 KiB * 2 + 44.0 KiB.
+# Counters cannot be read from inside this process; the figure is carried here from that profile run.
+GATEUP_GEMV_TRAFFIC_BYTES = 23453696
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16/fp16 matrix rate
 PREFILL_BATCH, PREFILL_LEN = 8, 1024
 
@@ -170,6 +174,9 @@ def main():
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-steps", type=int, default=96)
+    ap.add_argument("--traffic-calibration", action="store_true",
+                    help="first run one 256 MiB device-to-device copy (a kernel of known traffic, for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--check-tokens", type=int, default=0,
                     help="also compare the first N greedy tokens with the oracle (slow: CPU decode)")
     args = ap.parse_args()
@@ -182,6 +189,13 @@ def main():
     import torch
 
     mynn = importlib.import_module("my-nn-engine_amd")
+    if args.traffic_calibration:
+        src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)  # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
     dt = {"f16": mynn.F16, "bf16": mynn.BF16}[args.dtype]
     eb = 2
     cfg = dict(TINYLLAMA, dtype=dt)
@@ -245,7 +259,8 @@ def main():
                    "step_algorithmic_bytes": step_bytes,
                    "step_hbm_frac": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": GATEUP_GEMV_TRAFFIC_BYTES if dom == "gemv_norm_gateup_swiglu" else None,
                      "bytes_per_launch": bytes_tot / calls, "avg_launch_us": round(ms_tot / calls * 1e3, 3),
                      "all_gemv_GBs": round(all_gemv_gbs, 1)},
     }
