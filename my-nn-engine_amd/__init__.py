@@ -53,7 +53,8 @@ _vp, _i, _sz, _f, _i64 = C.c_void_p, C.c_int, C.c_size_t, C.c_float, C.c_int64
 class ModelConfig(C.Structure):
     _fields_ = [("n_layers", _i), ("hidden", _i), ("n_heads", _i), ("n_kv_heads", _i), ("head_dim", _i),
                 ("ffn", _i), ("vocab", _i), ("max_seq", _i), ("eps", _f), ("rope_theta", _f), ("dtype", _i),
-                ("seq_q", _i), ("batch", _i), ("weights_int8", _i)]
+                ("seq_q", _i), ("batch", _i), ("weights_int8", _i), ("quant_kv_cache", _i),
+                ("quantize_activations", _i)]
 
 
 class KernelTime(C.Structure):
@@ -310,19 +311,24 @@ class Decoder:
       prefill and a decode model can share them (PersistentBuffers in the reference).
     """
 
-    def __init__(self, cfg, weights, seq_q=1, batch=1, kv=None):
+    def __init__(self, cfg, weights, seq_q=1, batch=1, kv=None, quant_kv_cache=False, quantize_activations=False):
         import torch
 
         tdt = {F16: torch.float16, BF16: torch.bfloat16}[cfg["dtype"]]
         quant = isinstance(weights["embed"], tuple)
         self.cfg = ModelConfig(cfg["n_layers"], cfg["hidden"], cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"],
                                cfg["ffn"], cfg["vocab"], cfg["max_seq"], float(cfg["eps"]), float(cfg["rope_theta"]),
-                               cfg["dtype"], seq_q, batch, int(quant))
+                               cfg["dtype"], seq_q, batch, int(quant), int(quant_kv_cache), int(quantize_activations))
         self.weights = weights  # keep the tensors alive
         if kv is None:
             shape = (batch, cfg["n_kv_heads"], cfg["max_seq"], cfg["head_dim"])
-            kv = [(torch.zeros(shape, dtype=tdt, device="cuda"), torch.zeros(shape, dtype=tdt, device="cuda"))
-                  for _ in range(cfg["n_layers"])]
+            if quant_kv_cache:  # (k i8, v i8, k_scale, v_scale) per layer
+                kv = [(torch.zeros(shape, dtype=torch.int8, device="cuda"), torch.zeros(shape, dtype=torch.int8, device="cuda"),
+                       torch.zeros(shape[:3], dtype=tdt, device="cuda"), torch.zeros(shape[:3], dtype=tdt, device="cuda"))
+                      for _ in range(cfg["n_layers"])]
+            else:
+                kv = [(torch.zeros(shape, dtype=tdt, device="cuda"), torch.zeros(shape, dtype=tdt, device="cuda"))
+                      for _ in range(cfg["n_layers"])]
         self.kv = kv
         init = []
 
@@ -343,8 +349,8 @@ class Decoder:
         init.append(_ptr(weights["final_norm"]))
         lin(weights["lm_head"])
         state = []
-        for k, v in kv:
-            state.extend([_ptr(k), _ptr(v)])
+        for bufs in kv:
+            state.extend([_ptr(t) for t in bufs])
         self._init = (_vp * len(init))(*init)
         self._state = (_vp * len(state))(*state)
         check(lib().mynn_model_configure(C.byref(self.cfg)))

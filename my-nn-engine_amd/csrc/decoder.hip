@@ -52,6 +52,7 @@ struct Layer {
     const void *norm1 = nullptr, *norm2 = nullptr;
     Lin qkv, o, gate, up, gu, down;  // qkv = rows of q,k,v concatenated; gu = gate/up rows interleaved
     void *k_cache = nullptr, *v_cache = nullptr;
+    void *k_scale = nullptr, *v_scale = nullptr;  // int8 KV cache: per-token scales [B,Hkv,max_seq]
     void *own_qkv_w = nullptr, *own_qkv_s = nullptr, *own_gu_w = nullptr, *own_gu_s = nullptr;
     // prefill executors: weights dequantised once to the 16-bit type, [N, Kp] (wt_gu: gate/up in groups of 32)
     void *wt_qkv = nullptr, *wt_o = nullptr, *wt_gu = nullptr, *wt_down = nullptr;
@@ -77,6 +78,8 @@ struct Model {
     size_t arena_bytes = 0;
     void *x = nullptr, *x2 = nullptr, *nrm = nullptr, *qkv = nullptr, *q = nullptr, *attn = nullptr, *g = nullptr,
          *u = nullptr, *hmid = nullptr, *proj = nullptr, *logits = nullptr;
+    int8_t *a8 = nullptr;    // W8A8: the current linear's activation rows as int8 [rows, max(H, QD, F)]
+    void *a8_scale = nullptr;  // and their per-row scales [rows]
     int64_t *d_ids = nullptr, *d_pos = nullptr;
     int32_t *d_past = nullptr, *d_active = nullptr, *d_next = nullptr, *d_tokens = nullptr, *d_step = nullptr;
     void *attn_scratch = nullptr, *attn_counters = nullptr;
@@ -160,6 +163,20 @@ static int linear_rows(Model &m, void *out, const void *act, const Lin &l, int M
     return launch_status("dense_linear_kernel");
 }
 
+// Options::quantize_activations: DynamicQuantizeLinear (per row, symmetric) then QuantizedMatMul.
+// `fresh` = the activation changed since the last call (q/k/v and gate/up share one quantisation,
+// as the pass caches it per value: quantize_activations.rs:121-130).
+static int linear_w8a8(Model &m, void *out, const void *act, const Lin &l, int M, bool fresh, const char *name) {
+    const double eb = dtype_size(m.cfg.dtype);
+    if (fresh) {
+        note(m, "dynamic_quantize", (double)M * l.K * (eb + 1) + M * eb);
+        TRY(mynn_dynamic_quantize_linear(m.a8, m.a8_scale, nullptr, act, M, l.K, m.cfg.dtype, 1, m.stream));
+    }
+    note(m, name, (double)l.N * l.K + (double)M * l.K + l.N * eb + (double)M * l.N * eb, 2.0 * M * l.N * l.K);
+    return mynn_quantized_matmul(out, nullptr, m.a8, m.a8_scale, (const int8_t *)l.w, l.scale, M, l.N, l.K, m.cfg.dtype,
+                                 m.stream);
+}
+
 template <typename T>
 static int enqueue_step(Model &m) {
     const mynn_model_config &c = m.cfg;
@@ -167,7 +184,8 @@ static int enqueue_step(Model &m) {
     const int H = c.hidden, Hq = c.n_heads, Hkv = c.n_kv_heads, D = c.head_dim, F = c.ffn, V = c.vocab;
     const int QD = Hq * D, KD = Hkv * D;
     const double eb = sizeof(T);
-    const bool fused = m.quant && rows == 1;
+    const bool w8a8 = c.quantize_activations != 0, kv8 = c.quant_kv_cache != 0;
+    const bool fused = m.quant && rows == 1 && !w8a8 && !kv8;
     hipStream_t s = m.stream;
     m.record.clear();
     for (hipEvent_t e : m.events) hipEventDestroy(e);
@@ -190,12 +208,14 @@ static int enqueue_step(Model &m) {
         } else {
             note(m, "rms_norm", 2.0 * rows * H * eb + H * eb);
             TRY(mynn_rms_norm(m.nrm, m.x, L.norm1, rows, H, c.eps, c.dtype, s));
-            if (m.resident16) TRY(gemm_rows(m, m.qkv, m.nrm, L.wt_qkv, nullptr, rows, L.qkv.N, H, GEMM_PLAIN, "linear_qkv"));
+            if (w8a8) TRY(linear_w8a8(m, m.qkv, m.nrm, L.qkv, rows, true, "qlinear_qkv"));
+            else if (m.resident16) TRY(gemm_rows(m, m.qkv, m.nrm, L.wt_qkv, nullptr, rows, L.qkv.N, H, GEMM_PLAIN, "linear_qkv"));
             else TRY(linear_rows<T>(m, m.qkv, m.nrm, L.qkv, rows, "linear_qkv"));
         }
         {
             AttnParams p{};
             p.out = m.attn; p.q = m.q; p.k = L.k_cache; p.v = L.v_cache; p.scale = softmax_scale;
+            p.k_scale = L.k_scale; p.v_scale = L.v_scale;
             p.is_causal = S > 1; p.B = B; p.Sq = S; p.Hq = Hq; p.Hkv = Hkv; p.cache_len = c.max_seq;
             p.d_active = m.d_active; p.nsplit = m.nsplit; p.slice = m.slice; p.heads_per_wg = m.heads_per_wg;
             attn_token_major_layout(p, D);
@@ -206,15 +226,19 @@ static int enqueue_step(Model &m) {
                 note(m, "attention_rope_append", (double)(QD + 2 * KD) * eb + 2.0 * KD * eb + QD * eb);
                 TRY(attention_decode_launch(p, D, c.dtype, 0, m.attn_scratch, m.attn_counters, s));
             } else {
-                note(m, "rope_kv_append", (double)rows * (QD + 2 * KD) * 2 * eb);
-                TRY(rope_kv_append<T>(m.q, L.k_cache, L.v_cache, m.qkv, m.cos_t, m.sin_t, m.d_pos, m.d_past, 0, B, S,
-                                      Hq, Hkv, D, c.max_seq, s));
+                note(m, kv8 ? "rope_quant_kv_append" : "rope_kv_append", (double)rows * (QD + 2 * KD) * 2 * eb);
+                if (kv8)
+                    TRY(rope_quant_kv_append<T>(m.q, (int8_t *)L.k_cache, (int8_t *)L.v_cache, L.k_scale, L.v_scale, m.qkv,
+                                                m.cos_t, m.sin_t, m.d_pos, m.d_past, B, S, Hq, Hkv, D, c.max_seq, s));
+                else
+                    TRY(rope_kv_append<T>(m.q, L.k_cache, L.v_cache, m.qkv, m.cos_t, m.sin_t, m.d_pos, m.d_past, 0, B, S,
+                                          Hq, Hkv, D, c.max_seq, s));
                 // bytes: q in, out; the K/V rows read depend on the context, which the host does not
                 // know under replay -- callers add 2*KD*eb per cached row when they report
                 // flops: the causal half of QK^T and PV over the new rows alone (exact when past_len is 0)
                 note(m, "attention", (double)rows * 2.0 * QD * eb, S > 1 ? 2.0 * B * Hq * D * (double)S * (S + 1) : 0.0);
-                if (S > 1 && attention_prefill_supported(p, D, c.dtype, 0)) TRY(attention_prefill_launch(p, D, c.dtype, s));
-                else TRY(attention_decode_launch(p, D, c.dtype, 0, m.attn_scratch, m.attn_counters, s));
+                if (S > 1 && attention_prefill_supported(p, D, c.dtype, kv8)) TRY(attention_prefill_launch(p, D, c.dtype, s));
+                else TRY(attention_decode_launch(p, D, c.dtype, kv8, m.attn_scratch, m.attn_counters, s));
             }
         }
         if (fused) {
@@ -224,6 +248,19 @@ static int enqueue_step(Model &m) {
             TRY(gemv_norm_swiglu<T>(m.hmid, m.x2, L.norm2, c.eps, (const int8_t *)L.gu.w, L.gu.scale, L.gu.N, H, s));
             note(m, "gemv_down_residual", (double)H * F + H * eb + F * eb + 2 * H * eb);
             TRY(gemv_residual<T>(m.x, m.hmid, (const int8_t *)L.down.w, L.down.scale, m.x2, H, F, s));
+        } else if (w8a8) {
+            TRY(linear_w8a8(m, m.proj, m.attn, L.o, rows, true, "qlinear_o"));
+            note(m, "add", 3.0 * rows * H * eb);
+            TRY(mynn_add(m.x2, m.x, m.proj, (size_t)rows * H, c.dtype, s));
+            note(m, "rms_norm", 2.0 * rows * H * eb + H * eb);
+            TRY(mynn_rms_norm(m.nrm, m.x2, L.norm2, rows, H, c.eps, c.dtype, s));
+            TRY(linear_w8a8(m, m.g, m.nrm, L.gate, rows, true, "qlinear_gate"));
+            TRY(linear_w8a8(m, m.u, m.nrm, L.up, rows, false, "qlinear_up"));
+            note(m, "swiglu", 3.0 * rows * F * eb);
+            TRY(mynn_swiglu(m.hmid, m.g, m.u, (size_t)rows * F, c.dtype, s));
+            TRY(linear_w8a8(m, m.proj, m.hmid, L.down, rows, true, "qlinear_down"));
+            note(m, "add", 3.0 * rows * H * eb);
+            TRY(mynn_add(m.x, m.x2, m.proj, (size_t)rows * H, c.dtype, s));
         } else if (m.resident16) {
             // residual adds and SwiGLU ride on the GEMM stores
             TRY(gemm_rows(m, m.x2, m.attn, L.wt_o, m.x, rows, H, QD, GEMM_RESIDUAL, "linear_o_residual"));
@@ -252,7 +289,8 @@ static int enqueue_step(Model &m) {
     } else {
         note(m, "rms_norm", 2.0 * rows * H * eb + H * eb);
         TRY(mynn_rms_norm(m.nrm, m.x, m.final_norm, rows, H, c.eps, c.dtype, s));
-        if (m.resident16) TRY(gemm_rows(m, m.logits, m.nrm, m.wt_lm_head, nullptr, rows, V, H, GEMM_PLAIN, "linear_lm_head"));
+        if (w8a8) TRY(linear_w8a8(m, m.logits, m.nrm, m.lm_head, rows, true, "qlinear_lm_head"));
+        else if (m.resident16) TRY(gemm_rows(m, m.logits, m.nrm, m.wt_lm_head, nullptr, rows, V, H, GEMM_PLAIN, "linear_lm_head"));
         else TRY(linear_rows<T>(m, m.logits, m.nrm, m.lm_head, rows, "linear_lm_head"));
     }
     // greedy token of the last row of each sequence; for a batch-1 decode step the same launch
@@ -335,9 +373,15 @@ static int build(Model &m, void **init, void **state) {
             TRY(interleave_rows(&L.own_gu_s, L.gate.scale, L.up.scale, F, eb));
             L.gu.w = L.own_gu_w; L.gu.scale = L.own_gu_s; L.gu.N = 2 * F; L.gu.K = H;
         }
-        L.k_cache = state[2 * li];
-        L.v_cache = state[2 * li + 1];
+        const int per_layer = c.quant_kv_cache ? 4 : 2;
+        L.k_cache = state[per_layer * li];
+        L.v_cache = state[per_layer * li + 1];
         MYNN_REQUIRE(L.k_cache && L.v_cache, MYNN_ERR_INVALID, "model_init: null KV buffer in layer %d", li);
+        if (c.quant_kv_cache) {
+            L.k_scale = state[per_layer * li + 2];
+            L.v_scale = state[per_layer * li + 3];
+            MYNN_REQUIRE(L.k_scale && L.v_scale, MYNN_ERR_INVALID, "model_init: null KV scale buffer in layer %d", li);
+        }
     }
     m.final_norm = init[i++];
     lin(m.lm_head, V, H);
@@ -349,7 +393,7 @@ static int build(Model &m, void **init, void **state) {
     // ---- prefill executors keep every linear weight dequantised to the 16-bit type (2 bytes per weight
     // on top of the int8 originals): the matrix-core GEMM reads them directly, and the values are
     // those of the per-call dequantisation, T(wq * scale)
-    if (m.quant && c.batch * c.seq_q >= 16 && H % 8 == 0 && QD % 8 == 0 && F % 32 == 0) {
+    if (m.quant && !c.quantize_activations && c.batch * c.seq_q >= 16 && H % 8 == 0 && QD % 8 == 0 && F % 32 == 0) {
         auto resident = [&](void **dst, const Lin &l) {
             MYNN_HIP(hipMalloc(dst, gemm_weight_bytes(l.N, l.K)));
             return dequant_weight_rows(*dst, (const int8_t *)l.w, l.scale, l.N, l.K, c.dtype, 0, 0, m.stream);
@@ -369,7 +413,7 @@ static int build(Model &m, void **init, void **state) {
 
     // ---- arena: every activation of one step, the device scalars, attention split scratch
     const int rows = c.batch * c.seq_q;
-    attn_plan(c.batch, c.seq_q, c.n_heads, c.n_kv_heads, c.head_dim, c.dtype, 0, c.max_seq, &m.slice, &m.nsplit, &m.heads_per_wg);
+    attn_plan(c.batch, c.seq_q, c.n_heads, c.n_kv_heads, c.head_dim, c.dtype, c.quant_kv_cache, c.max_seq, &m.slice, &m.nsplit, &m.heads_per_wg);
     m.token_cap = c.max_seq + 8;
     ArenaPlan plan;
     size_t o_x = plan.take((size_t)rows * H * eb), o_x2 = plan.take((size_t)rows * H * eb);
@@ -378,6 +422,8 @@ static int build(Model &m, void **init, void **state) {
     size_t o_g = plan.take((size_t)rows * F * eb), o_u = plan.take((size_t)rows * F * eb);
     size_t o_h = plan.take((size_t)rows * F * eb), o_p = plan.take((size_t)rows * H * eb);
     size_t o_l = plan.take((size_t)rows * V * eb);
+    const size_t kmax = (size_t)(F > H ? (F > QD ? F : QD) : (H > QD ? H : QD));
+    size_t o_a8 = plan.take(c.quantize_activations ? (size_t)rows * kmax : 0), o_a8s = plan.take((size_t)rows * eb);
     size_t o_ids = plan.take((size_t)rows * 8), o_pos = plan.take((size_t)c.seq_q * 8);
     size_t o_sc = plan.take(256), o_tok = plan.take((size_t)m.token_cap * 4);
     size_t o_as = plan.take(attn_scratch_bytes(c.batch, c.n_heads, c.seq_q, c.head_dim, m.nsplit));
@@ -388,6 +434,7 @@ static int build(Model &m, void **init, void **state) {
     m.x = m.arena + o_x; m.x2 = m.arena + o_x2; m.nrm = m.arena + o_n; m.qkv = m.arena + o_qkv; m.q = m.arena + o_q;
     m.attn = m.arena + o_attn; m.g = m.arena + o_g; m.u = m.arena + o_u; m.hmid = m.arena + o_h; m.proj = m.arena + o_p;
     m.logits = m.arena + o_l;
+    m.a8 = (int8_t *)(m.arena + o_a8); m.a8_scale = m.arena + o_a8s;
     m.d_ids = (int64_t *)(m.arena + o_ids); m.d_pos = (int64_t *)(m.arena + o_pos);
     m.d_past = (int32_t *)(m.arena + o_sc); m.d_active = m.d_past + 1; m.d_step = m.d_past + 2;
     m.d_next = m.d_past + 8;  // up to 56 sequences' tokens after the scalars
@@ -499,6 +546,10 @@ extern "C" int mynn_model_configure(const mynn_model_config *cfg) {
     MYNN_REQUIRE(cfg->n_heads % cfg->n_kv_heads == 0, MYNN_ERR_INVALID, "model_configure: heads not a multiple of kv heads");
     MYNN_REQUIRE(cfg->dtype == MYNN_F16 || cfg->dtype == MYNN_BF16, MYNN_ERR_UNSUPPORTED,
                  "model_configure: dtype %d (fp16 or bf16 only)", cfg->dtype);
+    MYNN_REQUIRE(!cfg->quantize_activations || (cfg->weights_int8 && cfg->hidden % 32 == 0 && cfg->ffn % 32 == 0),
+                 MYNN_ERR_UNSUPPORTED, "model_configure: quantize_activations needs int8 weights and K %% 32 == 0");
+    MYNN_REQUIRE(!cfg->quant_kv_cache || (cfg->head_dim % 2 == 0 && cfg->head_dim <= 128), MYNN_ERR_UNSUPPORTED,
+                 "model_configure: quant_kv_cache needs an even head_dim <= 128 (got %d)", cfg->head_dim);
     MYNN_REQUIRE(cfg->seq_q <= cfg->max_seq, MYNN_ERR_INVALID, "model_configure: prefill_len %d > max_seq %d", cfg->seq_q,
                  cfg->max_seq);
     std::lock_guard<std::mutex> lk(g_mu);

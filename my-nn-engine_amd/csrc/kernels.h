@@ -58,5 +58,11 @@ template <typename T>
 int rope_kv_append(void *q_out, void *k_cache, void *v_cache, const void *qkv, const void *cos_t, const void *sin_t,
                    const int64_t *position, const int32_t *d_past, int past_host, int B, int S, int Hq, int Hkv, int D,
                    int max_seq, hipStream_t s);
+// the same for an int8 KV cache: k (after RoPE, rounded to T) and v are quantised per token row into
+// the caches and their scale rows [B,Hkv,max_seq] (QuantizingKVCacheUpdate, CPU backend rounding)
+template <typename T>
+int rope_quant_kv_append(void *q_out, int8_t *k_cache, int8_t *v_cache, void *k_scale, void *v_scale, const void *qkv,
+                         const void *cos_t, const void *sin_t, const int64_t *position, const int32_t *d_past, int B,
+                         int S, int Hq, int Hkv, int D, int max_seq, hipStream_t s);
 
 }  // namespace mynn

@@ -81,6 +81,77 @@ __global__ __launch_bounds__(256) void rope_kv_append_vec_kernel(T *q_out, T *k_
     }
 }
 
+// int8 KV cache (BuildOptions::quant_kv_cache): RoPE(q) -> q_out; RoPE(k) rounded to T and v are quantised
+// per token row with the rule of quantizing_kvcache_update (CPU backend rounding: s = amax/127,
+// q = trunc(x * 127/amax +- 0.5) clamped to [-128,127]) into the int8 caches and their scale rows
+// [B,Hkv,max_seq].  One wave per (token, head); needs D <= 128.
+template <typename T>
+__global__ __launch_bounds__(64) void rope_quant_kv_append_kernel(T *q_out, int8_t *k_cache, int8_t *v_cache, T *k_scale,
+                                                                 T *v_scale, const T *qkv, const T *cos_t, const T *sin_t,
+                                                                 const int64_t *position, const int32_t *d_past, int S,
+                                                                 int Hq, int Hkv, int D, int max_seq) {
+    const int s = blockIdx.x, head = blockIdx.y, b = blockIdx.z, lane = threadIdx.x;
+    const int half = D / 2;
+    const int past = *d_past;
+    const size_t row = (size_t)b * S + s;
+    const T *src = qkv + row * (size_t)(Hq + 2 * Hkv) * D + (size_t)head * D;
+    // lane j < D/2 owns elements j and j + D/2
+    float lo = 0.f, hi = 0.f;
+    const bool on = lane < half;
+    if (on) {
+        lo = Elem<T>::ld(src, lane);
+        hi = Elem<T>::ld(src, lane + half);
+        if (head < Hq + Hkv) {
+            const size_t tab = (size_t)position[s] * D;
+            const float cl = Elem<T>::ld(cos_t, tab + lane), ch = Elem<T>::ld(cos_t, tab + lane + half);
+            const float sl = Elem<T>::ld(sin_t, tab + lane), sh = Elem<T>::ld(sin_t, tab + lane + half);
+            const float rl = Elem<T>::rnd(lo * cl - hi * sl), rh = Elem<T>::rnd(hi * ch + lo * sh);
+            lo = rl;
+            hi = rh;
+        }
+    }
+    if (head < Hq) {
+        if (on) {
+            T *dst = q_out + row * (size_t)Hq * D + (size_t)head * D;
+            Elem<T>::st(dst, lane, lo);
+            Elem<T>::st(dst, lane + half, hi);
+        }
+        return;
+    }
+    const bool is_k = head < Hq + Hkv;
+    const int hk = is_k ? head - Hq : head - Hq - Hkv;
+    const size_t tok = ((size_t)b * Hkv + hk) * max_seq + past + s;
+    const float amax = wave_max(fmaxf(fabsf(lo), fabsf(hi)));
+    const float inv = amax == 0.f ? 0.f : 127.0f / amax;
+    if (lane == 0) Elem<T>::st(is_k ? k_scale : v_scale, tok, amax * (1.0f / 127.0f));
+    if (on) {
+        int8_t *dst = (is_k ? k_cache : v_cache) + tok * D;
+        const float a = lo * inv, c = hi * inv;
+        int qa = (int)(a + (a >= 0.f ? 0.5f : -0.5f)), qc = (int)(c + (c >= 0.f ? 0.5f : -0.5f));
+        qa = qa < -128 ? -128 : (qa > 127 ? 127 : qa);
+        qc = qc < -128 ? -128 : (qc > 127 ? 127 : qc);
+        dst[lane] = (int8_t)qa;
+        dst[lane + half] = (int8_t)qc;
+    }
+}
+
+template <typename T>
+int rope_quant_kv_append(void *q_out, int8_t *k_cache, int8_t *v_cache, void *k_scale, void *v_scale, const void *qkv,
+                         const void *cos_t, const void *sin_t, const int64_t *position, const int32_t *d_past, int B,
+                         int S, int Hq, int Hkv, int D, int max_seq, hipStream_t s) {
+    MYNN_REQUIRE(D % 2 == 0 && D <= 128, MYNN_ERR_UNSUPPORTED, "int8 KV append: head_dim %d", D);
+    MYNN_REQUIRE(S <= 65535 * 32 && Hq + 2 * Hkv <= 65535 && B <= 65535, MYNN_ERR_UNSUPPORTED, "int8 KV append: grid");
+    MYNN_REQUIRE(d_past, MYNN_ERR_INVALID, "int8 KV append: null past_len");
+    MYNN_LAUNCH(rope_quant_kv_append_kernel<T>, dim3(S, Hq + 2 * Hkv, B), dim3(64), 0, s, (T *)q_out, k_cache, v_cache,
+                (T *)k_scale, (T *)v_scale, (const T *)qkv, (const T *)cos_t, (const T *)sin_t, position, d_past, S, Hq,
+                Hkv, D, max_seq);
+    return launch_status("rope_quant_kv_append_kernel");
+}
+template int rope_quant_kv_append<bf16_t>(void *, int8_t *, int8_t *, void *, void *, const void *, const void *, const void *,
+                                          const int64_t *, const int32_t *, int, int, int, int, int, int, hipStream_t);
+template int rope_quant_kv_append<f16_t>(void *, int8_t *, int8_t *, void *, void *, const void *, const void *, const void *,
+                                         const int64_t *, const int32_t *, int, int, int, int, int, int, hipStream_t);
+
 template <typename T>
 int rope_kv_append(void *q_out, void *k_cache, void *v_cache, const void *qkv, const void *cos_t, const void *sin_t,
                    const int64_t *position, const int32_t *d_past, int past_host, int B, int S, int Hq, int Hkv, int D,

@@ -93,6 +93,9 @@ _sig("orc_model_set_linear", None, _vp, _i, _i, Linear)
 _sig("orc_model_set_norm", None, _vp, _i, _i, _vp)
 _sig("orc_model_reset", None, _vp)
 _sig("orc_model_set_gemm_mode", None, _vp, _i)
+_sig("orc_model_set_options", None, _vp, _i, _i)
+_sig("orc_model_k_scale", _vp, _vp, _i)
+_sig("orc_model_v_scale", _vp, _vp, _i)
 _sig("orc_model_past_len", _ll, _vp)
 _sig("orc_model_set_past_len", None, _vp, _ll)
 _sig("orc_model_forward", None, _vp, _vp, _vp, _sz, _ll, _ll, _i, _vp)
@@ -387,6 +390,11 @@ class Model:
         """-1: CPU backend's kernel choice (default); 2: CUDA backend's."""
         _lib.orc_model_set_gemm_mode(self._h, int(mode))
 
+    def set_options(self, quant_kv_cache=False, quantize_activations=False):
+        """BuildOptions::quant_kv_cache / Options::quantize_activations; before the first forward."""
+        self.quant_kv_cache = bool(quant_kv_cache)
+        _lib.orc_model_set_options(self._h, int(quant_kv_cache), int(quantize_activations))
+
     @property
     def past_len(self):
         return _lib.orc_model_past_len(self._h)
@@ -424,7 +432,16 @@ class Model:
         shape = (self.cfg.n_kv_heads, self.cfg.max_seq, self.cfg.head_dim)
         kp = _lib.orc_model_k_cache(self._h, layer)
         vp = _lib.orc_model_v_cache(self._h, layer)
-        typ = C.c_float if self.dt == F32 else C.c_uint16
+        typ = C.c_int8 if getattr(self, "quant_kv_cache", False) else (C.c_float if self.dt == F32 else C.c_uint16)
         k = np.ctypeslib.as_array(C.cast(kp, C.POINTER(typ)), (n,)).reshape(shape).copy()
         v = np.ctypeslib.as_array(C.cast(vp, C.POINTER(typ)), (n,)).reshape(shape).copy()
         return k, v
+
+    def kv_scales(self, layer):
+        """quant_kv_cache: the per-token scales [Hkv, max_seq] of layer's k and v caches."""
+        n = self.cfg.n_kv_heads * self.cfg.max_seq
+        typ = C.c_float if self.dt == F32 else C.c_uint16
+        ks = np.ctypeslib.as_array(C.cast(_lib.orc_model_k_scale(self._h, layer), C.POINTER(typ)), (n,))
+        vs = np.ctypeslib.as_array(C.cast(_lib.orc_model_v_scale(self._h, layer), C.POINTER(typ)), (n,))
+        shape = (self.cfg.n_kv_heads, self.cfg.max_seq)
+        return ks.reshape(shape).copy(), vs.reshape(shape).copy()

@@ -534,7 +534,8 @@ void orc_streaming_kv_position(int64_t *out, size_t sink, size_t window, size_t 
 struct orc_layer {
     orc_linear lin[7];
     const void *norm[2];
-    void *k_cache, *v_cache; /* [Hkv, max_seq, D] dtype */
+    void *k_cache, *v_cache; /* [Hkv, max_seq, D] dtype, or int8 with quant_kv_cache */
+    void *k_scale, *v_scale; /* quant_kv_cache: [Hkv, max_seq] dtype */
 };
 struct orc_model {
     orc_model_cfg cfg;
@@ -544,6 +545,8 @@ struct orc_model {
     void *cos_t, *sin_t;
     long long past_len;
     int gemm_mode; /* -1: CPU backend's dispatch; 2: CUDA backend's (M >= 16 -> W rounded first) */
+    int quant_kv_cache;       /* BuildOptions::quant_kv_cache (decoder.rs:672, 405-470) */
+    int quantize_activations; /* Options::quantize_activations (transform/optimize/quantize_activations.rs) */
     void *last_hidden;
     size_t last_S;
 };
@@ -568,7 +571,10 @@ orc_model *orc_model_create(const orc_model_cfg *cfg) {
 }
 void orc_model_destroy(orc_model *m) {
     if (!m) return;
-    for (int l = 0; l < m->cfg.n_layers; l++) { free(m->layers[l].k_cache); free(m->layers[l].v_cache); }
+    for (int l = 0; l < m->cfg.n_layers; l++) {
+        free(m->layers[l].k_cache); free(m->layers[l].v_cache);
+        free(m->layers[l].k_scale); free(m->layers[l].v_scale);
+    }
     free(m->layers); free(m->cos_t); free(m->sin_t); free(m->last_hidden); free(m);
 }
 void orc_model_set_embed(orc_model *m, orc_linear w) { m->embed = w; }
@@ -578,6 +584,22 @@ void orc_model_set_linear(orc_model *m, int layer, int which, orc_linear w) { m-
 void orc_model_set_norm(orc_model *m, int layer, int which, const void *w) { m->layers[layer].norm[which] = w; }
 void orc_model_reset(orc_model *m) { m->past_len = 0; }
 void orc_model_set_gemm_mode(orc_model *m, int mode) { m->gemm_mode = mode; }
+/* must be called before the first forward: the caches change element type */
+void orc_model_set_options(orc_model *m, int quant_kv_cache, int quantize_activations) {
+    m->quant_kv_cache = quant_kv_cache;
+    m->quantize_activations = quantize_activations;
+    size_t rows = (size_t)m->cfg.n_kv_heads * (size_t)m->cfg.max_seq;
+    for (int l = 0; l < m->cfg.n_layers && quant_kv_cache; l++) {
+        struct orc_layer *L = &m->layers[l];
+        free(L->k_cache); free(L->v_cache); free(L->k_scale); free(L->v_scale);
+        L->k_cache = calloc(rows * (size_t)m->cfg.head_dim, 1);
+        L->v_cache = calloc(rows * (size_t)m->cfg.head_dim, 1);
+        L->k_scale = calloc(rows, esize(m->cfg.dtype));
+        L->v_scale = calloc(rows, esize(m->cfg.dtype));
+    }
+}
+const void *orc_model_k_scale(const orc_model *m, int layer) { return m->layers[layer].k_scale; }
+const void *orc_model_v_scale(const orc_model *m, int layer) { return m->layers[layer].v_scale; }
 long long orc_model_past_len(const orc_model *m) { return m->past_len; }
 void orc_model_set_past_len(orc_model *m, long long p) { m->past_len = p; }
 const void *orc_model_k_cache(const orc_model *m, int layer) { return m->layers[layer].k_cache; }
@@ -589,6 +611,17 @@ const void *orc_model_last_hidden(const orc_model *m) { return m->last_hidden; }
 static void linear(const orc_model *m, void *out, const void *x, const orc_linear *w, size_t S,
                    size_t N, size_t K) {
     int dt = m->cfg.dtype;
+    if (w->q && m->quantize_activations && K % 32 == 0) {
+        /* DequantMatMul -> DynamicQuantizeLinear(axis 0, symmetric) + QuantizedMatMul
+         * (quantize_activations.rs:63-84, 121-183); re-quantising a shared activation per
+         * consumer gives the same int8 rows as the pass's cached value */
+        int8_t *a8 = (int8_t *)malloc(S * K);
+        void *as = malloc(S * esize(dt));
+        orc_dynquant_i8(a8, as, x, S, K, dt);
+        orc_quantized_matmul(out, NULL, a8, as, w->q, w->scale, S, N, K, dt);
+        free(a8); free(as);
+        return;
+    }
     if (w->q) {
         /* kernel choice per backend: CPU (translator.rs:3002-3115) M==1 fused decode else
          * dequantise+sgemm; CUDA (cuda.rs:1518-1652) M>=16 && K%8==0 tensor cores else
@@ -660,10 +693,17 @@ void orc_model_forward(orc_model *m, const int64_t *ids, const int64_t *position
         to_heads(vh, vb, S, Hkv, D, eb);
         orc_rope(qr, qh, m->cos_t, m->sin_t, positions, Hq, S, D, dt);
         orc_rope(kr, kh, m->cos_t, m->sin_t, positions, Hkv, S, D, dt);
-        orc_kv_cache_update(L->k_cache, kr, past_len, Hkv, S, (size_t)c->max_seq, D, eb);
-        orc_kv_cache_update(L->v_cache, vh, past_len, Hkv, S, (size_t)c->max_seq, D, eb);
-        orc_attention(ao, qr, L->k_cache, L->v_cache, NULL, NULL, active, 1, Hq, Hkv, S,
-                      (size_t)c->max_seq, D, is_causal, scale, dt, 0);
+        if (m->quant_kv_cache) {
+            orc_quantizing_kv_cache_update((int8_t *)L->k_cache, L->k_scale, kr, past_len, Hkv, S, (size_t)c->max_seq, D, dt);
+            orc_quantizing_kv_cache_update((int8_t *)L->v_cache, L->v_scale, vh, past_len, Hkv, S, (size_t)c->max_seq, D, dt);
+            orc_attention(ao, qr, L->k_cache, L->v_cache, L->k_scale, L->v_scale, active, 1, Hq, Hkv, S,
+                          (size_t)c->max_seq, D, is_causal, scale, dt, 1);
+        } else {
+            orc_kv_cache_update(L->k_cache, kr, past_len, Hkv, S, (size_t)c->max_seq, D, eb);
+            orc_kv_cache_update(L->v_cache, vh, past_len, Hkv, S, (size_t)c->max_seq, D, eb);
+            orc_attention(ao, qr, L->k_cache, L->v_cache, NULL, NULL, active, 1, Hq, Hkv, S,
+                          (size_t)c->max_seq, D, is_causal, scale, dt, 0);
+        }
         from_heads(ab, ao, S, Hq, D, eb);
         linear(m, ob, ab, &L->lin[3], S, H, QD);
         orc_add(x2, x, ob, S * H, dt);                 /* attn residual */

@@ -182,6 +182,13 @@ void orc_model_reset(orc_model *m);                 /* past_len = 0 (session.rs:
 /* which backend's DequantMatMul kernel choice the linears follow: -1 the CPU backend's (default),
  * 2 the CUDA backend's (rows >= 16: weight rounded to the 16-bit type before the product) */
 void orc_model_set_gemm_mode(orc_model *m, int mode);
+/* BuildOptions::quant_kv_cache (crates/llm/src/decoder.rs:672, 405-470: int8 caches + per-token scales,
+ * QuantizingKVCacheUpdate, attention scale slots) and Options::quantize_activations
+ * (src/transform/optimize/quantize_activations.rs: DynamicQuantizeLinear + QuantizedMatMul for every
+ * int8 linear with K % 32 == 0).  Call before the first forward. */
+void orc_model_set_options(orc_model *m, int quant_kv_cache, int quantize_activations);
+const void *orc_model_k_scale(const orc_model *m, int layer);
+const void *orc_model_v_scale(const orc_model *m, int layer);
 long long orc_model_past_len(const orc_model *m);
 void orc_model_set_past_len(orc_model *m, long long p);
 /* One graph run with S tokens: positions[s], writes KV rows past_len..past_len+S-1, attends

@@ -184,3 +184,47 @@ def test_prefill_then_decode_shares_kv_and_matches_decode_only(g, dt):
         c = g.mynn.LlmSession(dec2, prefill=pre)
         c.generate_ids(list(range(100)), 1)
     b.close(), dec.close(), pre.close(), dec2.close()
+
+
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+@pytest.mark.parametrize("kv8,w8a8", [(True, False), (False, True), (True, True)])
+def test_int8_kv_cache_and_w8a8_executor_vs_oracle(g, dt, kv8, w8a8):
+    """BuildOptions::quant_kv_cache (int8 caches + per-token scales, QuantizingKVCacheUpdate, attention
+    scale slots; crates/llm/src/decoder.rs:405-470) and Options::quantize_activations
+    (DynamicQuantizeLinear + QuantizedMatMul for every int8 linear; quantize_activations.rs) in the
+    executor: a 16-token prefill chunk, then decode steps over the same caches, against the oracle
+    with the same options."""
+    cfg, w = llm_weights.synthetic_int8(SMALL, dt, seed=41)
+    ref = orc.Model(cfg, w)
+    ref.set_options(quant_kv_cache=kv8, quantize_activations=w8a8)
+    ref.set_gemm_mode(2)
+    dw = dev_weights(g, w, dt)
+    dec = g.mynn.Decoder(cfg, dw, quant_kv_cache=kv8, quantize_activations=w8a8)
+    pre = g.mynn.Decoder(cfg, dw, seq_q=16, kv=dec.kv, quant_kv_cache=kv8, quantize_activations=w8a8)
+    rng = np.random.default_rng(3)
+    ids = rng.integers(0, cfg["vocab"], 16)
+    want = ref.forward(ids, np.arange(16), 0, 16, True)
+    _, got = pre.step(ids, np.arange(16), 0, 16, want_logits=True)
+    assert max_err_rel_to_max(g.f32(got, dt), g.f32(want, dt)) <= 2e-2
+    past = 16
+    for t in [7, 500, 31, 999, 2, 640]:
+        want = ref.forward([t], [past], past, past + 1, False)
+        nxt, got = dec.step([t], [past], past, past + 1, want_logits=True)
+        assert max_err_rel_to_max(g.f32(got, dt), g.f32(want, dt)) <= 2e-2, past
+        assert nxt[0] == orc.argmax_last(got[0], dt)
+        past += 1
+    if kv8:
+        for l in range(cfg["n_layers"]):
+            k_ref, v_ref = ref.kv_cache(l)
+            ks_ref, vs_ref = ref.kv_scales(l)
+            k_gpu, v_gpu, ks_gpu, vs_gpu = [g.to_host(t)[0] for t in dec.kv[l]]
+            assert k_gpu.dtype == np.int8 and not k_gpu[:, past:].any() and not v_gpu[:, past:].any()
+            # the projections differ in summation order by a spacing of T here and there; when that hits
+            # the row's amax every code of the row moves by up to 127 * 2^-8 (bf16), plus its own rounding
+            assert np.abs(k_gpu[:, :past].astype(int) - k_ref[:, :past].astype(int)).max() <= 2
+            assert np.abs(v_gpu[:, :past].astype(int) - v_ref[:, :past].astype(int)).max() <= 2
+            assert np.mean(k_gpu[:, :past] == k_ref[:, :past]) > 0.85
+            # a scale is amax/127 rounded to T: amax one spacing of T apart, then one more rounding
+            assert max_abs_rel(g.f32(ks_gpu[:, :past], dt), g.f32(ks_ref[:, :past], dt)) <= 2e-2
+            assert max_abs_rel(g.f32(vs_gpu[:, :past], dt), g.f32(vs_ref[:, :past], dt)) <= 2e-2
+    pre.close(), dec.close()

@@ -74,3 +74,37 @@ def test_forward_rows_are_causal():
     ids2[3:] = [31999, 4]
     b = m.forward(ids2, pos, 0, 5, True)
     assert np.array_equal(a[:3], b[:3]) and not np.array_equal(a[3], b[3])
+
+
+@pytest.mark.parametrize("dt", [orc.F32, orc.BF16])
+def test_quant_kv_cache_and_quantize_activations_options_stay_close_to_the_plain_model(dt):
+    """The two int8 options change storage/arithmetic precision, not the function: an int8 KV cache
+    (127 levels per token row) and W8A8 linears (127 levels per activation row) must leave the logits
+    within a few percent of the plain model's, the caches must dequantise to the plain caches within
+    half a quantisation step, and the options must actually change the arithmetic."""
+    cfg = dict(n_layers=2, hidden=64, n_heads=4, n_kv_heads=2, head_dim=16, ffn=96, vocab=200, max_seq=24,
+               eps=1e-5, rope_theta=10000.0)
+    cfg, w = llm_weights.synthetic_int8(cfg, dt, seed=2)
+    ids = np.random.default_rng(0).integers(0, cfg["vocab"], 10)
+    pos = np.arange(10)
+    plain = orc.Model(cfg, w)
+    base = orc.to_f32(plain.forward(ids, pos, 0, 10, True), dt)
+    for kv8, w8a8 in [(True, False), (False, True), (True, True)]:
+        m = orc.Model(cfg, w)
+        m.set_options(quant_kv_cache=kv8, quantize_activations=w8a8)
+        got = orc.to_f32(m.forward(ids, pos, 0, 10, True), dt)
+        err = np.abs(got - base).max() / np.abs(base).max()
+        assert 0 < err < 0.08, (kv8, w8a8, err)
+        if kv8 and not w8a8:
+            for l in range(cfg["n_layers"]):
+                kq, vq = m.kv_cache(l)
+                ks, vs = m.kv_scales(l)
+                kp, vp = plain.kv_cache(l)
+                assert kq.dtype == np.int8
+                kd = kq[:, :10].astype(np.float32) * orc.to_f32(ks, dt)[:, :10, None]
+                if l == 0:  # layer 0 sees identical inputs in both models
+                    step = orc.to_f32(ks, dt)[:, :10, None]
+                    # half a step from the rounding, plus 127 codes times the rounding of the stored scale
+                    slack = 0.5 * 1.02 + (127 * 2.0 ** -8 if dt == orc.BF16 else 0.0)
+                    assert np.all(np.abs(kd - orc.to_f32(kp, dt)[:, :10]) <= slack * step + 1e-6)
+                assert np.abs(kq[:, :10]).max() == 127 and not kq[:, 10:].any()
