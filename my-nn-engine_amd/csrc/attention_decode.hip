@@ -8,8 +8,8 @@
 //      heads and reduces inside the group; scores go to LDS,
 //   3. V is parked in LDS; one wave per query head does max / exp / sum over the slice,
 //   4. thread (head, d) accumulates sum_k p[head,k] * V[k,d] from LDS -- no cross-lane merging.
-// Longer caches are cut into slices over gridDim.y; the last workgroup of a (batch, kv head, row)
-// to finish merges the slices (a counter in device memory; nobody spins).
+// Longer caches are cut into slices over gridDim.y; a small second launch (attn_merge_kernel) merges
+// the slices' partial results.
 //
 // FUSE form (decoder executor, one new token): the kernel also applies RoPE to q and to the new
 // k row, appends k/v to the cache and attends to the new row from registers -- the reference's
@@ -49,7 +49,6 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
     __shared__ float q_s[G][D];
     __shared__ float new_s[2][D];  // FUSE: rotated k row and v row of the new token (values rounded to T)
     __shared__ float ml_s[G][2];
-    __shared__ int sm_last;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int grp = tid / LPK, dc = tid % LPK;
@@ -268,36 +267,6 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
             }
         }
     }
-    if (p.nsplit == 1) return;
-
-    // ---- 5. last workgroup of this (batch, kv head, row) merges the slices
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) {
-        unsigned prev = atomicAdd(&p.counters[(size_t)blockIdx.x * Sq + sq], 1u);
-        sm_last = (prev == (unsigned)p.nsplit - 1);
-    }
-    __syncthreads();
-    if (!sm_last) return;
-    __threadfence();
-    for (int idx = tid; idx < G * D; idx += kAttnThreads) {
-        const int g = idx / D, d = idx % D;
-        const size_t row = row_base + (size_t)g * Sq;
-        const float *ml = p.part_ml + row * p.nsplit * 2;
-        const float *po = p.part_o + row * p.nsplit * D;
-        float mt = -INFINITY;
-        for (int s = 0; s < p.nsplit; s++) mt = fmaxf(mt, __builtin_nontemporal_load(&ml[2 * s]));
-        float lt = 0.f, ot = 0.f;
-        for (int s = 0; s < p.nsplit; s++) {
-            const float ms = __builtin_nontemporal_load(&ml[2 * s]);
-            const float c = (ms == -INFINITY) ? 0.f : fast_exp(ms - mt);
-            lt = fmaf(__builtin_nontemporal_load(&ml[2 * s + 1]), c, lt);
-            ot = fmaf(__builtin_nontemporal_load(&po[s * D + d]), c, ot);
-        }
-        const size_t oo = (size_t)b * p.o_bs + (size_t)(head0 + g) * p.o_hs + (size_t)sq * p.o_rs + d;
-        Elem<T>::st(out, oo, ot / lt);
-    }
-    if (tid == 0) p.counters[(size_t)blockIdx.x * Sq + sq] = 0;  // ready for the next launch
 }
 
 // LDS the kernel may use per workgroup for the V slice, the scores and the v scales
@@ -370,10 +339,15 @@ bool attention_fused_supported(int D, int G) {
 // Slice length, number of slices and query heads per workgroup for a launch.  kv_len = longest key
 // range any row can have.  All heads of a kv head share one workgroup (one K/V read) unless that
 // leaves fewer than ~64 workgroups; then the heads are divided, halving until there are enough.
-void attn_plan(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, int *slice, int *nsplit,
-               int *heads_per_wg) {
-    const size_t kv_elem = kv_int8 ? 1 : dtype_size(dtype);
+void attn_plan(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, bool fused, int *slice,
+               int *nsplit, int *heads_per_wg) {
     const int Gt = Hq / Hkv;
+    if (!fused && attn_stream_eligible(B, Sq, Hq, Hkv, D, dtype, kv_int8, kv_len)) {
+        attn_stream_plan(B, Hkv, kv_len, slice, nsplit);
+        *heads_per_wg = Gt;
+        return;
+    }
+    const size_t kv_elem = kv_int8 ? 1 : dtype_size(dtype);
     const int rows = slice_rows(D, Gt, kv_elem);
     int n = (kv_len + rows - 1) / rows;
     if (n < 1) n = 1;
@@ -393,8 +367,7 @@ size_t attn_counter_bytes(int B, int Hq, int Sq) {
     return ((size_t)B * Hq * Sq * sizeof(unsigned) + 255) / 256 * 256;
 }
 
-// scratch = [part_o | part_ml] (contents need not survive); counters = one unsigned per
-// (batch, kv head, row), zero on entry and zero again when the kernel has finished
+// scratch = [part_o | part_ml] (contents need not survive); `counters` is unused (kept for callers)
 int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *scratch, void *counters,
                             hipStream_t s) {
     if (p.nsplit > 1) {
@@ -404,7 +377,11 @@ int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *s
         p.counters = (unsigned *)counters;
     }
     const bool fuse = p.qkv != nullptr;
-    return dispatch_dtype(dtype, [&](auto *t) {
+    // the plan (attn_plan, with the same kv_len) was made for the streaming kernel when it is eligible
+    const int kv_len = p.d_active ? p.cache_len : (p.active < p.cache_len ? p.active : p.cache_len);
+    if (!fuse && attn_stream_eligible(p.B, p.Sq, p.Hq, p.Hkv, D, dtype, kv_int8, kv_len))
+        return attention_stream_launch(p, D, dtype, s);
+    int rc = dispatch_dtype(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
         if constexpr (sizeof(T) == 2) {
             if (fuse) {
@@ -416,6 +393,8 @@ int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *s
         }
         return kv_int8 ? launch_d<T, true, false>(p, D, s) : launch_d<T, false, false>(p, D, s);
     });
+    if (rc || p.nsplit == 1) return rc;
+    return attention_merge_launch(p, D, dtype, s);
 }
 
 // ---- library-owned scratch for the op-level entry point: grown on demand.  The counters live
@@ -465,7 +444,7 @@ extern "C" int mynn_attention(void *out, const void *Q, const void *K, const voi
     if (Sq > 1 && attention_prefill_supported(p, head_dim, dtype, kv_int8))
         return attention_prefill_launch(p, head_dim, dtype, st);
     int kv_len = d_active ? cache_seq_len : (active_seq_kv < cache_seq_len ? active_seq_kv : cache_seq_len);
-    attn_plan(B, Sq, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, kv_len, &p.slice, &p.nsplit, &p.heads_per_wg);
+    attn_plan(B, Sq, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, kv_len, false, &p.slice, &p.nsplit, &p.heads_per_wg);
     MYNN_REQUIRE(p.nsplit <= 65535, MYNN_ERR_UNSUPPORTED, "attention: cache of %d rows needs too many slices", kv_len);
     if (p.nsplit > 1) {
         int rc = ensure(g_scratch, attn_scratch_bytes(B, num_q_heads, Sq, head_dim, p.nsplit), false, st);

@@ -80,6 +80,36 @@ def test_decode_attention_head_shapes_and_active_length(g, dt, Hq, Hkv, D):
     assert np.array_equal(got3, got)
 
 
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+@pytest.mark.parametrize("B,Hq,Hkv,D,L,active", [(8, 32, 8, 128, 1100, 1037), (16, 32, 4, 64, 700, 613),
+                                                 (8, 8, 8, 64, 600, 600), (4, 16, 8, 64, 1200, 1111),
+                                                 (32, 32, 8, 128, 160, 129)])
+def test_streaming_decode_attention_vs_oracle(g, dt, B, Hq, Hkv, D, L, active):
+    """Batch x context products large enough for the streaming kernel (matrix-core scores, online
+    softmax, key ranges merged by the last workgroup): ragged active lengths, the length read on the
+    device, and rows beyond it poisoned."""
+    import torch
+
+    assert B * Hkv * min(active, L) >= 32768 or B * Hkv * L >= 32768
+    rng = np.random.default_rng(B * 31 + D + active)
+    q = orc.to_storage(rng.standard_normal((B, Hq, 1, D)), dt)
+    k = orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt)
+    v = orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt)
+    k[:, :, active:] = orc.to_storage(np.full((B, Hkv, L - active, D), np.nan), dt)
+    v[:, :, active:] = orc.to_storage(np.full((B, Hkv, L - active, D), np.nan), dt)
+    want = orc.attention(q, k, v, dt, D ** -0.5, False, active)
+    exact = orc.attention_f64(q, k, v, dt, D ** -0.5, False, active)
+    dq, dk, dv = g.to_dev(q, dt), g.to_dev(k, dt), g.to_dev(v, dt)
+    d_active = torch.tensor([active], dtype=torch.int32, device="cuda")
+    for rep in range(2):  # the second call finds the merge counters as the first left them
+        got = g.to_host(g.mynn.attention(dq, dk, dv, D ** -0.5, False, active=L, d_active=d_active))
+        assert max_abs_rel(g.f32(got, dt), g.f32(want, dt)) <= 1e-2, rep
+        assert max_abs_rel(g.f32(got, dt), exact) <= 1e-2, rep
+    if B * Hkv * active >= 32768:
+        got = g.to_host(g.mynn.attention(dq, dk, dv, D ** -0.5, False, active))
+        assert max_abs_rel(g.f32(got, dt), exact) <= 1e-2
+
+
 @pytest.mark.parametrize("dt", [orc.F32, orc.F16, orc.BF16])
 def test_attention_invariants_on_gpu(g, dt):
     rng = np.random.default_rng(11)
