@@ -3,17 +3,21 @@
 //
 // attention_decode.hip is built for latency (one pass, everything in flight at once, one workgroup
 // per CU); with tens of megabytes of K/V per launch the job is bandwidth instead, and this kernel
-// keeps the loads streaming: a workgroup of 4 waves walks its key range in tiles of 16 keys per wave,
-// the next tile's K and V already in registers while the current one is used.
-//   scores   S^T[16 keys x 16 heads] = K_tile . Q^T with v_mfma_f32_16x16x32 (K rows are the A operand
-//            straight from global memory: lane l holds key l%16, dims 8*(l/16)..+7 of each 32-dim block;
-//            heads beyond G are zero columns),
-//   softmax  online, per head, f32; the tile's p values and the rescale factors cross to the layout of
-//            the next step through a 1 KB LDS patch per wave,
-//   P.V      on the vector ALUs: a lane owns one key of the pass and 8 dims, and accumulates
-//            o[g][8 dims] for all G heads from one 16-byte V load (8 FMAs per head per key),
-// then lanes and waves are combined, and key ranges by a small second launch (attn_merge_kernel).
-// Replaces the reference's attention_decode (attention.cuh:495-606) for these shapes.
+// keeps the loads streaming: a workgroup of 4 waves walks its key range in tiles of 32 keys per wave,
+// the next tile's K and V already in registers while the current one is used.  Both products run on
+// the matrix cores (v_mfma_f32_16x16x32), with the query heads as the 16 columns (zero beyond G):
+//   scores   S[keys x heads] = K_tile . Q^T; K rows are the A operand straight from global memory
+//            (lane l holds key l%16, dims 8*(l/16)..+7 of each 32-dim block),
+//   softmax  online, per head, f32; a lane holds one head (l%16), so rescaling its accumulators is
+//            lane-local; the tile's p values go to LDS as [head][key] in the storage type,
+//   P.V      O^T[dims x heads] += V^T . P; V needs its keys along the reduction, so the tile is parked
+//            in LDS (row stride 136 bytes: conflict-free) and read back two dims at a time, each pair of
+//            keys split into an "even dims" and an "odd dims" operand by one v_perm -- the 16 rows of
+//            an MFMA tile are dims 32c + 2r (+1),
+// then waves are combined through LDS and key ranges by a small second launch (attn_merge_kernel).
+// P enters the second product as a sum of two storage-type values.  Replaces the reference's attention_decode (attention.cuh:495-606) for these shapes.
+#include <type_traits>
+
 #include "attention.h"
 #include "mfma.h"
 
@@ -32,16 +36,24 @@ template <> struct Mfma16<bf16_t> {
     }
 };
 
-constexpr int kStreamWaves = 4, kStreamThreads = kStreamWaves * 64, kStreamTile = 16;
+constexpr int kStreamWaves = 4, kStreamThreads = kStreamWaves * 64, kStreamTile = 32;
 
 template <typename T, int D, int G>
 __global__ __launch_bounds__(kStreamThreads) void attn_stream_kernel(AttnParams p) {
-    constexpr int KB = D / 32;        // 32-dim blocks of a key row (MFMA K steps)
-    constexpr int LPK = D / 8;        // lanes per key in the P.V layout
-    constexpr int KPP = 64 / LPK;     // keys per P.V pass of a wave
-    constexpr int NP = kStreamTile / KPP;  // passes per tile
-    __shared__ float p_s[kStreamWaves][kStreamTile][16];  // p[key][head] of the wave's tile
-    __shared__ float a_s[kStreamWaves][16];               // rescale factor per head
+    constexpr int KB = D / 32;              // 32-dim blocks of a key row
+    constexpr int LPK = D / 8;              // lanes per key row when a tile is loaded 16 bytes per lane
+    constexpr int KPP = 64 / LPK;           // key rows per load pass of a wave
+    constexpr int NP = kStreamTile / KPP;   // load passes per tile (V)
+    constexpr int VST = D + 4;              // V tile row stride in elements (D*2 + 8 bytes)
+    constexpr int PST = kStreamTile + 8;    // p tile row stride in elements (16-byte aligned rows)
+    __shared__ __align__(16) uint16_t v_s[kStreamWaves][kStreamTile * VST];
+    // the storage type keeps 8 (bf16) or 11 (fp16) bits of p, and over thousands of keys that rounding shows
+    // in small outputs: a second tile holds the remainder p - T(p) and feeds a second product
+    constexpr bool kSplitP = true;
+    // fp16 has the bits but not the range: p of a far-away key is subnormal or zero in fp16 while
+    // thousands of them still add up, so p is stored times 2^12 and the factor taken out at the end
+    constexpr float kPScale = std::is_same<T, f16_t>::value ? 4096.f : 1.f;
+    __shared__ __align__(16) uint16_t p_s[kStreamWaves][(kSplitP ? 2 : 1) * 16 * PST];
     __shared__ float m_s[kStreamWaves][G], l_s[kStreamWaves][G];
     __shared__ float o_s[kStreamWaves][G][D];
 
@@ -54,52 +66,66 @@ __global__ __launch_bounds__(kStreamThreads) void attn_stream_kernel(AttnParams 
     const int k0 = split * p.slice, k1 = min(bound, k0 + p.slice);
     const size_t kv_base = (size_t)bhkv * p.cache_len;
     const T *Kp = (const T *)p.k + kv_base * D, *Vp = (const T *)p.v + kv_base * D;
+    const int col = lane & 15, quad = lane >> 4;  // MFMA column (head) and row/k group of this lane
 
-    // Q^T as the MFMA B operand: lane l = head l%16 (zero beyond G), dims 8*(l/16)..+7 of each block
+    // Q^T as the B operand of the score product: column = head, k = dims 8*quad..+7 of each block
     U4 qf[KB];
     {
-        const int h = lane & 15;
-        const T *qrow = (const T *)p.q + (size_t)b * p.q_bs + (size_t)(head0 + (h < G ? h : 0)) * p.q_hs;
+        const T *qrow = (const T *)p.q + (size_t)b * p.q_bs + (size_t)(head0 + (col < G ? col : 0)) * p.q_hs;
 #pragma unroll
         for (int j = 0; j < KB; j++) {
-            qf[j] = *(const U4 *)(qrow + j * 32 + (lane >> 4) * 8);
-            if (h >= G) qf[j] = U4{0u, 0u, 0u, 0u};
+            qf[j] = *(const U4 *)(qrow + j * 32 + quad * 8);
+            if (col >= G) qf[j] = U4{0u, 0u, 0u, 0u};
         }
     }
 
-    // running state.  Scores layout (after the MFMA): lane l = head l%16, keys 4*(l/16)+e of the tile.
-    float m_run = -INFINITY, l_run = 0.f;  // of head l%16 (the 4 lanes sharing a head hold partial l)
-    float o[G][8];
+    // running state of head `col`: maximum, partial sum (the 4 quads hold parts), O^T accumulators
+    // acc[c][par][e] = dim 32c + 2*(4*quad + e) + par
+    float m_run = -INFINITY, l_run = 0.f;
+    f4_t acc[KB][2];
 #pragma unroll
-    for (int g = 0; g < G; g++)
+    for (int c = 0; c < KB; c++)
 #pragma unroll
-        for (int e = 0; e < 8; e++) o[g][e] = 0.f;
+        for (int par = 0; par < 2; par++) acc[c][par] = f4_t{0.f, 0.f, 0.f, 0.f};
 
-    const int kk_m = lane & 15, kd_m = (lane >> 4) * 8;   // K load: key within tile, dim offset within a block
-    const int kk_v = lane / LPK, vd = (lane % LPK) * 8;   // V load: key within pass, dim offset
-    auto load_tile = [&](int t0, U4 *kr, U4 *vr) {
+    const int vk = lane / LPK, vd = (lane % LPK) * 8;  // V load: key row within a pass, dim offset
+    auto load_tile = [&](int t0, U4 (*kr)[KB], U4 *vr) {
         // rows past the range re-read the last valid row; their scores are masked below
-        const int krow = min(t0 + kk_m, k1 - 1);
 #pragma unroll
-        for (int j = 0; j < KB; j++) kr[j] = *(const U4 *)(Kp + (size_t)krow * D + j * 32 + kd_m);
+        for (int a = 0; a < 2; a++) {
+            const int krow = min(t0 + a * 16 + col, k1 - 1);
+#pragma unroll
+            for (int j = 0; j < KB; j++) kr[a][j] = *(const U4 *)(Kp + (size_t)krow * D + j * 32 + quad * 8);
+        }
 #pragma unroll
         for (int q = 0; q < NP; q++) {
-            const int vrow = min(t0 + q * KPP + kk_v, k1 - 1);
+            const int vrow = min(t0 + q * KPP + vk, k1 - 1);
             vr[q] = *(const U4 *)(Vp + (size_t)vrow * D + vd);
         }
     };
 
-    auto process = [&](int t, const U4 *kr, const U4 *vr) {
-        // ---- scores of this tile
-        f4_t s4 = {0.f, 0.f, 0.f, 0.f};
+    uint16_t *vt = v_s[wave], *pt = p_s[wave];
+    auto process = [&](int t, const U4 (*kr)[KB], const U4 *vr) {
+        // ---- park V: [key][dim], two 8-byte stores per lane and pass
 #pragma unroll
-        for (int j = 0; j < KB; j++) s4 = Mfma16<T>::run(kr[j], qf[j], s4);
-        float sv[4], tmax = -INFINITY;
+        for (int q = 0; q < NP; q++) {
+            uint2 *dst = (uint2 *)&vt[(q * KPP + vk) * VST + vd];
+            dst[0] = uint2{vr[q].x, vr[q].y};
+            dst[1] = uint2{vr[q].z, vr[q].w};
+        }
+        // ---- scores: lane = head col, keys 16a + 4*quad + e
+        float sv[2][4], tmax = -INFINITY;
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const int key = t + (lane >> 4) * 4 + e;
-            sv[e] = key < k1 ? s4[e] * p.scale : -INFINITY;
-            tmax = fmaxf(tmax, sv[e]);
+        for (int a = 0; a < 2; a++) {
+            f4_t s4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < KB; j++) s4 = Mfma16<T>::run(kr[a][j], qf[j], s4);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int key = t + a * 16 + quad * 4 + e;
+                sv[a][e] = key < k1 ? s4[e] * p.scale : -INFINITY;
+                tmax = fmaxf(tmax, sv[a][e]);
+            }
         }
         tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
@@ -108,38 +134,50 @@ __global__ __launch_bounds__(kStreamThreads) void attn_stream_kernel(AttnParams 
         m_run = m_new;
         float psum = 0.f;
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const float pe = fast_exp(sv[e] - m_new);
-            psum += pe;
-            p_s[wave][(lane >> 4) * 4 + e][lane & 15] = pe;
+        for (int a = 0; a < 2; a++) {
+            float pe[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                pe[e] = fast_exp(sv[a][e] - m_new);  // 0 for keys past the range
+                psum += pe[e];
+            }
+            // p[head][16a + 4*quad .. +3] in the storage type
+            *(uint2 *)&pt[col * PST + a * 16 + quad * 4] =
+                uint2{pack2<T>(pe[0] * kPScale, pe[1] * kPScale), pack2<T>(pe[2] * kPScale, pe[3] * kPScale)};
+            if constexpr (kSplitP) {
+                float lo[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) lo[e] = pe[e] * kPScale - Elem<T>::rnd(pe[e] * kPScale);
+                *(uint2 *)&pt[16 * PST + col * PST + a * 16 + quad * 4] = uint2{pack2<T>(lo[0], lo[1]), pack2<T>(lo[2], lo[3])};
+            }
         }
         l_run = l_run * alpha + psum;
-        if (lane < 16) a_s[wave][lane] = alpha;
+        if (alpha != 1.f) {
+#pragma unroll
+            for (int c = 0; c < KB; c++)
+#pragma unroll
+                for (int par = 0; par < 2; par++) acc[c][par] *= alpha;
+        }
         __builtin_amdgcn_wave_barrier();
-        // ---- P.V: rescale the accumulators when some head's maximum moved, then add this tile
-        float al[G];
-        bool moved = false;
+        // ---- O^T += V^T . P: B operand = p[head col][keys 8*quad..+7]; A operands from V dword pairs
+        const U4 pf = *(const U4 *)&pt[col * PST + quad * 8];
+        U4 pl = U4{0u, 0u, 0u, 0u};
+        if constexpr (kSplitP) pl = *(const U4 *)&pt[16 * PST + col * PST + quad * 8];
 #pragma unroll
-        for (int g = 0; g < G; g++) {
-            al[g] = a_s[wave][g];
-            moved |= al[g] != 1.f;
-        }
-        if (moved) {
+        for (int c = 0; c < KB; c++) {
+            uint32_t w[8];
 #pragma unroll
-            for (int g = 0; g < G; g++)
-#pragma unroll
-                for (int e = 0; e < 8; e++) o[g][e] *= al[g];
-        }
-#pragma unroll
-        for (int q = 0; q < NP; q++) {
-            float vf[8];
-            widen8<T>(vr[q], vf);
-            const float *pk = p_s[wave][q * KPP + kk_v];  // 0 for keys past the range
-#pragma unroll
-            for (int g = 0; g < G; g++) {
-                const float pg = pk[g];
-#pragma unroll
-                for (int e = 0; e < 8; e++) o[g][e] = fmaf(pg, vf[e], o[g][e]);
+            for (int i = 0; i < 8; i++) w[i] = *(const uint32_t *)&vt[(quad * 8 + i) * VST + c * 32 + col * 2];
+            U4 ev, od;  // keys 8*quad..+7 at dim 32c + 2*col and at the next dim
+            ev.x = __builtin_amdgcn_perm(w[1], w[0], 0x05040100u); od.x = __builtin_amdgcn_perm(w[1], w[0], 0x07060302u);
+            ev.y = __builtin_amdgcn_perm(w[3], w[2], 0x05040100u); od.y = __builtin_amdgcn_perm(w[3], w[2], 0x07060302u);
+            ev.z = __builtin_amdgcn_perm(w[5], w[4], 0x05040100u); od.z = __builtin_amdgcn_perm(w[5], w[4], 0x07060302u);
+            ev.w = __builtin_amdgcn_perm(w[7], w[6], 0x05040100u); od.w = __builtin_amdgcn_perm(w[7], w[6], 0x07060302u);
+            acc[c][0] = Mfma16<T>::run(ev, pf, acc[c][0]);
+            acc[c][1] = Mfma16<T>::run(od, pf, acc[c][1]);
+            if constexpr (kSplitP) {
+                acc[c][0] = Mfma16<T>::run(ev, pl, acc[c][0]);
+                acc[c][1] = Mfma16<T>::run(od, pl, acc[c][1]);
             }
         }
         __builtin_amdgcn_wave_barrier();
@@ -148,7 +186,7 @@ __global__ __launch_bounds__(kStreamThreads) void attn_stream_kernel(AttnParams 
     // two register sets, named so that the wait for one never covers the other; the load of the tile
     // after next is issued unconditionally (rows clamp to the last valid one) to keep the loop free of
     // branches around loads
-    U4 kA[KB], vA[NP], kB[KB], vB[NP];
+    U4 kA[2][KB], vA[NP], kB[2][KB], vB[NP];
     const int tstep = kStreamWaves * kStreamTile;
     int t = k0 + wave * kStreamTile;
     if (t < k1) {
@@ -165,27 +203,21 @@ __global__ __launch_bounds__(kStreamThreads) void attn_stream_kernel(AttnParams 
         }
     }
 
-    // ---- combine inside the wave: l over the 4 lanes of a head, o over the KPP key slots
+    // ---- this wave's results to LDS: l over the 4 quads of a head; lane (head col, quad) holds the
+    // dims 32c + 2*(4*quad + e) + par of O^T
     l_run += __shfl_xor(l_run, 16, 64);
     l_run += __shfl_xor(l_run, 32, 64);
-#pragma unroll
-    for (int g = 0; g < G; g++)
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            float v = o[g][e];
-#pragma unroll
-            for (int off = LPK; off < 64; off <<= 1) v += __shfl_xor(v, off, 64);
-            o[g][e] = v;
-        }
     if (lane < G) {
         m_s[wave][lane] = m_run;
         l_s[wave][lane] = l_run;
     }
-    if (lane < LPK) {
+    if (col < G) {
 #pragma unroll
-        for (int g = 0; g < G; g++)
+        for (int c = 0; c < KB; c++)
 #pragma unroll
-            for (int e = 0; e < 8; e++) o_s[wave][g][lane * 8 + e] = o[g][e];
+            for (int par = 0; par < 2; par++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) o_s[wave][col][c * 32 + 2 * (4 * quad + e) + par] = acc[c][par][e] * (1.0f / kPScale);
     }
     __syncthreads();
 
@@ -263,7 +295,7 @@ bool attn_stream_eligible(int B, int Sq, int Hq, int Hkv, int D, int dtype, int 
 
 // key rows per workgroup and number of key ranges: as many workgroups as the device holds at once
 // (three per CU at the kernel's register count) and no more, so that there is no short second round;
-// ranges a multiple of the 64 keys a workgroup takes per step and at least 128 long
+// ranges a multiple of the 128 keys a workgroup takes per step
 void attn_stream_plan(int B, int Hkv, int kv_len, int *slice, int *nsplit) {
     const int step = kStreamWaves * kStreamTile;
     static int slots = 0;
