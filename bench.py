@@ -164,10 +164,66 @@ def prefill_main(args, mynn, cfg):
     print(json.dumps(out))
 
 
+def attention_main(args, mynn):
+    """GQA decode attention op at the largest shape of configs[1]: 16 sequences x 4096 cached keys,
+    32 query heads over 4 KV heads of 64 dims, fp16 cache, softmax scale 1/8.  One step = one
+    attention call; the caches rotate over > 256 MB so no call finds its K/V in the Infinity Cache."""
+    import torch
+
+    B, L, Hq, Hkv, D = 16, 4096, 32, 4, 64
+    K = 200 if args.steps is None else args.steps
+    W = 10 if args.warmup is None else args.warmup
+    tdt = {"f16": torch.float16, "bf16": torch.bfloat16}[args.dtype]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(args.seed)
+    n = 6  # 6 x 67 MB of K/V
+    ks = [torch.randn((B, Hkv, L, D), generator=gen, device="cuda", dtype=tdt) for _ in range(n)]
+    vs = [torch.randn((B, Hkv, L, D), generator=gen, device="cuda", dtype=tdt) for _ in range(n)]
+    q = torch.randn((B, Hq, 1, D), generator=gen, device="cuda", dtype=tdt)
+    for i in range(W):
+        mynn.attention(q, ks[i % n], vs[i % n], 0.125, active=L)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(K):
+        mynn.attention(q, ks[i % n], vs[i % n], 0.125, active=L)
+    stop.record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    gpu_ms = start.elapsed_time(stop) / K  # launches are queued ahead of the GPU: this is device time per call
+    nbytes = 2 * B * Hkv * L * D * 2 + 2 * B * Hq * D * 2
+    achieved = nbytes / (gpu_ms * 1e-3) / 1e9
+    out = {
+        "metric": "GQA decode attention op: achieved HBM GB/s vs peak (configs[1], B=16, L=4096)",
+        "value": round(achieved, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(elapsed * 1e3 / K, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32 softmax and accumulate over %s K/V" % args.dtype, "data": "synthetic",
+        "config": {"workload": "configs[1]: attention op, B=16, Hq=32, Hkv=4, D=64, L=4096, scale 0.125, seq_q=1",
+                   "seed": args.seed, "rotating_kv_sets": n, "device_ms_per_call": round(gpu_ms, 4)},
+        "roofline": {"bound": "hbm", "kernel": "attn_stream_kernel + attn_merge_kernel", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "bytes_per_launch": nbytes, "avg_launch_us": round(gpu_ms * 1e3, 2)},
+    }
+    if not args.no_cpu_baseline:
+        import numpy as np
+        import oracle as orc
+
+        dt = {"f16": orc.F16, "bf16": orc.BF16}[args.dtype]
+        hq, hk, hv = [t.view(torch.int16).cpu().numpy().view(np.uint16) for t in (q, ks[0], vs[0])]
+        t0 = time.perf_counter()
+        orc.attention(hq, hk, hv, dt, 0.125)
+        cpu = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": round(nbytes / cpu / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": "one call at the same shape, C port of the reference CPU attention "
+                                         "(single thread, as the reference)"}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--workload", choices=["decode", "prefill"], default="decode")
+    ap.add_argument("--workload", choices=["decode", "prefill", "attention"], default="decode")
     ap.add_argument("--steps", type=int, default=None, help="default 256 (decode) / 5 (prefill)")
     ap.add_argument("--warmup", type=int, default=None, help="default 16 (decode) / 2 (prefill)")
     ap.add_argument("--dtype", choices=["f16", "bf16"], default="f16")
@@ -201,6 +257,8 @@ def main():
     cfg = dict(TINYLLAMA, dtype=dt)
     if args.workload == "prefill":
         return prefill_main(args, mynn, cfg)
+    if args.workload == "attention":
+        return attention_main(args, mynn)
     K = 256 if args.steps is None else args.steps
     W = 16 if args.warmup is None else args.warmup
     assert PROMPT_LEN + max(K, W) <= cfg["max_seq"], "steps/warmup do not fit max_seq %d" % cfg["max_seq"]

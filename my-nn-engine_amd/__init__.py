@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libmynn_hip.so")
 CSRC = os.path.join(_HERE, "csrc")
 
-F32, BF16, F16 = 0, 1, 2
+F32, BF16, F16, I8 = 0, 1, 2, 3
 
 
 class MynnError(RuntimeError):
@@ -98,6 +98,17 @@ SIGNATURES = {
     "mynn_model_decode_loop": (_i, [_vp, C.c_int32, _i64, _i, _vp]),
     "mynn_model_profile_step": (_i, [_vp, C.c_int32, _i64, C.POINTER(KernelTime), _i]),
     "mynn_model_profile": (_i, [_vp, _vp, _vp, _i64, _i64, C.POINTER(KernelTime), _i]),
+    "mynn_weights_open": (_vp, [C.c_char_p]),
+    "mynn_weights_close": (None, [_vp]),
+    "mynn_weights_count": (_i, [_vp]),
+    "mynn_weights_name": (C.c_char_p, [_vp, _i]),
+    "mynn_weights_find": (_i, [_vp, C.c_char_p, C.POINTER(_i), C.POINTER(_i64), C.POINTER(_i), C.POINTER(_vp),
+                               C.POINTER(_sz)]),
+    "mynn_quantize_safetensors_int8": (_i, [C.c_char_p, C.c_char_p, C.POINTER(_i), C.POINTER(_i)]),
+    "mynn_weights_upload": (_vp, [_vp, _vp]),
+    "mynn_device_weights_initializer": (C.POINTER(_vp), [_vp]),
+    "mynn_device_weights_int8": (_i, [_vp]),
+    "mynn_device_weights_free": (None, [_vp]),
     "mynn_quantize_per_channel": (_i, [_vp, _vp, _vp, _sz, _sz, _i]),
     "mynn_rope_table": (_i, [_vp, _vp, _i, _i, _f, _i]),
     "mynn_llm_create": (_vp, [_vp, _vp, _i, _i, _i64]),
@@ -301,6 +312,70 @@ def argmax_last(logits):
 LIN_NAMES = ("q", "k", "v", "o", "gate", "up", "down")
 
 
+class Weights:
+    """HfWeights: a .safetensors file or model directory, memory-mapped (crates/llm/src/hf_weights.rs)."""
+
+    def __init__(self, path):
+        self.handle = lib().mynn_weights_open(str(path).encode())
+        if not self.handle:
+            raise MynnError(lib().mynn_last_error().decode())
+
+    def names(self):
+        return [lib().mynn_weights_name(self.handle, i).decode() for i in range(lib().mynn_weights_count(self.handle))]
+
+    def find(self, name):
+        """(dtype code, shape, numpy view of the mapped bytes)."""
+        import numpy as np
+
+        dt, nd, ptr, nb = _i(), _i(), _vp(), _sz()
+        shape = (_i64 * 8)()
+        check(lib().mynn_weights_find(self.handle, name.encode(), C.byref(dt), shape, C.byref(nd), C.byref(ptr), C.byref(nb)))
+        npdt = {F32: np.float32, BF16: np.uint16, F16: np.uint16, I8: np.int8}[dt.value]
+        buf = (C.c_char * nb.value).from_address(ptr.value) if nb.value else b""
+        arr = np.frombuffer(buf, dtype=npdt).reshape([shape[i] for i in range(nd.value)])
+        return dt.value, tuple(arr.shape), arr
+
+    def close(self):
+        if getattr(self, "handle", None) and _lib is not None:
+            _lib.mynn_weights_close(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def quantize_safetensors_int8(src, dst):
+    """crates/llm/src/quantize.rs quantize_safetensors_int8(_dir): returns (quantized, passthrough)."""
+    q, p = _i(), _i()
+    check(lib().mynn_quantize_safetensors_int8(str(src).encode(), str(dst).encode(), C.byref(q), C.byref(p)))
+    return q.value, p.value
+
+
+class DeviceWeights:
+    """A checkpoint uploaded in `initializer` order (mynn_weights_upload); owns the device memory."""
+
+    def __init__(self, weights, cfg_struct):
+        self.handle = lib().mynn_weights_upload(weights.handle, C.byref(cfg_struct))
+        if not self.handle:
+            raise MynnError(lib().mynn_last_error().decode())
+        self.int8 = bool(lib().mynn_device_weights_int8(self.handle))
+        self.initializer = lib().mynn_device_weights_initializer(self.handle)
+
+    def close(self):
+        if getattr(self, "handle", None) and _lib is not None:
+            _lib.mynn_device_weights_free(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 class Decoder:
     """Thin holder around model_init / model_step / model_destroy.
 
@@ -315,7 +390,8 @@ class Decoder:
         import torch
 
         tdt = {F16: torch.float16, BF16: torch.bfloat16}[cfg["dtype"]]
-        quant = isinstance(weights["embed"], tuple)
+        from_file = isinstance(weights, (str, os.PathLike, Weights))
+        quant = True if from_file else isinstance(weights["embed"], tuple)
         self.cfg = ModelConfig(cfg["n_layers"], cfg["hidden"], cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"],
                                cfg["ffn"], cfg["vocab"], cfg["max_seq"], float(cfg["eps"]), float(cfg["rope_theta"]),
                                cfg["dtype"], seq_q, batch, int(quant), int(quant_kv_cache), int(quantize_activations))
@@ -330,6 +406,20 @@ class Decoder:
                 kv = [(torch.zeros(shape, dtype=tdt, device="cuda"), torch.zeros(shape, dtype=tdt, device="cuda"))
                       for _ in range(cfg["n_layers"])]
         self.kv = kv
+        state = []
+        for bufs in kv:
+            state.extend([_ptr(t) for t in bufs])
+        self._state = (_vp * len(state))(*state)
+        if from_file:
+            # a checkpoint: read, convert and upload by the library (names as the reference's ModelSpec)
+            src = weights if isinstance(weights, Weights) else Weights(weights)
+            self.weights = DeviceWeights(src, self.cfg)
+            self.cfg.weights_int8 = int(self.weights.int8)
+            check(lib().mynn_model_configure(C.byref(self.cfg)))
+            self.handle = lib().model_init(self.weights.initializer, self._state)
+            if not self.handle:
+                raise MynnError("model_init failed: %s" % lib().mynn_last_error().decode())
+            return
         init = []
 
         def lin(w):
@@ -348,11 +438,7 @@ class Decoder:
                 lin(weights["layers.%d.%s" % (l, nm)])
         init.append(_ptr(weights["final_norm"]))
         lin(weights["lm_head"])
-        state = []
-        for bufs in kv:
-            state.extend([_ptr(t) for t in bufs])
         self._init = (_vp * len(init))(*init)
-        self._state = (_vp * len(state))(*state)
         check(lib().mynn_model_configure(C.byref(self.cfg)))
         torch.cuda.synchronize()
         self.handle = lib().model_init(self._init, self._state)
