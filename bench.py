@@ -220,10 +220,93 @@ def attention_main(args, mynn):
     print(json.dumps(out))
 
 
+LLAMA3_8B = dict(n_layers=32, hidden=4096, n_heads=32, n_kv_heads=8, head_dim=128, ffn=14336, vocab=128256,
+                 max_seq=2304, eps=1e-5, rope_theta=500000.0)
+
+
+def decode_batch_main(args, mynn):
+    """configs[4]: Llama-3-8B-shape int8 decoder, 32 sequences decoded together at a context of 2048
+    tokens.  The caches are filled with random K/V rows instead of running the 65,536-token prefill: the
+    cost of a decode step does not depend on their values.  One step = one new token for each sequence."""
+    import numpy as np
+    import torch
+
+    B, ctx = 32, 2048
+    K = 32 if args.steps is None else args.steps
+    W = 4 if args.warmup is None else args.warmup
+    dt = {"f16": mynn.F16, "bf16": mynn.BF16}[args.dtype]
+    tdt = {"f16": torch.float16, "bf16": torch.bfloat16}[args.dtype]
+    cfg = dict(LLAMA3_8B, dtype=dt)
+    assert ctx + W + K <= cfg["max_seq"]
+    weights = make_weights(cfg, dt, args.seed)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(args.seed + 1)
+    shape = (B, cfg["n_kv_heads"], cfg["max_seq"], cfg["head_dim"])
+    kv = []
+    for _ in range(cfg["n_layers"]):
+        k = torch.zeros(shape, dtype=tdt, device="cuda")
+        v = torch.zeros(shape, dtype=tdt, device="cuda")
+        k[:, :, :ctx] = torch.randn((B, shape[1], ctx, shape[3]), generator=gen, device="cuda", dtype=tdt)
+        v[:, :, :ctx] = torch.randn((B, shape[1], ctx, shape[3]), generator=gen, device="cuda", dtype=tdt)
+        kv.append((k, v))
+    torch.cuda.synchronize()
+    dec = mynn.Decoder(cfg, weights, batch=B, kv=kv)
+    stats = dec.stats()
+    rng = np.random.default_rng(args.seed)
+    toks = rng.integers(0, cfg["vocab"], B).tolist()
+    past = ctx
+    for _ in range(W):
+        toks, _ = dec.step(toks, [past], past, past + 1)
+        past += 1
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(K):
+        toks, _ = dec.step(toks, [past], past, past + 1)
+        past += 1
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / K
+
+    agg = {}
+    for _ in range(2):
+        for name, ms, nbytes, flops in dec.profile(toks, [past], past, past + 1):
+            a = agg.setdefault(name, [0, 0.0, 0.0])
+            a[0] += 1
+            a[1] += ms
+            a[2] += nbytes
+    eb = 2
+    H, F, V = cfg["hidden"], cfg["ffn"], cfg["vocab"]
+    QD, KD = cfg["n_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
+    w_bytes = cfg["n_layers"] * (QD * H + 2 * KD * H + H * QD + 3 * F * H) + V * H
+    kv_bytes = cfg["n_layers"] * B * 2 * KD * eb * (ctx + W + K // 2)
+    step_bytes = w_bytes + kv_bytes
+    lin = {k: v for k, v in agg.items() if k.startswith("linear_")}
+    dom = max(lin, key=lambda k: lin[k][1])
+    calls, ms_tot, bytes_tot = lin[dom]
+    achieved = bytes_tot / (ms_tot * 1e-3) / 1e9
+    out = {
+        "metric": "decode tok/s, batch 32 at context 2048, Llama-3-8B-shape int8 (aggregate over the batch)",
+        "value": round(B * K / elapsed, 1), "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32 accumulate over int8 weights, %s activations/KV" % args.dtype, "data": "synthetic",
+        "config": {"workload": "configs[4]: Llama-3-8B-shape int8 decoder, batch 32, context 2048 (caches filled with "
+                               "random rows), %d decode steps timed" % K,
+                   "batch": B, "context": ctx, "launches_per_step": stats["launches_per_step"], "hipgraph": stats["graph"],
+                   "seed": args.seed, "step_algorithmic_bytes": step_bytes,
+                   "step_hbm_frac": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                   "per_kernel_ms": {k: round(v[1] / 2, 3) for k, v in sorted(agg.items(), key=lambda kv: -kv[1][1])}},
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "bytes_per_launch": bytes_tot / calls,
+                     "avg_launch_us": round(ms_tot / calls * 1e3, 2)},
+    }
+    dec.close()
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--workload", choices=["decode", "prefill", "attention"], default="decode")
+    ap.add_argument("--workload", choices=["decode", "prefill", "attention", "decode_batch"], default="decode")
     ap.add_argument("--steps", type=int, default=None, help="default 256 (decode) / 5 (prefill)")
     ap.add_argument("--warmup", type=int, default=None, help="default 16 (decode) / 2 (prefill)")
     ap.add_argument("--dtype", choices=["f16", "bf16"], default="f16")
@@ -259,6 +342,8 @@ def main():
         return prefill_main(args, mynn, cfg)
     if args.workload == "attention":
         return attention_main(args, mynn)
+    if args.workload == "decode_batch":
+        return decode_batch_main(args, mynn)
     K = 256 if args.steps is None else args.steps
     W = 16 if args.warmup is None else args.warmup
     assert PROMPT_LEN + max(K, W) <= cfg["max_seq"], "steps/warmup do not fit max_seq %d" % cfg["max_seq"]

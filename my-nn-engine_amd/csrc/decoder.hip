@@ -56,6 +56,8 @@ struct Layer {
     void *own_qkv_w = nullptr, *own_qkv_s = nullptr, *own_gu_w = nullptr, *own_gu_s = nullptr;
     // prefill executors: weights dequantised once to the 16-bit type, [N, Kp] (wt_gu: gate/up in groups of 32)
     void *wt_qkv = nullptr, *wt_o = nullptr, *wt_gu = nullptr, *wt_down = nullptr;
+    // few-row executors: int8 weights re-tiled so that a wave streams them sequentially
+    void *pk_qkv = nullptr, *pk_o = nullptr, *pk_gu = nullptr, *pk_down = nullptr;
 };
 
 struct Launch {
@@ -70,8 +72,10 @@ struct Model {
     Lin embed, lm_head;
     const void *final_norm = nullptr;
     std::vector<Layer> layers;
-    void *wt_lm_head = nullptr;
+    void *wt_lm_head = nullptr, *pk_lm_head = nullptr;
     bool resident16 = false;  // the wt_* copies exist and the matrix-core path with fused stores is used
+    bool skinny = false;      // 16..64 rows: int8 weights streamed once through the few-row matrix-core kernel
+    float *skinny_scratch = nullptr;
     void *cos_t = nullptr, *sin_t = nullptr;
     // arena
     char *arena = nullptr;
@@ -163,6 +167,16 @@ static int linear_rows(Model &m, void *out, const void *act, const Lin &l, int M
     return launch_status("dense_linear_kernel");
 }
 
+// one few-row GEMM against int8 weights (two launches: products, then sum/scale/store)
+static int skinny_rows(Model &m, void *out, const void *act, const Lin &l, const void *packed, const void *res, int M, int epi,
+                       const char *name) {
+    const double eb = dtype_size(m.cfg.dtype), n_out = epi == GEMM_SWIGLU ? l.N / 2 : l.N;
+    note(m, name, (double)l.N * l.K + l.N * eb + (double)M * l.K * eb + (double)M * n_out * eb * (epi == GEMM_RESIDUAL ? 2 : 1),
+         2.0 * M * l.N * l.K);
+    return dequant_gemm_skinny(out, act, (const int8_t *)(packed ? packed : l.w), packed != nullptr, l.scale, res, M, l.N, l.K,
+                               m.cfg.dtype, epi, m.skinny_scratch, m.stream);
+}
+
 // Options::quantize_activations: DynamicQuantizeLinear (per row, symmetric) then QuantizedMatMul.
 // `fresh` = the activation changed since the last call (q/k/v and gate/up share one quantisation,
 // as the pass caches it per value: quantize_activations.rs:121-130).
@@ -208,7 +222,8 @@ static int enqueue_step(Model &m) {
         } else {
             note(m, "rms_norm", 2.0 * rows * H * eb + H * eb);
             TRY(mynn_rms_norm(m.nrm, m.x, L.norm1, rows, H, c.eps, c.dtype, s));
-            if (w8a8) TRY(linear_w8a8(m, m.qkv, m.nrm, L.qkv, rows, true, "qlinear_qkv"));
+            if (m.skinny) TRY(skinny_rows(m, m.qkv, m.nrm, L.qkv, L.pk_qkv, nullptr, rows, GEMM_PLAIN, "linear_qkv"));
+            else if (w8a8) TRY(linear_w8a8(m, m.qkv, m.nrm, L.qkv, rows, true, "qlinear_qkv"));
             else if (m.resident16) TRY(gemm_rows(m, m.qkv, m.nrm, L.wt_qkv, nullptr, rows, L.qkv.N, H, GEMM_PLAIN, "linear_qkv"));
             else TRY(linear_rows<T>(m, m.qkv, m.nrm, L.qkv, rows, "linear_qkv"));
         }
@@ -248,6 +263,12 @@ static int enqueue_step(Model &m) {
             TRY(gemv_norm_swiglu<T>(m.hmid, m.x2, L.norm2, c.eps, (const int8_t *)L.gu.w, L.gu.scale, L.gu.N, H, s));
             note(m, "gemv_down_residual", (double)H * F + H * eb + F * eb + 2 * H * eb);
             TRY(gemv_residual<T>(m.x, m.hmid, (const int8_t *)L.down.w, L.down.scale, m.x2, H, F, s));
+        } else if (m.skinny) {
+            TRY(skinny_rows(m, m.x2, m.attn, L.o, L.pk_o, m.x, rows, GEMM_RESIDUAL, "linear_o_residual"));
+            note(m, "rms_norm", 2.0 * rows * H * eb + H * eb);
+            TRY(mynn_rms_norm(m.nrm, m.x2, L.norm2, rows, H, c.eps, c.dtype, s));
+            TRY(skinny_rows(m, m.hmid, m.nrm, L.gu, L.pk_gu, nullptr, rows, GEMM_SWIGLU, "linear_gateup_swiglu"));
+            TRY(skinny_rows(m, m.x, m.hmid, L.down, L.pk_down, m.x2, rows, GEMM_RESIDUAL, "linear_down_residual"));
         } else if (w8a8) {
             TRY(linear_w8a8(m, m.proj, m.attn, L.o, rows, true, "qlinear_o"));
             note(m, "add", 3.0 * rows * H * eb);
@@ -289,7 +310,8 @@ static int enqueue_step(Model &m) {
     } else {
         note(m, "rms_norm", 2.0 * rows * H * eb + H * eb);
         TRY(mynn_rms_norm(m.nrm, m.x, m.final_norm, rows, H, c.eps, c.dtype, s));
-        if (w8a8) TRY(linear_w8a8(m, m.logits, m.nrm, m.lm_head, rows, true, "qlinear_lm_head"));
+        if (m.skinny) TRY(skinny_rows(m, m.logits, m.nrm, m.lm_head, m.pk_lm_head, nullptr, rows, GEMM_PLAIN, "linear_lm_head"));
+        else if (w8a8) TRY(linear_w8a8(m, m.logits, m.nrm, m.lm_head, rows, true, "qlinear_lm_head"));
         else if (m.resident16) TRY(gemm_rows(m, m.logits, m.nrm, m.wt_lm_head, nullptr, rows, V, H, GEMM_PLAIN, "linear_lm_head"));
         else TRY(linear_rows<T>(m, m.logits, m.nrm, m.lm_head, rows, "linear_lm_head"));
     }
@@ -393,7 +415,28 @@ static int build(Model &m, void **init, void **state) {
     // ---- prefill executors keep every linear weight dequantised to the 16-bit type (2 bytes per weight
     // on top of the int8 originals): the matrix-core GEMM reads them directly, and the values are
     // those of the per-call dequantisation, T(wq * scale)
-    if (m.quant && !c.quantize_activations && c.batch * c.seq_q >= 16 && H % 8 == 0 && QD % 8 == 0 && F % 32 == 0) {
+    {
+        const int rows_ = c.batch * c.seq_q;
+        m.skinny = m.quant && !c.quantize_activations && skinny_gemm_supported(rows_, QD + 2 * KD, H) &&
+                   skinny_gemm_supported(rows_, H, QD) && skinny_gemm_supported(rows_, 2 * F, H) &&
+                   skinny_gemm_supported(rows_, H, F) && skinny_gemm_supported(rows_, V, H);
+    }
+    if (m.skinny) {
+        // one more int8 copy of every linear weight, tiled for sequential streaming (1 byte per weight)
+        auto pack = [&](void **dst, const Lin &l) {
+            MYNN_HIP(hipMalloc(dst, skinny_packed_bytes(l.N, l.K)));
+            return skinny_pack_weight(*dst, (const int8_t *)l.w, l.N, l.K, m.stream);
+        };
+        for (Layer &L : m.layers) {
+            TRY(pack(&L.pk_qkv, L.qkv));
+            TRY(pack(&L.pk_o, L.o));
+            TRY(pack(&L.pk_gu, L.gu));
+            TRY(pack(&L.pk_down, L.down));
+        }
+        TRY(pack(&m.pk_lm_head, m.lm_head));
+        MYNN_HIP(hipStreamSynchronize(m.stream));
+    }
+    if (m.quant && !m.skinny && !c.quantize_activations && c.batch * c.seq_q >= 16 && H % 8 == 0 && QD % 8 == 0 && F % 32 == 0) {
         auto resident = [&](void **dst, const Lin &l) {
             MYNN_HIP(hipMalloc(dst, gemm_weight_bytes(l.N, l.K)));
             return dequant_weight_rows(*dst, (const int8_t *)l.w, l.scale, l.N, l.K, c.dtype, 0, 0, m.stream);
@@ -428,6 +471,14 @@ static int build(Model &m, void **init, void **state) {
     size_t o_h = plan.take((size_t)rows * F * eb), o_p = plan.take((size_t)rows * H * eb);
     size_t o_l = plan.take((size_t)rows * V * eb);
     const size_t kmax = (size_t)(F > H ? (F > QD ? F : QD) : (H > QD ? H : QD));
+    size_t sk_bytes = 0;
+    if (m.skinny) {
+        const size_t cand[5] = {skinny_scratch_bytes(rows, QD + 2 * KD, H), skinny_scratch_bytes(rows, H, QD),
+                                skinny_scratch_bytes(rows, 2 * F, H), skinny_scratch_bytes(rows, H, F),
+                                skinny_scratch_bytes(rows, V, H)};
+        for (size_t b : cand) sk_bytes = b > sk_bytes ? b : sk_bytes;
+    }
+    size_t o_sk = plan.take(sk_bytes);
     size_t o_a8 = plan.take(c.quantize_activations ? (size_t)rows * kmax : 0), o_a8s = plan.take((size_t)rows * eb);
     size_t o_ids = plan.take((size_t)rows * 8), o_pos = plan.take((size_t)c.seq_q * 8);
     size_t o_sc = plan.take(256), o_tok = plan.take((size_t)m.token_cap * 4);
@@ -440,6 +491,7 @@ static int build(Model &m, void **init, void **state) {
     m.attn = m.arena + o_attn; m.g = m.arena + o_g; m.u = m.arena + o_u; m.hmid = m.arena + o_h; m.proj = m.arena + o_p;
     m.logits = m.arena + o_l;
     m.a8 = (int8_t *)(m.arena + o_a8); m.a8_scale = m.arena + o_a8s;
+    m.skinny_scratch = (float *)(m.arena + o_sk);
     m.d_ids = (int64_t *)(m.arena + o_ids); m.d_pos = (int64_t *)(m.arena + o_pos);
     m.d_past = (int32_t *)(m.arena + o_sc); m.d_active = m.d_past + 1; m.d_step = m.d_past + 2;
     m.d_next = m.d_past + 8;  // up to 56 sequences' tokens after the scalars
@@ -450,8 +502,9 @@ static int build(Model &m, void **init, void **state) {
     MYNN_HIP(hipHostMalloc((void **)&m.h_stage, m.stage_bytes, hipHostMallocDefault));
     MYNN_HIP(hipDeviceSynchronize());
 
-    // ---- capture the decode step once
-    if (rows == 1) {
+    // ---- capture the decode step once (one new token per sequence, any batch: every launch reads its
+    // positions and lengths from device memory)
+    if (c.seq_q == 1) {
         hipError_t e = hipStreamBeginCapture(m.stream, hipStreamCaptureModeThreadLocal);
         if (e == hipSuccess) {
             int rc = enqueue(m);
@@ -494,8 +547,13 @@ static void destroy(Model *m) {
         if (L.wt_o) hipFree(L.wt_o);
         if (L.wt_gu) hipFree(L.wt_gu);
         if (L.wt_down) hipFree(L.wt_down);
+        if (L.pk_qkv) hipFree(L.pk_qkv);
+        if (L.pk_o) hipFree(L.pk_o);
+        if (L.pk_gu) hipFree(L.pk_gu);
+        if (L.pk_down) hipFree(L.pk_down);
     }
     if (m->wt_lm_head) hipFree(m->wt_lm_head);
+    if (m->pk_lm_head) hipFree(m->pk_lm_head);
     if (m->cos_t) hipFree(m->cos_t);
     if (m->sin_t) hipFree(m->sin_t);
     if (m->arena) hipFree(m->arena);

@@ -19,6 +19,16 @@ int dequant_gemv_dispatch(void *out, const void *act, const int8_t *wq, const vo
                           int act_dtype, int out_dtype, hipStream_t s);
 
 // gemm.hip -- matrix-core DequantMatMul, M >= 16, 16-bit types
+// skinny.hip -- 16 <= M <= 64 rows against int8 weights streamed once (scale after the sum); `scratch` holds
+// skinny_scratch_bytes(M, N, K) of f32 partial sums; epi is one of GEMM_* (SWIGLU: interleaved gate/up rows)
+bool skinny_gemm_supported(int M, int N, int K);
+size_t skinny_scratch_bytes(int M, int N, int K);
+// `packed`: wq is a tiled copy (skinny_packed_bytes, made by skinny_pack_weight) that a wave reads sequentially
+size_t skinny_packed_bytes(int N, int K);
+int skinny_pack_weight(void *dst, const int8_t *wq, int N, int K, hipStream_t s);
+int dequant_gemm_skinny(void *out, const void *act, const int8_t *wq, bool packed, const void *scale, const void *res, int M,
+                        int N, int K, int dtype, int epi, float *scratch, hipStream_t s);
+
 // matrix-core GEMM pieces.  A dequantised weight is [N, Kp] of the 16-bit type, Kp = K rounded up to 64,
 // zero padded (gemm_weight_bytes); dequant_weight_rows writes one (group/which: see gemm.hip), and
 // gemm_nt_mfma multiplies by it: out = store(act . wt^T) with the store one of GEMM_*.

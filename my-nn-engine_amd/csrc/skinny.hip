@@ -1,0 +1,259 @@
+// DequantMatMul for a few dozen activation rows (16 <= M <= 64: batched decode, short prefill
+// chunks): the int8 weight matrix is still the whole cost, so it is streamed ONCE, as int8, and turned
+// into matrix-core operands in registers -- unlike the large-M path, which multiplies by a 16-bit
+// copy of the weights (twice the bytes) in 256-row tiles that M rows would leave mostly empty.
+//
+//   out[m,n] = T(scale[n] * sum_k act[m,k] * wq[n,k])   (scale after the f32 sum, as the reference's
+//   small-M kernels: dequant_gemv.cuh:12-59, dequant_matmul.cuh:12-51; int8 -> 16-bit is exact)
+//
+// A wave owns 32 weight rows (the A operand of v_mfma_f32_32x32x16, rows n) against up to two tiles of
+// 32 activation rows (B operand, columns m).  The reduction index of an MFMA is free to permute as long
+// as both operands agree, so a lane takes 64 CONTIGUOUS bytes of its weight row per step of 128 k
+// (a full 128-byte line per row and step across the two lane halves) and the matching activation
+// elements (staged through LDS once per workgroup and step).  Four steps' loads are in flight per wave
+// (HBM latency under load is microseconds); when the matrix has too few rows to fill the device the K range is split over gridDim.y.  Partial sums [ksplit][M][N] (f32) are summed,
+// scaled and stored by a second launch that also applies the residual or SwiGLU.
+#include <type_traits>
+
+#include "kernels.h"
+#include "mfma.h"
+
+namespace mynn {
+
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+
+// 8 int8 (two dwords) -> 8 values of T packed in a U4; exact
+template <typename T> __device__ inline U4 i8x8_to_operand(uint32_t w0, uint32_t w1) {
+    if constexpr (std::is_same<T, f16_t>::value) {
+        // byte b + 128 under an 0x64 high byte is the fp16 number 1024 + (b + 128); subtract 1152
+        const h2_t bias = {(_Float16)1152.f, (_Float16)1152.f};
+        const uint32_t x0 = w0 ^ 0x80808080u, x1 = w1 ^ 0x80808080u;
+        auto two = [&](uint32_t x, uint32_t sel) {
+            const h2_t h = __builtin_bit_cast(h2_t, __builtin_amdgcn_perm(0x64646464u, x, sel)) - bias;
+            return __builtin_bit_cast(uint32_t, h);
+        };
+        return U4{two(x0, 0x04010400u), two(x0, 0x04030402u), two(x1, 0x04010400u), two(x1, 0x04030402u)};
+    } else {
+        // |b| <= 128 has at most 8 significant bits: the upper half of its f32 form is the bf16 value
+        auto two = [&](uint32_t w, int sh) {
+            const float a = (float)(int8_t)((w >> sh) & 0xFF), b = (float)(int8_t)((w >> (sh + 8)) & 0xFF);
+            return __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, b), __builtin_bit_cast(uint32_t, a), 0x07060302u);
+        };
+        return U4{two(w0, 0), two(w0, 16), two(w1, 0), two(w1, 16)};
+    }
+}
+
+constexpr int kSkinnyWaves = 4, kSkinnyThreads = kSkinnyWaves * 64, kSkinnyK = 128, kSkinnyStages = 5;
+
+constexpr int kSkinnyLd = kSkinnyK + 8;  // LDS row stride of the activation chunk (272 bytes: conflict-free 128-bit reads)
+
+// PACKED: wq is the tiled copy made by skinny_pack_kernel -- for every (32 rows, 128 k) tile the 4 KB a
+// wave needs, in the order its four load instructions want them (instruction j, lane l -> 16 bytes at
+// j*1024 + l*16): one sequential stream per wave instead of 128-byte pieces of 32 rows a row pitch apart
+// (measured 2.3 TB/s for the row-major form: DRAM pages are opened for 128 bytes each).
+template <typename T, int MT, bool PACKED>
+__global__ __launch_bounds__(kSkinnyThreads) void skinny_gemm_kernel(float *part, const T *act, const int8_t *wq, int M,
+                                                                    int N, int K, int iters_per_split) {
+    // the activation chunk [32*MT rows][128 k] of the current step, shared by the four waves
+    __shared__ __align__(16) uint16_t a_s[2][MT * 32 * kSkinnyLd];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, h = lane >> 5;
+    const int n0 = (blockIdx.x * kSkinnyWaves + wave) * 32;
+    const int iters = K / kSkinnyK;
+    const int it0 = blockIdx.y * iters_per_split, it1 = min(it0 + iters_per_split, iters);
+    if (it0 >= it1) return;  // whole workgroup
+    // waves past N recompute the last rows (row-major) or read the zero-padded last tile (packed), store nothing
+    const int8_t *wrow = PACKED ? wq + (size_t)min(n0 / 32, (N - 1) / 32) * iters * 4096 + lane * 16
+                                : wq + (size_t)min(n0 + r, N - 1) * K + 64 * h;
+
+    f16x_t acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[mt][e] = 0.f;
+
+    // cooperative activation load: 16 lanes per row (256 contiguous bytes), 16 rows per pass of the workgroup
+    constexpr int AP = MT * 2;
+    const int arow = tid >> 4, acol = (tid & 15) * 8;
+    const T *ap[AP];
+#pragma unroll
+    for (int q = 0; q < AP; q++) ap[q] = act + (size_t)min(arow + 16 * q, M - 1) * K + acol;
+    // one step's loads: 64 bytes of this lane's weight row and this thread's share of the activation
+    // chunk.  kSkinnyStages - 1 steps are in flight at any time; everything is consumed in the order it was
+    // issued, so the counter wait for one step never drains a younger one.  Steps past the range re-read
+    // the last one (unused).
+    struct Stage {
+        U4 w[4], a[AP];
+    };
+    // Workgroups walk their K range from different starting steps: all rows of the matrix are a multiple of
+    // 128 bytes apart, so in lockstep every request in flight would carry the same low address bits and
+    // land on the same few memory channels.
+    const int len = it1 - it0, rot = (int)((blockIdx.x * 7u + blockIdx.y * 3u) % (unsigned)len);
+    auto load = [&](int it, Stage &st) {
+        int step = min(it, it1 - 1) - it0 + rot;
+        if (step >= len) step -= len;
+        const size_t k = (size_t)(it0 + step) * kSkinnyK;
+        const U4 *src = (const U4 *)(wrow + (PACKED ? (size_t)(it0 + step) * 4096 : k));
+#pragma unroll
+        for (int j = 0; j < 4; j++) st.w[j] = __builtin_nontemporal_load(src + (PACKED ? j * 64 : j));
+#pragma unroll
+        for (int q = 0; q < AP; q++) st.a[q] = *(const U4 *)(ap[q] + k);
+    };
+    auto store_act = [&](int buf, const Stage &st) {
+#pragma unroll
+        for (int q = 0; q < AP; q++) *(U4 *)&a_s[buf][(arow + 16 * q) * kSkinnyLd + acol] = st.a[q];
+    };
+    auto compute = [&](int buf, const Stage &st) {
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+            const U4 &q = st.w[s >> 1];
+            const U4 a = (s & 1) ? i8x8_to_operand<T>(q.z, q.w) : i8x8_to_operand<T>(q.x, q.y);
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) {
+                const U4 b = *(const U4 *)&a_s[buf][(mt * 32 + r) * kSkinnyLd + 64 * h + 8 * s];
+                acc[mt] = Mfma<T>::run(a, b, acc[mt]);
+            }
+        }
+    };
+
+    constexpr int S = kSkinnyStages;
+    Stage st[S];
+    int it = it0;
+#pragma unroll
+    for (int j = 0; j < S - 1; j++) load(it + j, st[j]);
+    store_act(0, st[0]);
+    __syncthreads();
+    int buf = 0;
+    bool more = true;
+    while (more) {
+#pragma unroll
+        for (int j = 0; j < S; j++) {  // fully unrolled: every stage index is a constant
+            if (more) {
+                load(it + S - 1, st[(j + S - 1) % S]);
+                compute(buf, st[j]);
+                store_act(buf ^ 1, st[(j + 1) % S]);  // the chunk of step it+1 for the other buffer
+                __syncthreads();
+                buf ^= 1;
+                more = ++it < it1;
+            }
+        }
+    }
+
+    // D[n][m]: lane holds column m = lane%32 and rows n = 8*(e/4) + 4*(lane/32) + e%4: four consecutive n
+    if (n0 >= N) return;
+    float *dst = part + (size_t)blockIdx.y * M * N;
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) {
+        const int m = mt * 32 + r;
+        if (m >= M) continue;
+#pragma unroll
+        for (int e4 = 0; e4 < 4; e4++) {
+            const int n = n0 + e4 * 8 + h * 4;
+            float *p = dst + (size_t)m * N + n;
+            if (n + 4 <= N && (N & 3) == 0) {
+                *(float4 *)p = float4{acc[mt][e4 * 4], acc[mt][e4 * 4 + 1], acc[mt][e4 * 4 + 2], acc[mt][e4 * 4 + 3]};
+            } else {
+                for (int x = 0; x < 4 && n + x < N; x++) p[x] = acc[mt][e4 * 4 + x];
+            }
+        }
+    }
+}
+
+// tile[(nb * iters + it)][j][l] (16 bytes) = W[nb*32 + l%32][it*128 + 64*(l/32) + 16*j ..]; rows past N are zero
+__global__ __launch_bounds__(256) void skinny_pack_kernel(U4 *dst, const int8_t *wq, int N, int K, size_t chunks) {
+    const size_t c = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (c >= chunks) return;
+    const int iters = K / kSkinnyK;
+    const int l = (int)(c & 63), j = (int)((c >> 6) & 3);
+    const size_t tile = c >> 8;
+    const int it = (int)(tile % iters);
+    const size_t row = (tile / iters) * 32 + (l & 31);
+    U4 v = U4{0u, 0u, 0u, 0u};
+    if (row < (size_t)N) v = *(const U4 *)(wq + row * K + (size_t)it * kSkinnyK + 64 * (l >> 5) + 16 * j);
+    dst[c] = v;
+}
+
+size_t skinny_packed_bytes(int N, int K) { return (size_t)((N + 31) / 32) * 32 * K; }
+int skinny_pack_weight(void *dst, const int8_t *wq, int N, int K, hipStream_t s) {
+    MYNN_REQUIRE(dst && wq && K % kSkinnyK == 0 && aligned16(wq) && aligned16(dst), MYNN_ERR_INVALID, "skinny pack: N=%d K=%d", N, K);
+    const size_t chunks = skinny_packed_bytes(N, K) / 16;
+    MYNN_LAUNCH(skinny_pack_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, s, (U4 *)dst, wq, N, K, chunks);
+    return launch_status("skinny_pack_kernel");
+}
+
+// sum of the K ranges, scale, store (with the residual or SwiGLU when asked); SWIGLU: rows of the weight
+// were gate/up interleaved (row 2i gate_i, 2i+1 up_i) and out is [M, N/2]
+template <typename T, int EPI>
+__global__ __launch_bounds__(256) void skinny_reduce_kernel(T *out, const float *part, const T *scale, const T *res, int M,
+                                                          int N, int ksplit) {
+    const int n_out = EPI == GEMM_SWIGLU ? N / 2 : N;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)M * n_out) return;
+    const int m = (int)(idx / n_out), c = (int)(idx % n_out);
+    auto total = [&](int n) {
+        float t = 0.f;
+        for (int s = 0; s < ksplit; s++) t += part[((size_t)s * M + m) * N + n];
+        return t;
+    };
+    if (EPI == GEMM_SWIGLU) {
+        const float g = Elem<T>::rnd(total(2 * c) * Elem<T>::ld(scale, 2 * c));
+        const float u = Elem<T>::rnd(total(2 * c + 1) * Elem<T>::ld(scale, 2 * c + 1));
+        const float sig = 1.0f / (1.0f + expf(-g));
+        Elem<T>::st(out, idx, (g * sig) * u);
+    } else {
+        float y = total(c) * Elem<T>::ld(scale, c);
+        if (EPI == GEMM_RESIDUAL) y = Elem<T>::rnd(y) + Elem<T>::ld(res, idx);
+        Elem<T>::st(out, idx, y);
+    }
+}
+
+bool skinny_gemm_supported(int M, int N, int K) { return M >= 16 && M <= 64 && K % kSkinnyK == 0 && K >= 2 * kSkinnyK && N >= 1; }
+
+// K ranges: enough waves to keep ~1000 in flight, each with at least as many steps as it has stages
+static int skinny_ksplit(int N, int K) {
+    const int waves_n = (N + 31) / 32, iters = K / kSkinnyK;
+    int ks = (1024 + waves_n - 1) / waves_n;
+    if (ks > iters / kSkinnyStages) ks = iters / kSkinnyStages;
+    return ks < 1 ? 1 : ks;
+}
+size_t skinny_scratch_bytes(int M, int N, int K) { return (size_t)skinny_ksplit(N, K) * M * N * sizeof(float); }
+
+int dequant_gemm_skinny(void *out, const void *act, const int8_t *wq, bool packed, const void *scale, const void *res, int M,
+                        int N, int K, int dtype, int epi, float *scratch, hipStream_t s) {
+    MYNN_REQUIRE(out && act && wq && scale && scratch, MYNN_ERR_INVALID, "dequant_matmul: null operand");
+    MYNN_REQUIRE(skinny_gemm_supported(M, N, K), MYNN_ERR_UNSUPPORTED, "dequant_matmul (few rows): M=%d N=%d K=%d", M, N, K);
+    MYNN_REQUIRE(aligned16(act) && aligned16(wq), MYNN_ERR_INVALID, "dequant_matmul: act and wq must be 16-byte aligned");
+    MYNN_REQUIRE(epi != GEMM_RESIDUAL || res, MYNN_ERR_INVALID, "dequant_matmul: residual store without a residual");
+    MYNN_REQUIRE(epi != GEMM_SWIGLU || N % 2 == 0, MYNN_ERR_INVALID, "dequant_matmul: SwiGLU store needs row pairs (N=%d)", N);
+    const int ksplit = skinny_ksplit(N, K), iters = K / kSkinnyK;
+    const int ips = (iters + ksplit - 1) / ksplit;
+    const int ks_used = (iters + ips - 1) / ips;
+    dim3 grid((N + 32 * kSkinnyWaves - 1) / (32 * kSkinnyWaves), ks_used);
+    const size_t n_out = (size_t)M * (epi == GEMM_SWIGLU ? N / 2 : N);
+    return dispatch_dtype16(dtype, [&](auto *t) {
+        using T = std::remove_pointer_t<decltype(t)>;
+        if (M <= 32 && packed)
+            MYNN_LAUNCH((skinny_gemm_kernel<T, 1, true>), grid, dim3(kSkinnyThreads), 0, s, scratch, (const T *)act, wq, M, N, K, ips);
+        else if (M <= 32)
+            MYNN_LAUNCH((skinny_gemm_kernel<T, 1, false>), grid, dim3(kSkinnyThreads), 0, s, scratch, (const T *)act, wq, M, N, K, ips);
+        else if (packed)
+            MYNN_LAUNCH((skinny_gemm_kernel<T, 2, true>), grid, dim3(kSkinnyThreads), 0, s, scratch, (const T *)act, wq, M, N, K, ips);
+        else
+            MYNN_LAUNCH((skinny_gemm_kernel<T, 2, false>), grid, dim3(kSkinnyThreads), 0, s, scratch, (const T *)act, wq, M, N, K, ips);
+        int rc = launch_status("skinny_gemm_kernel");
+        if (rc) return rc;
+        const dim3 rg((unsigned)((n_out + 255) / 256));
+        if (epi == GEMM_RESIDUAL)
+            MYNN_LAUNCH((skinny_reduce_kernel<T, GEMM_RESIDUAL>), rg, dim3(256), 0, s, (T *)out, scratch, (const T *)scale,
+                        (const T *)res, M, N, ks_used);
+        else if (epi == GEMM_SWIGLU)
+            MYNN_LAUNCH((skinny_reduce_kernel<T, GEMM_SWIGLU>), rg, dim3(256), 0, s, (T *)out, scratch, (const T *)scale,
+                        (const T *)res, M, N, ks_used);
+        else
+            MYNN_LAUNCH((skinny_reduce_kernel<T, GEMM_PLAIN>), rg, dim3(256), 0, s, (T *)out, scratch, (const T *)scale,
+                        (const T *)res, M, N, ks_used);
+        return launch_status("skinny_reduce_kernel");
+    });
+}
+
+}  // namespace mynn

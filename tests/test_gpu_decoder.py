@@ -228,3 +228,47 @@ def test_int8_kv_cache_and_w8a8_executor_vs_oracle(g, dt, kv8, w8a8):
             assert max_abs_rel(g.f32(ks_gpu[:, :past], dt), g.f32(ks_ref[:, :past], dt)) <= 2e-2
             assert max_abs_rel(g.f32(vs_gpu[:, :past], dt), g.f32(vs_ref[:, :past], dt)) <= 2e-2
     pre.close(), dec.close()
+
+
+FEWROWS = dict(SMALL, ffn=768)  # every K a multiple of 128: 16..64 rows take the few-row int8 GEMM
+
+
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+@pytest.mark.parametrize("rows", [16, 32, 48])
+def test_few_row_gemm_prefill_chunk_vs_oracle(g, dt, rows):
+    """16 <= rows <= 64: linears stream the int8 weights once through the few-row matrix-core kernel
+    (scale after the sum, K split over workgroups, residual / SwiGLU in the reducing launch)."""
+    cfg, w = llm_weights.synthetic_int8(FEWROWS, dt, seed=51)
+    ref = orc.Model(cfg, w)
+    dec = g.mynn.Decoder(cfg, dev_weights(g, w, dt), seq_q=rows)
+    names = [n for n, _, _, _ in dec.profile(np.zeros(rows, np.int64), np.arange(rows), 0, rows)]
+    assert "linear_gateup_swiglu" in names and "swiglu" not in names
+    rng = np.random.default_rng(rows)
+    past = 0
+    for chunk in range(2):
+        ids = rng.integers(0, cfg["vocab"], rows)
+        pos = np.arange(past, past + rows)
+        want = ref.forward(ids, pos, past, past + rows, True)
+        _, got = dec.step(ids, pos, past, past + rows, want_logits=True)
+        assert max_err_rel_to_max(g.f32(got, dt), g.f32(want, dt)) <= 1e-2, chunk
+        past += rows
+    dec.close()
+
+
+@pytest.mark.parametrize("dt", [orc.F16])
+def test_batched_decode_equals_independent_sequences(g, dt):
+    """Batch 16 decode (the shape of the batched-serving config, scaled down): every sequence must follow
+    its own batch-1 oracle, sharing nothing but the weights."""
+    B = 16
+    cfg, w = llm_weights.synthetic_int8(FEWROWS, dt, seed=61)
+    dec = g.mynn.Decoder(cfg, dev_weights(g, w, dt), batch=B)
+    refs = [orc.Model(cfg, w) for _ in range(B)]
+    rng = np.random.default_rng(4)
+    for step in range(5):
+        toks = rng.integers(0, cfg["vocab"], B)
+        nxt, got = dec.step(toks, [step], step, step + 1, want_logits=True)
+        for b in range(B):
+            want = refs[b].forward([toks[b]], [step], step, step + 1, False)
+            assert max_err_rel_to_max(g.f32(got[b:b + 1], dt), g.f32(want, dt)) <= 1e-2, (step, b)
+            assert nxt[b] == orc.argmax_last(got[b], dt)
+    dec.close()
