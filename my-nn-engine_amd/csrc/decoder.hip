@@ -318,10 +318,14 @@ static int enqueue_step(Model &m) {
     // greedy token of the last row of each sequence; for a batch-1 decode step the same launch
     // moves the device-side loop state on (token -> next input, position / past / active + 1)
     note(m, rows == 1 ? "argmax_advance" : "argmax_last", (double)B * V * eb);
-    for (int b = 0; b < B; b++) {
+    if (S == 1) {
+        // the last (only) rows of all sequences are contiguous: one launch, one workgroup per sequence
         AdvanceState adv{};
         if (rows == 1) adv = AdvanceState{m.d_ids, m.d_pos, m.d_past, m.d_active, m.d_tokens, m.d_step, m.token_cap};
-        TRY(argmax_rows<T>(m.d_next + b, (const T *)m.logits + ((size_t)b * S + (S - 1)) * V, 1, V, adv, s));
+        TRY(argmax_rows<T>(m.d_next, m.logits, B, V, adv, s));
+    } else {
+        for (int b = 0; b < B; b++)
+            TRY(argmax_rows<T>(m.d_next + b, (const T *)m.logits + ((size_t)b * S + (S - 1)) * V, 1, V, AdvanceState{}, s));
     }
     launch_timer() = LaunchTimer{};
     m.launches = (int)m.record.size();
