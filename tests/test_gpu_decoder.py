@@ -272,3 +272,29 @@ def test_batched_decode_equals_independent_sequences(g, dt):
             assert max_err_rel_to_max(g.f32(got[b:b + 1], dt), g.f32(want, dt)) <= 1e-2, (step, b)
             assert nxt[b] == orc.argmax_last(got[b], dt)
     dec.close()
+
+
+def test_full_size_tinyllama_shape_greedy_tokens_match_oracle(g):
+    """The benchmark's own model (TinyLlama-1.1B shape, int8, fp16 activations, seed 1234, GPU-generated
+    weights): a 16-token prompt and 24 greedy tokens through the captured decode step, against the oracle
+    on the same weights, teacher-forced with the GPU's tokens; a disagreement must be a tie within 8
+    spacings of fp16 in the oracle's own logits."""
+    import os
+    import sys
+    import torch
+
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import bench
+
+    dt = orc.F16
+    cfg = dict(bench.TINYLLAMA, dtype=dt, max_seq=64)
+    weights = bench.make_weights(cfg, dt, 1234)
+    torch.cuda.synchronize()
+    dec = g.mynn.Decoder(cfg, weights)
+    assert dec.stats()["graph"] and dec.stats()["launches_per_step"] == 113
+    ref = orc.Model(dict(cfg), bench.to_host_weights(weights))
+    prompt = np.random.default_rng(1234).integers(0, cfg["vocab"], 16).tolist()
+    gpu_ids, ref_ids, near = g.greedy_compare(ref, dec, prompt, 24, dt)
+    assert all(abs(gap) <= 8 for _, gap in near), near
+    assert sum(a == b for a, b in zip(gpu_ids, ref_ids)) >= 22
+    dec.close()
