@@ -244,13 +244,26 @@ def decode_batch_main(args, mynn):
     shape = (B, cfg["n_kv_heads"], cfg["max_seq"], cfg["head_dim"])
     kv = []
     for _ in range(cfg["n_layers"]):
-        k = torch.zeros(shape, dtype=tdt, device="cuda")
-        v = torch.zeros(shape, dtype=tdt, device="cuda")
-        k[:, :, :ctx] = torch.randn((B, shape[1], ctx, shape[3]), generator=gen, device="cuda", dtype=tdt)
-        v[:, :, :ctx] = torch.randn((B, shape[1], ctx, shape[3]), generator=gen, device="cuda", dtype=tdt)
-        kv.append((k, v))
+        if args.kv_int8:
+            bufs = []
+            for _ in range(2):
+                c = torch.zeros(shape, dtype=torch.int8, device="cuda")
+                c[:, :, :ctx] = torch.randint(-127, 128, (B, shape[1], ctx, shape[3]), generator=gen, device="cuda",
+                                              dtype=torch.int8)
+                bufs.append(c)
+            for _ in range(2):
+                sc = torch.zeros(shape[:3], dtype=tdt, device="cuda")
+                sc[:, :, :ctx] = (torch.rand((B, shape[1], ctx), generator=gen, device="cuda") * 0.02 + 0.01).to(tdt)
+                bufs.append(sc)
+            kv.append(tuple(bufs))
+        else:
+            k = torch.zeros(shape, dtype=tdt, device="cuda")
+            v = torch.zeros(shape, dtype=tdt, device="cuda")
+            k[:, :, :ctx] = torch.randn((B, shape[1], ctx, shape[3]), generator=gen, device="cuda", dtype=tdt)
+            v[:, :, :ctx] = torch.randn((B, shape[1], ctx, shape[3]), generator=gen, device="cuda", dtype=tdt)
+            kv.append((k, v))
     torch.cuda.synchronize()
-    dec = mynn.Decoder(cfg, weights, batch=B, kv=kv)
+    dec = mynn.Decoder(cfg, weights, batch=B, kv=kv, quant_kv_cache=args.kv_int8)
     stats = dec.stats()
     rng = np.random.default_rng(args.seed)
     toks = rng.integers(0, cfg["vocab"], B).tolist()
@@ -278,7 +291,8 @@ def decode_batch_main(args, mynn):
     H, F, V = cfg["hidden"], cfg["ffn"], cfg["vocab"]
     QD, KD = cfg["n_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
     w_bytes = cfg["n_layers"] * (QD * H + 2 * KD * H + H * QD + 3 * F * H) + V * H
-    kv_bytes = cfg["n_layers"] * B * 2 * KD * eb * (ctx + W + K // 2)
+    kv_row = KD + cfg["n_kv_heads"] * eb if args.kv_int8 else KD * eb  # bytes of one token's k (or v) over all kv heads
+    kv_bytes = cfg["n_layers"] * B * 2 * kv_row * (ctx + W + K // 2)
     step_bytes = w_bytes + kv_bytes
     lin = {k: v for k, v in agg.items() if k.startswith("linear_")}
     dom = max(lin, key=lambda k: lin[k][1])
@@ -288,9 +302,10 @@ def decode_batch_main(args, mynn):
         "metric": "decode tok/s, batch 32 at context 2048, Llama-3-8B-shape int8 (aggregate over the batch)",
         "value": round(B * K / elapsed, 1), "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32 accumulate over int8 weights, %s activations/KV" % args.dtype, "data": "synthetic",
+        "dtype": "f32 accumulate over int8 weights, %s activations, %s KV" % (args.dtype, "int8" if args.kv_int8 else args.dtype),
+        "data": "synthetic",
         "config": {"workload": "configs[4]: Llama-3-8B-shape int8 decoder, batch 32, context 2048 (caches filled with "
-                               "random rows), %d decode steps timed" % K,
+                               "random rows%s), %d decode steps timed" % (", int8 KV cache" if args.kv_int8 else "", K),
                    "batch": B, "context": ctx, "launches_per_step": stats["launches_per_step"], "hipgraph": stats["graph"],
                    "seed": args.seed, "step_algorithmic_bytes": step_bytes,
                    "step_hbm_frac": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
@@ -316,6 +331,8 @@ def main():
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="first run one 256 MiB device-to-device copy (a kernel of known traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--kv-int8", action="store_true",
+                    help="decode_batch: int8 KV cache with per-token scales (BuildOptions::quant_kv_cache)")
     ap.add_argument("--check-tokens", type=int, default=0,
                     help="also compare the first N greedy tokens with the oracle (slow: CPU decode)")
     args = ap.parse_args()

@@ -39,8 +39,8 @@ inline void attn_token_major_layout(AttnParams &p, int D) {
     p.q_rs = p.o_rs = (long)p.Hq * D;
 }
 
-void attn_plan(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, bool fused, int *slice,
-               int *nsplit, int *heads_per_wg);
+void attn_plan(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, int cache_len, bool fused,
+               int *slice, int *nsplit, int *heads_per_wg);
 bool attention_fused_supported(int D, int G);
 size_t attn_scratch_bytes(int B, int Hq, int Sq, int D, int nsplit);
 size_t attn_counter_bytes(int B, int Hq, int Sq);
@@ -48,9 +48,9 @@ int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *s
 int attention_prefill_launch(const AttnParams &p, int D, int dtype, hipStream_t s);
 bool attention_prefill_supported(const AttnParams &p, int D, int dtype, int kv_int8);
 // streaming decode kernel (attention_stream.hip): taken when eligible; attn_plan then returns its plan
-bool attn_stream_eligible(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len);
+bool attn_stream_eligible(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, int cache_len);
 void attn_stream_plan(int B, int Hkv, int kv_len, int *slice, int *nsplit);
-int attention_stream_launch(const AttnParams &p, int D, int dtype, hipStream_t s);
+int attention_stream_launch(const AttnParams &p, int D, int dtype, int kv_int8, hipStream_t s);
 // out = merge of the nsplit partial results in p.part_o / p.part_ml (its own launch)
 int attention_merge_launch(const AttnParams &p, int D, int dtype, hipStream_t s);
 

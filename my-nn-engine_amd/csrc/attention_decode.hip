@@ -339,10 +339,10 @@ bool attention_fused_supported(int D, int G) {
 // Slice length, number of slices and query heads per workgroup for a launch.  kv_len = longest key
 // range any row can have.  All heads of a kv head share one workgroup (one K/V read) unless that
 // leaves fewer than ~64 workgroups; then the heads are divided, halving until there are enough.
-void attn_plan(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, bool fused, int *slice,
-               int *nsplit, int *heads_per_wg) {
+void attn_plan(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, int cache_len, bool fused,
+               int *slice, int *nsplit, int *heads_per_wg) {
     const int Gt = Hq / Hkv;
-    if (!fused && attn_stream_eligible(B, Sq, Hq, Hkv, D, dtype, kv_int8, kv_len)) {
+    if (!fused && attn_stream_eligible(B, Sq, Hq, Hkv, D, dtype, kv_int8, kv_len, cache_len)) {
         attn_stream_plan(B, Hkv, kv_len, slice, nsplit);
         *heads_per_wg = Gt;
         return;
@@ -379,8 +379,8 @@ int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *s
     const bool fuse = p.qkv != nullptr;
     // the plan (attn_plan, with the same kv_len) was made for the streaming kernel when it is eligible
     const int kv_len = p.d_active ? p.cache_len : (p.active < p.cache_len ? p.active : p.cache_len);
-    if (!fuse && attn_stream_eligible(p.B, p.Sq, p.Hq, p.Hkv, D, dtype, kv_int8, kv_len))
-        return attention_stream_launch(p, D, dtype, s);
+    if (!fuse && attn_stream_eligible(p.B, p.Sq, p.Hq, p.Hkv, D, dtype, kv_int8, kv_len, p.cache_len))
+        return attention_stream_launch(p, D, dtype, kv_int8, s);
     int rc = dispatch_dtype(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
         if constexpr (sizeof(T) == 2) {
@@ -444,7 +444,8 @@ extern "C" int mynn_attention(void *out, const void *Q, const void *K, const voi
     if (Sq > 1 && attention_prefill_supported(p, head_dim, dtype, kv_int8))
         return attention_prefill_launch(p, head_dim, dtype, st);
     int kv_len = d_active ? cache_seq_len : (active_seq_kv < cache_seq_len ? active_seq_kv : cache_seq_len);
-    attn_plan(B, Sq, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, kv_len, false, &p.slice, &p.nsplit, &p.heads_per_wg);
+    attn_plan(B, Sq, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, kv_len, cache_seq_len, false, &p.slice, &p.nsplit,
+              &p.heads_per_wg);
     MYNN_REQUIRE(p.nsplit <= 65535, MYNN_ERR_UNSUPPORTED, "attention: cache of %d rows needs too many slices", kv_len);
     if (p.nsplit > 1) {
         int rc = ensure(g_scratch, attn_scratch_bytes(B, num_q_heads, Sq, head_dim, p.nsplit), false, st);

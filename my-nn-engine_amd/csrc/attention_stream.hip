@@ -1,5 +1,5 @@
 // Streaming GQA decode attention for large (batch x context) products: one query row per sequence,
-// 16-bit K/V, head_dim 64 or 128, up to 8 query heads per kv head.
+// 16-bit or int8 (per-token scales) K/V, head_dim 64 or 128, up to 8 query heads per kv head.
 //
 // attention_decode.hip is built for latency (one pass, everything in flight at once, one workgroup
 // per CU); with tens of megabytes of K/V per launch the job is bandwidth instead, and this kernel
@@ -38,7 +38,9 @@ template <> struct Mfma16<bf16_t> {
 
 constexpr int kStreamWaves = 4, kStreamThreads = kStreamWaves * 64, kStreamTile = 32;
 
-template <typename T, int D, int G>
+// KVI8: int8 caches with one scale per token row (QuantizingKVCacheUpdate): K and V are widened exactly to
+// the 16-bit type in registers, the key's k scale multiplies its score and its v scale its p.
+template <typename T, int D, int G, bool KVI8>
 __global__ __launch_bounds__(kStreamThreads) void attn_stream_kernel(AttnParams p) {
     constexpr int KB = D / 32;              // 32-dim blocks of a key row
     constexpr int LPK = D / 8;              // lanes per key row when a tile is loaded 16 bytes per lane
@@ -65,7 +67,14 @@ __global__ __launch_bounds__(kStreamThreads) void attn_stream_kernel(AttnParams 
     const int bound = min(active, p.cache_len);
     const int k0 = split * p.slice, k1 = min(bound, k0 + p.slice);
     const size_t kv_base = (size_t)bhkv * p.cache_len;
-    const T *Kp = (const T *)p.k + kv_base * D, *Vp = (const T *)p.v + kv_base * D;
+    using TKV = typename std::conditional<KVI8, int8_t, T>::type;
+    using Chunk = typename std::conditional<KVI8, uint2, U4>::type;  // 8 elements of a cached row
+    const TKV *Kp = (const TKV *)p.k + kv_base * D, *Vp = (const TKV *)p.v + kv_base * D;
+    const T *ksc = (const T *)p.k_scale + kv_base, *vsc = (const T *)p.v_scale + kv_base;  // KVI8 only
+    auto operand = [](const Chunk &c) -> U4 {
+        if constexpr (KVI8) return i8x8_to_operand<T>(c.x, c.y);
+        else return c;
+    };
     const int col = lane & 15, quad = lane >> 4;  // MFMA column (head) and row/k group of this lane
 
     // Q^T as the B operand of the score product: column = head, k = dims 8*quad..+7 of each block
@@ -89,29 +98,45 @@ __global__ __launch_bounds__(kStreamThreads) void attn_stream_kernel(AttnParams 
         for (int par = 0; par < 2; par++) acc[c][par] = f4_t{0.f, 0.f, 0.f, 0.f};
 
     const int vk = lane / LPK, vd = (lane % LPK) * 8;  // V load: key row within a pass, dim offset
-    auto load_tile = [&](int t0, U4 (*kr)[KB], U4 *vr) {
+    // (KVI8: the scales of the lane's 2 x 4 score keys travel with the tile, 8 bytes per load; the cache
+    // length is a multiple of 32 there, so a tile never reaches past its row of scales)
+    auto load_tile = [&](int t0, Chunk (*kr)[KB], Chunk *vr, uint2 *sr) {
+        if constexpr (KVI8) {
+#pragma unroll
+            for (int a = 0; a < 2; a++) {
+                sr[a] = *(const uint2 *)(ksc + t0 + a * 16 + quad * 4);
+                sr[2 + a] = *(const uint2 *)(vsc + t0 + a * 16 + quad * 4);
+            }
+        }
         // rows past the range re-read the last valid row; their scores are masked below
 #pragma unroll
         for (int a = 0; a < 2; a++) {
             const int krow = min(t0 + a * 16 + col, k1 - 1);
 #pragma unroll
-            for (int j = 0; j < KB; j++) kr[a][j] = *(const U4 *)(Kp + (size_t)krow * D + j * 32 + quad * 8);
+            for (int j = 0; j < KB; j++) kr[a][j] = *(const Chunk *)(Kp + (size_t)krow * D + j * 32 + quad * 8);
         }
 #pragma unroll
         for (int q = 0; q < NP; q++) {
             const int vrow = min(t0 + q * KPP + vk, k1 - 1);
-            vr[q] = *(const U4 *)(Vp + (size_t)vrow * D + vd);
+            vr[q] = *(const Chunk *)(Vp + (size_t)vrow * D + vd);
         }
     };
 
     uint16_t *vt = v_s[wave], *pt = p_s[wave];
-    auto process = [&](int t, const U4 (*kr)[KB], const U4 *vr) {
+    auto scale_of = [](const uint2 &four, int e) -> float {  // element e of four packed storage-type values
+        const uint32_t w = e < 2 ? four.x : four.y;
+        const uint16_t b = (uint16_t)((e & 1) ? w >> 16 : w & 0xFFFFu);
+        T v = __builtin_bit_cast(T, b);
+        return Elem<T>::ld(&v, 0);
+    };
+    auto process = [&](int t, const Chunk (*kr)[KB], const Chunk *vr, const uint2 *sr) {
         // ---- park V: [key][dim], two 8-byte stores per lane and pass
 #pragma unroll
         for (int q = 0; q < NP; q++) {
             uint2 *dst = (uint2 *)&vt[(q * KPP + vk) * VST + vd];
-            dst[0] = uint2{vr[q].x, vr[q].y};
-            dst[1] = uint2{vr[q].z, vr[q].w};
+            const U4 v = operand(vr[q]);
+            dst[0] = uint2{v.x, v.y};
+            dst[1] = uint2{v.z, v.w};
         }
         // ---- scores: lane = head col, keys 16a + 4*quad + e
         float sv[2][4], tmax = -INFINITY;
@@ -119,11 +144,13 @@ __global__ __launch_bounds__(kStreamThreads) void attn_stream_kernel(AttnParams 
         for (int a = 0; a < 2; a++) {
             f4_t s4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int j = 0; j < KB; j++) s4 = Mfma16<T>::run(kr[a][j], qf[j], s4);
+            for (int j = 0; j < KB; j++) s4 = Mfma16<T>::run(operand(kr[a][j]), qf[j], s4);
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int key = t + a * 16 + quad * 4 + e;
-                sv[a][e] = key < k1 ? s4[e] * p.scale : -INFINITY;
+                float sc = s4[e];
+                if constexpr (KVI8) sc *= scale_of(sr[a], e);
+                sv[a][e] = key < k1 ? sc * p.scale : -INFINITY;
                 tmax = fmaxf(tmax, sv[a][e]);
             }
         }
@@ -140,6 +167,7 @@ __global__ __launch_bounds__(kStreamThreads) void attn_stream_kernel(AttnParams 
             for (int e = 0; e < 4; e++) {
                 pe[e] = fast_exp(sv[a][e] - m_new);  // 0 for keys past the range
                 psum += pe[e];
+                if constexpr (KVI8) pe[e] = t + a * 16 + quad * 4 + e < k1 ? pe[e] * scale_of(sr[2 + a], e) : 0.f;
             }
             // p[head][16a + 4*quad .. +3] in the storage type
             *(uint2 *)&pt[col * PST + a * 16 + quad * 4] =
@@ -186,18 +214,19 @@ __global__ __launch_bounds__(kStreamThreads) void attn_stream_kernel(AttnParams 
     // two register sets, named so that the wait for one never covers the other; the load of the tile
     // after next is issued unconditionally (rows clamp to the last valid one) to keep the loop free of
     // branches around loads
-    U4 kA[2][KB], vA[NP], kB[2][KB], vB[NP];
+    Chunk kA[2][KB], vA[NP], kB[2][KB], vB[NP];
+    uint2 sA[4], sB[4];
     const int tstep = kStreamWaves * kStreamTile;
     int t = k0 + wave * kStreamTile;
     if (t < k1) {
-        load_tile(t, kA, vA);
+        load_tile(t, kA, vA, sA);
         while (true) {
-            load_tile(t + tstep, kB, vB);
-            process(t, kA, vA);
+            load_tile(min(t + tstep, p.cache_len - kStreamTile), kB, vB, sB);
+            process(t, kA, vA, sA);
             t += tstep;
             if (t >= k1) break;
-            load_tile(t + tstep, kA, vA);
-            process(t, kB, vB);
+            load_tile(min(t + tstep, p.cache_len - kStreamTile), kA, vA, sA);
+            process(t, kB, vB, sB);
             t += tstep;
             if (t >= k1) break;
         }
@@ -287,10 +316,10 @@ int attention_merge_launch(const AttnParams &p, int D, int dtype, hipStream_t s)
 }
 
 // ---- host side ---------------------------------------------------------------------------------
-bool attn_stream_eligible(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len) {
+bool attn_stream_eligible(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, int cache_len) {
     const int G = Hq / Hkv;
-    return Sq == 1 && !kv_int8 && dtype != MYNN_F32 && (D == 64 || D == 128) && (G == 1 || G == 2 || G == 4 || G == 8) &&
-           (long)B * Hkv * kv_len >= 32768;
+    return Sq == 1 && dtype != MYNN_F32 && (!kv_int8 || cache_len % kStreamTile == 0) && (D == 64 || D == 128) &&
+           (G == 1 || G == 2 || G == 4 || G == 8) && (long)B * Hkv * kv_len >= 32768;
 }
 
 // key rows per workgroup and number of key ranges: as many workgroups as the device holds at once
@@ -316,20 +345,22 @@ void attn_stream_plan(int B, int Hkv, int kv_len, int *slice, int *nsplit) {
     *nsplit = (kv_len + rows - 1) / rows;
 }
 
-template <typename T, int D>
+template <typename T, int D, bool KVI8>
 static int stream_g(const AttnParams &p, hipStream_t s) {
     dim3 grid(p.B * p.Hkv, p.nsplit), block(kStreamThreads);
     switch (p.Hq / p.Hkv) {
-    case 1: MYNN_LAUNCH((attn_stream_kernel<T, D, 1>), grid, block, 0, s, p); break;
-    case 2: MYNN_LAUNCH((attn_stream_kernel<T, D, 2>), grid, block, 0, s, p); break;
-    case 4: MYNN_LAUNCH((attn_stream_kernel<T, D, 4>), grid, block, 0, s, p); break;
-    case 8: MYNN_LAUNCH((attn_stream_kernel<T, D, 8>), grid, block, 0, s, p); break;
+    case 1: MYNN_LAUNCH((attn_stream_kernel<T, D, 1, KVI8>), grid, block, 0, s, p); break;
+    case 2: MYNN_LAUNCH((attn_stream_kernel<T, D, 2, KVI8>), grid, block, 0, s, p); break;
+    case 4: MYNN_LAUNCH((attn_stream_kernel<T, D, 4, KVI8>), grid, block, 0, s, p); break;
+    case 8: MYNN_LAUNCH((attn_stream_kernel<T, D, 8, KVI8>), grid, block, 0, s, p); break;
     default: return fail(MYNN_ERR_UNSUPPORTED, "streaming attention: %d query heads per kv head", p.Hq / p.Hkv);
     }
     return launch_status("attn_stream_kernel");
 }
 
-int attention_stream_launch(const AttnParams &p, int D, int dtype, hipStream_t s) {
+int attention_stream_launch(const AttnParams &p, int D, int dtype, int kv_int8, hipStream_t s) {
+    MYNN_REQUIRE(!kv_int8 || (p.k_scale && p.v_scale && p.cache_len % kStreamTile == 0), MYNN_ERR_INVALID,
+                 "streaming attention: int8 KV needs scales and a cache length that is a multiple of %d", kStreamTile);
     MYNN_REQUIRE(p.q_rs >= 0 && aligned16(p.q) && aligned16(p.k) && aligned16(p.v) && p.q_bs % 8 == 0 && p.q_hs % 8 == 0,
                  MYNN_ERR_INVALID, "streaming attention: q, k, v must be 16-byte aligned");
     MYNN_REQUIRE(p.nsplit == 1 || (p.part_o && p.part_ml), MYNN_ERR_INVALID,
@@ -337,8 +368,13 @@ int attention_stream_launch(const AttnParams &p, int D, int dtype, hipStream_t s
     MYNN_REQUIRE(p.slice % (kStreamWaves * kStreamTile) == 0 && p.nsplit <= 65535, MYNN_ERR_INVALID,
                  "streaming attention: slice %d, %d ranges", p.slice, p.nsplit);
     int rc;
-    if (dtype == MYNN_F16) rc = D == 64 ? stream_g<f16_t, 64>(p, s) : stream_g<f16_t, 128>(p, s);
-    else rc = D == 64 ? stream_g<bf16_t, 64>(p, s) : stream_g<bf16_t, 128>(p, s);
+    if (kv_int8) {
+        if (dtype == MYNN_F16) rc = D == 64 ? stream_g<f16_t, 64, true>(p, s) : stream_g<f16_t, 128, true>(p, s);
+        else rc = D == 64 ? stream_g<bf16_t, 64, true>(p, s) : stream_g<bf16_t, 128, true>(p, s);
+    } else {
+        if (dtype == MYNN_F16) rc = D == 64 ? stream_g<f16_t, 64, false>(p, s) : stream_g<f16_t, 128, false>(p, s);
+        else rc = D == 64 ? stream_g<bf16_t, 64, false>(p, s) : stream_g<bf16_t, 128, false>(p, s);
+    }
     if (rc || p.nsplit == 1) return rc;
     return attention_merge_launch(p, D, dtype, s);
 }

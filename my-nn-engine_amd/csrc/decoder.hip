@@ -463,7 +463,7 @@ static int build(Model &m, void **init, void **state) {
     {
         const bool fused_attn = m.quant && rows == 1 && !c.quantize_activations && !c.quant_kv_cache &&
                                 attention_fused_supported(c.head_dim, c.n_heads / c.n_kv_heads);
-        attn_plan(c.batch, c.seq_q, c.n_heads, c.n_kv_heads, c.head_dim, c.dtype, c.quant_kv_cache, c.max_seq, fused_attn,
+        attn_plan(c.batch, c.seq_q, c.n_heads, c.n_kv_heads, c.head_dim, c.dtype, c.quant_kv_cache, c.max_seq, c.max_seq, fused_attn,
                   &m.slice, &m.nsplit, &m.heads_per_wg);
     }
     m.token_cap = c.max_seq + 8;

@@ -20,29 +20,6 @@
 
 namespace mynn {
 
-typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
-
-// 8 int8 (two dwords) -> 8 values of T packed in a U4; exact
-template <typename T> __device__ inline U4 i8x8_to_operand(uint32_t w0, uint32_t w1) {
-    if constexpr (std::is_same<T, f16_t>::value) {
-        // byte b + 128 under an 0x64 high byte is the fp16 number 1024 + (b + 128); subtract 1152
-        const h2_t bias = {(_Float16)1152.f, (_Float16)1152.f};
-        const uint32_t x0 = w0 ^ 0x80808080u, x1 = w1 ^ 0x80808080u;
-        auto two = [&](uint32_t x, uint32_t sel) {
-            const h2_t h = __builtin_bit_cast(h2_t, __builtin_amdgcn_perm(0x64646464u, x, sel)) - bias;
-            return __builtin_bit_cast(uint32_t, h);
-        };
-        return U4{two(x0, 0x04010400u), two(x0, 0x04030402u), two(x1, 0x04010400u), two(x1, 0x04030402u)};
-    } else {
-        // |b| <= 128 has at most 8 significant bits: the upper half of its f32 form is the bf16 value
-        auto two = [&](uint32_t w, int sh) {
-            const float a = (float)(int8_t)((w >> sh) & 0xFF), b = (float)(int8_t)((w >> (sh + 8)) & 0xFF);
-            return __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, b), __builtin_bit_cast(uint32_t, a), 0x07060302u);
-        };
-        return U4{two(w0, 0), two(w0, 16), two(w1, 0), two(w1, 16)};
-    }
-}
-
 constexpr int kSkinnyWaves = 4, kSkinnyThreads = kSkinnyWaves * 64, kSkinnyK = 128, kSkinnyStages = 5;
 
 constexpr int kSkinnyLd = kSkinnyK + 8;  // LDS row stride of the activation chunk (272 bytes: conflict-free 128-bit reads)

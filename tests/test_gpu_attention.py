@@ -188,6 +188,29 @@ def test_int8_kv_attention(g, dt):
 
 
 @pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+@pytest.mark.parametrize("B,Hq,Hkv,D,L,active", [(16, 32, 4, 64, 700, 613), (8, 32, 8, 128, 1100, 1037)])
+def test_streaming_decode_attention_int8_kv(g, dt, B, Hq, Hkv, D, L, active):
+    """The streaming kernel over an int8 cache with per-token scales (k scale on the score, v scale on p),
+    rows beyond the active length poisoned with the most negative code and a NaN scale."""
+    rng = np.random.default_rng(active + D)
+    q = orc.to_storage(rng.standard_normal((B, Hq, 1, D)), dt)
+    kc = np.zeros((B, Hkv, L, D), np.int8)
+    vc = np.zeros((B, Hkv, L, D), np.int8)
+    ks = orc.to_storage(np.zeros((B, Hkv, L)), dt)
+    vs = orc.to_storage(np.zeros((B, Hkv, L)), dt)
+    orc.quantizing_kv_cache_update(kc, ks, orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt), 0, dt)
+    orc.quantizing_kv_cache_update(vc, vs, orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt), 0, dt)
+    kc[:, :, active:] = -128
+    vc[:, :, active:] = -128
+    ks[:, :, active:] = orc.to_storage(np.full((B, Hkv, L - active), np.nan), dt)
+    vs[:, :, active:] = orc.to_storage(np.full((B, Hkv, L - active), np.nan), dt)
+    want = orc.attention(q, kc, vc, dt, D ** -0.5, False, active, k_scale=ks, v_scale=vs)
+    got = g.to_host(g.mynn.attention(g.to_dev(q, dt), g.to_dev(kc), g.to_dev(vc), D ** -0.5, False, active,
+                                     k_scale=g.to_dev(ks, dt), v_scale=g.to_dev(vs, dt)))
+    assert max_abs_rel(g.f32(got, dt), g.f32(want, dt)) <= 1e-2
+
+
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
 @pytest.mark.parametrize("B,Hq,Hkv,S,D,past,causal", [
     (1, 8, 2, 128, 64, 0, True),
     (2, 4, 4, 100, 64, 0, True),      # ragged: rows past the last 128-row block, MHA
