@@ -22,7 +22,6 @@ struct AttnParams {
     const int64_t *d_pos;
     float *part_o;            // [B*Hq*Sq, nsplit, D]
     float *part_ml;           // [B*Hq*Sq, nsplit, 2]
-    unsigned *counters;       // [B*Hkv*Sq], zero between launches
     // element strides of Q and out: batch, head, row.  Reference layout [B,Hq,Sq,D] is
     // (Hq*Sq*D, Sq*D, D); token-major [B,Sq,Hq*D] is (Sq*Hq*D, D, Hq*D).
     long q_bs, q_hs, q_rs, o_bs, o_hs, o_rs;
@@ -43,8 +42,7 @@ void attn_plan(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, in
                int *slice, int *nsplit, int *heads_per_wg);
 bool attention_fused_supported(int D, int G);
 size_t attn_scratch_bytes(int B, int Hq, int Sq, int D, int nsplit);
-size_t attn_counter_bytes(int B, int Hq, int Sq);
-int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *scratch, void *counters, hipStream_t s);
+int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *scratch, hipStream_t s);
 int attention_prefill_launch(const AttnParams &p, int D, int dtype, hipStream_t s);
 bool attention_prefill_supported(const AttnParams &p, int D, int dtype, int kv_int8);
 // streaming decode kernel (attention_stream.hip): taken when eligible; attn_plan then returns its plan

@@ -362,19 +362,12 @@ size_t attn_scratch_bytes(int B, int Hq, int Sq, int D, int nsplit) {
     size_t bytes = rows * nsplit * (D + 2) * sizeof(float);
     return (bytes + 255) / 256 * 256;
 }
-size_t attn_counter_bytes(int B, int Hq, int Sq) {
-    // one per (batch, kv head, part, row); at most one part per query head
-    return ((size_t)B * Hq * Sq * sizeof(unsigned) + 255) / 256 * 256;
-}
-
-// scratch = [part_o | part_ml] (contents need not survive); `counters` is unused (kept for callers)
-int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *scratch, void *counters,
-                            hipStream_t s) {
+// scratch = [part_o | part_ml] of attn_scratch_bytes (contents need not survive the call)
+int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *scratch, hipStream_t s) {
     if (p.nsplit > 1) {
         size_t rows = (size_t)p.B * p.Hq * p.Sq;
         p.part_o = (float *)scratch;
         p.part_ml = p.part_o + rows * p.nsplit * D;
-        p.counters = (unsigned *)counters;
     }
     const bool fuse = p.qkv != nullptr;
     // the plan (attn_plan, with the same kv_len) was made for the streaming kernel when it is eligible
@@ -397,14 +390,12 @@ int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *s
     return attention_merge_launch(p, D, dtype, s);
 }
 
-// ---- library-owned scratch for the op-level entry point: grown on demand.  The counters live
-// in their own allocation so that partial results of an earlier, differently shaped call can
-// never be mistaken for a count.
+// ---- library-owned scratch for the op-level entry point: grown on demand
 struct Grown {
     void *ptr = nullptr;
     size_t bytes = 0;
 };
-static Grown g_scratch, g_counters;
+static Grown g_scratch;
 static int ensure(Grown &g, size_t bytes, bool zero, hipStream_t s) {
     if (bytes <= g.bytes) return 0;
     MYNN_HIP(hipStreamSynchronize(s));
@@ -450,8 +441,6 @@ extern "C" int mynn_attention(void *out, const void *Q, const void *K, const voi
     if (p.nsplit > 1) {
         int rc = ensure(g_scratch, attn_scratch_bytes(B, num_q_heads, Sq, head_dim, p.nsplit), false, st);
         if (rc) return rc;
-        rc = ensure(g_counters, attn_counter_bytes(B, num_q_heads, Sq), true, st);
-        if (rc) return rc;
     }
-    return attention_decode_launch(p, head_dim, dtype, kv_int8, g_scratch.ptr, g_counters.ptr, st);
+    return attention_decode_launch(p, head_dim, dtype, kv_int8, g_scratch.ptr, st);
 }

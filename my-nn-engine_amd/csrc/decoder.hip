@@ -86,7 +86,7 @@ struct Model {
     void *a8_scale = nullptr;  // and their per-row scales [rows]
     int64_t *d_ids = nullptr, *d_pos = nullptr;
     int32_t *d_past = nullptr, *d_active = nullptr, *d_next = nullptr, *d_tokens = nullptr, *d_step = nullptr;
-    void *attn_scratch = nullptr, *attn_counters = nullptr;
+    void *attn_scratch = nullptr;
     int nsplit = 1, slice = 0, heads_per_wg = 1;
     int token_cap = 0;
     // host staging (pinned)
@@ -239,7 +239,7 @@ static int enqueue_step(Model &m) {
                 // RoPE(q), RoPE(k), both cache appends and the attention in one launch
                 p.qkv = m.qkv; p.cos_t = m.cos_t; p.sin_t = m.sin_t; p.d_pos = m.d_pos;
                 note(m, "attention_rope_append", (double)(QD + 2 * KD) * eb + 2.0 * KD * eb + QD * eb);
-                TRY(attention_decode_launch(p, D, c.dtype, 0, m.attn_scratch, m.attn_counters, s));
+                TRY(attention_decode_launch(p, D, c.dtype, 0, m.attn_scratch, s));
             } else {
                 note(m, kv8 ? "rope_quant_kv_append" : "rope_kv_append", (double)rows * (QD + 2 * KD) * 2 * eb);
                 if (kv8)
@@ -253,7 +253,7 @@ static int enqueue_step(Model &m) {
                 // flops: the causal half of QK^T and PV over the new rows alone (exact when past_len is 0)
                 note(m, "attention", (double)rows * 2.0 * QD * eb, S > 1 ? 2.0 * B * Hq * D * (double)S * (S + 1) : 0.0);
                 if (S > 1 && attention_prefill_supported(p, D, c.dtype, kv8)) TRY(attention_prefill_launch(p, D, c.dtype, s));
-                else TRY(attention_decode_launch(p, D, c.dtype, kv8, m.attn_scratch, m.attn_counters, s));
+                else TRY(attention_decode_launch(p, D, c.dtype, kv8, m.attn_scratch, s));
             }
         }
         if (fused) {
@@ -487,7 +487,6 @@ static int build(Model &m, void **init, void **state) {
     size_t o_ids = plan.take((size_t)rows * 8), o_pos = plan.take((size_t)c.seq_q * 8);
     size_t o_sc = plan.take(256), o_tok = plan.take((size_t)m.token_cap * 4);
     size_t o_as = plan.take(attn_scratch_bytes(c.batch, c.n_heads, c.seq_q, c.head_dim, m.nsplit));
-    size_t o_ac = plan.take(attn_counter_bytes(c.batch, c.n_heads, c.seq_q));
     m.arena_bytes = plan.off;
     MYNN_HIP(hipMalloc((void **)&m.arena, m.arena_bytes));
     MYNN_HIP(hipMemset(m.arena, 0, m.arena_bytes));
@@ -501,7 +500,7 @@ static int build(Model &m, void **init, void **state) {
     m.d_next = m.d_past + 8;  // up to 56 sequences' tokens after the scalars
     MYNN_REQUIRE(c.batch <= 56, MYNN_ERR_UNSUPPORTED, "batch %d > 56", c.batch);
     m.d_tokens = (int32_t *)(m.arena + o_tok);
-    m.attn_scratch = m.arena + o_as; m.attn_counters = m.arena + o_ac;
+    m.attn_scratch = m.arena + o_as;
     m.stage_bytes = align_up((size_t)rows * 8 + (size_t)c.seq_q * 8 + 64 + (size_t)m.token_cap * 4, 256) + 512;
     MYNN_HIP(hipHostMalloc((void **)&m.h_stage, m.stage_bytes, hipHostMallocDefault));
     MYNN_HIP(hipDeviceSynchronize());
