@@ -84,6 +84,77 @@ __device__ inline void tile_of(int b, int nblocks, int tiles_m, int tiles_n, int
     tn = in_band / rows_here;
 }
 
+// ---- store of a workgroup tile.  The MFMAs take the weight fragment as their first operand, so an
+// accumulator tile is the transpose of the output tile: lane l holds output row l % 32 and, in elements
+// 4q..4q+3, the four neighbouring output columns 8q + 4*(l/32) + 0..3 -- one 8-byte piece of a row.  Each
+// wave turns one 32-row strip of its tile at a time into row-major 16-bit values in its own LDS patch (the
+// operand buffers are free by now) and writes it out, and reads the residual, 16 bytes per lane, rows
+// contiguous.
+template <typename T, typename G, int EPI>
+__device__ __forceinline__ void gemm_store(f16x_t (&acc)[G::TI][G::TJ], uint16_t *lds, T *C, const T *R, int M, int N, int m0,
+                                           int n0, int wrow, int wcol, int lane, int wave) {
+    constexpr int TI = G::TI, TJ = G::TJ;
+    constexpr int EST = G::EST;
+    constexpr int OC = EPI == GEMM_SWIGLU ? TJ * 16 : TJ * 32;  // output columns of the wave tile
+    constexpr int CPR = OC / 8;                                 // 16-byte chunks per strip row
+    const int ldc = EPI == GEMM_SWIGLU ? N >> 1 : N;
+    const int c0 = EPI == GEMM_SWIGLU ? (n0 + wcol) >> 1 : n0 + wcol;
+    T *patch = (T *)lds + (size_t)wave * 32 * EST;
+    const bool vec_ok = (ldc & 7) == 0;
+#pragma unroll
+    for (int i = 0; i < TI; i++) {
+        T *prow = patch + (lane & 31) * EST + (lane >> 5) * 4;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            if (EPI == GEMM_SWIGLU) {
+#pragma unroll
+                for (int j = 0; j < TJ; j += 2) {
+                    float o[4];
+#pragma unroll
+                    for (int x = 0; x < 4; x++) {
+                        const float g = Elem<T>::rnd(acc[i][j][4 * q + x]), u = Elem<T>::rnd(acc[i][j + 1][4 * q + x]);
+                        const float sig = 1.0f / (1.0f + expf(-g));
+                        o[x] = (g * sig) * u;
+                    }
+                    *(uint2 *)(prow + j * 16 + 8 * q) = uint2{pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3])};
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < TJ; j++)
+                    *(uint2 *)(prow + j * 32 + 8 * q) = uint2{pack2<T>(acc[i][j][4 * q], acc[i][j][4 * q + 1]),
+                                                              pack2<T>(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3])};
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        const int row0 = m0 + wrow + i * 32;
+#pragma unroll
+        for (int q = 0; q < 32 * CPR / 64; q++) {
+            const int ch = q * 64 + lane, r = ch / CPR, cc = (ch % CPR) * 8;
+            const int row = row0 + r, col = c0 + cc;
+            if (row >= M || col >= ldc) continue;
+            U4 v = *(const U4 *)&patch[r * EST + cc];
+            const size_t at = (size_t)row * ldc + col;
+            if (vec_ok && col + 8 <= ldc) {
+                if (EPI == GEMM_RESIDUAL) {
+                    float fv[8], fr8[8];
+                    widen8<T>(v, fv);
+                    widen8<T>(*(const U4 *)(R + at), fr8);
+                    v = U4{pack2<T>(fr8[0] + fv[0], fr8[1] + fv[1]), pack2<T>(fr8[2] + fv[2], fr8[3] + fv[3]),
+                           pack2<T>(fr8[4] + fv[4], fr8[5] + fv[5]), pack2<T>(fr8[6] + fv[6], fr8[7] + fv[7])};
+                }
+                *(U4 *)(C + at) = v;
+            } else {
+                for (int x = 0; x < 8 && col + x < ldc; x++) {
+                    const float f = Elem<T>::ld(patch, r * EST + cc + x);
+                    if (EPI == GEMM_RESIDUAL) Elem<T>::st(C, at + x, Elem<T>::ld(R, at + x) + f);
+                    else C[at + x] = patch[r * EST + cc + x];
+                }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
 // KTAIL: K is not a multiple of 2*BK, so the last steps mask the columns of A past K.
 // EPI: GEMM_PLAIN C = T(acc); GEMM_RESIDUAL C = T(R + T(acc)) with R laid out like C;
 // GEMM_SWIGLU: B's rows are gate/up interleaved in groups of 32, C is [M, N/2] and
@@ -149,7 +220,7 @@ __global__ __launch_bounds__(G::THREADS) void gemm_nt_mfma_kernel(T *C, const T 
 #pragma unroll
             for (int i = 0; i < TI; i++)
 #pragma unroll
-                for (int j = 0; j < TJ; j++) acc[i][j] = Mfma<T>::run(fa[i], fb[j], acc[i][j]);
+                for (int j = 0; j < TJ; j++) acc[i][j] = Mfma<T>::run(fb[j], fa[i], acc[i][j]);
         }
     };
 
@@ -171,61 +242,152 @@ __global__ __launch_bounds__(G::THREADS) void gemm_nt_mfma_kernel(T *C, const T 
         __syncthreads();
     }
 
-    // ---- store.  D[r][c] of a 32 x 32 tile sits in lane c + 32*((r/4)%2), element 4*(r/8) + r%4.
-    // Each wave turns one 32-row strip of its tile at a time into row-major 16-bit values in its own
-    // LDS patch and writes it out (and reads the residual) 16 bytes per lane, rows contiguous.
-    constexpr int EST = G::EST;
-    constexpr int OC = EPI == GEMM_SWIGLU ? TJ * 16 : TJ * 32;  // output columns of the wave tile
-    constexpr int CPR = OC / 8;                                 // 16-byte chunks per strip row
-    const int ldc = EPI == GEMM_SWIGLU ? N >> 1 : N;
-    const int c0 = EPI == GEMM_SWIGLU ? (n0 + wcol) >> 1 : n0 + wcol;
-    T *patch = (T *)lds + (size_t)wave * 32 * EST;
-    const bool vec_ok = (ldc & 7) == 0;
+    gemm_store<T, G, EPI>(acc, lds, C, R, M, N, m0, n0, wrow, wcol, lane, wave);
+}
+
+// ---- the same product with the operand tiles copied global -> LDS by the load unit itself
+// (global_load_lds_dwordx4: no register staging, no LDS store instructions).  A wave's load instruction
+// fills 1 KB of LDS lane by lane, so padding is impossible; instead the 16-byte chunks of a tile (8 per
+// row at K step 64) are placed at position 8*row + (chunk ^ ((row >> 1) & 7)), which keeps the chunks of a
+// row together (one full 128-byte line per row in global memory) and makes the 128-bit fragment reads
+// conflict-free.  Two LDS stages of 64 KB: the loads of tile kt+2 are issued as soon as everyone has
+// finished reading tile kt and fly during tile kt+1; one barrier per K tile, a bare s_barrier with explicit
+// counter waits.  Fragments of the next 16-k step are read while the current one multiplies.
+// 256 x 256 tile, 8 waves of 128 x 64.  Needs K % 64 == 0.
+using TileDma = GemmTile<256, 256, 2, 4>;
+constexpr int DBK = 64;
+constexpr int kDmaStage = 2 * 256 * DBK;  // elements per stage: A tile then B tile (64 KB)
+constexpr size_t kDmaLds = (size_t)2 * kDmaStage * 2;
+
+template <typename T, typename G, int EPI>
+__global__ __launch_bounds__(G::THREADS) void gemm_nt_dma_kernel(T *C, const T *A, const T *B, const T *R, int M, int N, int K,
+                                                                 int Kp) {
+    static_assert(G::BM == 256 && G::BN == 256, "tile");
+    constexpr int TI = G::TI, TJ = G::TJ, KS = DBK / 16;
+    constexpr int CH = 2048 / G::THREADS;  // 16-byte chunks per thread per operand tile
+    extern __shared__ __align__(16) uint16_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / G::WN, wn = wave % G::WN;
+    const int wrow = wm * TI * 32, wcol = wn * TJ * 32;
+    const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
+    int tm, tn;
+    tile_of(blockIdx.x, gridDim.x, tiles_m, tiles_n, tm, tn);
+    const int m0 = tm * 256, n0 = tn * 256;
+
+    // this lane's chunks of each operand tile: LDS position P = (CH*wave + i)*64 + lane
+    const T *asrc[CH], *bsrc[CH];
+#pragma unroll
+    for (int i = 0; i < CH; i++) {
+        const int P = (CH * wave + i) * 64 + lane, r = P >> 3, c = (P & 7) ^ ((r >> 1) & 7);
+        asrc[i] = A + (size_t)min(m0 + r, M - 1) * K + c * 8;
+        bsrc[i] = B + (size_t)min(n0 + r, N - 1) * Kp + c * 8;
+    }
+    auto issue = [&](int kt, int stage) {
+        uint16_t *dst = lds + stage * kDmaStage + (CH * wave) * 512;  // wave-uniform; the lane offset is implicit
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(asrc[i] + (size_t)kt * DBK),
+                                             (__attribute__((address_space(3))) void *)(dst + i * 512), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(bsrc[i] + (size_t)kt * DBK),
+                                             (__attribute__((address_space(3))) void *)(dst + 256 * DBK + i * 512), 16, 0, 0);
+        }
+    };
+
+    f16x_t acc[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; i++)
+#pragma unroll
+        for (int j = 0; j < TJ; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+
+    // fragment addresses (elements) inside a stage: row r, chunk c = 2*ks + g  ->  (8r + (c ^ swz)) * 8
+    const int fr = lane & 31, g = lane >> 5;
+    int arow8[TI], aswz[TI], brow8[TJ], bswz[TJ];
 #pragma unroll
     for (int i = 0; i < TI; i++) {
-#pragma unroll
-        for (int e = 0; e < 16; e++) {
-            const int r = (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-            if (EPI == GEMM_SWIGLU) {
-#pragma unroll
-                for (int j = 0; j < TJ; j += 2) {
-                    const float g = Elem<T>::rnd(acc[i][j][e]), u = Elem<T>::rnd(acc[i][j + 1][e]);
-                    const float sig = 1.0f / (1.0f + expf(-g));
-                    Elem<T>::st(patch, r * EST + j * 16 + (lane & 31), (g * sig) * u);
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < TJ; j++) Elem<T>::st(patch, r * EST + j * 32 + (lane & 31), acc[i][j][e]);
-            }
-        }
-        __builtin_amdgcn_wave_barrier();
-        const int row0 = m0 + wrow + i * 32;
-#pragma unroll
-        for (int q = 0; q < 32 * CPR / 64; q++) {
-            const int ch = q * 64 + lane, r = ch / CPR, cc = (ch % CPR) * 8;
-            const int row = row0 + r, col = c0 + cc;
-            if (row >= M || col >= ldc) continue;
-            U4 v = *(const U4 *)&patch[r * EST + cc];
-            const size_t at = (size_t)row * ldc + col;
-            if (vec_ok && col + 8 <= ldc) {
-                if (EPI == GEMM_RESIDUAL) {
-                    float fv[8], fr8[8];
-                    widen8<T>(v, fv);
-                    widen8<T>(*(const U4 *)(R + at), fr8);
-                    v = U4{pack2<T>(fr8[0] + fv[0], fr8[1] + fv[1]), pack2<T>(fr8[2] + fv[2], fr8[3] + fv[3]),
-                           pack2<T>(fr8[4] + fv[4], fr8[5] + fv[5]), pack2<T>(fr8[6] + fv[6], fr8[7] + fv[7])};
-                }
-                *(U4 *)(C + at) = v;
-            } else {
-                for (int x = 0; x < 8 && col + x < ldc; x++) {
-                    const float f = Elem<T>::ld(patch, r * EST + cc + x);
-                    if (EPI == GEMM_RESIDUAL) Elem<T>::st(C, at + x, Elem<T>::ld(R, at + x) + f);
-                    else C[at + x] = patch[r * EST + cc + x];
-                }
-            }
-        }
-        __builtin_amdgcn_wave_barrier();
+        const int r = wrow + i * 32 + fr;
+        arow8[i] = 64 * r;
+        aswz[i] = (r >> 1) & 7;
     }
+#pragma unroll
+    for (int j = 0; j < TJ; j++) {
+        const int r = wcol + j * 32 + fr;
+        brow8[j] = 256 * DBK + 64 * r;
+        bswz[j] = (r >> 1) & 7;
+    }
+    auto read_frags = [&](const uint16_t *st, int ks, U4 *fa, U4 *fb) {
+        const int c = 2 * ks + g;
+#pragma unroll
+        for (int i = 0; i < TI; i++) fa[i] = *(const U4 *)&st[arow8[i] + ((c ^ aswz[i]) << 3)];
+#pragma unroll
+        for (int j = 0; j < TJ; j++) fb[j] = *(const U4 *)&st[brow8[j] + ((c ^ bswz[j]) << 3)];
+    };
+
+    auto multiply = [&](const U4 *fa, const U4 *fb) {
+#pragma unroll
+        for (int i = 0; i < TI; i++)
+#pragma unroll
+            for (int j = 0; j < TJ; j++) acc[i][j] = Mfma<T>::run(fb[j], fa[i], acc[i][j]);
+    };
+
+    // Schedule of one K tile (4 steps of 16): steps 0..2 multiply while the fragments of the next step are
+    // read; then the one synchronisation point of the tile -- this wave's reads of the tile are complete
+    // and its share of the next tile has landed, so after the barrier the next tile is whole and the stage
+    // of this one is free; step 3 multiplies while the loads of tile kt+2 are issued into that stage and the
+    // first fragments of tile kt+1 are read.  Left alone the instruction scheduler sinks every LDS read to
+    // just before its first use and exposes the LDS latency once per step; the sched_group_barrier
+    // sequences pin the interleaving (one read or load, then its share of the MFMAs).
+    const int nk = K / DBK;
+    U4 fa[2][TI], fb[2][TJ];
+    issue(0, 0);
+    issue(min(1, nk - 1), 1);
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    read_frags(lds, 0, fa[0], fb[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int kt = 0; kt < nk; kt++) {
+        const uint16_t *st = lds + (kt & 1) * kDmaStage, *nx = lds + ((kt + 1) & 1) * kDmaStage;
+#pragma unroll
+        for (int ks = 0; ks + 1 < KS; ks++) {
+            read_frags(st, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+            multiply(fa[ks & 1], fb[ks & 1]);
+#pragma unroll
+            for (int n = 0; n < TI + TJ; n++) {  // reads early in the step, so the last has landed by its end
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, TI * TJ - (TI + TJ), 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(nx, 0, fa[0], fb[0]);     // (after the last tile: stale data, never used)
+        issue(min(kt + 2, nk - 1), kt & 1);  // (past the end: a repeat of the last tile, never read)
+        multiply(fa[(KS - 1) & 1], fb[(KS - 1) & 1]);
+        // LDS reads first (the compiler keeps them ahead of the LDS-writing loads anyway), two per MFMA,
+        // then the loads spread over the remaining MFMAs
+        constexpr int RD_MFMA = (TI + TJ) / 2, LD_MFMA = TI * TJ - RD_MFMA;
+#pragma unroll
+        for (int n = 0; n < RD_MFMA; n++) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+#pragma unroll
+        for (int n = 0; n < LD_MFMA; n++) {
+            __builtin_amdgcn_sched_group_barrier(0x010, (2 * CH + LD_MFMA - 1) / LD_MFMA, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // the repeat of the last tile too, before LDS is reused
+    __syncthreads();
+    gemm_store<T, G, EPI>(acc, lds, C, R, M, N, m0, n0, wrow, wcol, lane, wave);
 }
 
 // library-owned workspace for the dequantised weight of the call in flight (grown on demand)
@@ -275,17 +437,35 @@ static int gemm_launch_tile(void *out, const void *act, const void *wt, const vo
     return launch_status("gemm_nt_mfma_kernel");
 }
 
-static int g_gemm_tile_override = 0;  // 0 = heuristic, 1 = 256x128, 2 = 256x256 (tuning/tests)
+template <typename T, typename G, int EPI>
+static int gemm_launch_dma(void *out, const void *act, const void *wt, const void *res, int M, int N, int K, hipStream_t s) {
+    static bool lds_set = false;
+    if (!lds_set) {
+        MYNN_HIP(hipFuncSetAttribute((const void *)gemm_nt_dma_kernel<T, G, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)kDmaLds));
+        lds_set = true;
+    }
+    const int tiles = ((M + 255) / 256) * ((N + 255) / 256);
+    MYNN_LAUNCH((gemm_nt_dma_kernel<T, G, EPI>), dim3(tiles), dim3(G::THREADS), kDmaLds, s, (T *)out, (const T *)act,
+                (const T *)wt, (const T *)res, M, N, K, gemm_kp(K));
+    return launch_status("gemm_nt_dma_kernel");
+}
+
+static int g_gemm_tile_override = 0;  // 0 = heuristic, 1 = 256x128, 2 = 256x256 via registers, 3 = 256x256 direct to LDS
 void gemm_set_tile(int which) { g_gemm_tile_override = which; }
 
 template <typename T, int EPI>
 static int gemm_launch(void *out, const void *act, const void *wt, const void *res, int M, int N, int K, hipStream_t s) {
-    // the large tile needs fewer LDS reads per MFMA (measured 10-20% faster) but runs one workgroup per
-    // CU, so a grid that is neither a whole number of rounds over the 256 CUs nor several rounds deep
-    // leaves too many of them idle
+    // the large tile needs fewer LDS reads per MFMA (measured 10-25% faster) but runs one workgroup per CU:
+    // it is chosen once it fills the 256 CUs at least once (a partly filled second round still wins: the
+    // CUs left running clock higher)
     const long big_tiles = (long)((M + 255) / 256) * ((N + 255) / 256);
-    bool big = big_tiles >= 2 * 256 || big_tiles % 256 == 0;
+    bool big = big_tiles >= 256;
     if (g_gemm_tile_override) big = g_gemm_tile_override == 2;
+    // the direct-to-LDS kernel is the faster 256 x 256 one (measured +5..20%); it needs whole 64-wide K steps
+    const bool dma_ok = K % 64 == 0 && g_gemm_tile_override != 2;
+    if (g_gemm_tile_override == 3) big = dma_ok;
+    if (big && dma_ok) return gemm_launch_dma<T, TileDma, EPI>(out, act, wt, res, M, N, K, s);
     if (big) return gemm_launch_tile<T, Tile256x256, EPI>(out, act, wt, res, M, N, K, s);
     return gemm_launch_tile<T, Tile256x128, EPI>(out, act, wt, res, M, N, K, s);
 }
@@ -335,7 +515,8 @@ int dequant_gemm_mfma(void *out, const void *act, const int8_t *wq, const void *
 }  // namespace mynn
 
 extern "C" int mynn_set_gemm_tile(int which) {
-    MYNN_REQUIRE(which >= 0 && which <= 2, MYNN_ERR_INVALID, "set_gemm_tile: %d is not 0 (automatic), 1 (256x128) or 2 (256x256)", which);
+    MYNN_REQUIRE(which >= 0 && which <= 3, MYNN_ERR_INVALID,
+                 "set_gemm_tile: %d is not 0 (automatic), 1 (256x128), 2 (256x256) or 3 (256x256, direct-to-LDS loads)", which);
     mynn::gemm_set_tile(which);
     return 0;
 }

@@ -57,6 +57,26 @@ def test_dequant_matmul_mfma_vs_oracle(g, dt, M, N, K):
     assert max_abs_rel(g.f32(got, dt), exact) <= 1e-2
 
 
+@pytest.mark.parametrize("tile", [1, 2, 3])
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+@pytest.mark.parametrize("M,N,K", [(200, 300, 512), (700, 520, 128), (128, 2560, 2048)])
+def test_dequant_matmul_every_workgroup_tile(g, dt, M, N, K, tile):
+    """Each workgroup tile / load scheme of the matrix-core GEMM (256x128; 256x256 with 8 or 4 waves;
+    256x256 with direct-to-LDS loads and swizzled tiles) on shapes with row and column tails."""
+    rng = np.random.default_rng(M + N + K)
+    act = orc.to_storage(rng.standard_normal((M, K)), dt)
+    W = rng.integers(-127, 128, (N, K)).astype(np.int8)
+    sc = orc.to_storage(rng.uniform(1e-3, 1e-2, N), dt)
+    want = orc.dequant_matmul(act, W, sc, dt, dt, mode=2)
+    g.mynn.set_gemm_tile(tile)
+    try:
+        got = g.to_host(g.mynn.dequant_matmul(g.to_dev(act, dt), g.to_dev(W), g.to_dev(sc, dt)))
+    finally:
+        g.mynn.set_gemm_tile(0)
+    assert max_abs_rel(g.f32(got, dt), g.f32(want, dt)) <= 1e-2
+    assert np.mean(got == want) > 0.97
+
+
 def test_dequant_matmul_linearity_at_prefill_size(g):
     """Size-independent property at the prefill shape (M = 8192): rows are independent, so any
     row block of the big product equals the product of that block alone."""
