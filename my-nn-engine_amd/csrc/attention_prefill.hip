@@ -12,6 +12,8 @@
 //                      registers; A = V^T read from LDS with two 8-byte reads
 // The rescale factor of the online softmax is a per-lane scalar because O^T keeps the same query
 // column per lane.  Key tiles past a wave's last causal position are skipped.
+#include <type_traits>
+
 #include "attention.h"
 #include "mfma.h"
 
@@ -93,7 +95,70 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(AttnParams p) 
     for (int t = 0; t < DT; t++)
 #pragma unroll
         for (int e = 0; e < 16; e++) o[t][e] = 0.f;
+    // running max in units of log2: scores are turned into exponents of two with one FMA each,
+    // p = 2^(s * scale * log2(e) - m); the softmax scale is positive, so the max may be taken on raw scores
     float m = -INFINITY, l = 0.f;
+    const float scale2 = p.scale * 1.4426950408889634f;
+    // keys every query row of this wave may see: tiles that end at or below it need no masking
+    const int wave_first = min(q_blk + wave * 32, Sq - 1);
+    const int wave_all = p.is_causal ? min(kv_bound, qoff + wave_first + 1) : kv_bound;
+
+    auto tile = [&](int buf, int k0, auto masked) {
+        constexpr bool MASKED = decltype(masked)::value;
+        // ---- S^T tile: rows = keys, cols = queries
+        f16x_t s;
+#pragma unroll
+        for (int e = 0; e < 16; e++) s[e] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            const U4 a = *(const U4 *)&Ks[buf][col * LDK + 16 * ks + 8 * g];
+            s = Mfma<T>::run(a, qf[ks], s);
+        }
+        // ---- online softmax for this lane's query over its 16 keys (+ partner lane's 16)
+        float mloc = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            if (MASKED) {
+                const int key = k0 + 8 * (e >> 2) + 4 * g + (e & 3);
+                if (key >= my_bound) s[e] = -INFINITY;
+            }
+            mloc = fmaxf(mloc, s[e]);
+        }
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+        const float mn = fmaxf(m, mloc * scale2);
+        float corr = 1.f;
+        float pe[16];
+        if (MASKED && mn == -INFINITY) {
+#pragma unroll
+            for (int e = 0; e < 16; e++) pe[e] = 0.f;
+        } else {
+            corr = __builtin_amdgcn_exp2f(m - mn);
+            float ls = 0.f;
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                pe[e] = __builtin_amdgcn_exp2f(fmaf(s[e], scale2, -mn));
+                ls += pe[e];
+            }
+            l = fmaf(l, corr, ls);
+            m = mn;
+        }
+#pragma unroll
+        for (int t2 = 0; t2 < DT; t2++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) o[t2][e] *= corr;
+        // ---- O^T += V^T . P^T, keys contracted in the order the D-layout delivers them
+#pragma unroll
+        for (int st = 0; st < 2; st++) {
+            const U4 pf = U4{pack2<T>(pe[8 * st + 0], pe[8 * st + 1]), pack2<T>(pe[8 * st + 2], pe[8 * st + 3]),
+                             pack2<T>(pe[8 * st + 4], pe[8 * st + 5]), pack2<T>(pe[8 * st + 6], pe[8 * st + 7])};
+#pragma unroll
+            for (int t2 = 0; t2 < DT; t2++) {
+                const uint16_t *vr = &Vt[buf][(32 * t2 + col) * LDV + 16 * st + 4 * g];
+                const uint2 lo = *(const uint2 *)vr, hi = *(const uint2 *)(vr + 8);
+                o[t2] = Mfma<T>::run(U4{lo.x, lo.y, hi.x, hi.y}, pf, o[t2]);
+            }
+        }
+    };
 
     if (ntiles > 0) {
         load_tile(0);
@@ -104,59 +169,8 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(AttnParams p) 
         const int buf = t & 1;
         if (t + 1 < ntiles) load_tile(t + 1);
         const int k0 = t * kPfKeys;
-        if (k0 < wave_bound) {
-            // ---- S^T tile: rows = keys, cols = queries
-            f16x_t s;
-#pragma unroll
-            for (int e = 0; e < 16; e++) s[e] = 0.f;
-#pragma unroll
-            for (int ks = 0; ks < KS; ks++) {
-                const U4 a = *(const U4 *)&Ks[buf][col * LDK + 16 * ks + 8 * g];
-                s = Mfma<T>::run(a, qf[ks], s);
-            }
-            // ---- online softmax for this lane's query over its 16 keys (+ partner lane's 16)
-            float mloc = -INFINITY;
-#pragma unroll
-            for (int e = 0; e < 16; e++) {
-                const int key = k0 + 8 * (e >> 2) + 4 * g + (e & 3);
-                s[e] = key < my_bound ? s[e] * p.scale : -INFINITY;
-                mloc = fmaxf(mloc, s[e]);
-            }
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
-            const float mn = fmaxf(m, mloc);
-            float corr = 1.f;
-            float pe[16];
-            if (mn == -INFINITY) {
-#pragma unroll
-                for (int e = 0; e < 16; e++) pe[e] = 0.f;
-            } else {
-                corr = fast_exp(m - mn);
-                float ls = 0.f;
-#pragma unroll
-                for (int e = 0; e < 16; e++) {
-                    pe[e] = fast_exp(s[e] - mn);
-                    ls += pe[e];
-                }
-                l = fmaf(l, corr, ls);
-                m = mn;
-            }
-#pragma unroll
-            for (int t2 = 0; t2 < DT; t2++)
-#pragma unroll
-                for (int e = 0; e < 16; e++) o[t2][e] *= corr;
-            // ---- O^T += V^T . P^T, keys contracted in the order the D-layout delivers them
-#pragma unroll
-            for (int st = 0; st < 2; st++) {
-                const U4 pf = U4{pack2<T>(pe[8 * st + 0], pe[8 * st + 1]), pack2<T>(pe[8 * st + 2], pe[8 * st + 3]),
-                                 pack2<T>(pe[8 * st + 4], pe[8 * st + 5]), pack2<T>(pe[8 * st + 6], pe[8 * st + 7])};
-#pragma unroll
-                for (int t2 = 0; t2 < DT; t2++) {
-                    const uint16_t *vr = &Vt[buf][(32 * t2 + col) * LDV + 16 * st + 4 * g];
-                    const uint2 lo = *(const uint2 *)vr, hi = *(const uint2 *)(vr + 8);
-                    o[t2] = Mfma<T>::run(U4{lo.x, lo.y, hi.x, hi.y}, pf, o[t2]);
-                }
-            }
-        }
+        if (k0 + kPfKeys <= wave_all) tile(buf, k0, std::false_type{});
+        else if (k0 < wave_bound) tile(buf, k0, std::true_type{});
         if (t + 1 < ntiles) {
             store_tile(buf ^ 1);
             __syncthreads();
@@ -185,6 +199,7 @@ bool attention_prefill_supported(const AttnParams &p, int D, int dtype, int kv_i
     if (kv_int8 || (dtype != MYNN_F16 && dtype != MYNN_BF16)) return false;
     if (D != 64 && D != 128) return false;
     if (p.Sq < 16) return false;  // a handful of rows: the per-row kernel wastes less
+    if (!(p.scale > 0.f)) return false;  // the running max is taken on unscaled scores
     // 16-byte loads of Q rows and 8-byte stores of out rows
     if ((p.q_rs % 8) || (p.q_hs % 8) || (p.q_bs % 8) || (p.o_rs % 4) || (p.o_hs % 4) || (p.o_bs % 4)) return false;
     if (((uintptr_t)p.q & 15) || ((uintptr_t)p.out & 7) || ((uintptr_t)p.k & 15) || ((uintptr_t)p.v & 15)) return false;
