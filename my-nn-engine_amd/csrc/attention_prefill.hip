@@ -3,9 +3,9 @@
 // shared memory, 16 lanes doing the softmax serially).
 //
 // One workgroup = 4 waves = 128 query rows of one (batch, query head); each wave owns 32 rows.
-// Per 32-key tile (staged once in LDS for the four waves, K row-major, V transposed):
+// Per 64-key tile (staged once in LDS for the four waves, K row-major, V transposed; two 32-key S^T tiles):
 //   S^T = K . Q^T      v_mfma_f32_32x32x16: A = K rows from LDS, B = Q kept in registers
-//   softmax            each lane owns ONE query column and 16 of the 32 keys of the tile, so the
+//   softmax            each lane owns ONE query column and 16 of the 32 keys of each S^T tile, so the
 //                      row max / sum are in-lane plus a single exchange with lane ^ 32
 //   O^T += V^T . P^T   the D-layout of S^T is already the B-operand layout of P^T (keys are
 //                      contracted in the permuted order 4g+0..3, 8+4g+0..3), so P never leaves
@@ -19,15 +19,15 @@
 
 namespace mynn {
 
-constexpr int kPfThreads = 256, kPfRows = 128, kPfKeys = 32;
+constexpr int kPfThreads = 256, kPfRows = 128, kPfKeys = 64;
 
 template <typename T, int D>
-__global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(AttnParams p) {
+__global__ __launch_bounds__(kPfThreads, D == 64 ? 3 : 2) void attn_prefill_kernel(AttnParams p) {
     constexpr int LDK = D + 8;          // K tile row stride (elements): conflict-free 16-byte reads
     constexpr int LDV = kPfKeys + 4;    // V^T tile row stride
     constexpr int KS = D / 16;          // k-steps of the S^T product
     constexpr int DT = D / 32;          // 32-row tiles of O^T
-    constexpr int CH = (kPfKeys * D / 8) / kPfThreads;  // 16-byte chunks per thread and tile (1 or 2)
+    constexpr int CH = (kPfKeys * D / 8) / kPfThreads;  // 16-byte chunks per thread and tile (2 or 4)
     static_assert(CH >= 1, "tile smaller than the workgroup");
     __shared__ __align__(16) uint16_t Ks[2][kPfKeys * LDK];
     __shared__ __align__(16) uint16_t Vt[2][D * LDV];
@@ -60,19 +60,16 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(AttnParams p) 
 
     const T *Kg = (const T *)p.k + (size_t)(b * p.Hkv + hkv) * p.cache_len * D;
     const T *Vg = (const T *)p.v + (size_t)(b * p.Hkv + hkv) * p.cache_len * D;
+    // a tile travels global -> registers (one iteration ahead of) -> LDS (one iteration ahead of) the MFMAs.
+    // Rows past the end are clamped to the last visible key: whatever they hold is masked out.
     U4 rk[CH], rv[CH];
     auto load_tile = [&](int t) {
 #pragma unroll
         for (int c = 0; c < CH; c++) {
             const int chunk = tid + c * kPfThreads;
-            const int key = t * kPfKeys + chunk / (D / 8), dd = (chunk % (D / 8)) * 8;
-            if (key < blk_bound) {
-                rk[c] = *(const U4 *)(Kg + (size_t)key * D + dd);
-                rv[c] = *(const U4 *)(Vg + (size_t)key * D + dd);
-            } else {
-                rk[c] = U4{0u, 0u, 0u, 0u};
-                rv[c] = U4{0u, 0u, 0u, 0u};
-            }
+            const int key = min(t * kPfKeys + chunk / (D / 8), blk_bound - 1), dd = (chunk % (D / 8)) * 8;
+            rk[c] = *(const U4 *)(Kg + (size_t)key * D + dd);
+            rv[c] = *(const U4 *)(Vg + (size_t)key * D + dd);
         }
     };
     auto store_tile = [&](int buf) {
@@ -103,42 +100,51 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(AttnParams p) 
     const int wave_first = min(q_blk + wave * 32, Sq - 1);
     const int wave_all = p.is_causal ? min(kv_bound, qoff + wave_first + 1) : kv_bound;
 
+    // one tile of 64 keys = two S^T tiles (rows = keys, cols = queries), one softmax update, 4 k-steps of P.V
     auto tile = [&](int buf, int k0, auto masked) {
         constexpr bool MASKED = decltype(masked)::value;
-        // ---- S^T tile: rows = keys, cols = queries
-        f16x_t s;
+        f16x_t s[2];
 #pragma unroll
-        for (int e = 0; e < 16; e++) s[e] = 0.f;
+        for (int hf = 0; hf < 2; hf++)
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-            const U4 a = *(const U4 *)&Ks[buf][col * LDK + 16 * ks + 8 * g];
-            s = Mfma<T>::run(a, qf[ks], s);
-        }
-        // ---- online softmax for this lane's query over its 16 keys (+ partner lane's 16)
+            for (int e = 0; e < 16; e++) s[hf][e] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+            for (int hf = 0; hf < 2; hf++) {
+                const U4 a = *(const U4 *)&Ks[buf][(32 * hf + col) * LDK + 16 * ks + 8 * g];
+                s[hf] = Mfma<T>::run(a, qf[ks], s[hf]);
+            }
+        // ---- online softmax for this lane's query over its 32 keys (+ partner lane's 32)
         float mloc = -INFINITY;
 #pragma unroll
-        for (int e = 0; e < 16; e++) {
-            if (MASKED) {
-                const int key = k0 + 8 * (e >> 2) + 4 * g + (e & 3);
-                if (key >= my_bound) s[e] = -INFINITY;
+        for (int hf = 0; hf < 2; hf++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                if (MASKED) {
+                    const int key = k0 + 32 * hf + 8 * (e >> 2) + 4 * g + (e & 3);
+                    if (key >= my_bound) s[hf][e] = -INFINITY;
+                }
+                mloc = fmaxf(mloc, s[hf][e]);
             }
-            mloc = fmaxf(mloc, s[e]);
-        }
         mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
         const float mn = fmaxf(m, mloc * scale2);
         float corr = 1.f;
-        float pe[16];
         if (MASKED && mn == -INFINITY) {
 #pragma unroll
-            for (int e = 0; e < 16; e++) pe[e] = 0.f;
+            for (int hf = 0; hf < 2; hf++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) s[hf][e] = 0.f;
         } else {
             corr = __builtin_amdgcn_exp2f(m - mn);
             float ls = 0.f;
 #pragma unroll
-            for (int e = 0; e < 16; e++) {
-                pe[e] = __builtin_amdgcn_exp2f(fmaf(s[e], scale2, -mn));
-                ls += pe[e];
-            }
+            for (int hf = 0; hf < 2; hf++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    s[hf][e] = __builtin_amdgcn_exp2f(fmaf(s[hf][e], scale2, -mn));
+                    ls += s[hf][e];
+                }
             l = fmaf(l, corr, ls);
             m = mn;
         }
@@ -148,9 +154,11 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(AttnParams p) 
             for (int e = 0; e < 16; e++) o[t2][e] *= corr;
         // ---- O^T += V^T . P^T, keys contracted in the order the D-layout delivers them
 #pragma unroll
-        for (int st = 0; st < 2; st++) {
-            const U4 pf = U4{pack2<T>(pe[8 * st + 0], pe[8 * st + 1]), pack2<T>(pe[8 * st + 2], pe[8 * st + 3]),
-                             pack2<T>(pe[8 * st + 4], pe[8 * st + 5]), pack2<T>(pe[8 * st + 6], pe[8 * st + 7])};
+        for (int st = 0; st < 4; st++) {
+            const f16x_t &ph = s[st >> 1];
+            const int e0 = 8 * (st & 1);
+            const U4 pf = U4{pack2<T>(ph[e0 + 0], ph[e0 + 1]), pack2<T>(ph[e0 + 2], ph[e0 + 3]),
+                             pack2<T>(ph[e0 + 4], ph[e0 + 5]), pack2<T>(ph[e0 + 6], ph[e0 + 7])};
 #pragma unroll
             for (int t2 = 0; t2 < DT; t2++) {
                 const uint16_t *vr = &Vt[buf][(32 * t2 + col) * LDV + 16 * st + 4 * g];
@@ -163,18 +171,17 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(AttnParams p) 
     if (ntiles > 0) {
         load_tile(0);
         store_tile(0);
+        if (ntiles > 1) load_tile(1);
     }
     __syncthreads();
     for (int t = 0; t < ntiles; t++) {
         const int buf = t & 1;
-        if (t + 1 < ntiles) load_tile(t + 1);
+        if (t + 1 < ntiles) store_tile(buf ^ 1);  // tile t+1, loaded an iteration ago; its buffer was released by the last barrier
+        if (t + 2 < ntiles) load_tile(t + 2);
         const int k0 = t * kPfKeys;
         if (k0 + kPfKeys <= wave_all) tile(buf, k0, std::false_type{});
         else if (k0 < wave_bound) tile(buf, k0, std::true_type{});
-        if (t + 1 < ntiles) {
-            store_tile(buf ^ 1);
-            __syncthreads();
-        }
+        __syncthreads();
     }
 
     // ---- out[query, d] = O^T[d, query] / l

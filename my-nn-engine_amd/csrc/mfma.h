@@ -25,16 +25,21 @@ template <> struct Mfma<bf16_t> {
     }
 };
 
-// two f32 -> one dword of two storage-type values (low half first)
-template <typename T> __device__ inline uint32_t pack2(float lo, float hi) {
-    T a, b;
-    Elem<T>::st(&a, 0, lo);
-    Elem<T>::st(&b, 0, hi);
-    return (uint32_t)__builtin_bit_cast(uint16_t, a) | ((uint32_t)__builtin_bit_cast(uint16_t, b) << 16);
-}
-
-
+// two f32 -> one dword of two storage-type values (low half first), round to nearest even: one packed
+// convert instruction.  The inputs are values ALREADY rounded to f32 (the empty asm keeps the compiler from
+// fusing the producing multiply into a mixed-precision op that would round the exact product once).
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
+template <typename T> __device__ inline uint32_t pack2(float lo, float hi);
+template <> __device__ inline uint32_t pack2<f16_t>(float lo, float hi) {
+    asm volatile("" : "+v"(lo), "+v"(hi));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2_t){lo, hi}, h2_t));
+}
+template <> __device__ inline uint32_t pack2<bf16_t>(float lo, float hi) {
+    asm volatile("" : "+v"(lo), "+v"(hi));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2_t){lo, hi}, bf2_t));
+}
 
 // 8 int8 (two dwords) -> 8 values of T packed in a U4; exact
 template <typename T> __device__ inline U4 i8x8_to_operand(uint32_t w0, uint32_t w1) {
