@@ -568,7 +568,7 @@ class LlmSession:
 
 def set_gemm_tile(which):
     """Workgroup tile of the matrix-core GEMM: 0 = per-shape choice, 1 = 256x128, 2 = 256x256 with
-    operands staged through registers, 3 = 256x256 with operands loaded straight into LDS."""
+    operands staged through registers, 3 = 256x256 and 4 = 256x320 with operands loaded straight into LDS."""
     check(lib().mynn_set_gemm_tile(int(which)))
 
 

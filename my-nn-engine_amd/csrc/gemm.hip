@@ -63,7 +63,6 @@ struct GemmTile {
     static constexpr int ROWS_PER_PASS = THREADS / 4;
     static constexpr int EST = BN / WN + 8;                              // store staging row stride
     static constexpr size_t LDS = (size_t)2 * (BM + BN) * LDT * 2;
-    static_assert(TJ % 2 == 0, "the SwiGLU store pairs neighbouring column tiles");
     static_assert((size_t)WM * WN * 32 * EST * 2 <= LDS, "store staging must fit the operand buffers");
 };
 using Tile256x128 = GemmTile<256, 128, 4, 2>;  // 64 x 64 per wave, 61 KB LDS, two workgroups per CU
@@ -95,6 +94,7 @@ __device__ __forceinline__ void gemm_store(f16x_t (&acc)[G::TI][G::TJ], uint16_t
                                            int n0, int wrow, int wcol, int lane, int wave) {
     constexpr int TI = G::TI, TJ = G::TJ;
     constexpr int EST = G::EST;
+    static_assert(EPI != GEMM_SWIGLU || TJ % 2 == 0, "the SwiGLU store pairs neighbouring column tiles");
     constexpr int OC = EPI == GEMM_SWIGLU ? TJ * 16 : TJ * 32;  // output columns of the wave tile
     constexpr int CPR = OC / 8;                                 // 16-byte chunks per strip row
     const int ldc = EPI == GEMM_SWIGLU ? N >> 1 : N;
@@ -113,7 +113,9 @@ __device__ __forceinline__ void gemm_store(f16x_t (&acc)[G::TI][G::TJ], uint16_t
 #pragma unroll
                     for (int x = 0; x < 4; x++) {
                         const float g = Elem<T>::rnd(acc[i][j][4 * q + x]), u = Elem<T>::rnd(acc[i][j + 1][4 * q + x]);
-                        const float sig = 1.0f / (1.0f + expf(-g));
+                        // hardware 2^x and reciprocal (about 1 ulp of f32 each, far below the 16-bit rounding that
+                        // follows); the exact expf and division cost ~35 instructions per element here
+                        const float sig = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.4426950408889634f));
                         o[x] = (g * sig) * u;
                     }
                     *(uint2 *)(prow + j * 16 + 8 * q) = uint2{pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3])};
@@ -253,43 +255,52 @@ __global__ __launch_bounds__(G::THREADS) void gemm_nt_mfma_kernel(T *C, const T 
 // conflict-free.  Two LDS stages of 64 KB: the loads of tile kt+2 are issued as soon as everyone has
 // finished reading tile kt and fly during tile kt+1; one barrier per K tile, a bare s_barrier with explicit
 // counter waits.  Fragments of the next 16-k step are read while the current one multiplies.
-// 256 x 256 tile, 8 waves of 128 x 64.  Needs K % 64 == 0.
+// 256 x 256 tile, 8 waves of 128 x 64; or 256 x 320, 8 waves of 64 x 160, for widths that this turns into
+// a whole number of rounds over the CUs (N = 2560: 256 tiles instead of 320).  Needs K % 64 == 0.
 using TileDma = GemmTile<256, 256, 2, 4>;
+using TileDma320 = GemmTile<256, 320, 4, 2>;
 constexpr int DBK = 64;
-constexpr int kDmaStage = 2 * 256 * DBK;  // elements per stage: A tile then B tile (64 KB)
-constexpr size_t kDmaLds = (size_t)2 * kDmaStage * 2;
+template <typename G> constexpr int dma_stage_elems() { return (G::BM + G::BN) * DBK; }  // A tile then B tile
+template <typename G> constexpr size_t dma_lds_bytes() { return (size_t)2 * dma_stage_elems<G>() * 2; }
 
 template <typename T, typename G, int EPI>
 __global__ __launch_bounds__(G::THREADS) void gemm_nt_dma_kernel(T *C, const T *A, const T *B, const T *R, int M, int N, int K,
                                                                  int Kp) {
-    static_assert(G::BM == 256 && G::BN == 256, "tile");
-    constexpr int TI = G::TI, TJ = G::TJ, KS = DBK / 16;
-    constexpr int CH = 2048 / G::THREADS;  // 16-byte chunks per thread per operand tile
+    constexpr int TI = G::TI, TJ = G::TJ, KS = DBK / 16, BM = G::BM, BN = G::BN;
+    constexpr int CHA = BM * 8 / G::THREADS, CHB = BN * 8 / G::THREADS;  // 16-byte chunks per thread per operand tile
+    constexpr int kDmaStage = dma_stage_elems<G>();
+    static_assert(BM * 8 % G::THREADS == 0 && BN * 8 % G::THREADS == 0, "whole load instructions per wave");
     extern __shared__ __align__(16) uint16_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / G::WN, wn = wave % G::WN;
     const int wrow = wm * TI * 32, wcol = wn * TJ * 32;
-    const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     int tm, tn;
     tile_of(blockIdx.x, gridDim.x, tiles_m, tiles_n, tm, tn);
-    const int m0 = tm * 256, n0 = tn * 256;
+    const int m0 = tm * BM, n0 = tn * BN;
 
     // this lane's chunks of each operand tile: LDS position P = (CH*wave + i)*64 + lane
-    const T *asrc[CH], *bsrc[CH];
+    const T *asrc[CHA], *bsrc[CHB];
 #pragma unroll
-    for (int i = 0; i < CH; i++) {
-        const int P = (CH * wave + i) * 64 + lane, r = P >> 3, c = (P & 7) ^ ((r >> 1) & 7);
+    for (int i = 0; i < CHA; i++) {
+        const int P = (CHA * wave + i) * 64 + lane, r = P >> 3, c = (P & 7) ^ ((r >> 1) & 7);
         asrc[i] = A + (size_t)min(m0 + r, M - 1) * K + c * 8;
+    }
+#pragma unroll
+    for (int i = 0; i < CHB; i++) {
+        const int P = (CHB * wave + i) * 64 + lane, r = P >> 3, c = (P & 7) ^ ((r >> 1) & 7);
         bsrc[i] = B + (size_t)min(n0 + r, N - 1) * Kp + c * 8;
     }
     auto issue = [&](int kt, int stage) {
-        uint16_t *dst = lds + stage * kDmaStage + (CH * wave) * 512;  // wave-uniform; the lane offset is implicit
+        uint16_t *dst = lds + stage * kDmaStage;  // wave-uniform destinations; the lane offset is implicit
 #pragma unroll
-        for (int i = 0; i < CH; i++) {
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(asrc[i] + (size_t)kt * DBK),
-                                             (__attribute__((address_space(3))) void *)(dst + i * 512), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(bsrc[i] + (size_t)kt * DBK),
-                                             (__attribute__((address_space(3))) void *)(dst + 256 * DBK + i * 512), 16, 0, 0);
+        for (int i = 0; i < (CHA > CHB ? CHA : CHB); i++) {
+            if (i < CHA)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(asrc[i] + (size_t)kt * DBK),
+                                                 (__attribute__((address_space(3))) void *)(dst + (CHA * wave + i) * 512), 16, 0, 0);
+            if (i < CHB)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(bsrc[i] + (size_t)kt * DBK),
+                                                 (__attribute__((address_space(3))) void *)(dst + BM * DBK + (CHB * wave + i) * 512), 16, 0, 0);
         }
     };
 
@@ -313,7 +324,7 @@ __global__ __launch_bounds__(G::THREADS) void gemm_nt_dma_kernel(T *C, const T *
 #pragma unroll
     for (int j = 0; j < TJ; j++) {
         const int r = wcol + j * 32 + fr;
-        brow8[j] = 256 * DBK + 64 * r;
+        brow8[j] = BM * DBK + 64 * r;
         bswz[j] = (r >> 1) & 7;
     }
     auto read_frags = [&](const uint16_t *st, int ks, U4 *fa, U4 *fb) {
@@ -372,7 +383,7 @@ __global__ __launch_bounds__(G::THREADS) void gemm_nt_dma_kernel(T *C, const T *
         multiply(fa[(KS - 1) & 1], fb[(KS - 1) & 1]);
         // LDS reads first (the compiler keeps them ahead of the LDS-writing loads anyway), two per MFMA,
         // then the loads spread over the remaining MFMAs
-        constexpr int RD_MFMA = (TI + TJ) / 2, LD_MFMA = TI * TJ - RD_MFMA;
+        constexpr int RD_MFMA = (TI + TJ + 1) / 2, LD_MFMA = TI * TJ - RD_MFMA;
 #pragma unroll
         for (int n = 0; n < RD_MFMA; n++) {
             __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
@@ -380,7 +391,7 @@ __global__ __launch_bounds__(G::THREADS) void gemm_nt_dma_kernel(T *C, const T *
         }
 #pragma unroll
         for (int n = 0; n < LD_MFMA; n++) {
-            __builtin_amdgcn_sched_group_barrier(0x010, (2 * CH + LD_MFMA - 1) / LD_MFMA, 0);
+            __builtin_amdgcn_sched_group_barrier(0x010, (CHA + CHB + LD_MFMA - 1) / LD_MFMA, 0);
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -442,16 +453,16 @@ static int gemm_launch_dma(void *out, const void *act, const void *wt, const voi
     static bool lds_set = false;
     if (!lds_set) {
         MYNN_HIP(hipFuncSetAttribute((const void *)gemm_nt_dma_kernel<T, G, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     (int)kDmaLds));
+                                     (int)dma_lds_bytes<G>()));
         lds_set = true;
     }
-    const int tiles = ((M + 255) / 256) * ((N + 255) / 256);
-    MYNN_LAUNCH((gemm_nt_dma_kernel<T, G, EPI>), dim3(tiles), dim3(G::THREADS), kDmaLds, s, (T *)out, (const T *)act,
+    const int tiles = ((M + G::BM - 1) / G::BM) * ((N + G::BN - 1) / G::BN);
+    MYNN_LAUNCH((gemm_nt_dma_kernel<T, G, EPI>), dim3(tiles), dim3(G::THREADS), dma_lds_bytes<G>(), s, (T *)out, (const T *)act,
                 (const T *)wt, (const T *)res, M, N, K, gemm_kp(K));
     return launch_status("gemm_nt_dma_kernel");
 }
 
-static int g_gemm_tile_override = 0;  // 0 = heuristic, 1 = 256x128, 2 = 256x256 via registers, 3 = 256x256 direct to LDS
+static int g_gemm_tile_override = 0;  // 0 = heuristic, 1 = 256x128, 2 = 256x256 via registers, 3 = 256x256 / 4 = 256x320 direct to LDS
 void gemm_set_tile(int which) { g_gemm_tile_override = which; }
 
 template <typename T, int EPI>
@@ -464,7 +475,14 @@ static int gemm_launch(void *out, const void *act, const void *wt, const void *r
     if (g_gemm_tile_override) big = g_gemm_tile_override == 2;
     // the direct-to-LDS kernel is the faster 256 x 256 one (measured +5..20%); it needs whole 64-wide K steps
     const bool dma_ok = K % 64 == 0 && g_gemm_tile_override != 2;
-    if (g_gemm_tile_override == 3) big = dma_ok;
+    if (g_gemm_tile_override == 3 || g_gemm_tile_override == 4) big = dma_ok;
+    if constexpr (EPI != GEMM_SWIGLU) {
+        // 320 columns per tile when that saves rounds over the CUs (rounds x tile width = time)
+        const long wide_tiles = (long)((M + 255) / 256) * ((N + 319) / 320);
+        const long cost256 = (big_tiles + 255) / 256 * 256, cost320 = (wide_tiles + 255) / 256 * 320;
+        const bool wide = g_gemm_tile_override ? g_gemm_tile_override == 4 : (big && cost320 < cost256);
+        if (wide && dma_ok) return gemm_launch_dma<T, TileDma320, EPI>(out, act, wt, res, M, N, K, s);
+    }
     if (big && dma_ok) return gemm_launch_dma<T, TileDma, EPI>(out, act, wt, res, M, N, K, s);
     if (big) return gemm_launch_tile<T, Tile256x256, EPI>(out, act, wt, res, M, N, K, s);
     return gemm_launch_tile<T, Tile256x128, EPI>(out, act, wt, res, M, N, K, s);
@@ -515,8 +533,8 @@ int dequant_gemm_mfma(void *out, const void *act, const int8_t *wq, const void *
 }  // namespace mynn
 
 extern "C" int mynn_set_gemm_tile(int which) {
-    MYNN_REQUIRE(which >= 0 && which <= 3, MYNN_ERR_INVALID,
-                 "set_gemm_tile: %d is not 0 (automatic), 1 (256x128), 2 (256x256) or 3 (256x256, direct-to-LDS loads)", which);
+    MYNN_REQUIRE(which >= 0 && which <= 4, MYNN_ERR_INVALID,
+                 "set_gemm_tile: %d is not 0 (automatic), 1 (256x128), 2 (256x256), 3 (256x256, direct-to-LDS loads) or 4 (256x320, direct-to-LDS loads)", which);
     mynn::gemm_set_tile(which);
     return 0;
 }

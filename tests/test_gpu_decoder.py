@@ -115,7 +115,7 @@ def test_generate_bookkeeping_and_errors(g):
     llm.close(), dec.close()
 
 
-@pytest.fixture(params=[0, 1, 2, 3], ids=["tile_auto", "tile_256x128", "tile_256x256", "tile_256x256_direct_lds"])
+@pytest.fixture(params=[0, 1, 2, 3, 4], ids=["tile_auto", "tile_256x128", "tile_256x256", "tile_256x256_direct_lds", "tile_256x320_direct_lds"])
 def gemm_tile(g, request):
     g.mynn.set_gemm_tile(request.param)
     yield request.param

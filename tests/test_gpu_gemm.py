@@ -57,7 +57,7 @@ def test_dequant_matmul_mfma_vs_oracle(g, dt, M, N, K):
     assert max_abs_rel(g.f32(got, dt), exact) <= 1e-2
 
 
-@pytest.mark.parametrize("tile", [1, 2, 3])
+@pytest.mark.parametrize("tile", [1, 2, 3, 4])
 @pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
 @pytest.mark.parametrize("M,N,K", [(200, 300, 512), (700, 520, 128), (128, 2560, 2048)])
 def test_dequant_matmul_every_workgroup_tile(g, dt, M, N, K, tile):
