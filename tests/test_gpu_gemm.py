@@ -59,10 +59,11 @@ def test_dequant_matmul_mfma_vs_oracle(g, dt, M, N, K):
 
 @pytest.mark.parametrize("tile", [1, 2, 3, 4])
 @pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
-@pytest.mark.parametrize("M,N,K", [(200, 300, 512), (700, 520, 128), (128, 2560, 2048)])
+@pytest.mark.parametrize("M,N,K", [(200, 300, 512), (700, 520, 128), (128, 2560, 2048), (300, 650, 64), (257, 321, 192)])
 def test_dequant_matmul_every_workgroup_tile(g, dt, M, N, K, tile):
-    """Each workgroup tile / load scheme of the matrix-core GEMM (256x128; 256x256 with 8 or 4 waves;
-    256x256 with direct-to-LDS loads and swizzled tiles) on shapes with row and column tails."""
+    """Each workgroup tile / load scheme of the matrix-core GEMM (256x128 and 256x256 staged through
+    registers; 256x256 and 256x320 with direct-to-LDS loads and swizzled tiles) on shapes with row and
+    column tails and 1, 2, 3, 8 and 32 K steps."""
     rng = np.random.default_rng(M + N + K)
     act = orc.to_storage(rng.standard_normal((M, K)), dt)
     W = rng.integers(-127, 128, (N, K)).astype(np.int8)
