@@ -28,6 +28,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # Counters cannot be read from inside this process; the figure is carried here from that profile run.
 GATEUP_GEMV_TRAFFIC_BYTES = 23453696
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16/fp16 matrix rate
+INT8_PEAK_TOPS = 5000.0    # MI355X published dense int8 matrix rate
 PREFILL_BATCH, PREFILL_LEN = 8, 1024
 
 TINYLLAMA = dict(n_layers=22, hidden=2048, n_heads=32, n_kv_heads=4, head_dim=64, ffn=5632, vocab=32000,
@@ -102,7 +103,7 @@ def prefill_main(args, mynn, cfg):
     cfg = dict(cfg, max_seq=S)
     weights = make_weights(cfg, cfg["dtype"], args.seed)
     torch.cuda.synchronize()
-    dec = mynn.Decoder(cfg, weights, seq_q=S, batch=B)
+    dec = mynn.Decoder(cfg, weights, seq_q=S, batch=B, quantize_activations=args.w8a8)
     rng = np.random.default_rng(args.seed)
     ids = rng.integers(0, cfg["vocab"], B * S)
     pos = np.arange(S)
@@ -129,22 +130,26 @@ def prefill_main(args, mynn, cfg):
     calls, ms_tot, _, fl_tot = mm[dom]
     achieved = fl_tot / (ms_tot * 1e-3) / 1e12
     step_flops = sum(v[3] for v in agg.values()) / 2
-    lin = {k: v for k, v in mm.items() if k.startswith("linear_")}
+    lin = {k: v for k, v in mm.items() if k.startswith("linear_") or k.startswith("qlinear_")}
+    # W8A8 (--w8a8): activations quantised per row, every linear an exact int8 x int8 -> int32 product
+    peak = INT8_PEAK_TOPS if args.w8a8 else MFMA_PEAK_TFLOPS
+    unit = "TOP/s" if args.w8a8 else "TFLOP/s"
     lin_tflops = sum(v[3] for v in lin.values()) / (sum(v[1] for v in lin.values()) * 1e-3) / 1e12
     out = {
-        "metric": "prefill tok/s 8x1024 TinyLlama-shape int8; MFMA utilisation",
+        "metric": "prefill tok/s 8x1024 TinyLlama-shape int8; MFMA utilisation" + (" (W8A8: quantize_activations)" if args.w8a8 else ""),
         "value": round(B * S * K / elapsed, 1), "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32 accumulate over %s (int8 weights dequantised to %s)" % (args.dtype, args.dtype),
+        "dtype": ("int32 accumulate over int8 activations x int8 weights, %s elsewhere" % args.dtype) if args.w8a8 else
+                 "f32 accumulate over %s (int8 weights dequantised to %s)" % (args.dtype, args.dtype),
         "data": "synthetic",
         "config": {"workload": "configs[3]: TinyLlama-1.1B-shape int8 decoder, prefill of 8 prompts x 1024 tokens, "
-                               "KV cache filled, logits for every row",
+                               "KV cache filled, logits for every row" + (", activations quantised to int8 per row" if args.w8a8 else ""),
                    "batch": B, "seq": S, "launches_per_step": dec.stats()["launches_per_step"], "seed": args.seed,
                    "step_flops": step_flops,
-                   "step_mfma_frac": round(step_flops / (ms_per_step * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4),
+                   "step_mfma_frac": round(step_flops / (ms_per_step * 1e-3) / 1e12 / peak, 4),
                    "per_kernel_ms": {k: round(v[1] / 2, 3) for k, v in sorted(agg.items(), key=lambda kv: -kv[1][1])}},
-        "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 1), "peak": MFMA_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(achieved / MFMA_PEAK_TFLOPS, 4), "traffic": None,
+        "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 1), "peak": peak,
+                     "unit": unit, "frac": round(achieved / peak, 4), "traffic": None,
                      "flops_per_launch": fl_tot / calls, "avg_launch_us": round(ms_tot / calls * 1e3, 2),
                      "all_linear_TFLOPs": round(lin_tflops, 1)},
     }
@@ -331,6 +336,8 @@ def main():
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="first run one 256 MiB device-to-device copy (a kernel of known traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--w8a8", action="store_true",
+                    help="prefill: quantise activations per row and run every linear as int8 x int8 (Options::quantize_activations)")
     ap.add_argument("--kv-int8", action="store_true",
                     help="decode_batch: int8 KV cache with per-token scales (BuildOptions::quant_kv_cache)")
     ap.add_argument("--check-tokens", type=int, default=0,

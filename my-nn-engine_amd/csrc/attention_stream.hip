@@ -217,15 +217,16 @@ __global__ __launch_bounds__(kStreamThreads) void attn_stream_kernel(AttnParams 
     Chunk kA[2][KB], vA[NP], kB[2][KB], vB[NP];
     uint2 sA[4], sB[4];
     const int tstep = kStreamWaves * kStreamTile;
+    const int last_tile = max(p.cache_len - kStreamTile, 0);  // start of the last whole tile (0 for a cache shorter than a tile)
     int t = k0 + wave * kStreamTile;
     if (t < k1) {
         load_tile(t, kA, vA, sA);
         while (true) {
-            load_tile(min(t + tstep, p.cache_len - kStreamTile), kB, vB, sB);
+            load_tile(min(t + tstep, last_tile), kB, vB, sB);
             process(t, kA, vA, sA);
             t += tstep;
             if (t >= k1) break;
-            load_tile(min(t + tstep, p.cache_len - kStreamTile), kA, vA, sA);
+            load_tile(min(t + tstep, last_tile), kA, vA, sA);
             process(t, kB, vB, sB);
             t += tstep;
             if (t >= k1) break;
@@ -319,7 +320,7 @@ int attention_merge_launch(const AttnParams &p, int D, int dtype, hipStream_t s)
 bool attn_stream_eligible(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, int cache_len) {
     const int G = Hq / Hkv;
     return Sq == 1 && dtype != MYNN_F32 && (!kv_int8 || cache_len % kStreamTile == 0) && (D == 64 || D == 128) &&
-           (G == 1 || G == 2 || G == 4 || G == 8) && (long)B * Hkv * kv_len >= 32768;
+           (G == 1 || G == 2 || G == 4 || G == 8) && cache_len >= kStreamTile && (long)B * Hkv * kv_len >= 32768;
 }
 
 // key rows per workgroup and number of key ranges: as many workgroups as the device holds at once

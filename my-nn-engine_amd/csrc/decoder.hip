@@ -58,6 +58,8 @@ struct Layer {
     void *wt_qkv = nullptr, *wt_o = nullptr, *wt_gu = nullptr, *wt_down = nullptr;
     // few-row executors: int8 weights re-tiled so that a wave streams them sequentially
     void *pk_qkv = nullptr, *pk_o = nullptr, *pk_gu = nullptr, *pk_down = nullptr;
+    // W8A8 prefill executors: int8 gate/up rows and their scales interleaved in groups of 32 (SwiGLU store)
+    void *q8_gu = nullptr, *q8_gu_scale = nullptr;
 };
 
 struct Launch {
@@ -73,6 +75,7 @@ struct Model {
     const void *final_norm = nullptr;
     std::vector<Layer> layers;
     void *wt_lm_head = nullptr, *pk_lm_head = nullptr;
+    bool w8a8_fused = false;  // W8A8 with the large int8 tiles: norm+quantise, residual and SwiGLU ride on the launches
     bool resident16 = false;  // the wt_* copies exist and the matrix-core path with fused stores is used
     bool skinny = false;      // 16..64 rows: int8 weights streamed once through the few-row matrix-core kernel
     float *skinny_scratch = nullptr;
@@ -91,7 +94,7 @@ struct Model {
     int token_cap = 0;
     // host staging (pinned)
     char *h_stage = nullptr;
-    size_t stage_bytes = 0;
+    size_t stage_bytes = 0, next_stage = 256;
     hipStream_t stream = nullptr;
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
@@ -191,6 +194,23 @@ static int linear_w8a8(Model &m, void *out, const void *act, const Lin &l, int M
                                  m.stream);
 }
 
+// W8A8 with the large int8 tiles: (RMSNorm +) per-row quantisation of the input, then the product with the
+// store that the layer needs (plain, + residual, SwiGLU over interleaved gate/up rows)
+static int qlinear_fused(Model &m, void *out, const void *act, const void *norm_w, const void *w, const void *scale, const void *res,
+                         int M, int N, int K, int epi, const char *name) {
+    const double eb = dtype_size(m.cfg.dtype);
+    if (norm_w) {
+        note(m, "rms_norm_quantize", (double)M * K * (eb + 1) + M * eb + K * eb);
+        TRY(rms_norm_dynquant(m.a8, m.a8_scale, m.nrm, act, norm_w, M, K, m.cfg.eps, m.cfg.dtype, m.stream));
+    } else {
+        note(m, "dynamic_quantize", (double)M * K * (eb + 1) + M * eb);
+        TRY(mynn_dynamic_quantize_linear(m.a8, m.a8_scale, nullptr, act, M, K, m.cfg.dtype, 1, m.stream));
+    }
+    const int n_out = epi == GEMM_SWIGLU ? N / 2 : N;
+    note(m, name, (double)N * K + (double)M * K + N * eb + (double)M * n_out * eb * (res ? 2 : 1), 2.0 * M * N * K);
+    return qgemm_dma(out, nullptr, m.a8, m.a8_scale, (const int8_t *)w, scale, res, M, N, K, m.cfg.dtype, epi, m.stream);
+}
+
 template <typename T>
 static int enqueue_step(Model &m) {
     const mynn_model_config &c = m.cfg;
@@ -219,6 +239,8 @@ static int enqueue_step(Model &m) {
         if (fused) {
             note(m, "gemv_norm_qkv", (double)L.qkv.N * H + L.qkv.N * eb + 2 * H * eb + L.qkv.N * eb);
             TRY(gemv_norm<T>(m.qkv, m.x, L.norm1, c.eps, (const int8_t *)L.qkv.w, L.qkv.scale, L.qkv.N, H, s));
+        } else if (m.w8a8_fused) {
+            TRY(qlinear_fused(m, m.qkv, m.x, L.norm1, L.qkv.w, L.qkv.scale, nullptr, rows, L.qkv.N, H, GEMM_PLAIN, "qlinear_qkv"));
         } else {
             note(m, "rms_norm", 2.0 * rows * H * eb + H * eb);
             TRY(mynn_rms_norm(m.nrm, m.x, L.norm1, rows, H, c.eps, c.dtype, s));
@@ -269,6 +291,10 @@ static int enqueue_step(Model &m) {
             TRY(mynn_rms_norm(m.nrm, m.x2, L.norm2, rows, H, c.eps, c.dtype, s));
             TRY(skinny_rows(m, m.hmid, m.nrm, L.gu, L.pk_gu, nullptr, rows, GEMM_SWIGLU, "linear_gateup_swiglu"));
             TRY(skinny_rows(m, m.x, m.hmid, L.down, L.pk_down, m.x2, rows, GEMM_RESIDUAL, "linear_down_residual"));
+        } else if (m.w8a8_fused) {
+            TRY(qlinear_fused(m, m.x2, m.attn, nullptr, L.o.w, L.o.scale, m.x, rows, H, QD, GEMM_RESIDUAL, "qlinear_o_residual"));
+            TRY(qlinear_fused(m, m.hmid, m.x2, L.norm2, L.q8_gu, L.q8_gu_scale, nullptr, rows, 2 * F, H, GEMM_SWIGLU, "qlinear_gateup_swiglu"));
+            TRY(qlinear_fused(m, m.x, m.hmid, nullptr, L.down.w, L.down.scale, m.x2, rows, H, F, GEMM_RESIDUAL, "qlinear_down_residual"));
         } else if (w8a8) {
             TRY(linear_w8a8(m, m.proj, m.attn, L.o, rows, true, "qlinear_o"));
             note(m, "add", 3.0 * rows * H * eb);
@@ -307,6 +333,8 @@ static int enqueue_step(Model &m) {
     if (fused) {
         note(m, "gemv_norm_lm_head", (double)V * H + V * eb + 2 * H * eb + V * eb);
         TRY(gemv_norm<T>(m.logits, m.x, m.final_norm, c.eps, (const int8_t *)m.lm_head.w, m.lm_head.scale, V, H, s));
+    } else if (m.w8a8_fused) {
+        TRY(qlinear_fused(m, m.logits, m.x, m.final_norm, m.lm_head.w, m.lm_head.scale, nullptr, rows, V, H, GEMM_PLAIN, "qlinear_lm_head"));
     } else {
         note(m, "rms_norm", 2.0 * rows * H * eb + H * eb);
         TRY(mynn_rms_norm(m.nrm, m.x, m.final_norm, rows, H, c.eps, c.dtype, s));
@@ -458,6 +486,27 @@ static int build(Model &m, void **init, void **state) {
         m.resident16 = true;
     }
 
+    // ---- W8A8 prefill executors: every linear is large enough for the 256-row int8 tiles; gate and up become one
+    // product whose store applies SwiGLU, so their rows (and scales) are interleaved in groups of 32 once
+    {
+        const int rows_ = c.batch * c.seq_q;
+        if (m.quant && c.quantize_activations && c.dtype != MYNN_F32 && F % 32 == 0 && qgemm_dma_supported(rows_, QD + 2 * KD, H) &&
+            qgemm_dma_supported(rows_, H, QD) && qgemm_dma_supported(rows_, 2 * F, H) && qgemm_dma_supported(rows_, H, F) &&
+            qgemm_dma_supported(rows_, V, H)) {
+            const size_t seb = dtype_size(c.dtype);
+            for (Layer &L : m.layers) {
+                MYNN_HIP(hipMalloc(&L.q8_gu, (size_t)2 * F * H));
+                MYNN_HIP(hipMalloc(&L.q8_gu_scale, (size_t)2 * F * seb));
+                TRY(interleave_row_groups(L.q8_gu, L.gate.w, F, (size_t)H, 32, 0, m.stream));
+                TRY(interleave_row_groups(L.q8_gu, L.up.w, F, (size_t)H, 32, 1, m.stream));
+                TRY(interleave_row_groups(L.q8_gu_scale, L.gate.scale, F, seb, 32, 0, m.stream));
+                TRY(interleave_row_groups(L.q8_gu_scale, L.up.scale, F, seb, 32, 1, m.stream));
+            }
+            MYNN_HIP(hipStreamSynchronize(m.stream));
+            m.w8a8_fused = true;
+        }
+    }
+
     // ---- arena: every activation of one step, the device scalars, attention split scratch
     const int rows = c.batch * c.seq_q;
     {
@@ -485,7 +534,7 @@ static int build(Model &m, void **init, void **state) {
     size_t o_sk = plan.take(sk_bytes);
     size_t o_a8 = plan.take(c.quantize_activations ? (size_t)rows * kmax : 0), o_a8s = plan.take((size_t)rows * eb);
     size_t o_ids = plan.take((size_t)rows * 8), o_pos = plan.take((size_t)c.seq_q * 8);
-    size_t o_sc = plan.take(256), o_tok = plan.take((size_t)m.token_cap * 4);
+    size_t o_sc = plan.take(32 + (size_t)c.batch * 4), o_tok = plan.take((size_t)m.token_cap * 4);
     size_t o_as = plan.take(attn_scratch_bytes(c.batch, c.n_heads, c.seq_q, c.head_dim, m.nsplit));
     m.arena_bytes = plan.off;
     MYNN_HIP(hipMalloc((void **)&m.arena, m.arena_bytes));
@@ -497,11 +546,11 @@ static int build(Model &m, void **init, void **state) {
     m.skinny_scratch = (float *)(m.arena + o_sk);
     m.d_ids = (int64_t *)(m.arena + o_ids); m.d_pos = (int64_t *)(m.arena + o_pos);
     m.d_past = (int32_t *)(m.arena + o_sc); m.d_active = m.d_past + 1; m.d_step = m.d_past + 2;
-    m.d_next = m.d_past + 8;  // up to 56 sequences' tokens after the scalars
-    MYNN_REQUIRE(c.batch <= 56, MYNN_ERR_UNSUPPORTED, "batch %d > 56", c.batch);
+    m.d_next = m.d_past + 8;  // one token per sequence after the scalars
     m.d_tokens = (int32_t *)(m.arena + o_tok);
     m.attn_scratch = m.arena + o_as;
-    m.stage_bytes = align_up((size_t)rows * 8 + (size_t)c.seq_q * 8 + 64 + (size_t)m.token_cap * 4, 256) + 512;
+    m.next_stage = align_up((size_t)c.batch * 4, 256);  // the sequences' next tokens live in the tail of the staging buffer
+    m.stage_bytes = align_up((size_t)rows * 8 + (size_t)c.seq_q * 8 + 64 + (size_t)m.token_cap * 4, 256) + 256 + m.next_stage;
     MYNN_HIP(hipHostMalloc((void **)&m.h_stage, m.stage_bytes, hipHostMallocDefault));
     MYNN_HIP(hipDeviceSynchronize());
 
@@ -549,6 +598,8 @@ static void destroy(Model *m) {
         if (L.wt_qkv) hipFree(L.wt_qkv);
         if (L.wt_o) hipFree(L.wt_o);
         if (L.wt_gu) hipFree(L.wt_gu);
+        if (L.q8_gu) hipFree(L.q8_gu);
+        if (L.q8_gu_scale) hipFree(L.q8_gu_scale);
         if (L.wt_down) hipFree(L.wt_down);
         if (L.pk_qkv) hipFree(L.pk_qkv);
         if (L.pk_o) hipFree(L.pk_o);
@@ -673,12 +724,12 @@ extern "C" int mynn_model_step(void *state, const int64_t *input_ids, const int6
     TRY(upload_inputs(m, input_ids, position_id, past_len, active_seq_kv));
     TRY(run_once(m));
     const mynn_model_config &c = m.cfg;
-    if (next_token) MYNN_HIP(hipMemcpyAsync(m.h_stage + m.stage_bytes - 256, m.d_next, (size_t)c.batch * 4, hipMemcpyDeviceToHost, m.stream));
+    if (next_token) MYNN_HIP(hipMemcpyAsync(m.h_stage + m.stage_bytes - m.next_stage, m.d_next, (size_t)c.batch * 4, hipMemcpyDeviceToHost, m.stream));
     if (logits_host)
         MYNN_HIP(hipMemcpyAsync(logits_host, m.logits, (size_t)c.batch * c.seq_q * c.vocab * dtype_size(c.dtype),
                                 hipMemcpyDeviceToHost, m.stream));
     MYNN_HIP(hipStreamSynchronize(m.stream));
-    if (next_token) memcpy(next_token, m.h_stage + m.stage_bytes - 256, (size_t)c.batch * 4);
+    if (next_token) memcpy(next_token, m.h_stage + m.stage_bytes - m.next_stage, (size_t)c.batch * 4);
     return 0;
 }
 

@@ -241,6 +241,117 @@ __global__ __launch_bounds__(kEwThreads) void dynquant_kernel(void *y_, T *y_sca
     }
 }
 
+// Symmetric per-row quantisation of 16-bit rows of at most 8 * 4 * kEwThreads values (a multiple of 8): the
+// row is read once with 128-bit loads and kept in registers; same arithmetic as dynquant_kernel<T, true>.
+// NORM: the row is first RMS-normalised exactly as rms_norm_vec_kernel does (rounded to the storage type)
+// and only the quantised form is written -- the normalised activations of a W8A8 layer have no other reader.
+template <typename T, bool NORM>
+__global__ __launch_bounds__(kEwThreads) void dynquant_rows_vec_kernel(int8_t *y, T *y_scale, const T *x, const T *w, int dim,
+                                                                       float eps) {
+    __shared__ float red[4];
+    const size_t base = (size_t)blockIdx.x * dim;
+    const int chunks = dim >> 3;
+    U4 v[4];
+    float ss = 0.f;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int c = threadIdx.x + q * kEwThreads;
+        v[q] = U4{0u, 0u, 0u, 0u};
+        if (c < chunks) {
+            v[q] = *(const U4 *)(x + base + (size_t)c * 8);
+            if (NORM) {
+                float f[8];
+                widen8<T>(v[q], f);
+#pragma unroll
+                for (int i = 0; i < 8; i++) ss += f[i] * f[i];
+            }
+        }
+    }
+    if (NORM) {
+        const float tot = block_sum(ss, red);
+        const float inv = 1.0f / sqrtf(tot / (float)dim + eps);
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const int c = threadIdx.x + q * kEwThreads;
+            if (c < chunks) {
+                float f[8], g[8];
+                widen8<T>(v[q], f);
+                widen8<T>(*(const U4 *)(w + (size_t)c * 8), g);
+                v[q].x = pack2<T>((f[0] * inv) * g[0], (f[1] * inv) * g[1]);
+                v[q].y = pack2<T>((f[2] * inv) * g[2], (f[3] * inv) * g[3]);
+                v[q].z = pack2<T>((f[4] * inv) * g[4], (f[5] * inv) * g[5]);
+                v[q].w = pack2<T>((f[6] * inv) * g[6], (f[7] * inv) * g[7]);
+            }
+        }
+    }
+    float amax = 0.f;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        float f[8];
+        widen8<T>(v[q], f);
+#pragma unroll
+        for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(f[i]));
+    }
+    amax = block_max(amax, red);
+    const float sc = amax > 0.f ? amax / 127.0f : 1.0f;
+    const float inv = 1.0f / sc;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int c = threadIdx.x + q * kEwThreads;
+        if (c < chunks) {
+            float f[8];
+            widen8<T>(v[q], f);
+            uint32_t b[2] = {0u, 0u};
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                float r = roundf(f[i] * inv);  // half away from zero
+                r = fminf(fmaxf(r, -127.f), 127.f);
+                b[i >> 2] |= ((uint32_t)(int)r & 0xFFu) << (8 * (i & 3));
+            }
+            *(uint2 *)(y + base + (size_t)c * 8) = uint2{b[0], b[1]};
+        }
+    }
+    if (threadIdx.x == 0) Elem<T>::st(y_scale, blockIdx.x, sc);
+}
+
+static bool dynquant_vec_ok(const void *y, const void *x, int dim) {
+    return dim % 8 == 0 && dim <= 8 * 4 * kEwThreads && aligned16(x) && ((uintptr_t)y & 7) == 0;
+}
+
+// RMSNorm followed by symmetric per-row quantisation (the pair RMSNormalization -> DynamicQuantizeLinear of a
+// W8A8 layer), one launch; falls back to the two operators for rows the vector kernel does not take.
+int rms_norm_dynquant(int8_t *y, void *y_scale, void *scratch_norm, const void *x, const void *w, int rows, int dim, float eps,
+                      int dtype, hipStream_t s) {
+    if (dtype != MYNN_F32 && dynquant_vec_ok(y, x, dim) && aligned16(w)) {
+        return dispatch_dtype16(dtype, [&](auto *t) {
+            using T = std::remove_pointer_t<decltype(t)>;
+            MYNN_LAUNCH((dynquant_rows_vec_kernel<T, true>), dim3(rows), dim3(kEwThreads), 0, s, y, (T *)y_scale, (const T *)x,
+                        (const T *)w, dim, eps);
+            return launch_status("dynquant_rows_vec_kernel");
+        });
+    }
+    int rc = mynn_rms_norm(scratch_norm, x, w, rows, dim, eps, dtype, s);
+    if (rc) return rc;
+    return mynn_dynamic_quantize_linear(y, y_scale, nullptr, scratch_norm, rows, dim, dtype, 1, s);
+}
+
+// dst rows [(r / group) * 2 * group + which * group + r % group] <- src rows r, row_bytes each (a multiple of 2):
+// the gate (which = 0) and up (1) halves of a fused gate/up weight whose SwiGLU store pairs column tiles
+__global__ void interleave_rows_kernel(uint16_t *dst, const uint16_t *src, size_t row_halfwords, size_t total, int group, int which) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const size_t r = i / row_halfwords, c = i % row_halfwords;
+    const size_t d = (r / group) * 2 * group + (size_t)which * group + r % group;
+    dst[d * row_halfwords + c] = src[i];
+}
+int interleave_row_groups(void *dst, const void *src, size_t rows, size_t row_bytes, int group, int which, hipStream_t s) {
+    MYNN_REQUIRE(dst && src && row_bytes % 2 == 0 && group > 0 && rows % group == 0, MYNN_ERR_INVALID, "interleave_row_groups: bad operand");
+    const size_t total = rows * (row_bytes / 2);
+    MYNN_LAUNCH(interleave_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, (uint16_t *)dst, (const uint16_t *)src,
+                row_bytes / 2, total, group, which);
+    return launch_status("interleave_rows_kernel");
+}
+
 // ---- greedy argmax, last maximum wins (reference crates/llm/src/session.rs:683-690) -----------
 // one workgroup of 1024 threads per row, 16-byte loads; (value, index) ordered by value, then index
 __device__ inline void argmax_take(float &bv, int &bi, float v, int i) {
@@ -428,6 +539,14 @@ extern "C" int mynn_dynamic_quantize_linear(void *y, void *y_scale, void *y_zero
     MYNN_REQUIRE(symmetric || y_zero_point, MYNN_ERR_INVALID, "dynamic_quantize_linear: asymmetric needs y_zero_point");
     return dispatch_dtype(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
+        if constexpr (sizeof(T) == 2) {
+            if (symmetric && dynquant_vec_ok(y, x, inner_size)) {
+                MYNN_LAUNCH((dynquant_rows_vec_kernel<T, false>), dim3(axis_dim), dim3(kEwThreads), 0, as_stream(s), (int8_t *)y,
+                            (T *)y_scale, (const T *)x, (const T *)nullptr, inner_size, 0.f);
+                if (y_zero_point) MYNN_HIP(hipMemsetAsync(y_zero_point, 0, axis_dim, as_stream(s)));
+                return launch_status("dynquant_rows_vec_kernel");
+            }
+        }
         if (symmetric)
             MYNN_LAUNCH((dynquant_kernel<T, true>), dim3(axis_dim), dim3(kEwThreads), 0, as_stream(s), y,
                                (T *)y_scale, y_zero_point, (const T *)x, inner_size);

@@ -89,8 +89,9 @@ __device__ inline void tile_of(int b, int nblocks, int tiles_m, int tiles_n, int
 // wave turns one 32-row strip of its tile at a time into row-major 16-bit values in its own LDS patch (the
 // operand buffers are free by now) and writes it out, and reads the residual, 16 bytes per lane, rows
 // contiguous.
-template <typename T, typename G, int EPI>
-__device__ __forceinline__ void gemm_store(f16x_t (&acc)[G::TI][G::TJ], uint16_t *lds, T *C, const T *R, int M, int N, int m0,
+// at(i, j, e): element e of the accumulator of MFMA tile (i, j), as f32 ready to be rounded.
+template <typename T, typename G, int EPI, typename AccAt>
+__device__ __forceinline__ void gemm_store(AccAt at, uint16_t *lds, T *C, const T *R, int M, int N, int m0,
                                            int n0, int wrow, int wcol, int lane, int wave) {
     constexpr int TI = G::TI, TJ = G::TJ;
     constexpr int EST = G::EST;
@@ -112,7 +113,7 @@ __device__ __forceinline__ void gemm_store(f16x_t (&acc)[G::TI][G::TJ], uint16_t
                     float o[4];
 #pragma unroll
                     for (int x = 0; x < 4; x++) {
-                        const float g = Elem<T>::rnd(acc[i][j][4 * q + x]), u = Elem<T>::rnd(acc[i][j + 1][4 * q + x]);
+                        const float g = Elem<T>::rnd(at(i, j, 4 * q + x)), u = Elem<T>::rnd(at(i, j + 1, 4 * q + x));
                         // hardware 2^x and reciprocal (about 1 ulp of f32 each, far below the 16-bit rounding that
                         // follows); the exact expf and division cost ~35 instructions per element here
                         const float sig = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.4426950408889634f));
@@ -123,8 +124,8 @@ __device__ __forceinline__ void gemm_store(f16x_t (&acc)[G::TI][G::TJ], uint16_t
             } else {
 #pragma unroll
                 for (int j = 0; j < TJ; j++)
-                    *(uint2 *)(prow + j * 32 + 8 * q) = uint2{pack2<T>(acc[i][j][4 * q], acc[i][j][4 * q + 1]),
-                                                              pack2<T>(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3])};
+                    *(uint2 *)(prow + j * 32 + 8 * q) = uint2{pack2<T>(at(i, j, 4 * q), at(i, j, 4 * q + 1)),
+                                                              pack2<T>(at(i, j, 4 * q + 2), at(i, j, 4 * q + 3))};
             }
         }
         __builtin_amdgcn_wave_barrier();
@@ -244,7 +245,7 @@ __global__ __launch_bounds__(G::THREADS) void gemm_nt_mfma_kernel(T *C, const T 
         __syncthreads();
     }
 
-    gemm_store<T, G, EPI>(acc, lds, C, R, M, N, m0, n0, wrow, wcol, lane, wave);
+    gemm_store<T, G, EPI>([&](int i, int j, int e) { return acc[i][j][e]; }, lds, C, R, M, N, m0, n0, wrow, wcol, lane, wave);
 }
 
 // ---- the same product with the operand tiles copied global -> LDS by the load unit itself
@@ -263,10 +264,20 @@ constexpr int DBK = 64;
 template <typename G> constexpr int dma_stage_elems() { return (G::BM + G::BN) * DBK; }  // A tile then B tile
 template <typename G> constexpr size_t dma_lds_bytes() { return (size_t)2 * dma_stage_elems<G>() * 2; }
 
-template <typename T, typename G, int EPI>
-__global__ __launch_bounds__(G::THREADS) void gemm_nt_dma_kernel(T *C, const T *A, const T *B, const T *R, int M, int N, int K,
-                                                                 int Kp) {
+// I8: the operands are int8 (QuantizedMatMul: A = activations quantised per row, B = the int8 weights), the
+// K tile is the same 128 bytes per row = 128 values, the MFMA is v_mfma_i32_32x32x32_i8 over the same 16-byte
+// fragments, the sum is exact int32 (optionally written out) and the store applies the two scales.
+typedef int i4x_t __attribute__((ext_vector_type(4)));
+typedef int i16x_t __attribute__((ext_vector_type(16)));
+
+template <typename T, typename G, int EPI, bool I8>
+__global__ __launch_bounds__(G::THREADS) void gemm_nt_dma_kernel(T *C, const void *A_, const void *B_, const T *R, int M, int N,
+                                                                 int K, int Kp, const T *a_scale, const T *b_scale,
+                                                                 int32_t *acc_out) {
     constexpr int TI = G::TI, TJ = G::TJ, KS = DBK / 16, BM = G::BM, BN = G::BN;
+    constexpr int EB = I8 ? 1 : 2;            // bytes per operand value
+    constexpr int TILE_B = DBK * 2;           // bytes of one row of a K tile
+    const char *A = (const char *)A_, *B = (const char *)B_;
     constexpr int CHA = BM * 8 / G::THREADS, CHB = BN * 8 / G::THREADS;  // 16-byte chunks per thread per operand tile
     constexpr int kDmaStage = dma_stage_elems<G>();
     static_assert(BM * 8 % G::THREADS == 0 && BN * 8 % G::THREADS == 0, "whole load instructions per wave");
@@ -280,37 +291,38 @@ __global__ __launch_bounds__(G::THREADS) void gemm_nt_dma_kernel(T *C, const T *
     const int m0 = tm * BM, n0 = tn * BN;
 
     // this lane's chunks of each operand tile: LDS position P = (CH*wave + i)*64 + lane
-    const T *asrc[CHA], *bsrc[CHB];
+    const char *asrc[CHA], *bsrc[CHB];
 #pragma unroll
     for (int i = 0; i < CHA; i++) {
         const int P = (CHA * wave + i) * 64 + lane, r = P >> 3, c = (P & 7) ^ ((r >> 1) & 7);
-        asrc[i] = A + (size_t)min(m0 + r, M - 1) * K + c * 8;
+        asrc[i] = A + (size_t)min(m0 + r, M - 1) * K * EB + c * 16;
     }
 #pragma unroll
     for (int i = 0; i < CHB; i++) {
         const int P = (CHB * wave + i) * 64 + lane, r = P >> 3, c = (P & 7) ^ ((r >> 1) & 7);
-        bsrc[i] = B + (size_t)min(n0 + r, N - 1) * Kp + c * 8;
+        bsrc[i] = B + (size_t)min(n0 + r, N - 1) * Kp * EB + c * 16;
     }
     auto issue = [&](int kt, int stage) {
         uint16_t *dst = lds + stage * kDmaStage;  // wave-uniform destinations; the lane offset is implicit
 #pragma unroll
         for (int i = 0; i < (CHA > CHB ? CHA : CHB); i++) {
             if (i < CHA)
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(asrc[i] + (size_t)kt * DBK),
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(asrc[i] + (size_t)kt * TILE_B),
                                                  (__attribute__((address_space(3))) void *)(dst + (CHA * wave + i) * 512), 16, 0, 0);
             if (i < CHB)
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(bsrc[i] + (size_t)kt * DBK),
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(bsrc[i] + (size_t)kt * TILE_B),
                                                  (__attribute__((address_space(3))) void *)(dst + BM * DBK + (CHB * wave + i) * 512), 16, 0, 0);
         }
     };
 
-    f16x_t acc[TI][TJ];
+    using acc_t = std::conditional_t<I8, i16x_t, f16x_t>;
+    acc_t acc[TI][TJ];
 #pragma unroll
     for (int i = 0; i < TI; i++)
 #pragma unroll
         for (int j = 0; j < TJ; j++)
 #pragma unroll
-            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0;
 
     // fragment addresses (elements) inside a stage: row r, chunk c = 2*ks + g  ->  (8r + (c ^ swz)) * 8
     const int fr = lane & 31, g = lane >> 5;
@@ -339,7 +351,13 @@ __global__ __launch_bounds__(G::THREADS) void gemm_nt_dma_kernel(T *C, const T *
 #pragma unroll
         for (int i = 0; i < TI; i++)
 #pragma unroll
-            for (int j = 0; j < TJ; j++) acc[i][j] = Mfma<T>::run(fb[j], fa[i], acc[i][j]);
+            for (int j = 0; j < TJ; j++) {
+                if constexpr (I8)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i4x_t, fb[j]), __builtin_bit_cast(i4x_t, fa[i]),
+                                                                      acc[i][j], 0, 0, 0);
+                else
+                    acc[i][j] = Mfma<T>::run(fb[j], fa[i], acc[i][j]);
+            }
     };
 
     // Schedule of one K tile (4 steps of 16): steps 0..2 multiply while the fragments of the next step are
@@ -349,7 +367,7 @@ __global__ __launch_bounds__(G::THREADS) void gemm_nt_dma_kernel(T *C, const T *
     // first fragments of tile kt+1 are read.  Left alone the instruction scheduler sinks every LDS read to
     // just before its first use and exposes the LDS latency once per step; the sched_group_barrier
     // sequences pin the interleaving (one read or load, then its share of the MFMAs).
-    const int nk = K / DBK;
+    const int nk = K * EB / TILE_B;
     U4 fa[2][TI], fb[2][TJ];
     issue(0, 0);
     issue(min(1, nk - 1), 1);
@@ -398,7 +416,40 @@ __global__ __launch_bounds__(G::THREADS) void gemm_nt_dma_kernel(T *C, const T *
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // the repeat of the last tile too, before LDS is reused
     __syncthreads();
-    gemm_store<T, G, EPI>(acc, lds, C, R, M, N, m0, n0, wrow, wcol, lane, wave);
+    if constexpr (I8) {
+        // accumulator tile = transposed output tile: lane l has output row l % 32 of strip i, and in elements
+        // 4q..4q+3 the columns 8q + 4*(l/32) + 0..3 of column tile j
+        if (acc_out) {
+#pragma unroll
+            for (int i = 0; i < TI; i++)
+#pragma unroll
+                for (int j = 0; j < TJ; j++)
+#pragma unroll
+                    for (int e = 0; e < 16; e++) {
+                        const int row = m0 + wrow + i * 32 + (lane & 31);
+                        const int col = n0 + wcol + j * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                        if (row < M && col < N) acc_out[(size_t)row * N + col] = acc[i][j][e];
+                    }
+        }
+        if (C) {
+            // the column scales of the tile as f32 in the top of LDS (above the store patches), the row scales in
+            // registers; out = T(((f32)sum * row scale) * column scale)
+            float *bs = (float *)((char *)lds + dma_lds_bytes<G>() - BN * sizeof(float));
+            for (int c = tid; c < BN; c += G::THREADS) bs[c] = n0 + c < N ? Elem<T>::ld(b_scale, n0 + c) : 0.f;
+            float asc[TI];
+#pragma unroll
+            for (int i = 0; i < TI; i++) {
+                const int row = m0 + wrow + i * 32 + (lane & 31);
+                asc[i] = row < M ? Elem<T>::ld(a_scale, row) : 0.f;
+            }
+            __syncthreads();
+            const float *bw = bs + wcol + 4 * (lane >> 5);
+            gemm_store<T, G, EPI>([&](int i, int j, int e) { return ((float)acc[i][j][e] * asc[i]) * bw[j * 32 + 8 * (e >> 2) + (e & 3)]; },
+                                  lds, C, R, M, N, m0, n0, wrow, wcol, lane, wave);
+        }
+    } else {
+        gemm_store<T, G, EPI>([&](int i, int j, int e) { return acc[i][j][e]; }, lds, C, R, M, N, m0, n0, wrow, wcol, lane, wave);
+    }
 }
 
 // library-owned workspace for the dequantised weight of the call in flight (grown on demand)
@@ -448,18 +499,44 @@ static int gemm_launch_tile(void *out, const void *act, const void *wt, const vo
     return launch_status("gemm_nt_mfma_kernel");
 }
 
-template <typename T, typename G, int EPI>
-static int gemm_launch_dma(void *out, const void *act, const void *wt, const void *res, int M, int N, int K, hipStream_t s) {
+template <typename T, typename G, int EPI, bool I8 = false>
+static int gemm_launch_dma(void *out, const void *act, const void *wt, const void *res, int M, int N, int K, hipStream_t s,
+                           const void *a_scale = nullptr, const void *b_scale = nullptr, int32_t *acc_out = nullptr) {
     static bool lds_set = false;
     if (!lds_set) {
-        MYNN_HIP(hipFuncSetAttribute((const void *)gemm_nt_dma_kernel<T, G, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize,
+        MYNN_HIP(hipFuncSetAttribute((const void *)gemm_nt_dma_kernel<T, G, EPI, I8>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)dma_lds_bytes<G>()));
         lds_set = true;
     }
     const int tiles = ((M + G::BM - 1) / G::BM) * ((N + G::BN - 1) / G::BN);
-    MYNN_LAUNCH((gemm_nt_dma_kernel<T, G, EPI>), dim3(tiles), dim3(G::THREADS), dma_lds_bytes<G>(), s, (T *)out, (const T *)act,
-                (const T *)wt, (const T *)res, M, N, K, gemm_kp(K));
+    MYNN_LAUNCH((gemm_nt_dma_kernel<T, G, EPI, I8>), dim3(tiles), dim3(G::THREADS), dma_lds_bytes<G>(), s, (T *)out, act, wt,
+                (const T *)res, M, N, K, I8 ? K : gemm_kp(K), (const T *)a_scale, (const T *)b_scale, acc_out);
     return launch_status("gemm_nt_dma_kernel");
+}
+
+// QuantizedMatMul on the matrix cores for a grid of at least one round of 256-row tiles: K % 128 == 0.
+// out (scaled, storage type; optionally + residual) and / or acc_out (exact int32).
+bool qgemm_dma_supported(int M, int N, int K) {
+    return K % 128 == 0 && (long)((M + 255) / 256) * ((N + 255) / 256) >= 128;
+}
+int qgemm_dma(void *out, int32_t *acc_out, const int8_t *lhs, const void *lhs_scale, const int8_t *rhs, const void *rhs_scale,
+              const void *res, int M, int N, int K, int dtype, int epi, hipStream_t s) {
+    MYNN_REQUIRE(qgemm_dma_supported(M, N, K), MYNN_ERR_UNSUPPORTED, "quantized_matmul (large tiles): M=%d N=%d K=%d", M, N, K);
+    MYNN_REQUIRE(epi != GEMM_RESIDUAL || res, MYNN_ERR_INVALID, "quantized_matmul: residual store without a residual");
+    MYNN_REQUIRE(epi != GEMM_SWIGLU || (N % 64 == 0 && !acc_out), MYNN_ERR_INVALID, "quantized_matmul: SwiGLU store needs N %% 64 == 0, N=%d", N);
+    return dispatch_dtype16(dtype, [&](auto *t) {
+        using T = std::remove_pointer_t<decltype(t)>;
+        const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256), t320 = (long)((M + 255) / 256) * ((N + 319) / 320);
+        const bool wide = (t320 + 255) / 256 * 320 < (t256 + 255) / 256 * 256;
+        if (epi == GEMM_SWIGLU)
+            return gemm_launch_dma<T, TileDma, GEMM_SWIGLU, true>(out, lhs, rhs, nullptr, M, N, K, s, lhs_scale, rhs_scale, nullptr);
+        if (epi == GEMM_RESIDUAL) {
+            if (wide) return gemm_launch_dma<T, TileDma320, GEMM_RESIDUAL, true>(out, lhs, rhs, res, M, N, K, s, lhs_scale, rhs_scale, acc_out);
+            return gemm_launch_dma<T, TileDma, GEMM_RESIDUAL, true>(out, lhs, rhs, res, M, N, K, s, lhs_scale, rhs_scale, acc_out);
+        }
+        if (wide) return gemm_launch_dma<T, TileDma320, GEMM_PLAIN, true>(out, lhs, rhs, nullptr, M, N, K, s, lhs_scale, rhs_scale, acc_out);
+        return gemm_launch_dma<T, TileDma, GEMM_PLAIN, true>(out, lhs, rhs, nullptr, M, N, K, s, lhs_scale, rhs_scale, acc_out);
+    });
 }
 
 static int g_gemm_tile_override = 0;  // 0 = heuristic, 1 = 256x128, 2 = 256x256 via registers, 3 = 256x256 / 4 = 256x320 direct to LDS

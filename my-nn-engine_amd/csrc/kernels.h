@@ -36,6 +36,17 @@ enum { GEMM_PLAIN = 0, GEMM_RESIDUAL = 1, GEMM_SWIGLU = 2 };
 size_t gemm_weight_bytes(int N, int K);
 int dequant_weight_rows(void *dst, const int8_t *wq, const void *scale, int N, int K, int dtype, int group, int which,
                         hipStream_t s);
+// RMSNormalization -> DynamicQuantizeLinear (symmetric, per row) in one launch; scratch_norm ([rows, dim] of
+// the storage type) is used only when the rows do not fit the vector kernel
+int rms_norm_dynquant(int8_t *y, void *y_scale, void *scratch_norm, const void *x, const void *w, int rows, int dim, float eps,
+                      int dtype, hipStream_t s);
+// row interleave of the two halves of a fused gate/up operand (groups of `group` rows)
+int interleave_row_groups(void *dst, const void *src, size_t rows, size_t row_bytes, int group, int which, hipStream_t s);
+// QuantizedMatMul (int8 x int8 -> exact int32 -> two scales) with the large direct-to-LDS tiles of the
+// matrix-core GEMM; res (optional) is added to the rounded result and rounded again
+bool qgemm_dma_supported(int M, int N, int K);
+int qgemm_dma(void *out, int32_t *acc_out, const int8_t *lhs, const void *lhs_scale, const int8_t *rhs, const void *rhs_scale,
+              const void *res, int M, int N, int K, int dtype, int epi, hipStream_t s);
 void gemm_set_tile(int which);  // 0 heuristic, 1 = 256x128, 2 = 256x256 workgroup tile
 int gemm_nt_mfma(void *out, const void *act, const void *wt, const void *res, int M, int N, int K, int dtype, int epi,
                  hipStream_t s);

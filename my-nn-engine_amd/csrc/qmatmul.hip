@@ -5,7 +5,8 @@
 // quantized_matmul_int8.cuh:112-269 (mma.m16n8k32.s8, 3-stage cp.async); CPU twin
 // src/codegen/cpu/kernels/qgemv_i8i8.rs:38-80.
 //   M < 16 : wave64 rows, 16 int8 per lane per load, v_dot4_i32_i8, integer butterfly
-//   M >= 16: v_mfma_i32_32x32x32_i8, 128x128 tile per workgroup, K step 32, padded LDS tiles
+//   M >= 16: v_mfma_i32_32x32x32_i8, 128x128 tile per workgroup, K step 32, padded LDS tiles;
+//            grids of >= 128 tiles of 256x256 with K % 128 == 0 use the direct-to-LDS kernel of gemm.hip
 // Integer accumulation is associative, so both are bit-exact whatever the order.
 #include "kernels.h"
 
@@ -184,6 +185,9 @@ extern "C" int mynn_quantized_matmul(void *out, int32_t *acc_out, const int8_t *
     MYNN_REQUIRE(aligned16(lhs) && aligned16(rhs), MYNN_ERR_INVALID, "quantized_matmul: operands must be 16-byte aligned");
     // int32 accumulators hold the exact sum as long as K * 128 * 128 < 2^31
     MYNN_REQUIRE(K <= 131071, MYNN_ERR_UNSUPPORTED, "quantized_matmul: K=%d could overflow the int32 accumulator", K);
+    // at least half a round of 256-row tiles and whole 128-value K steps: the large direct-to-LDS tiles
+    if (dtype != MYNN_F32 && qgemm_dma_supported(M, N, K) && (!out || aligned16(out)))
+        return qgemm_dma(out, acc_out, lhs, lhs_scale, rhs, rhs_scale, nullptr, M, N, K, dtype, GEMM_PLAIN, as_stream(s));
     return dispatch_dtype(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
         return qmatmul_launch<T>(out, acc_out, lhs, lhs_scale, rhs, rhs_scale, M, N, K, as_stream(s));

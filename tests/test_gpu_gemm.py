@@ -128,6 +128,27 @@ def test_quantized_matmul_bit_exact(g, dt, M, N, K):
     assert np.array_equal(g.to_host(out), want_out)
 
 
+@pytest.mark.parametrize("dt", [orc.BF16, orc.F16])
+@pytest.mark.parametrize("M,N,K", [(4096, 2048, 128), (4000, 2100, 384), (8192, 2560, 256)])
+def test_quantized_matmul_large_tiles_bit_exact(g, dt, M, N, K):
+    """Grids of at least half a round of 256-row tiles take the direct-to-LDS int8 kernel (256x256 and, for
+    N = 2560, 256x320 tiles; 1, 3 and 2 K steps; row and column tails): int32 sums and scaled output bit
+    for bit against the oracle."""
+    rng = np.random.default_rng(M + N + K)
+    lhs = rng.integers(-128, 128, (M, K)).astype(np.int8)
+    rhs = rng.integers(-128, 128, (N, K)).astype(np.int8)
+    ls = orc.to_storage(rng.uniform(1e-3, 1e-1, M), dt)
+    rs = orc.to_storage(rng.uniform(1e-3, 1e-2, N), dt)
+    out, acc = g.mynn.quantized_matmul(g.to_dev(lhs), g.to_dev(ls, dt), g.to_dev(rhs), g.to_dev(rs, dt))
+    want_acc = (lhs.astype(np.float64) @ rhs.astype(np.float64).T).astype(np.int32)  # exact: |sum| < 2^53
+    assert np.array_equal(g.to_host(acc), want_acc)
+    want_out = orc.to_storage((want_acc.astype(np.float32) * g.f32(ls, dt)[:, None]) * g.f32(rs, dt)[None, :], dt)
+    assert np.array_equal(g.to_host(out), want_out)
+    sub = slice(0, 64)
+    ref_out, ref_acc = orc.quantized_matmul(lhs[sub], ls[sub], rhs, rs, dt)
+    assert np.array_equal(want_acc[sub], ref_acc) and np.array_equal(want_out[sub], ref_out)
+
+
 def test_quantized_matmul_extremes(g):
     K = 4096
     lhs = np.full((32, K), -128, np.int8)
