@@ -241,21 +241,23 @@ __global__ __launch_bounds__(kEwThreads) void dynquant_kernel(void *y_, T *y_sca
     }
 }
 
-// Symmetric per-row quantisation of 16-bit rows of at most 8 * 4 * kEwThreads values (a multiple of 8): the
-// row is read once with 128-bit loads and kept in registers; same arithmetic as dynquant_kernel<T, true>.
+// Symmetric per-row quantisation of 16-bit rows of at most 8 * 64 * NCH values (a multiple of 8): one wave
+// per row, the row read once with 128-bit loads and kept in registers, reductions inside the wave (no
+// workgroup barrier); same arithmetic as dynquant_kernel<T, true>.
 // NORM: the row is first RMS-normalised exactly as rms_norm_vec_kernel does (rounded to the storage type)
 // and only the quantised form is written -- the normalised activations of a W8A8 layer have no other reader.
-template <typename T, bool NORM>
-__global__ __launch_bounds__(kEwThreads) void dynquant_rows_vec_kernel(int8_t *y, T *y_scale, const T *x, const T *w, int dim,
-                                                                       float eps) {
-    __shared__ float red[4];
-    const size_t base = (size_t)blockIdx.x * dim;
+template <typename T, bool NORM, int NCH>
+__global__ __launch_bounds__(kEwThreads) void dynquant_rows_vec_kernel(int8_t *y, T *y_scale, int8_t *y_zp, const T *x, const T *w,
+                                                                       int rows, int dim, float eps) {
+    const int lane = threadIdx.x & 63, row = blockIdx.x * (kEwThreads / 64) + (threadIdx.x >> 6);
+    if (row >= rows) return;  // whole wave
+    const size_t base = (size_t)row * dim;
     const int chunks = dim >> 3;
-    U4 v[4];
+    U4 v[NCH];
     float ss = 0.f;
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-        const int c = threadIdx.x + q * kEwThreads;
+    for (int q = 0; q < NCH; q++) {
+        const int c = lane + q * 64;
         v[q] = U4{0u, 0u, 0u, 0u};
         if (c < chunks) {
             v[q] = *(const U4 *)(x + base + (size_t)c * 8);
@@ -268,11 +270,11 @@ __global__ __launch_bounds__(kEwThreads) void dynquant_rows_vec_kernel(int8_t *y
         }
     }
     if (NORM) {
-        const float tot = block_sum(ss, red);
+        const float tot = wave_sum(ss);
         const float inv = 1.0f / sqrtf(tot / (float)dim + eps);
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const int c = threadIdx.x + q * kEwThreads;
+        for (int q = 0; q < NCH; q++) {
+            const int c = lane + q * 64;
             if (c < chunks) {
                 float f[8], g[8];
                 widen8<T>(v[q], f);
@@ -286,18 +288,18 @@ __global__ __launch_bounds__(kEwThreads) void dynquant_rows_vec_kernel(int8_t *y
     }
     float amax = 0.f;
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
+    for (int q = 0; q < NCH; q++) {
         float f[8];
         widen8<T>(v[q], f);
 #pragma unroll
         for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(f[i]));
     }
-    amax = block_max(amax, red);
+    amax = wave_max(amax);
     const float sc = amax > 0.f ? amax / 127.0f : 1.0f;
     const float inv = 1.0f / sc;
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-        const int c = threadIdx.x + q * kEwThreads;
+    for (int q = 0; q < NCH; q++) {
+        const int c = lane + q * 64;
         if (c < chunks) {
             float f[8];
             widen8<T>(v[q], f);
@@ -311,11 +313,29 @@ __global__ __launch_bounds__(kEwThreads) void dynquant_rows_vec_kernel(int8_t *y
             *(uint2 *)(y + base + (size_t)c * 8) = uint2{b[0], b[1]};
         }
     }
-    if (threadIdx.x == 0) Elem<T>::st(y_scale, blockIdx.x, sc);
+    if (lane == 0) {
+        Elem<T>::st(y_scale, row, sc);
+        if (y_zp) y_zp[row] = 0;
+    }
+}
+
+template <typename T, bool NORM>
+static int dynquant_rows_vec(int8_t *y, void *y_scale, int8_t *y_zp, const void *x, const void *w, int rows, int dim, float eps, hipStream_t s) {
+    const dim3 grid((rows + kEwThreads / 64 - 1) / (kEwThreads / 64)), block(kEwThreads);
+    const int nch = (dim / 8 + 63) / 64;
+    if (nch <= 4)
+        MYNN_LAUNCH((dynquant_rows_vec_kernel<T, NORM, 4>), grid, block, 0, s, y, (T *)y_scale, y_zp, (const T *)x, (const T *)w, rows, dim, eps);
+    else if (nch <= 8)
+        MYNN_LAUNCH((dynquant_rows_vec_kernel<T, NORM, 8>), grid, block, 0, s, y, (T *)y_scale, y_zp, (const T *)x, (const T *)w, rows, dim, eps);
+    else if (nch <= 12)
+        MYNN_LAUNCH((dynquant_rows_vec_kernel<T, NORM, 12>), grid, block, 0, s, y, (T *)y_scale, y_zp, (const T *)x, (const T *)w, rows, dim, eps);
+    else
+        MYNN_LAUNCH((dynquant_rows_vec_kernel<T, NORM, 16>), grid, block, 0, s, y, (T *)y_scale, y_zp, (const T *)x, (const T *)w, rows, dim, eps);
+    return launch_status("dynquant_rows_vec_kernel");
 }
 
 static bool dynquant_vec_ok(const void *y, const void *x, int dim) {
-    return dim % 8 == 0 && dim <= 8 * 4 * kEwThreads && aligned16(x) && ((uintptr_t)y & 7) == 0;
+    return dim % 8 == 0 && dim <= 8 * 64 * 16 && aligned16(x) && ((uintptr_t)y & 7) == 0;
 }
 
 // RMSNorm followed by symmetric per-row quantisation (the pair RMSNormalization -> DynamicQuantizeLinear of a
@@ -325,9 +345,7 @@ int rms_norm_dynquant(int8_t *y, void *y_scale, void *scratch_norm, const void *
     if (dtype != MYNN_F32 && dynquant_vec_ok(y, x, dim) && aligned16(w)) {
         return dispatch_dtype16(dtype, [&](auto *t) {
             using T = std::remove_pointer_t<decltype(t)>;
-            MYNN_LAUNCH((dynquant_rows_vec_kernel<T, true>), dim3(rows), dim3(kEwThreads), 0, s, y, (T *)y_scale, (const T *)x,
-                        (const T *)w, dim, eps);
-            return launch_status("dynquant_rows_vec_kernel");
+            return dynquant_rows_vec<T, true>(y, y_scale, nullptr, x, w, rows, dim, eps, s);
         });
     }
     int rc = mynn_rms_norm(scratch_norm, x, w, rows, dim, eps, dtype, s);
@@ -541,10 +559,8 @@ extern "C" int mynn_dynamic_quantize_linear(void *y, void *y_scale, void *y_zero
         using T = std::remove_pointer_t<decltype(t)>;
         if constexpr (sizeof(T) == 2) {
             if (symmetric && dynquant_vec_ok(y, x, inner_size)) {
-                MYNN_LAUNCH((dynquant_rows_vec_kernel<T, false>), dim3(axis_dim), dim3(kEwThreads), 0, as_stream(s), (int8_t *)y,
-                            (T *)y_scale, (const T *)x, (const T *)nullptr, inner_size, 0.f);
-                if (y_zero_point) MYNN_HIP(hipMemsetAsync(y_zero_point, 0, axis_dim, as_stream(s)));
-                return launch_status("dynquant_rows_vec_kernel");
+                return dynquant_rows_vec<T, false>((int8_t *)y, y_scale, (int8_t *)y_zero_point, x, nullptr, axis_dim, inner_size, 0.f,
+                                                   as_stream(s));
             }
         }
         if (symmetric)
