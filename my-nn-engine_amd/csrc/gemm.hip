@@ -8,10 +8,12 @@
 //
 // Two steps: (1) W_T[n,k] = T(wq[n,k] * scale[n]) -- a pure streaming pass (~3 bytes moved per
 // weight) into a library-owned workspace per call, or once into a resident copy that a prefill
-// executor keeps; (2) C = A . W_T^T with v_mfma_f32_32x32x16_{f16,bf16}: 256x128 output tile per
-// workgroup of 8 waves (4x2, 64x64 per wave = 2x2 MFMA tiles), K step 32, operands staged through
-// padded LDS tiles (conflict-free 128-bit reads), two register stages of global loads in flight.
+// executor keeps; (2) C = A . W_T^T with v_mfma_f32_32x32x16_{f16,bf16}.  Grids of at least one round
+// of 256 x 256 tiles with K % 64 == 0 run gemm_nt_dma_kernel (operand tiles loaded straight into LDS,
+// swizzled, 256 x 256 or 256 x 320 per workgroup of 8 waves); the rest runs gemm_nt_mfma_kernel (256 x 128
+// or 256 x 256, K step 32, operands staged through registers into padded LDS tiles, any K % 8 == 0).
 // The store can add a residual (o_proj, down_proj) or apply SwiGLU to interleaved gate/up columns.
+// The int8 form of gemm_nt_dma_kernel is QuantizedMatMul for large grids (qgemm_dma).
 #include "kernels.h"
 #include "mfma.h"
 

@@ -47,7 +47,7 @@ int interleave_row_groups(void *dst, const void *src, size_t rows, size_t row_by
 bool qgemm_dma_supported(int M, int N, int K);
 int qgemm_dma(void *out, int32_t *acc_out, const int8_t *lhs, const void *lhs_scale, const int8_t *rhs, const void *rhs_scale,
               const void *res, int M, int N, int K, int dtype, int epi, hipStream_t s);
-void gemm_set_tile(int which);  // 0 heuristic, 1 = 256x128, 2 = 256x256 workgroup tile
+void gemm_set_tile(int which);  // 0 heuristic; 1 = 256x128, 2 = 256x256 (register staged); 3 = 256x256, 4 = 256x320 (direct to LDS)
 int gemm_nt_mfma(void *out, const void *act, const void *wt, const void *res, int M, int N, int K, int dtype, int epi,
                  hipStream_t s);
 // the two halves of dequant_gemm_mfma: W_T = T(wq * scale) into the library workspace, then out = act . W_T^T
