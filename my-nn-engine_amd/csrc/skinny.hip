@@ -28,9 +28,12 @@ constexpr int kSkinnyLd = kSkinnyK + 8;  // LDS row stride of the activation chu
 // wave needs, in the order its four load instructions want them (instruction j, lane l -> 16 bytes at
 // j*1024 + l*16): one sequential stream per wave instead of 128-byte pieces of 32 rows a row pitch apart
 // (measured 2.3 TB/s for the row-major form: DRAM pages are opened for 128 bytes each).
-template <typename T, int MT, bool PACKED>
+// FEPI < 0: partial sums to `part` (several K ranges, summed by skinny_reduce_kernel).  FEPI = GEMM_*: the
+// workgroup covers the whole K range and stores the finished output itself (scale, residual or SwiGLU).
+template <typename T, int MT, bool PACKED, int FEPI>
 __global__ __launch_bounds__(kSkinnyThreads) void skinny_gemm_kernel(float *part, const T *act, const int8_t *wq, int M,
-                                                                    int N, int K, int iters_per_split) {
+                                                                    int N, int K, int iters_per_split, T *out,
+                                                                    const T *scale, const T *res) {
     // the activation chunk [32*MT rows][128 k] of the current step, shared by the four waves
     __shared__ __align__(16) uint16_t a_s[2][MT * 32 * kSkinnyLd];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -118,6 +121,38 @@ __global__ __launch_bounds__(kSkinnyThreads) void skinny_gemm_kernel(float *part
 
     // D[n][m]: lane holds column m = lane%32 and rows n = 8*(e/4) + 4*(lane/32) + e%4: four consecutive n
     if (n0 >= N) return;
+    if constexpr (FEPI >= 0) {
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+            const int m = mt * 32 + r;
+            if (m >= M) continue;
+#pragma unroll
+            for (int e4 = 0; e4 < 4; e4++) {
+                const int n = n0 + e4 * 8 + h * 4;
+                float y[4];
+#pragma unroll
+                for (int x = 0; x < 4; x++) y[x] = n + x < N ? acc[mt][e4 * 4 + x] * Elem<T>::ld(scale, n + x) : 0.f;
+                if constexpr (FEPI == GEMM_SWIGLU) {
+                    // rows 2i / 2i+1 of the weight are gate_i / up_i; out is [M, N/2]
+                    T *o = out + (size_t)m * (N >> 1) + (n >> 1);
+#pragma unroll
+                    for (int x = 0; x < 2; x++) {
+                        if (n + 2 * x + 1 < N) {
+                            const float g = Elem<T>::rnd(y[2 * x]), u = Elem<T>::rnd(y[2 * x + 1]);
+                            const float sig = 1.0f / (1.0f + expf(-g));
+                            Elem<T>::st(o, x, (g * sig) * u);
+                        }
+                    }
+                } else {
+                    const size_t at = (size_t)m * N + n;
+#pragma unroll
+                    for (int x = 0; x < 4; x++)
+                        if (n + x < N) Elem<T>::st(out, at + x, y[x]);
+                }
+            }
+        }
+        return;
+    }
     float *dst = part + (size_t)blockIdx.y * M * N;
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
@@ -189,6 +224,7 @@ bool skinny_gemm_supported(int M, int N, int K) { return M >= 16 && M <= 64 && K
 // K ranges: enough waves to keep ~1000 in flight, each with at least as many steps as it has stages
 static int skinny_ksplit(int N, int K) {
     const int waves_n = (N + 31) / 32, iters = K / kSkinnyK;
+    if (waves_n >= 768) return 1;  // three waves per CU already: one launch that stores the finished output
     int ks = (1024 + waves_n - 1) / waves_n;
     if (ks > iters / kSkinnyStages) ks = iters / kSkinnyStages;
     return ks < 1 ? 1 : ks;
@@ -209,15 +245,25 @@ int dequant_gemm_skinny(void *out, const void *act, const int8_t *wq, bool packe
     const size_t n_out = (size_t)M * (epi == GEMM_SWIGLU ? N / 2 : N);
     return dispatch_dtype16(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
-        if (M <= 32 && packed)
-            MYNN_LAUNCH((skinny_gemm_kernel<T, 1, true>), grid, dim3(kSkinnyThreads), 0, s, scratch, (const T *)act, wq, M, N, K, ips);
-        else if (M <= 32)
-            MYNN_LAUNCH((skinny_gemm_kernel<T, 1, false>), grid, dim3(kSkinnyThreads), 0, s, scratch, (const T *)act, wq, M, N, K, ips);
-        else if (packed)
-            MYNN_LAUNCH((skinny_gemm_kernel<T, 2, true>), grid, dim3(kSkinnyThreads), 0, s, scratch, (const T *)act, wq, M, N, K, ips);
-        else
-            MYNN_LAUNCH((skinny_gemm_kernel<T, 2, false>), grid, dim3(kSkinnyThreads), 0, s, scratch, (const T *)act, wq, M, N, K, ips);
-        int rc = launch_status("skinny_gemm_kernel");
+        auto gemm = [&](auto fepi) {
+            constexpr int FEPI = decltype(fepi)::value;
+            T *o = (T *)out;
+            const T *sc = (const T *)scale, *rs = (const T *)res;
+            if (M <= 32 && packed)
+                MYNN_LAUNCH((skinny_gemm_kernel<T, 1, true, FEPI>), grid, dim3(kSkinnyThreads), 0, s, scratch, (const T *)act, wq, M, N, K, ips, o, sc, rs);
+            else if (M <= 32)
+                MYNN_LAUNCH((skinny_gemm_kernel<T, 1, false, FEPI>), grid, dim3(kSkinnyThreads), 0, s, scratch, (const T *)act, wq, M, N, K, ips, o, sc, rs);
+            else if (packed)
+                MYNN_LAUNCH((skinny_gemm_kernel<T, 2, true, FEPI>), grid, dim3(kSkinnyThreads), 0, s, scratch, (const T *)act, wq, M, N, K, ips, o, sc, rs);
+            else
+                MYNN_LAUNCH((skinny_gemm_kernel<T, 2, false, FEPI>), grid, dim3(kSkinnyThreads), 0, s, scratch, (const T *)act, wq, M, N, K, ips, o, sc, rs);
+            return launch_status("skinny_gemm_kernel");
+        };
+        // the whole K range in one workgroup: no partial sums, no second launch (the wide shapes: gate/up and
+        // lm_head; a residual store never meets this width, it keeps the two-launch form)
+        if (ks_used == 1 && epi == GEMM_SWIGLU) return gemm(std::integral_constant<int, GEMM_SWIGLU>{});
+        if (ks_used == 1 && epi == GEMM_PLAIN) return gemm(std::integral_constant<int, GEMM_PLAIN>{});
+        int rc = gemm(std::integral_constant<int, -1>{});
         if (rc) return rc;
         const dim3 rg((unsigned)((n_out + 255) / 256));
         if (epi == GEMM_RESIDUAL)

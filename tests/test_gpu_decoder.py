@@ -319,6 +319,27 @@ def test_few_row_gemm_prefill_chunk_vs_oracle(g, dt, rows):
     dec.close()
 
 
+WIDE = dict(SMALL, n_layers=1, ffn=12288, vocab=24576)  # gate/up and lm_head wide enough to skip the K split
+
+
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+@pytest.mark.parametrize("rows", [32, 48])
+def test_few_row_gemm_unsplit_store_vs_oracle(g, dt, rows):
+    """Few-row int8 GEMM on matrices of >= 24576 rows: one launch per linear that applies the scale (and
+    SwiGLU) itself instead of writing partial sums for a second one."""
+    cfg, w = llm_weights.synthetic_int8(WIDE, dt, seed=77)
+    dw = dev_weights(g, w, dt)
+    pre = g.mynn.Decoder(cfg, dw, seq_q=rows)
+    ids = np.random.default_rng(rows).integers(0, cfg["vocab"], rows)
+    names = [k[0] for k in pre.profile(ids, np.arange(rows), 0, rows)]
+    assert "linear_gateup_swiglu" in names
+    ref = orc.Model(cfg, w)
+    want = ref.forward(ids, np.arange(rows), 0, rows, True)
+    _, got = pre.step(ids, np.arange(rows), 0, rows, want_logits=True)
+    assert max_err_rel_to_max(g.f32(got, dt), g.f32(want, dt)) <= 1e-2
+    pre.close()
+
+
 @pytest.mark.parametrize("dt", [orc.F16])
 def test_batched_decode_equals_independent_sequences(g, dt):
     """Batch 16 decode (the shape of the batched-serving config, scaled down): every sequence must follow
