@@ -70,6 +70,40 @@ def test_int8_decoder_step_logits_and_kv_vs_oracle(g, dt):
     dec.close()
 
 
+SHORT_CACHE = {
+    64: dict(SMALL, n_layers=2, hidden=256, n_heads=4, n_kv_heads=2, head_dim=64, max_seq=512),
+    128: dict(SMALL, n_layers=2, hidden=256, n_heads=2, n_kv_heads=1, head_dim=128, max_seq=256),
+}
+
+
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+@pytest.mark.parametrize("D", [64, 128])
+def test_decode_attention_short_cache_every_pass_vs_oracle(g, dt, D):
+    """Head dims 64 and 128 with a cache one workgroup covers (512 / 256 rows): the decode step's attention
+    keeps every key in registers, a lane group per key and pass.  Token by token through most of the cache,
+    so that every pass and every wave gets keys, and the rows the kernel appends, against the oracle."""
+    cfg, w = llm_weights.synthetic_int8(SHORT_CACHE[D], dt, seed=13 + D)
+    ref = orc.Model(cfg, w)
+    dec = g.mynn.Decoder(cfg, dev_weights(g, w, dt))
+    n = cfg["max_seq"] - 5
+    toks = np.random.default_rng(D).integers(0, cfg["vocab"], n)
+    for i, t in enumerate(toks):
+        want = ref.forward([t], [i], i, i + 1, False)
+        if i % 37 == 0 or i >= n - 3:
+            nxt, got = dec.step([t], [i], i, i + 1, want_logits=True)
+            assert max_err_rel_to_max(g.f32(got, dt), g.f32(want, dt)) <= 1e-2, i
+            assert nxt[0] == orc.argmax_last(got[0], dt)
+        else:
+            dec.step([t], [i], i, i + 1)
+    for l in range(cfg["n_layers"]):
+        k_ref, v_ref = ref.kv_cache(l)
+        k_gpu, v_gpu = g.to_host(dec.kv[l][0])[0], g.to_host(dec.kv[l][1])[0]
+        assert max_err_rel_to_max(g.f32(k_gpu[:, :n], dt), g.f32(k_ref[:, :n], dt)) <= 1e-2
+        assert max_err_rel_to_max(g.f32(v_gpu[:, :n], dt), g.f32(v_ref[:, :n], dt)) <= 1e-2
+        assert not k_gpu[:, n:].any() and not v_gpu[:, n:].any()
+    dec.close()
+
+
 @pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
 def test_int8_greedy_tokens_vs_oracle_small(g, dt):
     """Greedy ids of the HIP path against the oracle on a small int8 model.  The oracle is
