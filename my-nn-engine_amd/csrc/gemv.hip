@@ -165,8 +165,14 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(GemvParams 
     const int nchunks = K >> 4;
     int g = blockIdx.x * kGemvWaves + wave;
 
-    U4 w[R][NC];
-    auto load_group = [&](int gg) {
+    // one row group's operands: R x NC weight chunks per lane, plus, in lane r < R, what the store of row r
+    // needs (scale, the next row's scale for SwiGLU, the residual) -- fetched with the weights, not after the sum
+    struct Group {
+        U4 w[R][NC];
+        float sc, sc1, res;
+    };
+    const T *scale = (const T *)p.scale;
+    auto load_group = [&](int gg, Group &G) {
 #pragma unroll
         for (int r = 0; r < R; r++) {
             const int row = gg * R + r < N ? gg * R + r : N - 1;
@@ -174,12 +180,17 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(GemvParams 
 #pragma unroll
             for (int j = 0; j < NC; j++) {
                 const int c = lane + j * kWave;
-                if (c < nchunks) w[r][j] = __builtin_nontemporal_load(&wrow[c]);
-                else w[r][j] = U4{0u, 0u, 0u, 0u};
+                if (c < nchunks) G.w[r][j] = __builtin_nontemporal_load(&wrow[c]);
+                else G.w[r][j] = U4{0u, 0u, 0u, 0u};
             }
         }
+        const int row = min(gg * R + min(lane, R - 1), N - 1);
+        G.sc = Elem<T>::ld(scale, row);
+        G.sc1 = EPI == EPI_SWIGLU ? Elem<T>::ld(scale, min(row + 1, N - 1)) : 0.f;
+        G.res = EPI == EPI_RESIDUAL ? Elem<T>::ld((const T *)p.residual, row) : 0.f;
     };
-    if (g < groups) load_group(g);  // in flight while the activation is staged
+    Group ga;
+    if (g < groups) load_group(g, ga);  // in flight while the activation is staged
 
     // ---- stage: thread t owns the 8-element pieces t, t + 256, ... of the row
     {
@@ -187,11 +198,13 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(GemvParams 
         const int npieces = K >> 3;
         constexpr int PMAX = (NC * 1024 / 8 + kGemvThreads - 1) / kGemvThreads;  // pieces per thread
         float f[PMAX][8];
+        U4 nwv[NORM ? PMAX : 1];  // the norm weights of this thread's pieces, fetched with the activation
         float ss = 0.f;
 #pragma unroll
         for (int q = 0; q < PMAX; q++) {
             const int pc = tid + q * kGemvThreads;
             if (pc < npieces) {
+                if constexpr (NORM) nwv[q] = ((const U4 *)p.norm_w)[pc];
                 widen8<T>(ap[pc], f[q]);
                 if constexpr (NORM) {
 #pragma unroll
@@ -215,7 +228,7 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(GemvParams 
             if (pc < npieces) {
                 if constexpr (NORM) {
                     float nw[8];
-                    widen8<T>(((const U4 *)p.norm_w)[pc], nw);
+                    widen8<T>(nwv[q], nw);
 #pragma unroll
                     for (int i = 0; i < 8; i++) f[q][i] = Elem<T>::rnd((f[q][i] * inv) * nw[i]);
                 }
@@ -227,12 +240,8 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(GemvParams 
     }
     __syncthreads();
 
-    const T *scale = (const T *)p.scale;
     T *out = (T *)p.out;
-    bool loaded = true;
-    for (; g < groups; g += total_waves) {
-        if (!loaded) load_group(g);
-        loaded = false;
+    auto compute = [&](int gg, Group &G) {
         float acc[R];
 #pragma unroll
         for (int r = 0; r < R; r++) acc[r] = 0.f;
@@ -250,8 +259,8 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(GemvParams 
 #pragma unroll
                 for (int r = 0; r < R; r++) {
                     float wf[16];
-                    pin(w[r][j]);
-                    widen16_i8(w[r][j], wf);
+                    pin(G.w[r][j]);
+                    widen16_i8(G.w[r][j], wf);
 #pragma unroll
                     for (int i = 0; i < 16; i++) acc[r] = fmaf(a[i], wf[i], acc[r]);
                 }
@@ -259,13 +268,13 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(GemvParams 
         }
 #pragma unroll
         for (int r = 0; r < R; r++) acc[r] = wave_sum(acc[r]);
-        const int row0 = g * R;
+        const int row0 = gg * R;
         if constexpr (EPI == EPI_SWIGLU) {
 #pragma unroll
             for (int r = 0; r < R; r += 2) {
                 if (lane == r && row0 + r + 1 < N) {
-                    float gt = Elem<T>::rnd(acc[r] * Elem<T>::ld(scale, row0 + r));
-                    float up = Elem<T>::rnd(acc[r + 1] * Elem<T>::ld(scale, row0 + r + 1));
+                    float gt = Elem<T>::rnd(acc[r] * G.sc);
+                    float up = Elem<T>::rnd(acc[r + 1] * G.sc1);
                     float sig = 1.0f / (1.0f + expf(-gt));
                     Elem<T>::st(out, (size_t)((row0 + r) >> 1), (gt * sig) * up);
                 }
@@ -274,20 +283,24 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(GemvParams 
 #pragma unroll
             for (int r = 0; r < R; r++) {
                 if (lane == r && row0 + r < N) {
-                    float y = acc[r] * Elem<T>::ld(scale, row0 + r);
-                    if constexpr (EPI == EPI_RESIDUAL) y = Elem<T>::rnd(y) + Elem<T>::ld((const T *)p.residual, row0 + r);
+                    float y = acc[r] * G.sc;
+                    if constexpr (EPI == EPI_RESIDUAL) y = Elem<T>::rnd(y) + G.res;
                     Elem<T>::st(out, row0 + r, y);
                 }
             }
         }
+    };
+    bool loaded = true;
+    for (; g < groups; g += total_waves) {
+        if (!loaded) load_group(g, ga);
+        loaded = false;
+        compute(g, ga);
     }
 }
-
-// waves are spread so that every wave gets the same number of row groups (no tail wave)
 template <typename T, int R, int NC, int EPI, bool NORM>
 static int launch_gemv1(const GemvParams &p, hipStream_t s) {
     const int groups = (p.N + R - 1) / R;
-    const int max_waves = 256 * 16;  // four resident waves per SIMD (measured best of 8/16/32)
+    const int max_waves = 256 * 16;  // four resident waves per SIMD (measured best of 8/16/24/32 per CU)
     const int passes = (groups + max_waves - 1) / max_waves;
     int waves = (groups + passes - 1) / passes;
     const int blocks = (waves + kGemvWaves - 1) / kGemvWaves;
