@@ -380,6 +380,15 @@ __global__ __launch_bounds__(1024) void argmax_last_kernel(int32_t *out, const T
     __shared__ float sv[16];
     __shared__ int si[16];
     const T *row = logits + (size_t)blockIdx.x * n;
+    // the loop state this launch moves on: read now, so that the tail is stores only
+    int st_step = 0, st_past = 0, st_active = 0;
+    int64_t st_pos = 0;
+    if (adv.ids && threadIdx.x == 0) {
+        st_step = *adv.step;
+        st_pos = adv.pos[0];
+        st_past = *adv.past;
+        st_active = *adv.active;
+    }
     float bv = -INFINITY;
     int bi = -1;
     if constexpr (sizeof(T) == 2) {
@@ -408,13 +417,12 @@ __global__ __launch_bounds__(1024) void argmax_last_kernel(int32_t *out, const T
             if (si[w] >= 0) argmax_take(bv, bi, sv[w], si[w]);
         out[blockIdx.x] = bi;
         if (adv.ids) {
-            const int i = *adv.step;
-            if (i < adv.cap) adv.tokens[i] = bi;
-            *adv.step = i + 1;
+            if (st_step < adv.cap) adv.tokens[st_step] = bi;
+            *adv.step = st_step + 1;
             adv.ids[0] = bi;
-            adv.pos[0] += 1;
-            *adv.past += 1;
-            *adv.active += 1;
+            adv.pos[0] = st_pos + 1;
+            *adv.past = st_past + 1;
+            *adv.active = st_active + 1;
         }
     }
 }
