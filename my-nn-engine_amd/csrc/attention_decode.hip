@@ -343,6 +343,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_short_kernel(AttnPar
     for (int e = 0; e < 8; e++) o[e] = 0.f;
 #pragma unroll
     for (int i = 0; i < kShortPasses; i++) {
+        if (i * KPP >= bound) break;  // no wave has keys in this pass or a later one
         const int key = i * KPP + wave * GPW + grp;
         float kf[8], vf[8];
         widen8<T>(kreg[i], kf);
