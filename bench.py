@@ -380,9 +380,15 @@ def main():
     prompt = rng.integers(0, cfg["vocab"], PROMPT_LEN).tolist()
 
     # prompt through the decode path, token by token (the reference's path without a prefill session)
+    # (each of these steps is a host round trip: inputs up, graph replay, token down -- timed for the record)
     first = None
+    t_host = None
     for i, t in enumerate(prompt):
+        if i == 16:
+            torch.cuda.synchronize()
+            t_host = time.perf_counter()
         first, _ = dec.step([t], [i], i, i + 1)
+    host_tok_s = (PROMPT_LEN - 16) / (time.perf_counter() - t_host)
     first = first[0]
 
     if W > 0:
@@ -423,6 +429,7 @@ def main():
                                "fed through the decode path then %d generated (timed: the generated tokens)" % K,
                    "prompt_len": PROMPT_LEN, "max_seq": cfg["max_seq"], "launches_per_step": stats["launches_per_step"],
                    "hipgraph": stats["graph"], "seed": args.seed,
+                   "host_roundtrip_tok_s": round(host_tok_s, 1),
                    "step_algorithmic_bytes": step_bytes,
                    "step_hbm_frac": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
