@@ -110,6 +110,41 @@ def test_streaming_decode_attention_vs_oracle(g, dt, B, Hq, Hkv, D, L, active):
         assert max_abs_rel(g.f32(got, dt), exact) <= 1e-2
 
 
+def test_decode_attention_seeded_shape_sweep(g):
+    """48 seeded shapes across the dispatch boundaries of the decode kernels (caches of 1..700 rows, shorter
+    and longer than a 32-key tile; batch x heads x context on either side of the streaming kernel's threshold;
+    1..8 query heads per kv head; head dims 32/64/128; the length passed by value or read on the device; the
+    tail of the cache poisoned) against the f64 formula."""
+    import torch
+
+    rng = np.random.default_rng(2024)
+    for case in range(48):
+        dt = [orc.F16, orc.BF16][case % 2]
+        D = [32, 64, 128][int(rng.integers(0, 3))]
+        Hkv = int(rng.choice([1, 2, 4, 8]))
+        G = int(rng.choice([1, 2, 4, 8]))
+        Hq = Hkv * G
+        L = int(rng.choice([1, 3, 17, 31, 32, 33, 64, 100, 257, 512, 700]))
+        B = int(rng.choice([1, 2, 5, 16, 40])) if L * Hkv < 3000 else int(rng.choice([1, 3, 12]))
+        active = int(rng.integers(1, L + 1))
+        q = orc.to_storage(rng.standard_normal((B, Hq, 1, D)), dt)
+        k = orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt)
+        v = orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt)
+        if active < L:
+            k[:, :, active:] = orc.to_storage(np.full((B, Hkv, L - active, D), np.nan), dt)
+            v[:, :, active:] = orc.to_storage(np.full((B, Hkv, L - active, D), np.nan), dt)
+        exact = orc.attention_f64(q, k, v, dt, D ** -0.5, False, active)
+        dq, dk, dv = g.to_dev(q, dt), g.to_dev(k, dt), g.to_dev(v, dt)
+        if case % 3 == 0:
+            d_active = torch.tensor([active], dtype=torch.int32, device="cuda")
+            got = g.mynn.attention(dq, dk, dv, D ** -0.5, False, active=L, d_active=d_active)
+        else:
+            got = g.mynn.attention(dq, dk, dv, D ** -0.5, False, active)
+        got = g.f32(g.to_host(got), dt)
+        assert not np.isnan(got).any(), (case, B, Hq, Hkv, D, L, active)
+        assert max_err_rel_to_max(got, exact) <= (4e-3 if dt == orc.BF16 else 1e-3), (case, B, Hq, Hkv, D, L, active)
+
+
 @pytest.mark.parametrize("dt", [orc.F32, orc.F16, orc.BF16])
 def test_attention_invariants_on_gpu(g, dt):
     rng = np.random.default_rng(11)

@@ -57,6 +57,31 @@ def test_dequant_matmul_mfma_vs_oracle(g, dt, M, N, K):
     assert max_abs_rel(g.f32(got, dt), exact) <= 1e-2
 
 
+def test_dequant_matmul_seeded_shape_sweep(g):
+    """40 seeded shapes across the kernel choices of DequantMatMul (one row, a few rows, 16 and more rows on the
+    matrix cores; K a multiple of 8 or not, shorter and longer than a K step; N with tails in every tile width)
+    against the f64 closed form of the kernel each shape takes (scale after the sum below 16 rows or for odd K,
+    weights rounded to the storage type first otherwise)."""
+    rng = np.random.default_rng(77)
+    for case in range(40):
+        dt = [orc.F16, orc.BF16][case % 2]
+        M = int(rng.choice([1, 2, 3, 7, 15, 16, 17, 33, 64, 65, 130, 260]))
+        N = int(rng.choice([1, 5, 31, 64, 100, 129, 255, 256, 257, 320, 700, 1030]))
+        K = int(rng.choice([8, 16, 24, 40, 64, 72, 128, 200, 512, 1032, 2048, 12, 100]))
+        act = orc.to_storage(rng.standard_normal((M, K)), dt)
+        W = rng.integers(-127, 128, (N, K)).astype(np.int8)
+        sc = orc.to_storage(rng.uniform(1e-3, 1e-2, N), dt)
+        got = g.f32(g.to_host(g.mynn.dequant_matmul(g.to_dev(act, dt), g.to_dev(W), g.to_dev(sc, dt))), dt)
+        a64, s64 = g.f32(act, dt).astype(np.float64), g.f32(sc, dt).astype(np.float64)
+        if M >= 16 and K % 8 == 0:
+            wr = g.f32(orc.to_storage(W.astype(np.float32) * g.f32(sc, dt)[:, None], dt), dt).astype(np.float64)
+            exact = a64 @ wr.T
+        else:
+            exact = (a64 @ W.astype(np.float64).T) * s64[None, :]
+        assert got.shape == (M, N) and not np.isnan(got).any(), (case, M, N, K)
+        assert max_abs_rel(got, exact) <= 1e-2, (case, M, N, K)
+
+
 @pytest.mark.parametrize("tile", [1, 2, 3, 4])
 @pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
 @pytest.mark.parametrize("M,N,K", [(200, 300, 512), (700, 520, 128), (128, 2560, 2048), (300, 650, 64), (257, 321, 192)])
