@@ -171,13 +171,14 @@ static int linear_rows(Model &m, void *out, const void *act, const Lin &l, int M
 }
 
 // one few-row GEMM against int8 weights (two launches: products, then sum/scale/store)
+// next_norm (residual store): the weights of the RMSNorm that reads this output next; *normed = m.nrm holds it
 static int skinny_rows(Model &m, void *out, const void *act, const Lin &l, const void *packed, const void *res, int M, int epi,
-                       const char *name) {
+                       const char *name, const void *next_norm = nullptr, bool *normed = nullptr) {
     const double eb = dtype_size(m.cfg.dtype), n_out = epi == GEMM_SWIGLU ? l.N / 2 : l.N;
     note(m, name, (double)l.N * l.K + l.N * eb + (double)M * l.K * eb + (double)M * n_out * eb * (epi == GEMM_RESIDUAL ? 2 : 1),
          2.0 * M * l.N * l.K);
     return dequant_gemm_skinny(out, act, (const int8_t *)(packed ? packed : l.w), packed != nullptr, l.scale, res, M, l.N, l.K,
-                               m.cfg.dtype, epi, m.skinny_scratch, m.stream);
+                               m.cfg.dtype, epi, m.skinny_scratch, m.stream, next_norm, m.cfg.eps, m.nrm, normed);
 }
 
 // Options::quantize_activations: DynamicQuantizeLinear (per row, symmetric) then QuantizedMatMul.
@@ -234,7 +235,9 @@ static int enqueue_step(Model &m) {
         TRY(mynn_gather_rows(m.x, m.embed.w, m.d_ids, rows, V, (size_t)H * sizeof(T), s));
     }
     const float softmax_scale = 1.0f / sqrtf((float)D);
-    for (Layer &L : m.layers) {
+    bool nrm_ready = false;  // m.nrm already holds the next RMSNorm's output (written by the launch that finished its input)
+    for (size_t li = 0; li < m.layers.size(); li++) {
+        Layer &L = m.layers[li];
         // ---- attention block
         if (fused) {
             note(m, "gemv_norm_qkv", (double)L.qkv.N * H + L.qkv.N * eb + 2 * H * eb + L.qkv.N * eb);
@@ -242,8 +245,11 @@ static int enqueue_step(Model &m) {
         } else if (m.w8a8_fused) {
             TRY(qlinear_fused(m, m.qkv, m.x, L.norm1, L.qkv.w, L.qkv.scale, nullptr, rows, L.qkv.N, H, GEMM_PLAIN, "qlinear_qkv"));
         } else {
-            note(m, "rms_norm", 2.0 * rows * H * eb + H * eb);
-            TRY(mynn_rms_norm(m.nrm, m.x, L.norm1, rows, H, c.eps, c.dtype, s));
+            if (!nrm_ready) {
+                note(m, "rms_norm", 2.0 * rows * H * eb + H * eb);
+                TRY(mynn_rms_norm(m.nrm, m.x, L.norm1, rows, H, c.eps, c.dtype, s));
+            }
+            nrm_ready = false;
             if (m.skinny) TRY(skinny_rows(m, m.qkv, m.nrm, L.qkv, L.pk_qkv, nullptr, rows, GEMM_PLAIN, "linear_qkv"));
             else if (w8a8) TRY(linear_w8a8(m, m.qkv, m.nrm, L.qkv, rows, true, "qlinear_qkv"));
             else if (m.resident16) TRY(gemm_rows(m, m.qkv, m.nrm, L.wt_qkv, nullptr, rows, L.qkv.N, H, GEMM_PLAIN, "linear_qkv"));
@@ -286,11 +292,15 @@ static int enqueue_step(Model &m) {
             note(m, "gemv_down_residual", (double)H * F + H * eb + F * eb + 2 * H * eb);
             TRY(gemv_residual<T>(m.x, m.hmid, (const int8_t *)L.down.w, L.down.scale, m.x2, H, F, s));
         } else if (m.skinny) {
-            TRY(skinny_rows(m, m.x2, m.attn, L.o, L.pk_o, m.x, rows, GEMM_RESIDUAL, "linear_o_residual"));
-            note(m, "rms_norm", 2.0 * rows * H * eb + H * eb);
-            TRY(mynn_rms_norm(m.nrm, m.x2, L.norm2, rows, H, c.eps, c.dtype, s));
+            bool normed = false;
+            TRY(skinny_rows(m, m.x2, m.attn, L.o, L.pk_o, m.x, rows, GEMM_RESIDUAL, "linear_o_residual", L.norm2, &normed));
+            if (!normed) {
+                note(m, "rms_norm", 2.0 * rows * H * eb + H * eb);
+                TRY(mynn_rms_norm(m.nrm, m.x2, L.norm2, rows, H, c.eps, c.dtype, s));
+            }
             TRY(skinny_rows(m, m.hmid, m.nrm, L.gu, L.pk_gu, nullptr, rows, GEMM_SWIGLU, "linear_gateup_swiglu"));
-            TRY(skinny_rows(m, m.x, m.hmid, L.down, L.pk_down, m.x2, rows, GEMM_RESIDUAL, "linear_down_residual"));
+            const void *next_norm = li + 1 < m.layers.size() ? m.layers[li + 1].norm1 : m.final_norm;
+            TRY(skinny_rows(m, m.x, m.hmid, L.down, L.pk_down, m.x2, rows, GEMM_RESIDUAL, "linear_down_residual", next_norm, &nrm_ready));
         } else if (m.w8a8_fused) {
             TRY(qlinear_fused(m, m.x2, m.attn, nullptr, L.o.w, L.o.scale, m.x, rows, H, QD, GEMM_RESIDUAL, "qlinear_o_residual"));
             TRY(qlinear_fused(m, m.hmid, m.x2, L.norm2, L.q8_gu, L.q8_gu_scale, nullptr, rows, 2 * F, H, GEMM_SWIGLU, "qlinear_gateup_swiglu"));
@@ -336,8 +346,10 @@ static int enqueue_step(Model &m) {
     } else if (m.w8a8_fused) {
         TRY(qlinear_fused(m, m.logits, m.x, m.final_norm, m.lm_head.w, m.lm_head.scale, nullptr, rows, V, H, GEMM_PLAIN, "qlinear_lm_head"));
     } else {
-        note(m, "rms_norm", 2.0 * rows * H * eb + H * eb);
-        TRY(mynn_rms_norm(m.nrm, m.x, m.final_norm, rows, H, c.eps, c.dtype, s));
+        if (!nrm_ready) {
+            note(m, "rms_norm", 2.0 * rows * H * eb + H * eb);
+            TRY(mynn_rms_norm(m.nrm, m.x, m.final_norm, rows, H, c.eps, c.dtype, s));
+        }
         if (m.skinny) TRY(skinny_rows(m, m.logits, m.nrm, m.lm_head, m.pk_lm_head, nullptr, rows, GEMM_PLAIN, "linear_lm_head"));
         else if (w8a8) TRY(linear_w8a8(m, m.logits, m.nrm, m.lm_head, rows, true, "qlinear_lm_head"));
         else if (m.resident16) TRY(gemm_rows(m, m.logits, m.nrm, m.wt_lm_head, nullptr, rows, V, H, GEMM_PLAIN, "linear_lm_head"));

@@ -27,7 +27,8 @@ size_t skinny_scratch_bytes(int M, int N, int K);
 size_t skinny_packed_bytes(int N, int K);
 int skinny_pack_weight(void *dst, const int8_t *wq, int N, int K, hipStream_t s);
 int dequant_gemm_skinny(void *out, const void *act, const int8_t *wq, bool packed, const void *scale, const void *res, int M,
-                        int N, int K, int dtype, int epi, float *scratch, hipStream_t s);
+                        int N, int K, int dtype, int epi, float *scratch, hipStream_t s, const void *norm_w = nullptr,
+                        float eps = 0.f, void *nrm_out = nullptr, bool *normed = nullptr);
 
 // matrix-core GEMM pieces.  A dequantised weight is [N, Kp] of the 16-bit type, Kp = K rounded up to 64,
 // zero padded (gemm_weight_bytes); dequant_weight_rows writes one (group/which: see gemm.hip), and

@@ -219,6 +219,60 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(T *out, const float 
     }
 }
 
+// The residual form of the reduction followed by the RMSNorm of the row it completes (the o projection before
+// the MLP's norm, the down projection before the next layer's): one workgroup per output row, four columns per
+// thread, every load issued before the first sum; x_out = T(T(sum * scale) + res), nrm_out = T((x * inv) * w)
+// with inv = 1 / sqrt(mean(x^2) + eps) over the stored (rounded) x, as the separate operators compute them.
+constexpr int kReduceNormThreads = 1024, kReduceNormMaxSplit = 8;
+template <typename T>
+__global__ __launch_bounds__(kReduceNormThreads) void skinny_reduce_norm_kernel(T *x_out, T *nrm_out, const float *part, const T *scale,
+                                                                              const T *res, const T *norm_w, int M, int N, int ksplit,
+                                                                              float eps) {
+    __shared__ float red[kReduceNormThreads / 64];
+    const int m = blockIdx.x, c0 = threadIdx.x * 4;
+    const bool live = c0 < N;
+    float4 pv[kReduceNormMaxSplit];
+    uint2 sc2 = uint2{0u, 0u}, rs2 = sc2, nw2 = sc2;
+#pragma unroll
+    for (int s = 0; s < kReduceNormMaxSplit; s++) {
+        pv[s] = float4{0.f, 0.f, 0.f, 0.f};
+        if (live && s < ksplit) pv[s] = *(const float4 *)(part + ((size_t)s * M + m) * N + c0);
+    }
+    if (live) {
+        sc2 = *(const uint2 *)(scale + c0);
+        rs2 = *(const uint2 *)(res + (size_t)m * N + c0);
+        nw2 = *(const uint2 *)(norm_w + c0);
+    }
+    float t[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < kReduceNormMaxSplit; s++) {  // the order of skinny_reduce_kernel: K ranges ascending
+        if (s < ksplit) {
+            t[0] += pv[s].x; t[1] += pv[s].y; t[2] += pv[s].z; t[3] += pv[s].w;
+        }
+    }
+    float sc[8], rs[8], nw[8], x[4];
+    widen8<T>(U4{sc2.x, sc2.y, 0u, 0u}, sc);
+    widen8<T>(U4{rs2.x, rs2.y, 0u, 0u}, rs);
+    widen8<T>(U4{nw2.x, nw2.y, 0u, 0u}, nw);
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        x[i] = Elem<T>::rnd(Elem<T>::rnd(t[i] * sc[i]) + rs[i]);
+        ss += x[i] * x[i];
+    }
+    if (live) *(uint2 *)(x_out + (size_t)m * N + c0) = uint2{pack2<T>(x[0], x[1]), pack2<T>(x[2], x[3])};
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    float tot = 0.f;
+#pragma unroll
+    for (int w = 0; w < kReduceNormThreads / 64; w++) tot += red[w];
+    const float inv = 1.0f / sqrtf(tot / (float)N + eps);
+    if (live)
+        *(uint2 *)(nrm_out + (size_t)m * N + c0) =
+            uint2{pack2<T>((x[0] * inv) * nw[0], (x[1] * inv) * nw[1]), pack2<T>((x[2] * inv) * nw[2], (x[3] * inv) * nw[3])};
+}
+
 bool skinny_gemm_supported(int M, int N, int K) { return M >= 16 && M <= 64 && K % kSkinnyK == 0 && K >= 2 * kSkinnyK && N >= 1; }
 
 // K ranges: enough waves to keep ~1000 in flight, each with at least as many steps as it has stages
@@ -231,8 +285,12 @@ static int skinny_ksplit(int N, int K) {
 }
 size_t skinny_scratch_bytes(int M, int N, int K) { return (size_t)skinny_ksplit(N, K) * M * N * sizeof(float); }
 
+// norm_w / nrm_out (optional, residual store only): also write the RMSNorm of the finished rows; *normed tells
+// whether this call did (it does when the K range is split, N % 4 == 0 and N <= 4096)
 int dequant_gemm_skinny(void *out, const void *act, const int8_t *wq, bool packed, const void *scale, const void *res, int M,
-                        int N, int K, int dtype, int epi, float *scratch, hipStream_t s) {
+                        int N, int K, int dtype, int epi, float *scratch, hipStream_t s, const void *norm_w, float eps,
+                        void *nrm_out, bool *normed) {
+    if (normed) *normed = false;
     MYNN_REQUIRE(out && act && wq && scale && scratch, MYNN_ERR_INVALID, "dequant_matmul: null operand");
     MYNN_REQUIRE(skinny_gemm_supported(M, N, K), MYNN_ERR_UNSUPPORTED, "dequant_matmul (few rows): M=%d N=%d K=%d", M, N, K);
     MYNN_REQUIRE(aligned16(act) && aligned16(wq), MYNN_ERR_INVALID, "dequant_matmul: act and wq must be 16-byte aligned");
@@ -265,6 +323,14 @@ int dequant_gemm_skinny(void *out, const void *act, const int8_t *wq, bool packe
         if (ks_used == 1 && epi == GEMM_PLAIN) return gemm(std::integral_constant<int, GEMM_PLAIN>{});
         int rc = gemm(std::integral_constant<int, -1>{});
         if (rc) return rc;
+        if (epi == GEMM_RESIDUAL && norm_w && nrm_out && normed && N % 4 == 0 && N <= 4 * kReduceNormThreads &&
+            ks_used <= kReduceNormMaxSplit && aligned16(out) && aligned16(res) && aligned16(nrm_out) && ((uintptr_t)norm_w & 7) == 0 &&
+            ((uintptr_t)scale & 7) == 0) {
+            MYNN_LAUNCH(skinny_reduce_norm_kernel<T>, dim3(M), dim3(kReduceNormThreads), 0, s, (T *)out, (T *)nrm_out, scratch,
+                        (const T *)scale, (const T *)res, (const T *)norm_w, M, N, ks_used, eps);
+            *normed = true;
+            return launch_status("skinny_reduce_norm_kernel");
+        }
         const dim3 rg((unsigned)((n_out + 255) / 256));
         if (epi == GEMM_RESIDUAL)
             MYNN_LAUNCH((skinny_reduce_kernel<T, GEMM_RESIDUAL>), rg, dim3(256), 0, s, (T *)out, scratch, (const T *)scale,

@@ -341,6 +341,8 @@ def test_few_row_gemm_prefill_chunk_vs_oracle(g, dt, rows):
     dec = g.mynn.Decoder(cfg, dev_weights(g, w, dt), seq_q=rows)
     names = [n for n, _, _, _ in dec.profile(np.zeros(rows, np.int64), np.arange(rows), 0, rows)]
     assert "linear_gateup_swiglu" in names and "swiglu" not in names
+    # every RMSNorm but the first rides on the launch that finishes its input (o / down projection + residual)
+    assert names.count("rms_norm") == 1
     rng = np.random.default_rng(rows)
     past = 0
     for chunk in range(2):
