@@ -173,12 +173,13 @@ static int linear_rows(Model &m, void *out, const void *act, const Lin &l, int M
 // one few-row GEMM against int8 weights (two launches: products, then sum/scale/store)
 // next_norm (residual store): the weights of the RMSNorm that reads this output next; *normed = m.nrm holds it
 static int skinny_rows(Model &m, void *out, const void *act, const Lin &l, const void *packed, const void *res, int M, int epi,
-                       const char *name, const void *next_norm = nullptr, bool *normed = nullptr) {
+                       const char *name, const void *next_norm = nullptr, bool *normed = nullptr, const SkinnyRope *rope = nullptr,
+                       bool *roped = nullptr) {
     const double eb = dtype_size(m.cfg.dtype), n_out = epi == GEMM_SWIGLU ? l.N / 2 : l.N;
     note(m, name, (double)l.N * l.K + l.N * eb + (double)M * l.K * eb + (double)M * n_out * eb * (epi == GEMM_RESIDUAL ? 2 : 1),
          2.0 * M * l.N * l.K);
     return dequant_gemm_skinny(out, act, (const int8_t *)(packed ? packed : l.w), packed != nullptr, l.scale, res, M, l.N, l.K,
-                               m.cfg.dtype, epi, m.skinny_scratch, m.stream, next_norm, m.cfg.eps, m.nrm, normed);
+                               m.cfg.dtype, epi, m.skinny_scratch, m.stream, next_norm, m.cfg.eps, m.nrm, normed, rope, roped);
 }
 
 // Options::quantize_activations: DynamicQuantizeLinear (per row, symmetric) then QuantizedMatMul.
@@ -239,6 +240,7 @@ static int enqueue_step(Model &m) {
     for (size_t li = 0; li < m.layers.size(); li++) {
         Layer &L = m.layers[li];
         // ---- attention block
+        bool roped = false;
         if (fused) {
             note(m, "gemv_norm_qkv", (double)L.qkv.N * H + L.qkv.N * eb + 2 * H * eb + L.qkv.N * eb);
             TRY(gemv_norm<T>(m.qkv, m.x, L.norm1, c.eps, (const int8_t *)L.qkv.w, L.qkv.scale, L.qkv.N, H, s));
@@ -250,7 +252,12 @@ static int enqueue_step(Model &m) {
                 TRY(mynn_rms_norm(m.nrm, m.x, L.norm1, rows, H, c.eps, c.dtype, s));
             }
             nrm_ready = false;
-            if (m.skinny) TRY(skinny_rows(m, m.qkv, m.nrm, L.qkv, L.pk_qkv, nullptr, rows, GEMM_PLAIN, "linear_qkv"));
+            if (m.skinny) {
+                // (16-bit KV cache) RoPE and both cache appends ride on the launch that sums the projection's K ranges
+                const SkinnyRope rp{m.q, L.k_cache, L.v_cache, m.cos_t, m.sin_t, m.d_pos, m.d_past, S, Hq, Hkv, D, c.max_seq};
+                TRY(skinny_rows(m, m.qkv, m.nrm, L.qkv, L.pk_qkv, nullptr, rows, GEMM_PLAIN, "linear_qkv", nullptr, nullptr,
+                                kv8 ? nullptr : &rp, &roped));
+            }
             else if (w8a8) TRY(linear_w8a8(m, m.qkv, m.nrm, L.qkv, rows, true, "qlinear_qkv"));
             else if (m.resident16) TRY(gemm_rows(m, m.qkv, m.nrm, L.wt_qkv, nullptr, rows, L.qkv.N, H, GEMM_PLAIN, "linear_qkv"));
             else TRY(linear_rows<T>(m, m.qkv, m.nrm, L.qkv, rows, "linear_qkv"));
@@ -269,8 +276,9 @@ static int enqueue_step(Model &m) {
                 note(m, "attention_rope_append", (double)(QD + 2 * KD) * eb + 2.0 * KD * eb + QD * eb);
                 TRY(attention_decode_launch(p, D, c.dtype, 0, m.attn_scratch, s));
             } else {
-                note(m, kv8 ? "rope_quant_kv_append" : "rope_kv_append", (double)rows * (QD + 2 * KD) * 2 * eb);
-                if (kv8)
+                if (!roped) note(m, kv8 ? "rope_quant_kv_append" : "rope_kv_append", (double)rows * (QD + 2 * KD) * 2 * eb);
+                if (roped) {
+                } else if (kv8)
                     TRY(rope_quant_kv_append<T>(m.q, (int8_t *)L.k_cache, (int8_t *)L.v_cache, L.k_scale, L.v_scale, m.qkv,
                                                 m.cos_t, m.sin_t, m.d_pos, m.d_past, B, S, Hq, Hkv, D, c.max_seq, s));
                 else

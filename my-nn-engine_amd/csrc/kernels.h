@@ -26,9 +26,19 @@ size_t skinny_scratch_bytes(int M, int N, int K);
 // `packed`: wq is a tiled copy (skinny_packed_bytes, made by skinny_pack_weight) that a wave reads sequentially
 size_t skinny_packed_bytes(int N, int K);
 int skinny_pack_weight(void *dst, const int8_t *wq, int N, int K, hipStream_t s);
+// rope (optional, plain store of a q|k|v projection): instead of storing the projection, rotate q and k by the
+// rows' positions and write q to q_out and k, v into the caches -- what rope_kv_append would do next
+struct SkinnyRope {
+    void *q_out, *k_cache, *v_cache;
+    const void *cos_t, *sin_t;
+    const int64_t *position;
+    const int32_t *d_past;
+    int S, Hq, Hkv, D, max_seq;
+};
 int dequant_gemm_skinny(void *out, const void *act, const int8_t *wq, bool packed, const void *scale, const void *res, int M,
                         int N, int K, int dtype, int epi, float *scratch, hipStream_t s, const void *norm_w = nullptr,
-                        float eps = 0.f, void *nrm_out = nullptr, bool *normed = nullptr);
+                        float eps = 0.f, void *nrm_out = nullptr, bool *normed = nullptr, const SkinnyRope *rope = nullptr,
+                        bool *roped = nullptr);
 
 // matrix-core GEMM pieces.  A dequantised weight is [N, Kp] of the 16-bit type, Kp = K rounded up to 64,
 // zero padded (gemm_weight_bytes); dequant_weight_rows writes one (group/which: see gemm.hip), and

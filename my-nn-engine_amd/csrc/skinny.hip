@@ -273,6 +273,76 @@ __global__ __launch_bounds__(kReduceNormThreads) void skinny_reduce_norm_kernel(
             uint2{pack2<T>((x[0] * inv) * nw[0], (x[1] * inv) * nw[1]), pack2<T>((x[2] * inv) * nw[2], (x[3] * inv) * nw[3])};
 }
 
+// The plain form of the reduction for a q|k|v projection, followed by what rope_kv_append_vec_kernel does with
+// the stored projection: one workgroup per token row, a thread per (head, 4 rotation pairs) or 4 values of v;
+// qkv values are rounded to the storage type before the rotation, exactly as if they had been stored.
+template <typename T>
+__global__ __launch_bounds__(kReduceNormThreads) void skinny_reduce_rope_kernel(const float *part, const T *scale, int M, int N, int ksplit,
+                                                                              T *q_out, T *k_cache, T *v_cache, const T *cos_t,
+                                                                              const T *sin_t, const int64_t *position,
+                                                                              const int32_t *d_past, int S, int Hq, int Hkv, int D,
+                                                                              int max_seq) {
+    const int m = blockIdx.x, b = m / S, sq = m % S;
+    const int half = D / 2, upr = half / 4, upv = D / 4;  // units per rotated head / per v head
+    const int rot_units = (Hq + Hkv) * upr, units = rot_units + Hkv * upv;
+    const int past = *d_past;
+    const size_t tab = (size_t)position[sq] * D;
+    auto total4 = [&](int col, float *t) {
+        float4 pv[kReduceNormMaxSplit];
+#pragma unroll
+        for (int s = 0; s < kReduceNormMaxSplit; s++) {
+            pv[s] = float4{0.f, 0.f, 0.f, 0.f};
+            if (s < ksplit) pv[s] = *(const float4 *)(part + ((size_t)s * M + m) * N + col);
+        }
+        const uint2 sc2 = *(const uint2 *)(scale + col);
+        float sc[8];
+        widen8<T>(U4{sc2.x, sc2.y, 0u, 0u}, sc);
+        t[0] = t[1] = t[2] = t[3] = 0.f;
+#pragma unroll
+        for (int s = 0; s < kReduceNormMaxSplit; s++)
+            if (s < ksplit) {
+                t[0] += pv[s].x; t[1] += pv[s].y; t[2] += pv[s].z; t[3] += pv[s].w;
+            }
+#pragma unroll
+        for (int i = 0; i < 4; i++) t[i] = Elem<T>::rnd(t[i] * sc[i]);
+    };
+    auto ld4 = [&](const T *p, float *f) {
+        const uint2 v = *(const uint2 *)p;
+        float w[8];
+        widen8<T>(U4{v.x, v.y, 0u, 0u}, w);
+#pragma unroll
+        for (int i = 0; i < 4; i++) f[i] = w[i];
+    };
+    for (int u = threadIdx.x; u < units; u += kReduceNormThreads) {
+        if (u >= rot_units) {
+            const int hv = (u - rot_units) / upv, j = ((u - rot_units) % upv) * 4;
+            float t[4];
+            total4((Hq + Hkv + hv) * D + j, t);
+            T *dst = v_cache + (((size_t)b * Hkv + hv) * max_seq + past + sq) * D + j;
+            *(uint2 *)dst = uint2{pack2<T>(t[0], t[1]), pack2<T>(t[2], t[3])};
+            continue;
+        }
+        const int head = u / upr, j = (u % upr) * 4;
+        float xl[4], xh[4], cl[4], ch[4], sl[4], sh[4];
+        total4(head * D + j, xl);
+        total4(head * D + j + half, xh);
+        ld4(cos_t + tab + j, cl);
+        ld4(cos_t + tab + j + half, ch);
+        ld4(sin_t + tab + j, sl);
+        ld4(sin_t + tab + j + half, sh);
+        T *dst = head < Hq ? q_out + (size_t)m * Hq * D + (size_t)head * D
+                           : k_cache + (((size_t)b * Hkv + (head - Hq)) * max_seq + past + sq) * D;
+        float ol[4], oh[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            ol[i] = xl[i] * cl[i] - xh[i] * sl[i];
+            oh[i] = xh[i] * ch[i] + xl[i] * sh[i];
+        }
+        *(uint2 *)(dst + j) = uint2{pack2<T>(ol[0], ol[1]), pack2<T>(ol[2], ol[3])};
+        *(uint2 *)(dst + j + half) = uint2{pack2<T>(oh[0], oh[1]), pack2<T>(oh[2], oh[3])};
+    }
+}
+
 bool skinny_gemm_supported(int M, int N, int K) { return M >= 16 && M <= 64 && K % kSkinnyK == 0 && K >= 2 * kSkinnyK && N >= 1; }
 
 // K ranges: enough waves to keep ~1000 in flight, each with at least as many steps as it has stages
@@ -289,8 +359,9 @@ size_t skinny_scratch_bytes(int M, int N, int K) { return (size_t)skinny_ksplit(
 // whether this call did (it does when the K range is split, N % 4 == 0 and N <= 4096)
 int dequant_gemm_skinny(void *out, const void *act, const int8_t *wq, bool packed, const void *scale, const void *res, int M,
                         int N, int K, int dtype, int epi, float *scratch, hipStream_t s, const void *norm_w, float eps,
-                        void *nrm_out, bool *normed) {
+                        void *nrm_out, bool *normed, const SkinnyRope *rope, bool *roped) {
     if (normed) *normed = false;
+    if (roped) *roped = false;
     MYNN_REQUIRE(out && act && wq && scale && scratch, MYNN_ERR_INVALID, "dequant_matmul: null operand");
     MYNN_REQUIRE(skinny_gemm_supported(M, N, K), MYNN_ERR_UNSUPPORTED, "dequant_matmul (few rows): M=%d N=%d K=%d", M, N, K);
     MYNN_REQUIRE(aligned16(act) && aligned16(wq), MYNN_ERR_INVALID, "dequant_matmul: act and wq must be 16-byte aligned");
@@ -330,6 +401,16 @@ int dequant_gemm_skinny(void *out, const void *act, const int8_t *wq, bool packe
                         (const T *)scale, (const T *)res, (const T *)norm_w, M, N, ks_used, eps);
             *normed = true;
             return launch_status("skinny_reduce_norm_kernel");
+        }
+        if (epi == GEMM_PLAIN && rope && roped && rope->D % 8 == 0 && N == (rope->Hq + 2 * rope->Hkv) * rope->D &&
+            ks_used <= kReduceNormMaxSplit && ((uintptr_t)scale & 7) == 0 && ((uintptr_t)rope->q_out & 7) == 0 &&
+            ((uintptr_t)rope->k_cache & 7) == 0 && ((uintptr_t)rope->v_cache & 7) == 0 && ((uintptr_t)rope->cos_t & 7) == 0 &&
+            ((uintptr_t)rope->sin_t & 7) == 0) {
+            MYNN_LAUNCH(skinny_reduce_rope_kernel<T>, dim3(M), dim3(kReduceNormThreads), 0, s, scratch, (const T *)scale, M, N, ks_used,
+                        (T *)rope->q_out, (T *)rope->k_cache, (T *)rope->v_cache, (const T *)rope->cos_t, (const T *)rope->sin_t,
+                        rope->position, rope->d_past, rope->S, rope->Hq, rope->Hkv, rope->D, rope->max_seq);
+            *roped = true;
+            return launch_status("skinny_reduce_rope_kernel");
         }
         const dim3 rg((unsigned)((n_out + 255) / 256));
         if (epi == GEMM_RESIDUAL)

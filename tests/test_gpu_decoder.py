@@ -333,14 +333,19 @@ FEWROWS = dict(SMALL, ffn=768)  # every K a multiple of 128: 16..64 rows take th
 
 @pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
 @pytest.mark.parametrize("rows", [16, 32, 48])
-def test_few_row_gemm_prefill_chunk_vs_oracle(g, dt, rows):
+@pytest.mark.parametrize("hidden", [256, 1536])
+def test_few_row_gemm_prefill_chunk_vs_oracle(g, dt, rows, hidden):
     """16 <= rows <= 64: linears stream the int8 weights once through the few-row matrix-core kernel
-    (scale after the sum, K split over workgroups, residual / SwiGLU in the reducing launch)."""
-    cfg, w = llm_weights.synthetic_int8(FEWROWS, dt, seed=51)
+    (scale after the sum, K split over workgroups, residual / SwiGLU in the reducing launch).  With the
+    longer rows (hidden 1536) the q|k|v projection's K range is split too, and the launch that sums it
+    applies RoPE and appends to the caches."""
+    shape = FEWROWS if hidden == 256 else dict(FEWROWS, hidden=1536, n_heads=48, n_kv_heads=12, n_layers=2)
+    cfg, w = llm_weights.synthetic_int8(shape, dt, seed=51)
     ref = orc.Model(cfg, w)
     dec = g.mynn.Decoder(cfg, dev_weights(g, w, dt), seq_q=rows)
     names = [n for n, _, _, _ in dec.profile(np.zeros(rows, np.int64), np.arange(rows), 0, rows)]
     assert "linear_gateup_swiglu" in names and "swiglu" not in names
+    assert ("rope_kv_append" in names) == (hidden == 256)
     # every RMSNorm but the first rides on the launch that finishes its input (o / down projection + residual)
     assert names.count("rms_norm") == 1
     rng = np.random.default_rng(rows)
