@@ -94,3 +94,16 @@ def test_mock_step_session_follows_logit_table():
     n = lib.mynn_llm_generate_ids(h2, prompt.ctypes.data_as(C.c_void_p), 3, 5, out.ctypes.data_as(C.c_void_p))
     assert n == 2 and out[:2].tolist() == [3, 4]
     lib.mynn_llm_destroy(h), lib.mynn_llm_destroy(h2)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py --gpus N with N > 1 (or a multi-rank launch) exits with a message instead of measuring anything."""
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2 and "ONE GPU" in r.stderr and not r.stdout.strip()
+    env = dict(os.environ, WORLD_SIZE="4")
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py")], capture_output=True, text=True, timeout=120, env=env)
+    assert r.returncode == 2 and "ONE GPU" in r.stderr
