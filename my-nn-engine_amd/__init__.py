@@ -76,6 +76,8 @@ SIGNATURES = {
     "mynn_dynamic_quantize_linear": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mynn_attention": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "mynn_kvcache_update": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
+    "mynn_kvcache_update_streaming": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "mynn_attention_streaming": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "mynn_quantizing_kvcache_update": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "mynn_rms_norm": (_i, [_vp, _vp, _vp, _i, _i, _f, _i, _vp]),
     "mynn_rope": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
@@ -246,6 +248,34 @@ def kvcache_update(cache, new_kv, offset):
     check(lib().mynn_kvcache_update(_ptr(cache), _ptr(new_kv), int(offset), B * H, new_kv.shape[2], max_seq, D,
                                     _dt(cache), _stream()))
     return cache
+
+
+def kvcache_update_streaming(cache, new_kv, offset, ring_sink, ring_window, ring_start):
+    """KVCacheUpdate through the sink + ring slot map (the reference's streaming-KV graph)."""
+    import torch
+
+    B, H, max_seq, D = cache.shape
+    check(lib().mynn_kvcache_update_streaming(_ptr(cache), _ptr(new_kv), int(offset), B * H, new_kv.shape[2], max_seq, D,
+                                              int(ring_sink), int(ring_window), int(ring_start),
+                                              I8 if cache.dtype == torch.int8 else _dt(cache), _stream()))
+    return cache
+
+
+def attention_streaming(q, k, v, scale, is_causal, active, ring_sink, ring_window, ring_start, q_pos_offset=None,
+                        k_scale=None, v_scale=None):
+    """Attention over the sink + ring layout: keys by recency rank, rank -> cache row by the ring map."""
+    import torch
+
+    B, Hq, Sq, D = q.shape
+    Hkv, cache_len = k.shape[1], k.shape[2]
+    if q_pos_offset is None:
+        q_pos_offset = active - Sq
+    out = torch.empty_like(q)
+    check(lib().mynn_attention_streaming(_ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(k_scale), _ptr(v_scale), float(scale),
+                                         int(is_causal), B, Sq, int(active), cache_len, int(q_pos_offset), Hq, Hkv, D,
+                                         _dt(q), int(k.dtype == torch.int8), int(ring_sink), int(ring_window),
+                                         int(ring_start), _stream()))
+    return out
 
 
 def quantizing_kvcache_update(cache, scale, new_kv, offset):

@@ -597,3 +597,104 @@ extern "C" int mynn_attention(void *out, const void *Q, const void *K, const voi
     }
     return attention_decode_launch(p, head_dim, dtype, kv_int8, g_scratch.ptr, st);
 }
+
+// ---- streaming KV (sink + ring cache): the slot map of the reference's kernels and the two operators that
+// take it.  Attention is order-free over its keys apart from the causal rule, which is stated in ranks, so
+// the rows are gathered into rank order (library-owned scratch) and handed to the kernels above.
+namespace mynn {
+
+__host__ __device__ inline int ring_phys_index(int rank, int sink, int window, int start) {
+    if (window == 0 || rank < sink) return rank;
+    return sink + (start + (rank - sink)) % window;
+}
+
+// dst[bh][r][:] = src[bh][ring_phys_index(r)][:] for r < rows (gather), or, SCATTER,
+// dst[bh][ring_phys_index(offset + r)][:] = src[bh][r][:]; rows of `units` 2-byte units
+template <bool SCATTER>
+__global__ void ring_rows_kernel(uint16_t *dst, const uint16_t *src, size_t units, int rows, int cache_len, int offset, int sink,
+                                 int window, int start, size_t total) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const size_t u = i % units, r = (i / units) % rows, bh = i / (units * rows);
+    if (SCATTER) {
+        // rows that share a slot: the last one in t order wins, as in the reference's sequential loop
+        // (two ranks share a ring slot exactly when both are past the sink and a multiple of the window apart)
+        const int slot = ring_phys_index(offset + (int)r, sink, window, start);
+        if (window > 0 && offset + (int)r >= sink && (int)r + window < rows) return;  // a later row takes the slot
+        dst[(bh * cache_len + slot) * units + u] = src[i];
+    } else {
+        dst[i] = src[(bh * cache_len + ring_phys_index((int)r, sink, window, start)) * units + u];
+    }
+}
+
+static Grown g_ring_k, g_ring_v, g_ring_ks, g_ring_vs;
+
+}  // namespace mynn
+
+extern "C" int mynn_kvcache_update_streaming(void *cache, const void *new_kv, int offset, int BH, int S_new, int max_seq, int D,
+                                             int ring_sink, int ring_window, int ring_start, int dtype, mynn_stream s) {
+    using namespace mynn;
+    MYNN_REQUIRE(cache && new_kv, MYNN_ERR_INVALID, "kvcache_update: null operand");
+    MYNN_REQUIRE(BH > 0 && S_new > 0 && D > 0 && offset >= 0, MYNN_ERR_INVALID, "kvcache_update: BH=%d S_new=%d D=%d offset=%d", BH,
+                 S_new, D, offset);
+    MYNN_REQUIRE(dtype_ok(dtype) || dtype == MYNN_I8, MYNN_ERR_INVALID, "kvcache_update: dtype %d", dtype);
+    MYNN_REQUIRE(ring_sink >= 0 && ring_window >= 0 && ring_start >= 0 && (ring_window == 0 || ring_start < ring_window),
+                 MYNN_ERR_INVALID, "kvcache_update: ring sink=%d window=%d start=%d", ring_sink, ring_window, ring_start);
+    if (ring_window == 0) {
+        MYNN_REQUIRE(offset + S_new <= max_seq, MYNN_ERR_INVALID, "kvcache_update: offset %d + %d rows exceeds max_seq %d", offset,
+                     S_new, max_seq);
+    } else {
+        MYNN_REQUIRE(ring_sink + ring_window <= max_seq, MYNN_ERR_INVALID, "kvcache_update: sink %d + window %d exceeds max_seq %d",
+                     ring_sink, ring_window, max_seq);
+    }
+    const size_t row_bytes = (size_t)D * (dtype == MYNN_I8 ? 1 : dtype_size(dtype));
+    MYNN_REQUIRE(row_bytes % 2 == 0, MYNN_ERR_UNSUPPORTED, "kvcache_update: rows of %zu bytes", row_bytes);
+    const size_t units = row_bytes / 2, total = (size_t)BH * S_new * units;
+    MYNN_LAUNCH((ring_rows_kernel<true>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, as_stream(s), (uint16_t *)cache,
+                (const uint16_t *)new_kv, units, S_new, max_seq, offset, ring_sink, ring_window, ring_start, total);
+    return launch_status("ring_rows_kernel");
+}
+
+extern "C" int mynn_attention_streaming(void *out, const void *Q, const void *K, const void *V, const void *k_scale,
+                                        const void *v_scale, float scale, int is_causal, int B, int Sq, int active_seq_kv,
+                                        int cache_seq_len, int q_pos_offset, int num_q_heads, int num_kv_heads, int head_dim,
+                                        int dtype, int kv_int8, int ring_sink, int ring_window, int ring_start, mynn_stream s) {
+    using namespace mynn;
+    MYNN_REQUIRE(ring_sink >= 0 && ring_window >= 0 && ring_start >= 0 && (ring_window == 0 || ring_start < ring_window),
+                 MYNN_ERR_INVALID, "attention: ring sink=%d window=%d start=%d", ring_sink, ring_window, ring_start);
+    if (ring_window == 0)
+        return mynn_attention(out, Q, K, V, k_scale, v_scale, scale, is_causal, B, Sq, active_seq_kv, nullptr, cache_seq_len,
+                              q_pos_offset, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, s);
+    MYNN_REQUIRE(out && Q && K && V, MYNN_ERR_INVALID, "attention: null operand");
+    MYNN_REQUIRE(B > 0 && Sq > 0 && cache_seq_len > 0 && num_q_heads > 0 && num_kv_heads > 0 && head_dim > 0, MYNN_ERR_INVALID,
+                 "attention: B=%d Sq=%d cache=%d Hq=%d Hkv=%d D=%d", B, Sq, cache_seq_len, num_q_heads, num_kv_heads, head_dim);
+    MYNN_REQUIRE(active_seq_kv >= 1, MYNN_ERR_INVALID, "attention: active_seq_kv=%d", active_seq_kv);
+    MYNN_REQUIRE(ring_sink + ring_window <= cache_seq_len, MYNN_ERR_INVALID, "attention: sink %d + window %d exceeds the cache of %d rows",
+                 ring_sink, ring_window, cache_seq_len);
+    MYNN_REQUIRE(!kv_int8 || (k_scale && v_scale), MYNN_ERR_INVALID, "attention: int8 KV needs k_scale and v_scale");
+    MYNN_REQUIRE(dtype_ok(dtype), MYNN_ERR_INVALID, "attention: dtype %d", dtype);
+    // ranks past sink + window would read ring rows a second time (the reference's kernels do); the session
+    // never asks for them, and the plain kernels clamp the same way
+    const int rows = active_seq_kv < ring_sink + ring_window ? active_seq_kv : ring_sink + ring_window;
+    const size_t eb = dtype_size(dtype), row_bytes = (size_t)head_dim * (kv_int8 ? 1 : eb);
+    MYNN_REQUIRE(row_bytes % 2 == 0 && eb % 2 == 0, MYNN_ERR_UNSUPPORTED, "attention: rows of %zu bytes", row_bytes);
+    const int BH = B * num_kv_heads;
+    hipStream_t st = as_stream(s);
+    auto gather = [&](Grown &gbuf, const void *src, size_t rb) -> int {
+        // (16 bytes of slack: the attention kernels want 16-byte aligned K / V, which hipMalloc gives)
+        int rc = ensure(gbuf, (size_t)BH * rows * rb + 16, false, st);
+        if (rc) return rc;
+        const size_t units = rb / 2, total = (size_t)BH * rows * units;
+        MYNN_LAUNCH((ring_rows_kernel<false>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, (uint16_t *)gbuf.ptr,
+                    (const uint16_t *)src, units, rows, cache_seq_len, 0, ring_sink, ring_window, ring_start, total);
+        return launch_status("ring_rows_kernel");
+    };
+    int rc = gather(g_ring_k, K, row_bytes);
+    if (!rc) rc = gather(g_ring_v, V, row_bytes);
+    if (!rc && kv_int8) rc = gather(g_ring_ks, k_scale, eb);
+    if (!rc && kv_int8) rc = gather(g_ring_vs, v_scale, eb);
+    if (rc) return rc;
+    return mynn_attention(out, Q, g_ring_k.ptr, g_ring_v.ptr, kv_int8 ? g_ring_ks.ptr : nullptr, kv_int8 ? g_ring_vs.ptr : nullptr, scale,
+                          is_causal, B, Sq, rows, nullptr, rows, q_pos_offset, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, s);
+}
+

@@ -247,6 +247,39 @@ def kv_cache_update(cache, new_kv, offset):
     return cache
 
 
+def ring_phys_index(rank, ring_sink, ring_window, ring_start):
+    """Cache row of the key with recency rank `rank` in the sink + ring layout
+    (src/codegen/cuda/cpp/common.cuh:55-60): the first ring_sink rows are fixed, the following ring_window
+    rows are a ring read from ring_start; ring_window == 0 switches the map off."""
+    if ring_window == 0 or rank < ring_sink:
+        return rank
+    return ring_sink + (ring_start + (rank - ring_sink)) % ring_window
+
+
+def kv_cache_update_streaming(cache, new_kv, offset, ring_sink, ring_window, ring_start):
+    """KVCacheUpdate with the ring inputs (src/codegen/cuda/cpp/kvcache_update.cuh:12-26): row t of new_kv goes
+    to row ring_phys_index(offset + t) of the cache, rows in increasing t (a later row wins a shared slot).
+    cache [B,H,max_seq,D] is updated in place (and returned)."""
+    assert cache.flags.c_contiguous
+    new_kv = _c(new_kv, cache.dtype)
+    for t in range(new_kv.shape[2]):
+        cache[:, :, ring_phys_index(offset + t, ring_sink, ring_window, ring_start)] = new_kv[:, :, t]
+    return cache
+
+
+def attention_streaming(q, k, v, dt, scale, is_causal, active, ring_sink, ring_window, ring_start, k_scale=None,
+                        v_scale=None):
+    """Attention over the sink + ring layout (src/codegen/cuda/cpp/attention.cuh:386-404, 436-438, 548-550):
+    keys are enumerated by recency rank 0..active-1, the key of rank r is cache row ring_phys_index(r), and
+    the causal rule compares query positions with ranks.  Restated as the plain attention of this module over
+    the rows gathered in rank order."""
+    rows = [ring_phys_index(r, ring_sink, ring_window, ring_start) for r in range(active)]
+    kg, vg = np.ascontiguousarray(k[:, :, rows]), np.ascontiguousarray(v[:, :, rows])
+    ks = np.ascontiguousarray(k_scale[:, :, rows]) if k_scale is not None else None
+    vs = np.ascontiguousarray(v_scale[:, :, rows]) if v_scale is not None else None
+    return attention(q, kg, vg, dt, scale, is_causal, active, ks, vs)
+
+
 def quantizing_kv_cache_update(cache, scale, new_kv, offset, dt):
     assert cache.flags.c_contiguous and cache.dtype == np.int8 and scale.flags.c_contiguous
     new_kv = _c(new_kv, np_dtype(dt))

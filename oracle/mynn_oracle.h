@@ -30,6 +30,9 @@
  *   orc_model_* (decoder executor and generate loop)   the reference's exact ids on its tiny random Llama
  *                             (crates/llm/tests/tinyllama_random.rs:20-24) in f32/bf16/f16 and three summation orders;
  *                             mock_decode expectations (crates/llm/tests/mock_decode.rs:30-87)
+ *   ring_phys_index, kv_cache_update_streaming, attention_streaming (numpy, oracle/__init__.py; sink + ring KV ops of the
+ *                             reference's CUDA kernels)   brute-force ring simulation, reduction to the plain update /
+ *                             attention when the ring has not wrapped, f64 attention over explicitly scattered rows
  * Parity unpinned: none.  What no offline check fixes bit for bit is the reference's own f32 summation
  * order (LLVM fast-math vectorisation, BLAS sgemm) and libm expf; those are covered by tolerance.
  */

@@ -294,3 +294,85 @@ def test_prefill_attention_rows_equal_decode_rows(g):
         one = g.mynn.attention(dq[:, :, row:row + 1].contiguous(), dk, dv, 0.125, False, row + 1)
         assert max_err_rel_to_max(full[:, :, row], g.f32(g.to_host(one), dt)[:, :, 0]) <= 2e-3, row
     assert np.array_equal(full[:, :, 0], np.repeat(g.f32(v, dt)[:, :, 0], Hq // Hkv, 1))  # first row sees one key
+
+
+# ---- streaming KV (sink + ring cache): the slot map of common.cuh:55-60 in KVCacheUpdate and Attention
+@pytest.mark.parametrize("kind", ["f16", "f32", "i8"])
+@pytest.mark.parametrize("offset,S_new,sink,window,start", [
+    (9, 5, 4, 16, 0),      # not wrapped: the plain update
+    (17, 5, 4, 16, 6),     # wraps inside the ring
+    (2, 7, 4, 16, 3),      # rows on both sides of the sink boundary
+    (20, 40, 4, 16, 9),    # more rows than ring slots: later rows win
+    (3, 6, 0, 0, 0),       # ring switched off
+])
+def test_kvcache_update_streaming_bit_exact(g, kind, offset, S_new, sink, window, start):
+    import torch
+
+    rng = np.random.default_rng(offset * 7 + S_new)
+    B, H, L, D = 2, 3, 64, 32
+    npdt = {"f16": np.uint16, "f32": np.float32, "i8": np.int8}[kind]
+    if kind == "f32":
+        cache = rng.standard_normal((B, H, L, D)).astype(np.float32)
+        new = rng.standard_normal((B, H, S_new, D)).astype(np.float32)
+    else:
+        hi = 65536 if kind == "f16" else 128
+        lo = 0 if kind == "f16" else -128
+        cache = rng.integers(lo, hi, (B, H, L, D)).astype(npdt)
+        new = rng.integers(lo, hi, (B, H, S_new, D)).astype(npdt)
+    want = orc.kv_cache_update_streaming(cache.copy(), new, offset, sink, window, start)
+    tdt = {"f16": torch.float16, "f32": torch.float32, "i8": torch.int8}[kind]
+    dc = torch.from_numpy(cache.view(np.int16) if kind == "f16" else cache).cuda()
+    dn = torch.from_numpy(new.view(np.int16) if kind == "f16" else new).cuda()
+    if kind == "f16":
+        dc, dn = dc.view(tdt), dn.view(tdt)
+    g.mynn.kvcache_update_streaming(dc, dn, offset, sink, window, start)
+    got = dc.view(torch.int16).cpu().numpy().view(np.uint16) if kind == "f16" else dc.cpu().numpy()
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+@pytest.mark.parametrize("Sq,causal,sink,window,start,active,D", [
+    (1, False, 4, 16, 11, 19, 64),    # decode over a wrapped ring
+    (1, False, 4, 28, 0, 9, 32),      # ring not full yet
+    (1, False, 0, 8, 5, 8, 128),      # no sink
+    (1, False, 4, 16, 3, 20, 64),     # the whole ring
+    (24, True, 4, 40, 17, 44, 64),    # causal prefill chunk over ranks (matrix-core kernel)
+    (6, True, 2, 16, 9, 13, 32),      # causal, per-row kernel
+    (1, False, 3, 0, 0, 12, 64),      # ring switched off: plain attention
+])
+def test_attention_streaming_vs_oracle(g, dt, Sq, causal, sink, window, start, active, D):
+    """Keys enumerated by recency rank through the ring map; rows that no rank maps to are poisoned."""
+    rng = np.random.default_rng(active * 13 + D + Sq)
+    B, Hq, Hkv, L = 2, 8, 2, 64
+    q = orc.to_storage(rng.standard_normal((B, Hq, Sq, D)), dt)
+    k = orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt)
+    v = orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt)
+    used = {orc.ring_phys_index(r, sink, window, start) for r in range(active)}
+    for row in range(L):
+        if row not in used:
+            k[:, :, row] = orc.to_storage(np.full((B, Hkv, D), np.nan), dt)
+            v[:, :, row] = orc.to_storage(np.full((B, Hkv, D), np.nan), dt)
+    want = orc.attention_streaming(q, k, v, dt, D ** -0.5, causal, active, sink, window, start)
+    got = g.to_host(g.mynn.attention_streaming(g.to_dev(q, dt), g.to_dev(k, dt), g.to_dev(v, dt), D ** -0.5, causal, active,
+                                               sink, window, start))
+    assert not np.isnan(g.f32(got, dt)).any()
+    assert max_err_rel_to_max(g.f32(got, dt), g.f32(want, dt)) <= 1e-2
+    # and against the f64 attention over the rank-ordered rows
+    rows = [orc.ring_phys_index(r, sink, window, start) for r in range(active)]
+    exact = orc.attention_f64(q, np.ascontiguousarray(k[:, :, rows]), np.ascontiguousarray(v[:, :, rows]), dt, D ** -0.5, causal, active)
+    assert max_err_rel_to_max(g.f32(got, dt), exact) <= (4e-3 if dt == orc.BF16 else 1e-3)
+
+
+def test_attention_streaming_int8_kv(g):
+    dt = orc.F16
+    rng = np.random.default_rng(8)
+    B, Hq, Hkv, L, D, sink, window, start, active = 2, 8, 2, 64, 64, 4, 32, 21, 30
+    q = orc.to_storage(rng.standard_normal((B, Hq, 1, D)), dt)
+    k = rng.integers(-127, 128, (B, Hkv, L, D)).astype(np.int8)
+    v = rng.integers(-127, 128, (B, Hkv, L, D)).astype(np.int8)
+    ks = orc.to_storage(rng.uniform(1e-3, 2e-2, (B, Hkv, L)), dt)
+    vs = orc.to_storage(rng.uniform(1e-3, 2e-2, (B, Hkv, L)), dt)
+    want = orc.attention_streaming(q, k, v, dt, D ** -0.5, False, active, sink, window, start, ks, vs)
+    got = g.to_host(g.mynn.attention_streaming(g.to_dev(q, dt), g.to_dev(k), g.to_dev(v), D ** -0.5, False, active, sink, window,
+                                               start, k_scale=g.to_dev(ks, dt), v_scale=g.to_dev(vs, dt)))
+    assert max_err_rel_to_max(g.f32(got, dt), g.f32(want, dt)) <= 1e-2

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import oracle as orc
-from conftest import close_either
+from conftest import close_either, max_abs_rel
 
 DT = [orc.F32, orc.BF16, orc.F16]
 
@@ -323,3 +323,57 @@ def test_ring_index_and_streaming_positions():
     # saturated: sink 2, window 4, stream_pos 9 -> ring_start (9-2)%4 = 3; slot 2+3 is the oldest
     pos = orc.streaming_kv_position(2, 4, 9, 8).tolist()
     assert pos == [0, 1, 3, 4, 5, 2, 6, 7]
+
+
+def test_ring_phys_index_is_the_sink_plus_ring_map():
+    """common.cuh:55-60 against a hand-kept ring: ranks below the sink are fixed, the next `window` ranks are a
+    bijection onto the ring rows starting at ring_start, window 0 is the identity."""
+    for sink, window in [(0, 4), (4, 16), (3, 5), (4, 28)]:
+        for start in range(window):
+            ring = [sink + (start + i) % window for i in range(window)]  # row of the i-th oldest ring entry
+            rows = [orc.ring_phys_index(r, sink, window, start) for r in range(sink + window)]
+            assert rows[:sink] == list(range(sink))
+            assert rows[sink:] == ring and sorted(rows) == list(range(sink + window))
+    assert [orc.ring_phys_index(r, 4, 0, 3) for r in range(10)] == list(range(10))
+
+
+def test_kv_cache_update_streaming_reduces_to_plain_update_and_wraps():
+    rng = np.random.default_rng(0)
+    B, H, L, D, sink, window = 2, 3, 24, 8, 4, 16
+    new = rng.standard_normal((B, H, 5, D)).astype(np.float32)
+    a = np.zeros((B, H, L, D), np.float32)
+    b = np.zeros_like(a)
+    # before the ring wraps (ring_start 0, rows below sink + window) it is the plain update
+    orc.kv_cache_update_streaming(a, new, 9, sink, window, 0)
+    orc.kv_cache_update(b, new, 9)
+    assert np.array_equal(a, b)
+    # wrapping: rows land at sink + (start + rank - sink) % window, later rows overwrite earlier ones
+    c = np.zeros_like(a)
+    orc.kv_cache_update_streaming(c, new, 17, sink, window, 6)
+    want = np.zeros_like(a)
+    for t in range(5):
+        want[:, :, sink + (6 + 17 + t - sink) % window] = new[:, :, t]
+    assert np.array_equal(c, want)
+    assert not c[:, :, sink + window:].any() and not c[:, :, :sink].any()
+
+
+@pytest.mark.parametrize("dt", [orc.F32, orc.F16])
+@pytest.mark.parametrize("causal,Sq", [(False, 1), (True, 6)])
+def test_attention_streaming_equals_attention_over_rank_ordered_rows(dt, causal, Sq):
+    """Keys written in rank order into a cache through the ring map, then read back by the streaming attention,
+    must give the attention over the rank-ordered rows themselves (f64 brute force): the two maps are inverse."""
+    rng = np.random.default_rng(3)
+    B, Hq, Hkv, D, L, sink, window, start, active = 2, 4, 2, 16, 32, 4, 16, 11, 19
+    q = orc.to_storage(rng.standard_normal((B, Hq, Sq, D)), dt)
+    k_rank = orc.to_storage(rng.standard_normal((B, Hkv, active, D)), dt)
+    v_rank = orc.to_storage(rng.standard_normal((B, Hkv, active, D)), dt)
+    k = orc.to_storage(np.full((B, Hkv, L, D), np.nan), dt)
+    v = orc.to_storage(np.full((B, Hkv, L, D), np.nan), dt)
+    for r in range(active):
+        row = sink + (start + r - sink) % window if r >= sink else r
+        k[:, :, row] = k_rank[:, :, r]
+        v[:, :, row] = v_rank[:, :, r]
+    got = orc.attention_streaming(q, k, v, dt, D ** -0.5, causal, active, sink, window, start)
+    exact = orc.attention_f64(q, k_rank, v_rank, dt, D ** -0.5, causal, active)
+    assert max_abs_rel(orc.to_f32(got, dt), exact) <= (1e-4 if dt == orc.F32 else 2e-3)
+
