@@ -77,6 +77,7 @@ SIGNATURES = {
     "mynn_attention": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "mynn_kvcache_update": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "mynn_kvcache_update_streaming": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "mynn_quantizing_kvcache_update_streaming": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "mynn_attention_streaming": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "mynn_quantizing_kvcache_update": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "mynn_rms_norm": (_i, [_vp, _vp, _vp, _i, _i, _f, _i, _vp]),
@@ -259,6 +260,14 @@ def kvcache_update_streaming(cache, new_kv, offset, ring_sink, ring_window, ring
                                               int(ring_sink), int(ring_window), int(ring_start),
                                               I8 if cache.dtype == torch.int8 else _dt(cache), _stream()))
     return cache
+
+
+def quantizing_kvcache_update_streaming(cache, scale, new_kv, offset, ring_sink, ring_window, ring_start):
+    B, H, max_seq, D = cache.shape
+    check(lib().mynn_quantizing_kvcache_update_streaming(_ptr(cache), _ptr(scale), _ptr(new_kv), int(offset), B * H,
+                                                         new_kv.shape[2], max_seq, D, int(ring_sink), int(ring_window),
+                                                         int(ring_start), _dt(new_kv), _stream()))
+    return cache, scale
 
 
 def attention_streaming(q, k, v, scale, is_causal, active, ring_sink, ring_window, ring_start, q_pos_offset=None,

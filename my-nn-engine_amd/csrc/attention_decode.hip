@@ -603,11 +603,6 @@ extern "C" int mynn_attention(void *out, const void *Q, const void *K, const voi
 // the rows are gathered into rank order (library-owned scratch) and handed to the kernels above.
 namespace mynn {
 
-__host__ __device__ inline int ring_phys_index(int rank, int sink, int window, int start) {
-    if (window == 0 || rank < sink) return rank;
-    return sink + (start + (rank - sink)) % window;
-}
-
 // dst[bh][r][:] = src[bh][ring_phys_index(r)][:] for r < rows (gather), or, SCATTER,
 // dst[bh][ring_phys_index(offset + r)][:] = src[bh][r][:]; rows of `units` 2-byte units
 template <bool SCATTER>

@@ -124,11 +124,14 @@ __global__ void kvcache_update_kernel(W *cache, const W *new_kv, int offset, int
 // one wave per token row
 template <typename T>
 __global__ __launch_bounds__(64) void quantizing_kvcache_update_kernel(int8_t *cache, T *scale, const T *new_kv,
-                                                                       int offset, int S_new, int max_seq, int D) {
+                                                                       int offset, int S_new, int max_seq, int D, int ring_sink,
+                                                                       int ring_window, int ring_start) {
     const size_t rowi = blockIdx.x;  // bh * S_new + t
     const int t = (int)(rowi % S_new);
     const size_t bh = rowi / S_new;
-    const size_t tok = bh * max_seq + offset + t;
+    // streaming KV: the row goes to its ring slot; of rows a whole window apart the later one keeps the slot
+    if (ring_window > 0 && offset + t >= ring_sink && t + ring_window < S_new) return;
+    const size_t tok = bh * max_seq + ring_phys_index(offset + t, ring_sink, ring_window, ring_start);
     const int lane = threadIdx.x;
     float amax = 0.f;
     for (int d = lane; d < D; d += 64) amax = fmaxf(amax, fabsf(Elem<T>::ld(new_kv, rowi * D + d)));
@@ -504,17 +507,31 @@ extern "C" int mynn_kvcache_update(void *cache, const void *new_kv, int offset, 
     return launch_status("kvcache_update_kernel");
 }
 
-extern "C" int mynn_quantizing_kvcache_update(int8_t *cache, void *scale, const void *new_kv, int offset, int BH,
-                                              int S_new, int max_seq, int D, int dtype, mynn_stream s) {
+extern "C" int mynn_quantizing_kvcache_update_streaming(int8_t *cache, void *scale, const void *new_kv, int offset, int BH,
+                                                        int S_new, int max_seq, int D, int ring_sink, int ring_window,
+                                                        int ring_start, int dtype, mynn_stream s) {
     MYNN_REQUIRE(cache && scale && new_kv, MYNN_ERR_INVALID, "quantizing_kvcache_update: null operand");
-    MYNN_REQUIRE(BH > 0 && S_new > 0 && D > 0 && offset >= 0 && offset + S_new <= max_seq, MYNN_ERR_INVALID,
-                 "quantizing_kvcache_update: offset %d + %d rows exceeds max_seq %d", offset, S_new, max_seq);
+    MYNN_REQUIRE(BH > 0 && S_new > 0 && D > 0 && offset >= 0, MYNN_ERR_INVALID, "quantizing_kvcache_update: BH=%d S_new=%d D=%d offset=%d",
+                 BH, S_new, D, offset);
+    MYNN_REQUIRE(ring_sink >= 0 && ring_window >= 0 && ring_start >= 0 && (ring_window == 0 || ring_start < ring_window),
+                 MYNN_ERR_INVALID, "quantizing_kvcache_update: ring sink=%d window=%d start=%d", ring_sink, ring_window, ring_start);
+    if (ring_window == 0)
+        MYNN_REQUIRE(offset + S_new <= max_seq, MYNN_ERR_INVALID, "quantizing_kvcache_update: offset %d + %d rows exceeds max_seq %d",
+                     offset, S_new, max_seq);
+    else
+        MYNN_REQUIRE(ring_sink + ring_window <= max_seq, MYNN_ERR_INVALID,
+                     "quantizing_kvcache_update: sink %d + window %d exceeds max_seq %d", ring_sink, ring_window, max_seq);
     return dispatch_dtype(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
         MYNN_LAUNCH(quantizing_kvcache_update_kernel<T>, dim3(BH * S_new), dim3(64), 0, as_stream(s), cache,
-                           (T *)scale, (const T *)new_kv, offset, S_new, max_seq, D);
+                           (T *)scale, (const T *)new_kv, offset, S_new, max_seq, D, ring_sink, ring_window, ring_start);
         return launch_status("quantizing_kvcache_update_kernel");
     });
+}
+
+extern "C" int mynn_quantizing_kvcache_update(int8_t *cache, void *scale, const void *new_kv, int offset, int BH,
+                                              int S_new, int max_seq, int D, int dtype, mynn_stream s) {
+    return mynn_quantizing_kvcache_update_streaming(cache, scale, new_kv, offset, BH, S_new, max_seq, D, 0, 0, 0, dtype, s);
 }
 
 extern "C" int mynn_dequantize_linear(void *out, const int8_t *x, const void *scale, size_t rows, size_t cols,

@@ -121,6 +121,12 @@ template <int width> __device__ inline float group_sum(float v) {
 // exp for softmax / SiLU: one definition for every kernel
 __device__ inline float fast_exp(float x) { return __expf(x); }
 
+// cache row of the key with recency rank `rank` in the sink + ring layout (reference common.cuh:55-60)
+__host__ __device__ inline int ring_phys_index(int rank, int sink, int window, int start) {
+    if (window == 0 || rank < sink) return rank;
+    return sink + (start + (rank - sink)) % window;
+}
+
 // ---- errors ---------------------------------------------------------------------------------
 void set_error(const char *fmt, ...);
 int fail(int code, const char *fmt, ...);

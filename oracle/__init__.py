@@ -267,6 +267,23 @@ def kv_cache_update_streaming(cache, new_kv, offset, ring_sink, ring_window, rin
     return cache
 
 
+def quantizing_kv_cache_update_streaming(cache, scale, new_kv, offset, ring_sink, ring_window, ring_start, dt):
+    """QuantizingKVCacheUpdate with the ring inputs (src/codegen/cuda/cpp/quantizing_kvcache_update.cuh:24-36):
+    each row is quantised as quantizing_kv_cache_update does and, with its scale, goes to row
+    ring_phys_index(offset + t), rows in increasing t."""
+    assert cache.flags.c_contiguous and cache.dtype == np.int8 and scale.flags.c_contiguous
+    B, H, _, D = cache.shape
+    S_new = new_kv.shape[2]
+    tmp_c = np.zeros((B, H, S_new, D), np.int8)
+    tmp_s = np.zeros((B, H, S_new), scale.dtype)
+    quantizing_kv_cache_update(tmp_c, tmp_s, new_kv, 0, dt)
+    for t in range(S_new):
+        row = ring_phys_index(offset + t, ring_sink, ring_window, ring_start)
+        cache[:, :, row] = tmp_c[:, :, t]
+        scale[:, :, row] = tmp_s[:, :, t]
+    return cache, scale
+
+
 def attention_streaming(q, k, v, dt, scale, is_causal, active, ring_sink, ring_window, ring_start, k_scale=None,
                         v_scale=None):
     """Attention over the sink + ring layout (src/codegen/cuda/cpp/attention.cuh:386-404, 436-438, 548-550):

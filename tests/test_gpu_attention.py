@@ -376,3 +376,17 @@ def test_attention_streaming_int8_kv(g):
     got = g.to_host(g.mynn.attention_streaming(g.to_dev(q, dt), g.to_dev(k), g.to_dev(v), D ** -0.5, False, active, sink, window,
                                                start, k_scale=g.to_dev(ks, dt), v_scale=g.to_dev(vs, dt)))
     assert max_err_rel_to_max(g.f32(got, dt), g.f32(want, dt)) <= 1e-2
+
+
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+@pytest.mark.parametrize("offset,S_new,sink,window,start", [(9, 5, 4, 16, 0), (17, 5, 4, 16, 6), (20, 40, 4, 16, 9), (3, 6, 0, 0, 0)])
+def test_quantizing_kvcache_update_streaming_bit_exact(g, dt, offset, S_new, sink, window, start):
+    rng = np.random.default_rng(offset + S_new)
+    B, H, L, D = 2, 3, 64, 32
+    new = orc.to_storage(rng.standard_normal((B, H, S_new, D)) * 3, dt)
+    cache = rng.integers(-128, 128, (B, H, L, D)).astype(np.int8)
+    scale = orc.to_storage(rng.uniform(0.01, 0.1, (B, H, L)), dt)
+    want_c, want_s = orc.quantizing_kv_cache_update_streaming(cache.copy(), scale.copy(), new, offset, sink, window, start, dt)
+    dc, ds = g.to_dev(cache), g.to_dev(scale, dt)
+    g.mynn.quantizing_kvcache_update_streaming(dc, ds, g.to_dev(new, dt), offset, sink, window, start)
+    assert np.array_equal(g.to_host(dc), want_c) and np.array_equal(g.to_host(ds), want_s)

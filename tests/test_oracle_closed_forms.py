@@ -377,3 +377,17 @@ def test_attention_streaming_equals_attention_over_rank_ordered_rows(dt, causal,
     exact = orc.attention_f64(q, k_rank, v_rank, dt, D ** -0.5, causal, active)
     assert max_abs_rel(orc.to_f32(got, dt), exact) <= (1e-4 if dt == orc.F32 else 2e-3)
 
+
+
+def test_quantizing_kv_cache_update_streaming_is_the_plain_rule_at_ring_rows():
+    rng = np.random.default_rng(1)
+    B, H, L, D, sink, window, start, offset = 1, 2, 24, 8, 4, 16, 5, 18
+    new = orc.to_storage(rng.standard_normal((B, H, 3, D)), orc.BF16)
+    c, s = np.zeros((B, H, L, D), np.int8), np.zeros((B, H, L), np.uint16)
+    orc.quantizing_kv_cache_update_streaming(c, s, new, offset, sink, window, start, orc.BF16)
+    pc, ps = np.zeros((B, H, L, D), np.int8), np.zeros((B, H, L), np.uint16)
+    orc.quantizing_kv_cache_update(pc, ps, new, 0, orc.BF16)
+    for t in range(3):
+        row = sink + (start + offset + t - sink) % window
+        assert np.array_equal(c[:, :, row], pc[:, :, t]) and np.array_equal(s[:, :, row], ps[:, :, t])
+    assert np.count_nonzero(s) == 3 * H
