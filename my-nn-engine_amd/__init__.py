@@ -78,7 +78,7 @@ SIGNATURES = {
     "mynn_kvcache_update": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "mynn_kvcache_update_streaming": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "mynn_quantizing_kvcache_update_streaming": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
-    "mynn_attention_streaming": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "mynn_attention_streaming": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "mynn_quantizing_kvcache_update": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "mynn_rms_norm": (_i, [_vp, _vp, _vp, _i, _i, _f, _i, _vp]),
     "mynn_rope": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
@@ -271,8 +271,9 @@ def quantizing_kvcache_update_streaming(cache, scale, new_kv, offset, ring_sink,
 
 
 def attention_streaming(q, k, v, scale, is_causal, active, ring_sink, ring_window, ring_start, q_pos_offset=None,
-                        k_scale=None, v_scale=None):
-    """Attention over the sink + ring layout: keys by recency rank, rank -> cache row by the ring map."""
+                        k_scale=None, v_scale=None, rope=None):
+    """Attention over the sink + ring layout: keys by recency rank, rank -> cache row by the ring map.
+    rope = (cos_table, sin_table, kv_position int64): rotate K inside the operator."""
     import torch
 
     B, Hq, Sq, D = q.shape
@@ -283,7 +284,8 @@ def attention_streaming(q, k, v, scale, is_causal, active, ring_sink, ring_windo
     check(lib().mynn_attention_streaming(_ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(k_scale), _ptr(v_scale), float(scale),
                                          int(is_causal), B, Sq, int(active), cache_len, int(q_pos_offset), Hq, Hkv, D,
                                          _dt(q), int(k.dtype == torch.int8), int(ring_sink), int(ring_window),
-                                         int(ring_start), _stream()))
+                                         int(ring_start), _ptr(rope[0]) if rope else None, _ptr(rope[1]) if rope else None,
+                                         _ptr(rope[2]) if rope else None, _stream()))
     return out
 
 

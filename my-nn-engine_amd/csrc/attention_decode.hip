@@ -622,7 +622,46 @@ __global__ void ring_rows_kernel(uint16_t *dst, const uint16_t *src, size_t unit
     }
 }
 
-static Grown g_ring_k, g_ring_v, g_ring_ks, g_ring_vs;
+static Grown g_ring_k, g_ring_v, g_ring_ks, g_ring_vs, g_ring_q, g_ring_o;
+
+// K rotated inside the operator (reference attention.cuh:407-420, 559-570): the key of rank r, dequantised,
+// is rotated by table row kv_position[r], everything in f32; V is dequantised.  Both land in rank order as f32.
+template <typename T, bool KVI8>
+__global__ void ring_rope_rows_kernel(float *kf, float *vf, const void *K, const void *V, const T *k_scale, const T *v_scale,
+                                      const T *cos_t, const T *sin_t, const int64_t *kv_position, int D, int rows, int cache_len,
+                                      int sink, int window, int start, size_t total) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int d = (int)(i % D), r = (int)((i / D) % rows);
+    const size_t bh = i / ((size_t)D * rows);
+    const size_t tok = bh * cache_len + ring_phys_index(r, sink, window, start);
+    const int half = D / 2, dp = d < half ? d + half : d - half;
+    const float sign = d < half ? -1.0f : 1.0f;
+    float k, kp, v;
+    if constexpr (KVI8) {
+        const float ks = Elem<T>::ld(k_scale, tok), vs = Elem<T>::ld(v_scale, tok);
+        k = (float)((const int8_t *)K)[tok * D + d] * ks;
+        kp = (float)((const int8_t *)K)[tok * D + dp] * ks;
+        v = (float)((const int8_t *)V)[tok * D + d] * vs;
+    } else {
+        k = Elem<T>::ld((const T *)K, tok * D + d);
+        kp = Elem<T>::ld((const T *)K, tok * D + dp);
+        v = Elem<T>::ld((const T *)V, tok * D + d);
+    }
+    const size_t tab = (size_t)kv_position[r] * D + d;
+    kf[i] = k * Elem<T>::ld(cos_t, tab) + (sign * kp) * Elem<T>::ld(sin_t, tab);
+    vf[i] = v;
+}
+template <typename T>
+__global__ void widen_rows_kernel(float *dst, const T *src, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = Elem<T>::ld(src, i);
+}
+template <typename T>
+__global__ void narrow_rows_kernel(T *dst, const float *src, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) Elem<T>::st(dst, i, src[i]);
+}
 
 }  // namespace mynn
 
@@ -653,11 +692,15 @@ extern "C" int mynn_kvcache_update_streaming(void *cache, const void *new_kv, in
 extern "C" int mynn_attention_streaming(void *out, const void *Q, const void *K, const void *V, const void *k_scale,
                                         const void *v_scale, float scale, int is_causal, int B, int Sq, int active_seq_kv,
                                         int cache_seq_len, int q_pos_offset, int num_q_heads, int num_kv_heads, int head_dim,
-                                        int dtype, int kv_int8, int ring_sink, int ring_window, int ring_start, mynn_stream s) {
+                                        int dtype, int kv_int8, int ring_sink, int ring_window, int ring_start,
+                                        const void *cos_t, const void *sin_t, const int64_t *kv_position, mynn_stream s) {
     using namespace mynn;
     MYNN_REQUIRE(ring_sink >= 0 && ring_window >= 0 && ring_start >= 0 && (ring_window == 0 || ring_start < ring_window),
                  MYNN_ERR_INVALID, "attention: ring sink=%d window=%d start=%d", ring_sink, ring_window, ring_start);
-    if (ring_window == 0)
+    const bool rope_on = cos_t || sin_t || kv_position;
+    MYNN_REQUIRE(!rope_on || (cos_t && sin_t && kv_position), MYNN_ERR_INVALID,
+                 "attention: the K rotation needs cos, sin and kv_position together");
+    if (ring_window == 0 && !rope_on)
         return mynn_attention(out, Q, K, V, k_scale, v_scale, scale, is_causal, B, Sq, active_seq_kv, nullptr, cache_seq_len,
                               q_pos_offset, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, s);
     MYNN_REQUIRE(out && Q && K && V, MYNN_ERR_INVALID, "attention: null operand");
@@ -670,11 +713,54 @@ extern "C" int mynn_attention_streaming(void *out, const void *Q, const void *K,
     MYNN_REQUIRE(dtype_ok(dtype), MYNN_ERR_INVALID, "attention: dtype %d", dtype);
     // ranks past sink + window would read ring rows a second time (the reference's kernels do); the session
     // never asks for them, and the plain kernels clamp the same way
-    const int rows = active_seq_kv < ring_sink + ring_window ? active_seq_kv : ring_sink + ring_window;
-    const size_t eb = dtype_size(dtype), row_bytes = (size_t)head_dim * (kv_int8 ? 1 : eb);
-    MYNN_REQUIRE(row_bytes % 2 == 0 && eb % 2 == 0, MYNN_ERR_UNSUPPORTED, "attention: rows of %zu bytes", row_bytes);
+    int rows = active_seq_kv < ring_sink + ring_window ? active_seq_kv : ring_sink + ring_window;
+    if (ring_window == 0) rows = active_seq_kv < cache_seq_len ? active_seq_kv : cache_seq_len;
     const int BH = B * num_kv_heads;
     hipStream_t st = as_stream(s);
+    if (rope_on) {
+        // f32 throughout, as the reference's kernel computes it: rotated / dequantised K and V in rank order, the
+        // queries widened, the f32 attention over them, one rounding of the result
+        MYNN_REQUIRE(head_dim % 2 == 0, MYNN_ERR_INVALID, "attention: head_dim %d", head_dim);
+        const size_t kv_n = (size_t)BH * rows * head_dim, q_n = (size_t)B * num_q_heads * Sq * head_dim;
+        int rc = ensure(g_ring_k, kv_n * 4, false, st);
+        if (!rc) rc = ensure(g_ring_v, kv_n * 4, false, st);
+        if (rc) return rc;
+        const void *qf = Q;
+        void *of = out;
+        if (dtype != MYNN_F32) {
+            rc = ensure(g_ring_q, q_n * 4, false, st);
+            if (!rc) rc = ensure(g_ring_o, q_n * 4, false, st);
+            if (rc) return rc;
+            qf = g_ring_q.ptr;
+            of = g_ring_o.ptr;
+        }
+        rc = dispatch_dtype(dtype, [&](auto *t) {
+            using T = std::remove_pointer_t<decltype(t)>;
+            const dim3 grid((unsigned)((kv_n + 255) / 256));
+            if (kv_int8)
+                MYNN_LAUNCH((ring_rope_rows_kernel<T, true>), grid, dim3(256), 0, st, (float *)g_ring_k.ptr, (float *)g_ring_v.ptr, K, V,
+                            (const T *)k_scale, (const T *)v_scale, (const T *)cos_t, (const T *)sin_t, kv_position, head_dim, rows,
+                            cache_seq_len, ring_sink, ring_window, ring_start, kv_n);
+            else
+                MYNN_LAUNCH((ring_rope_rows_kernel<T, false>), grid, dim3(256), 0, st, (float *)g_ring_k.ptr, (float *)g_ring_v.ptr, K, V,
+                            (const T *)nullptr, (const T *)nullptr, (const T *)cos_t, (const T *)sin_t, kv_position, head_dim, rows,
+                            cache_seq_len, ring_sink, ring_window, ring_start, kv_n);
+            if (dtype != MYNN_F32)
+                MYNN_LAUNCH(widen_rows_kernel<T>, dim3((unsigned)((q_n + 255) / 256)), dim3(256), 0, st, (float *)g_ring_q.ptr, (const T *)Q, q_n);
+            return launch_status("ring_rope_rows_kernel");
+        });
+        if (rc) return rc;
+        rc = mynn_attention(of, qf, g_ring_k.ptr, g_ring_v.ptr, nullptr, nullptr, scale, is_causal, B, Sq, rows, nullptr, rows, q_pos_offset,
+                            num_q_heads, num_kv_heads, head_dim, MYNN_F32, 0, s);
+        if (rc || dtype == MYNN_F32) return rc;
+        return dispatch_dtype16(dtype, [&](auto *t) {
+            using T = std::remove_pointer_t<decltype(t)>;
+            MYNN_LAUNCH(narrow_rows_kernel<T>, dim3((unsigned)((q_n + 255) / 256)), dim3(256), 0, st, (T *)out, (const float *)g_ring_o.ptr, q_n);
+            return launch_status("narrow_rows_kernel");
+        });
+    }
+    const size_t eb = dtype_size(dtype), row_bytes = (size_t)head_dim * (kv_int8 ? 1 : eb);
+    MYNN_REQUIRE(row_bytes % 2 == 0 && eb % 2 == 0, MYNN_ERR_UNSUPPORTED, "attention: rows of %zu bytes", row_bytes);
     auto gather = [&](Grown &gbuf, const void *src, size_t rb) -> int {
         // (16 bytes of slack: the attention kernels want 16-byte aligned K / V, which hipMalloc gives)
         int rc = ensure(gbuf, (size_t)BH * rows * rb + 16, false, st);

@@ -285,16 +285,37 @@ def quantizing_kv_cache_update_streaming(cache, scale, new_kv, offset, ring_sink
 
 
 def attention_streaming(q, k, v, dt, scale, is_causal, active, ring_sink, ring_window, ring_start, k_scale=None,
-                        v_scale=None):
+                        v_scale=None, rope=None):
     """Attention over the sink + ring layout (src/codegen/cuda/cpp/attention.cuh:386-404, 436-438, 548-550):
     keys are enumerated by recency rank 0..active-1, the key of rank r is cache row ring_phys_index(r), and
     the causal rule compares query positions with ranks.  Restated as the plain attention of this module over
-    the rows gathered in rank order."""
+    the rows gathered in rank order.
+
+    rope = (cos_table, sin_table, kv_position) switches on the rotation of K inside the operator
+    (attention.cuh:407-420, 559-570): the dequantised key of RANK r is rotated (half-split) by row
+    kv_position[r] of the tables, all in f32, before the dot product; scores, softmax and P.V stay f32, so the
+    restatement runs the f32 attention over the rotated / dequantised rows and rounds the result once."""
     rows = [ring_phys_index(r, ring_sink, ring_window, ring_start) for r in range(active)]
-    kg, vg = np.ascontiguousarray(k[:, :, rows]), np.ascontiguousarray(v[:, :, rows])
-    ks = np.ascontiguousarray(k_scale[:, :, rows]) if k_scale is not None else None
-    vs = np.ascontiguousarray(v_scale[:, :, rows]) if v_scale is not None else None
-    return attention(q, kg, vg, dt, scale, is_causal, active, ks, vs)
+    if rope is None:
+        kg, vg = np.ascontiguousarray(k[:, :, rows]), np.ascontiguousarray(v[:, :, rows])
+        ks = np.ascontiguousarray(k_scale[:, :, rows]) if k_scale is not None else None
+        vs = np.ascontiguousarray(v_scale[:, :, rows]) if v_scale is not None else None
+        return attention(q, kg, vg, dt, scale, is_causal, active, ks, vs)
+    cos_t, sin_t, kv_position = rope
+    D = q.shape[-1]
+    half = D // 2
+    if k.dtype == np.int8:
+        kf = k[:, :, rows].astype(np.float32) * to_f32(k_scale, dt)[:, :, rows, None]
+        vf = v[:, :, rows].astype(np.float32) * to_f32(v_scale, dt)[:, :, rows, None]
+    else:
+        kf, vf = to_f32(k, dt)[:, :, rows], to_f32(v, dt)[:, :, rows]
+    pos = np.asarray(kv_position, np.int64)[:active]
+    c, sn = to_f32(cos_t, dt)[pos], to_f32(sin_t, dt)[pos]  # [active, D]
+    pair = np.concatenate([kf[..., half:], kf[..., :half]], axis=-1)
+    sign = np.concatenate([-np.ones(half, np.float32), np.ones(half, np.float32)])
+    krot = (kf * c + (sign * pair) * sn).astype(np.float32)
+    out = attention(to_f32(q, dt), np.ascontiguousarray(krot), np.ascontiguousarray(vf), F32, scale, is_causal, active)
+    return to_storage(out, dt)
 
 
 def quantizing_kv_cache_update(cache, scale, new_kv, offset, dt):

@@ -390,3 +390,58 @@ def test_quantizing_kvcache_update_streaming_bit_exact(g, dt, offset, S_new, sin
     dc, ds = g.to_dev(cache), g.to_dev(scale, dt)
     g.mynn.quantizing_kvcache_update_streaming(dc, ds, g.to_dev(new, dt), offset, sink, window, start)
     assert np.array_equal(g.to_host(dc), want_c) and np.array_equal(g.to_host(ds), want_s)
+
+
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16, orc.F32])
+@pytest.mark.parametrize("kv8,Sq,causal,window", [(True, 1, False, 16), (False, 1, False, 16), (True, 5, True, 16), (True, 1, False, 0)])
+def test_attention_streaming_with_k_rotation_inside_the_operator(g, dt, kv8, Sq, causal, window):
+    """Operator slots 10-12: the dequantised key of rank r is rotated by table row kv_position[r] (ranks, as the
+    reference's kernels index it), f32 throughout.  Against the oracle and, for the decode row, an explicit f64 loop."""
+    import torch
+
+    if kv8 and dt == orc.F32:
+        pytest.skip("int8 KV comes with 16-bit scales")
+    rng = np.random.default_rng(17 + Sq + window)
+    B, Hq, Hkv, L, D, sink, start, active = 2, 4, 2, 48, 32, 4, 7 if window else 0, 15
+    q = orc.to_storage(rng.standard_normal((B, Hq, Sq, D)), dt)
+    if kv8:
+        k = rng.integers(-127, 128, (B, Hkv, L, D)).astype(np.int8)
+        v = rng.integers(-127, 128, (B, Hkv, L, D)).astype(np.int8)
+        ks = orc.to_storage(rng.uniform(1e-3, 2e-2, (B, Hkv, L)), dt)
+        vs = orc.to_storage(rng.uniform(1e-3, 2e-2, (B, Hkv, L)), dt)
+    else:
+        k = orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt)
+        v = orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt)
+        ks = vs = None
+    cos_t, sin_t = orc.rope_table(L, D, 10000.0, dt)
+    kvpos = rng.integers(0, L, L).astype(np.int64)
+    want = orc.attention_streaming(q, k, v, dt, D ** -0.5, causal, active, sink, window, start, ks, vs, rope=(cos_t, sin_t, kvpos))
+    dev = lambda a: g.to_dev(a, dt) if a is not None and a.dtype != np.int8 else (g.to_dev(a) if a is not None else None)
+    got = g.to_host(g.mynn.attention_streaming(dev(q), dev(k), dev(v), D ** -0.5, causal, active, sink, window, start,
+                                               k_scale=dev(ks), v_scale=dev(vs),
+                                               rope=(dev(cos_t), dev(sin_t), torch.from_numpy(kvpos).cuda())))
+    assert max_err_rel_to_max(g.f32(got, dt), g.f32(want, dt)) <= (1e-2 if dt != orc.F32 else 1e-5)
+    if Sq == 1:
+        qf, cf, sf = [orc.to_f32(a, dt).astype(np.float64) for a in (q, cos_t, sin_t)]
+        out = np.zeros((B, Hq, 1, D))
+        for b in range(B):
+            for h in range(Hq):
+                hk = h // (Hq // Hkv)
+                sc, vv = [], []
+                for r in range(active):
+                    slot = orc.ring_phys_index(r, sink, window, start)
+                    if kv8:
+                        kk = k[b, hk, slot].astype(np.float64) * float(orc.to_f32(ks[b, hk, slot:slot + 1], dt)[0])
+                        vr = v[b, hk, slot].astype(np.float64) * float(orc.to_f32(vs[b, hk, slot:slot + 1], dt)[0])
+                    else:
+                        kk = orc.to_f32(k[b, hk, slot], dt).astype(np.float64)
+                        vr = orc.to_f32(v[b, hk, slot], dt).astype(np.float64)
+                    p = int(kvpos[r])
+                    rot = np.concatenate([kk[:D // 2] * cf[p, :D // 2] - kk[D // 2:] * sf[p, :D // 2],
+                                          kk[D // 2:] * cf[p, D // 2:] + kk[:D // 2] * sf[p, D // 2:]])
+                    sc.append(float(qf[b, h, 0] @ rot) * D ** -0.5)
+                    vv.append(vr)
+                sc = np.array(sc)
+                w = np.exp(sc - sc.max())
+                out[b, h, 0] = (w / w.sum()) @ np.array(vv)
+        assert max_err_rel_to_max(g.f32(got, dt), out) <= (4e-3 if dt == orc.BF16 else 1e-3 if dt == orc.F16 else 1e-5)
