@@ -19,8 +19,6 @@
 #include "attention.h"
 #include "kernels.h"
 
-#include "decode_persistent.h"
-
 namespace mynn {
 
 // ---- plain (un-quantised) linear: out[m,n] = T(sum_k act[m,k] * w[n,k]), one wave per element.
@@ -102,13 +100,6 @@ struct Model {
     hipGraphExec_t graph_exec = nullptr;
     bool use_graph = false;
     int launches = 0;
-    // single-launch decode step: per-layer pointer table, two sets of hand-over words, grid size;
-    // its error word and step counter sit behind the loop-state scalars (d_past[3], d_past[4])
-    bool persistent = false;
-    PdLayer *pd_layers = nullptr;
-    uint64_t *pd_hand = nullptr;
-    size_t pd_set_words = 0;
-    int pd_nb = 0;
     // per-launch record of the last enqueue (names + algorithmic bytes), events when profiling
     std::vector<Launch> record;
     bool profiling = false;
@@ -118,7 +109,6 @@ struct Model {
 static mynn_model_config g_cfg{};
 static bool g_cfg_set = false;
 static int g_weights_quantized = 1;
-static int g_decode_persistent = 1;  // batch-1 decode executors use the single-launch step when the shape allows
 static std::mutex g_mu;
 
 static size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -236,30 +226,6 @@ static int enqueue_step(Model &m) {
     m.record.clear();
     for (hipEvent_t e : m.events) hipEventDestroy(e);
     m.events.clear();
-
-    if (m.persistent) {
-        // the whole step in one launch; bytes = the sum of what the per-op launches below would note
-        const double NQ = QD + 2 * KD;
-        double bytes = H + eb + H * eb;
-        bytes += (double)c.n_layers * ((NQ * H + NQ * eb + 2 * H * eb + NQ * eb) + (NQ * eb + 2.0 * KD * eb + QD * eb) +
-                                       ((double)H * QD + H * eb + QD * eb + 2 * H * eb) +
-                                       (2.0 * F * H + 2.0 * F * eb + 2 * H * eb + F * eb) + ((double)H * F + H * eb + F * eb + 2 * H * eb));
-        bytes += (double)V * H + V * eb + 2 * H * eb + V * eb + V * eb;
-        note(m, "decode_step_persistent", bytes);
-        PdParams p{};
-        p.layers = m.pd_layers; p.n_layers = c.n_layers; p.H = H; p.Hq = Hq; p.Hkv = Hkv; p.F = F; p.V = V; p.max_seq = c.max_seq;
-        p.eps = c.eps; p.softmax_scale = 1.0f / sqrtf((float)D);
-        p.embed_w = (const int8_t *)m.embed.w; p.embed_s = m.embed.scale; p.final_norm = m.final_norm;
-        p.lm_w = (const int8_t *)m.lm_head.w; p.lm_s = m.lm_head.scale; p.cos_t = m.cos_t; p.sin_t = m.sin_t;
-        p.hand = m.pd_hand; p.set_words = (int)m.pd_set_words; p.logits = m.logits; p.next = m.d_next;
-        p.adv = AdvanceState{m.d_ids, m.d_pos, m.d_past, m.d_active, m.d_tokens, m.d_step, m.token_cap};
-        p.err = m.d_past + 3; p.epoch = (unsigned *)(m.d_past + 4); p.spin_limit = 400000;
-        const PdShape shape{c.n_layers, H, Hq, Hkv, D, F, V, c.max_seq};
-        TRY(decode_persistent_launch(p, shape, c.dtype, m.pd_nb, s));
-        launch_timer() = LaunchTimer{};
-        m.launches = (int)m.record.size();
-        return 0;
-    }
 
     // embed: DequantizeLinear(table) -> Gather(ids), one row per token
     if (m.quant) {
@@ -608,35 +574,6 @@ static int build(Model &m, void **init, void **state) {
     MYNN_HIP(hipHostMalloc((void **)&m.h_stage, m.stage_bytes, hipHostMallocDefault));
     MYNN_HIP(hipDeviceSynchronize());
 
-    // ---- batch-1 decode: the single-launch step when the shape, the alignment and the device allow
-    if (m.quant && rows == 1 && !c.quantize_activations && !c.quant_kv_cache && g_decode_persistent) {
-        int dev = 0, cus = 0;
-        MYNN_HIP(hipGetDevice(&dev));
-        MYNN_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-        const PdShape shape{c.n_layers, H, c.n_heads, c.n_kv_heads, c.head_dim, F, V, c.max_seq};
-        bool ok = decode_persistent_supported(shape, c.dtype, cus) && aligned16(m.embed.w) && aligned16(m.lm_head.w) &&
-                  aligned16(m.final_norm);
-        for (const Layer &L : m.layers)
-            ok = ok && aligned16(L.qkv.w) && aligned16(L.o.w) && aligned16(L.gu.w) && aligned16(L.down.w) && aligned16(L.norm1) &&
-                 aligned16(L.norm2) && aligned16(L.k_cache) && aligned16(L.v_cache);
-        if (ok) {
-            std::vector<PdLayer> hl(c.n_layers);
-            for (int li = 0; li < c.n_layers; li++) {
-                const Layer &L = m.layers[li];
-                hl[li] = PdLayer{(const int8_t *)L.qkv.w, (const int8_t *)L.o.w, (const int8_t *)L.gu.w, (const int8_t *)L.down.w,
-                                 L.qkv.scale, L.o.scale, L.gu.scale, L.down.scale, L.norm1, L.norm2, L.k_cache, L.v_cache};
-            }
-            m.pd_nb = cus;
-            m.pd_set_words = decode_persistent_set_words(shape, cus);
-            MYNN_HIP(hipMalloc((void **)&m.pd_layers, hl.size() * sizeof(PdLayer)));
-            MYNN_HIP(hipMemcpy(m.pd_layers, hl.data(), hl.size() * sizeof(PdLayer), hipMemcpyHostToDevice));
-            MYNN_HIP(hipMalloc((void **)&m.pd_hand, 2 * m.pd_set_words * 8));
-            MYNN_HIP(hipMemset(m.pd_hand, 0xFF, 2 * m.pd_set_words * 8));
-            MYNN_HIP(hipDeviceSynchronize());
-            m.persistent = true;
-        }
-    }
-
     // ---- capture the decode step once (one new token per sequence, any batch: every launch reads its
     // positions and lengths from device memory)
     if (c.seq_q == 1) {
@@ -689,8 +626,6 @@ static void destroy(Model *m) {
         if (L.pk_gu) hipFree(L.pk_gu);
         if (L.pk_down) hipFree(L.pk_down);
     }
-    if (m->pd_layers) hipFree(m->pd_layers);
-    if (m->pd_hand) hipFree(m->pd_hand);
     if (m->wt_lm_head) hipFree(m->wt_lm_head);
     if (m->pk_lm_head) hipFree(m->pk_lm_head);
     if (m->cos_t) hipFree(m->cos_t);
@@ -724,14 +659,6 @@ static int upload_inputs(Model &m, const int64_t *ids, const int64_t *pos, int64
     MYNN_HIP(hipMemcpyAsync(m.d_pos, h_pos, (size_t)c.seq_q * 8, hipMemcpyHostToDevice, m.stream));
     MYNN_HIP(hipMemcpyAsync(m.d_past, h_sc, 12, hipMemcpyHostToDevice, m.stream));
     return 0;
-}
-
-// single-launch step: a wait that ran out left the error word set (read back by the caller after the
-// stream has drained); the hand-over buffers are emptied again so that the next step starts clean
-static int persistent_failed(Model &m) {
-    (void)hipMemset(m.pd_hand, 0xFF, 2 * m.pd_set_words * 8);
-    (void)hipMemset(m.d_past + 3, 0, 4);
-    return fail(MYNN_ERR_STATE, "decode step (single launch): a wait between workgroups ran out (is the device shared?)");
 }
 
 static int run_once(Model &m) {
@@ -797,11 +724,6 @@ extern "C" void *model_init(void **initializer, void **session_state) {
 }
 
 extern "C" void model_destroy(void *state) { destroy((Model *)state); }
-extern "C" int mynn_set_decode_persistent(int on) {
-    std::lock_guard<std::mutex> lk(g_mu);
-    g_decode_persistent = on != 0;
-    return 0;
-}
 extern "C" void model_device_sync(void) { (void)hipDeviceSynchronize(); }
 extern "C" int model_memcpy(void *dst, const void *src, size_t n, int kind) {
     return (int)hipMemcpy(dst, src, n, (hipMemcpyKind)kind);
@@ -822,20 +744,12 @@ extern "C" int mynn_model_step(void *state, const int64_t *input_ids, const int6
     TRY(upload_inputs(m, input_ids, position_id, past_len, active_seq_kv));
     TRY(run_once(m));
     const mynn_model_config &c = m.cfg;
-    char *h_next = m.h_stage + m.stage_bytes - m.next_stage;
-    // (single-launch step: the error word travels in the same copy, d_past[3] .. d_next[0])
-    if (m.persistent) MYNN_HIP(hipMemcpyAsync(h_next, m.d_past + 3, 24, hipMemcpyDeviceToHost, m.stream));
-    else if (next_token) MYNN_HIP(hipMemcpyAsync(h_next, m.d_next, (size_t)c.batch * 4, hipMemcpyDeviceToHost, m.stream));
+    if (next_token) MYNN_HIP(hipMemcpyAsync(m.h_stage + m.stage_bytes - m.next_stage, m.d_next, (size_t)c.batch * 4, hipMemcpyDeviceToHost, m.stream));
     if (logits_host)
         MYNN_HIP(hipMemcpyAsync(logits_host, m.logits, (size_t)c.batch * c.seq_q * c.vocab * dtype_size(c.dtype),
                                 hipMemcpyDeviceToHost, m.stream));
     MYNN_HIP(hipStreamSynchronize(m.stream));
-    if (m.persistent) {
-        if (*(const int32_t *)h_next) return persistent_failed(m);
-        if (next_token) memcpy(next_token, h_next + 20, 4);
-        return 0;
-    }
-    if (next_token) memcpy(next_token, h_next, (size_t)c.batch * 4);
+    if (next_token) memcpy(next_token, m.h_stage + m.stage_bytes - m.next_stage, (size_t)c.batch * 4);
     return 0;
 }
 
@@ -887,10 +801,7 @@ extern "C" int mynn_model_decode_loop(void *state, int32_t token, int64_t past_l
     TRY(upload_inputs(m, &id, &pos, past_len, past_len + 1));
     for (int i = 0; i < n_steps; i++) TRY(run_once(m));
     MYNN_HIP(hipMemcpyAsync(m.h_stage, m.d_tokens, (size_t)n_steps * 4, hipMemcpyDeviceToHost, m.stream));
-    char *h_err = m.h_stage + m.stage_bytes - m.next_stage;
-    if (m.persistent) MYNN_HIP(hipMemcpyAsync(h_err, m.d_past + 3, 4, hipMemcpyDeviceToHost, m.stream));
     MYNN_HIP(hipStreamSynchronize(m.stream));
-    if (m.persistent && *(const int32_t *)h_err) return persistent_failed(m);
     memcpy(out_tokens, m.h_stage, (size_t)n_steps * 4);
     return 0;
 }
