@@ -27,6 +27,11 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # --pmc FETCH_SIZE (x2.000, scaled by a 256 MiB copy) + WRITE_SIZE (x1.000): 11430.0 KiB * 2 + 44.0 KiB.
 # Counters cannot be read from inside this process; the figure is carried here from that profile run.
 GATEUP_GEMV_TRAFFIC_BYTES = 23453696
+# the same for the dominant kernels of the other workloads (profiles/prefill_and_batched_decode_pmc_hbm_traffic.md):
+# prefill gate/up GEMM + SwiGLU (f16, 8192 x 11264 x 2048): 287320.4 KiB * 2 + 90112.0 KiB;
+# batched-decode gate/up few-row GEMM (Llama-3-8B shape, 32 rows): 61689.4 KiB * 2 + 896.3 KiB
+PREFILL_GATEUP_GEMM_TRAFFIC_BYTES = 680706867
+BATCHED_GATEUP_GEMM_TRAFFIC_BYTES = 127257702
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16/fp16 matrix rate
 INT8_PEAK_TOPS = 5000.0    # MI355X published dense int8 matrix rate
 PREFILL_BATCH, PREFILL_LEN = 8, 1024
@@ -149,7 +154,8 @@ def prefill_main(args, mynn, cfg):
                    "step_mfma_frac": round(step_flops / (ms_per_step * 1e-3) / 1e12 / peak, 4),
                    "per_kernel_ms": {k: round(v[1] / 2, 3) for k, v in sorted(agg.items(), key=lambda kv: -kv[1][1])}},
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 1), "peak": peak,
-                     "unit": unit, "frac": round(achieved / peak, 4), "traffic": None,
+                     "unit": unit, "frac": round(achieved / peak, 4),
+                     "traffic": PREFILL_GATEUP_GEMM_TRAFFIC_BYTES if dom == "linear_gateup_swiglu" and args.dtype == "f16" else None,
                      "flops_per_launch": fl_tot / calls, "avg_launch_us": round(ms_tot / calls * 1e3, 2),
                      "all_linear_TFLOPs": round(lin_tflops, 1)},
     }
@@ -316,7 +322,9 @@ def decode_batch_main(args, mynn):
                    "step_hbm_frac": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                    "per_kernel_ms": {k: round(v[1] / 2, 3) for k, v in sorted(agg.items(), key=lambda kv: -kv[1][1])}},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "bytes_per_launch": bytes_tot / calls,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": BATCHED_GATEUP_GEMM_TRAFFIC_BYTES if dom == "linear_gateup_swiglu" and not args.kv_int8 else None,
+                     "bytes_per_launch": bytes_tot / calls,
                      "avg_launch_us": round(ms_tot / calls * 1e3, 2)},
     }
     dec.close()
