@@ -72,6 +72,7 @@ SIGNATURES = {
     "mynn_dequant_gemv": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mynn_dequant_matmul": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "mynn_set_gemm_tile": (_i, [_i]),
+    "mynn_set_fuse_qkv_attention": (_i, [_i]),
     "mynn_quantized_matmul": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mynn_dynamic_quantize_linear": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mynn_attention": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
@@ -611,6 +612,12 @@ def set_gemm_tile(which):
     """Workgroup tile of the matrix-core GEMM: 0 = per-shape choice, 1 = 256x128, 2 = 256x256 with
     operands staged through registers, 3 = 256x256 and 4 = 256x320 with operands loaded straight into LDS."""
     check(lib().mynn_set_gemm_tile(int(which)))
+
+
+def set_fuse_qkv_attention(on):
+    """Batch-1 decode executors built after this call run a layer's q|k|v projection and attention in one
+    launch (True, the default, when the shape allows) or in two (False)."""
+    check(lib().mynn_set_fuse_qkv_attention(1 if on else 0))
 
 
 def quantize_per_channel(w_f32, scale_dt):

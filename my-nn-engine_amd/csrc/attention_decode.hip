@@ -22,6 +22,7 @@
 
 #include "attention.h"
 #include "mfma.h"
+#include "attention_short.h"
 
 namespace mynn {
 
@@ -274,141 +275,25 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
     }
 }
 
-// ---- FUSE form for a cache that one workgroup covers in registers (cache_len <= 8 passes of 64 / (D/8) keys
-// per wave and 8 waves): one workgroup per query head, and everything between the loads and the final merge
-// stays inside a wave -- a group of D/8 lanes owns a key per pass, keeps an online softmax (m, l) and the
-// 8 output dims of its lane over its keys, groups meet by shuffles, waves through one LDS exchange.  No V
-// parking, one barrier.  The latency of a decode step's attention is what this buys (short contexts are
-// launch- and latency-bound, not bandwidth-bound).
-constexpr int kShortPasses = 8;
-
+// ---- FUSE form for a cache that one workgroup covers in registers: one workgroup per query head, the
+// body is attn_short_body (attention_short.h)
 template <typename T, int D>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_short_kernel(AttnParams p) {
-    constexpr int LPK = D / 8, GPW = 64 / LPK, KPP = kAttnWaves * GPW;  // lanes per key, keys per wave / workgroup and pass
-    __shared__ float part_s[kAttnWaves][D + 2];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int dc = lane % LPK, grp = lane / LPK;
+    static_assert(kAttnWaves == kShortWaves, "the short form is written for 8 waves");
+    __shared__ float part_s[kShortWaves][D + 2];
+    const int tid = threadIdx.x;
     const int b = blockIdx.x / p.Hq, h = blockIdx.x % p.Hq;
     const int Gt = p.Hq / p.Hkv, hkv = h / Gt;
     const int active = p.d_active ? *p.d_active : p.active;
     const int bound = min(active, p.cache_len);
-    const int new_row = active - 1;  // cache row of the token being decoded
     const size_t kv_base = (size_t)(b * p.Hkv + hkv) * p.cache_len;
-    const T *Kc = (const T *)p.k + kv_base * D + dc * 8, *Vc = (const T *)p.v + kv_base * D + dc * 8;
-
-    // ---- all K / V loads of this lane
-    U4 kreg[kShortPasses], vreg[kShortPasses];
-#pragma unroll
-    for (int i = 0; i < kShortPasses; i++) {
-        const int key = i * KPP + wave * GPW + grp;
-        kreg[i] = vreg[i] = U4{0u, 0u, 0u, 0u};
-        if (key < bound && key != new_row) {
-            kreg[i] = *(const U4 *)(Kc + (size_t)key * D);
-            vreg[i] = *(const U4 *)(Vc + (size_t)key * D);
-        }
-    }
-
-    // ---- this lane's 8 dims of the rotated query, of the rotated new key and of the new value
-    constexpr int half = D / 2;
-    const int d0 = dc * 8, dp = d0 < half ? d0 + half : d0 - half;
     const T *row = (const T *)p.qkv + (size_t)b * (p.Hq + 2 * p.Hkv) * D;
-    const size_t tab = (size_t)(*p.d_pos) * D + d0;
-    float c[8], sn[8], q[8], kn[8], vn[8];
-    widen8<T>(*(const U4 *)((const T *)p.cos_t + tab), c);
-    widen8<T>(*(const U4 *)((const T *)p.sin_t + tab), sn);
-    const U4 v_new = *(const U4 *)(row + (size_t)(p.Hq + p.Hkv + hkv) * D + d0);
-    widen8<T>(v_new, vn);
-    {
-        float own[8], oth[8];
-        const T *src = row + (size_t)h * D;
-        widen8<T>(*(const U4 *)(src + d0), own);
-        widen8<T>(*(const U4 *)(src + dp), oth);
-#pragma unroll
-        for (int e = 0; e < 8; e++) q[e] = Elem<T>::rnd(d0 < half ? own[e] * c[e] - oth[e] * sn[e] : own[e] * c[e] + oth[e] * sn[e]);
-        src = row + (size_t)(p.Hq + hkv) * D;
-        widen8<T>(*(const U4 *)(src + d0), own);
-        widen8<T>(*(const U4 *)(src + dp), oth);
-#pragma unroll
-        for (int e = 0; e < 8; e++) kn[e] = Elem<T>::rnd(d0 < half ? own[e] * c[e] - oth[e] * sn[e] : own[e] * c[e] + oth[e] * sn[e]);
-    }
-    if (h % Gt == 0 && wave == 0 && grp == 0) {  // one lane group appends the new row
-        *(U4 *)((T *)p.k + (kv_base + new_row) * D + d0) =
-            U4{pack2<T>(kn[0], kn[1]), pack2<T>(kn[2], kn[3]), pack2<T>(kn[4], kn[5]), pack2<T>(kn[6], kn[7])};
-        *(U4 *)((T *)p.v + (kv_base + new_row) * D + d0) = v_new;
-    }
-
-    // ---- online softmax over this lane group's keys
-    float m = -INFINITY, l = 0.f, o[8];
-#pragma unroll
-    for (int e = 0; e < 8; e++) o[e] = 0.f;
-#pragma unroll
-    for (int i = 0; i < kShortPasses; i++) {
-        if (i * KPP >= bound) break;  // no wave has keys in this pass or a later one
-        const int key = i * KPP + wave * GPW + grp;
-        float kf[8], vf[8];
-        widen8<T>(kreg[i], kf);
-        widen8<T>(vreg[i], vf);
-        if (key == new_row) {
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                kf[e] = kn[e];
-                vf[e] = vn[e];
-            }
-        }
-        float sc = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; e++) sc = fmaf(q[e], kf[e], sc);
-        sc = group_sum<LPK>(sc) * p.scale;
-        if (key < bound) {
-            const float mn = fmaxf(m, sc);
-            const float corr = fast_exp(m - mn), pe = fast_exp(sc - mn);
-            l = l * corr + pe;
-#pragma unroll
-            for (int e = 0; e < 8; e++) o[e] = o[e] * corr + pe * vf[e];
-            m = mn;
-        }
-    }
-    // ---- lane groups of the wave meet (lanes of equal dc), then the waves through LDS
-    auto merge = [&](float m2, float l2, const float *o2) {
-        const float mn = fmaxf(m, m2);
-        const float a = m == -INFINITY ? 0.f : fast_exp(m - mn), bb = m2 == -INFINITY ? 0.f : fast_exp(m2 - mn);
-        l = l * a + l2 * bb;
-#pragma unroll
-        for (int e = 0; e < 8; e++) o[e] = o[e] * a + o2[e] * bb;
-        m = mn;
-    };
-#pragma unroll
-    for (int off = LPK; off < 64; off <<= 1) {
-        float o2[8];
-        const float m2 = __shfl_xor(m, off, 64), l2 = __shfl_xor(l, off, 64);
-#pragma unroll
-        for (int e = 0; e < 8; e++) o2[e] = __shfl_xor(o[e], off, 64);
-        merge(m2, l2, o2);
-    }
-    if (grp == 0) {
-#pragma unroll
-        for (int e = 0; e < 8; e++) part_s[wave][d0 + e] = o[e];
-        if (dc == 0) {
-            part_s[wave][D] = m;
-            part_s[wave][D + 1] = l;
-        }
-    }
-    __syncthreads();
-    if (tid < D) {
-        float mt = -INFINITY;
-#pragma unroll
-        for (int w = 0; w < kAttnWaves; w++) mt = fmaxf(mt, part_s[w][D]);
-        float lt = 0.f, ot = 0.f;
-#pragma unroll
-        for (int w = 0; w < kAttnWaves; w++) {
-            const float mw = part_s[w][D];
-            const float a = mw == -INFINITY ? 0.f : fast_exp(mw - mt);
-            lt += part_s[w][D + 1] * a;
-            ot += part_s[w][tid] * a;
-        }
-        const size_t oo = (size_t)b * p.o_bs + (size_t)h * p.o_hs + tid;
-        Elem<T>::st((T *)p.out, oo, ot / lt);
-    }
+    const size_t tab = (size_t)(*p.d_pos) * D;
+    float r;
+    if (attn_short_body<T, D>(row + (size_t)h * D, row + (size_t)(p.Hq + hkv) * D, row + (size_t)(p.Hq + p.Hkv + hkv) * D,
+                              (T *)p.k + kv_base * D, (T *)p.v + kv_base * D, bound, active - 1, h % Gt == 0,
+                              (const T *)p.cos_t + tab, (const T *)p.sin_t + tab, p.scale, part_s, tid, r, [] {}))
+        Elem<T>::st((T *)p.out, (size_t)b * p.o_bs + (size_t)h * p.o_hs + tid, r);
 }
 
 bool attention_short_supported(const AttnParams &p, int D, int dtype) {

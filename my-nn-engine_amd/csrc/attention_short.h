@@ -1,0 +1,143 @@
+// Decode attention for a cache that one workgroup covers in registers (cache_len <= 8 passes of
+// 64 / (D/8) keys per wave and 8 waves): one workgroup of 512 threads per query head, and everything
+// between the loads and the final merge stays inside a wave -- a group of D/8 lanes owns a key per
+// pass, keeps an online softmax (m, l) and the 8 output dims of its lane over its keys, groups meet by
+// shuffles, waves through one LDS exchange.  No V parking, one barrier.  RoPE of the query and of the new
+// key, and both cache appends, are part of it.  Shared by the stand-alone kernel and the single-launch
+// decode step.
+#pragma once
+#include "mynn_common.h"
+#include "mfma.h"
+
+namespace mynn {
+
+constexpr int kShortPasses = 8;
+constexpr int kShortWaves = 8;
+
+// qsrc / ksrc / vsrc: the D raw projection values of this query head, of its kv head's new key and new value
+// (any address space).  Kc / Vc: cache rows of this (batch, kv head), row stride D.  cs / sn: the RoPE table
+// rows of the token's position.  append: this workgroup writes the new row into the caches.
+// part_s: kShortWaves x (D + 2) floats of LDS.  Every thread of the 512 calls it; threads tid < D get the
+// output dim tid in `result` and return true.  `ready()` runs once the cache loads are on their way and before
+// qsrc / ksrc / vsrc are read: a caller whose projection values arrive late waits for them there.
+template <typename T, int D, typename Ready>
+__device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, const T *vsrc, T *Kcache, T *Vcache, int bound,
+                                                int new_row, bool append, const T *cs, const T *snp, float scale,
+                                                float (*part_s)[D + 2], int tid, float &result, Ready ready) {
+    constexpr int LPK = D / 8, GPW = 64 / LPK, KPP = kShortWaves * GPW;  // lanes per key, keys per wave / workgroup and pass
+    const int lane = tid & 63, wave = tid >> 6;
+    const int dc = lane % LPK, grp = lane / LPK;
+    const T *Kc = Kcache + dc * 8, *Vc = Vcache + dc * 8;
+
+    // ---- all K / V loads of this lane
+    U4 kreg[kShortPasses], vreg[kShortPasses];
+#pragma unroll
+    for (int i = 0; i < kShortPasses; i++) {
+        const int key = i * KPP + wave * GPW + grp;
+        kreg[i] = vreg[i] = U4{0u, 0u, 0u, 0u};
+        if (key < bound && key != new_row) {
+            kreg[i] = *(const U4 *)(Kc + (size_t)key * D);
+            vreg[i] = *(const U4 *)(Vc + (size_t)key * D);
+        }
+    }
+
+    ready();
+    // ---- this lane's 8 dims of the rotated query, of the rotated new key and of the new value
+    constexpr int half = D / 2;
+    const int d0 = dc * 8, dp = d0 < half ? d0 + half : d0 - half;
+    float c[8], sn[8], q[8], kn[8], vn[8];
+    widen8<T>(*(const U4 *)(cs + d0), c);
+    widen8<T>(*(const U4 *)(snp + d0), sn);
+    const U4 v_new = *(const U4 *)(vsrc + d0);
+    widen8<T>(v_new, vn);
+    {
+        float own[8], oth[8];
+        widen8<T>(*(const U4 *)(qsrc + d0), own);
+        widen8<T>(*(const U4 *)(qsrc + dp), oth);
+#pragma unroll
+        for (int e = 0; e < 8; e++) q[e] = Elem<T>::rnd(d0 < half ? own[e] * c[e] - oth[e] * sn[e] : own[e] * c[e] + oth[e] * sn[e]);
+        widen8<T>(*(const U4 *)(ksrc + d0), own);
+        widen8<T>(*(const U4 *)(ksrc + dp), oth);
+#pragma unroll
+        for (int e = 0; e < 8; e++) kn[e] = Elem<T>::rnd(d0 < half ? own[e] * c[e] - oth[e] * sn[e] : own[e] * c[e] + oth[e] * sn[e]);
+    }
+    if (append && wave == 0 && grp == 0) {  // one lane group appends the new row
+        *(U4 *)(Kcache + (size_t)new_row * D + d0) =
+            U4{pack2<T>(kn[0], kn[1]), pack2<T>(kn[2], kn[3]), pack2<T>(kn[4], kn[5]), pack2<T>(kn[6], kn[7])};
+        *(U4 *)(Vcache + (size_t)new_row * D + d0) = v_new;
+    }
+
+    // ---- online softmax over this lane group's keys
+    float m = -INFINITY, l = 0.f, o[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) o[e] = 0.f;
+#pragma unroll
+    for (int i = 0; i < kShortPasses; i++) {
+        if (i * KPP >= bound) break;  // no wave has keys in this pass or a later one
+        const int key = i * KPP + wave * GPW + grp;
+        float kf[8], vf[8];
+        widen8<T>(kreg[i], kf);
+        widen8<T>(vreg[i], vf);
+        if (key == new_row) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                kf[e] = kn[e];
+                vf[e] = vn[e];
+            }
+        }
+        float sc = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) sc = fmaf(q[e], kf[e], sc);
+        sc = group_sum<LPK>(sc) * scale;
+        if (key < bound) {
+            const float mn = fmaxf(m, sc);
+            const float corr = fast_exp(m - mn), pe = fast_exp(sc - mn);
+            l = l * corr + pe;
+#pragma unroll
+            for (int e = 0; e < 8; e++) o[e] = o[e] * corr + pe * vf[e];
+            m = mn;
+        }
+    }
+    // ---- lane groups of the wave meet (lanes of equal dc), then the waves through LDS
+    auto merge = [&](float m2, float l2, const float *o2) {
+        const float mn = fmaxf(m, m2);
+        const float a = m == -INFINITY ? 0.f : fast_exp(m - mn), bb = m2 == -INFINITY ? 0.f : fast_exp(m2 - mn);
+        l = l * a + l2 * bb;
+#pragma unroll
+        for (int e = 0; e < 8; e++) o[e] = o[e] * a + o2[e] * bb;
+        m = mn;
+    };
+#pragma unroll
+    for (int off = LPK; off < 64; off <<= 1) {
+        float o2[8];
+        const float m2 = __shfl_xor(m, off, 64), l2 = __shfl_xor(l, off, 64);
+#pragma unroll
+        for (int e = 0; e < 8; e++) o2[e] = __shfl_xor(o[e], off, 64);
+        merge(m2, l2, o2);
+    }
+    if (grp == 0) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) part_s[wave][d0 + e] = o[e];
+        if (dc == 0) {
+            part_s[wave][D] = m;
+            part_s[wave][D + 1] = l;
+        }
+    }
+    __syncthreads();
+    if (tid >= D) return false;
+    float mt = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kShortWaves; w++) mt = fmaxf(mt, part_s[w][D]);
+    float lt = 0.f, ot = 0.f;
+#pragma unroll
+    for (int w = 0; w < kShortWaves; w++) {
+        const float mw = part_s[w][D];
+        const float a = mw == -INFINITY ? 0.f : fast_exp(mw - mt);
+        lt += part_s[w][D + 1] * a;
+        ot += part_s[w][tid] * a;
+    }
+    result = ot / lt;
+    return true;
+}
+
+}  // namespace mynn

@@ -100,6 +100,9 @@ struct Model {
     hipGraphExec_t graph_exec = nullptr;
     bool use_graph = false;
     int launches = 0;
+    // batch-1 decode: projection and attention share a launch; m.qkv is then the hand-over vector between them
+    // (all 0xFFFF between uses) and d_past[3] the error word of its bounded waits
+    bool qkv_attn = false;
     // per-launch record of the last enqueue (names + algorithmic bytes), events when profiling
     std::vector<Launch> record;
     bool profiling = false;
@@ -109,6 +112,7 @@ struct Model {
 static mynn_model_config g_cfg{};
 static bool g_cfg_set = false;
 static int g_weights_quantized = 1;
+static int g_fuse_qkv_attention = 1;  // batch-1 decode executors built from now on share a launch between q|k|v and attention
 static std::mutex g_mu;
 
 static size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -241,7 +245,16 @@ static int enqueue_step(Model &m) {
         Layer &L = m.layers[li];
         // ---- attention block
         bool roped = false;
-        if (fused) {
+        if (fused && m.qkv_attn) {
+            // RMSNorm + q|k|v projection, RoPE, both cache appends and the attention in one launch
+            note(m, "qkv_attention", (double)L.qkv.N * H + L.qkv.N * eb + 2 * H * eb + 2.0 * KD * eb + QD * eb);
+            QkvAttnParams p{};
+            p.x = m.x; p.norm_w = L.norm1; p.eps = c.eps; p.wq = (const int8_t *)L.qkv.w; p.scale = L.qkv.scale;
+            p.N = L.qkv.N; p.K = H; p.qkv = (uint64_t *)m.qkv; p.out = m.attn; p.k_cache = L.k_cache; p.v_cache = L.v_cache;
+            p.cos_t = m.cos_t; p.sin_t = m.sin_t; p.d_pos = m.d_pos; p.d_active = m.d_active; p.Hq = Hq; p.Hkv = Hkv;
+            p.max_seq = c.max_seq; p.softmax_scale = softmax_scale; p.err = m.d_past + 3; p.spin_limit = 400000;
+            TRY(qkv_attention_launch(p, D, c.dtype, s));
+        } else if (fused) {
             note(m, "gemv_norm_qkv", (double)L.qkv.N * H + L.qkv.N * eb + 2 * H * eb + L.qkv.N * eb);
             TRY(gemv_norm<T>(m.qkv, m.x, L.norm1, c.eps, (const int8_t *)L.qkv.w, L.qkv.scale, L.qkv.N, H, s));
         } else if (m.w8a8_fused) {
@@ -262,7 +275,7 @@ static int enqueue_step(Model &m) {
             else if (m.resident16) TRY(gemm_rows(m, m.qkv, m.nrm, L.wt_qkv, nullptr, rows, L.qkv.N, H, GEMM_PLAIN, "linear_qkv"));
             else TRY(linear_rows<T>(m, m.qkv, m.nrm, L.qkv, rows, "linear_qkv"));
         }
-        {
+        if (!(fused && m.qkv_attn)) {
             AttnParams p{};
             p.out = m.attn; p.q = m.q; p.k = L.k_cache; p.v = L.v_cache; p.scale = softmax_scale;
             p.k_scale = L.k_scale; p.v_scale = L.v_scale;
@@ -294,7 +307,9 @@ static int enqueue_step(Model &m) {
         }
         if (fused) {
             note(m, "gemv_o_residual", (double)H * QD + H * eb + QD * eb + 2 * H * eb);
-            TRY(gemv_residual<T>(m.x2, m.attn, (const int8_t *)L.o.w, L.o.scale, m.x, H, QD, s));
+            // (the o projection also empties the hand-over vector of the fused launch before its next use)
+            TRY(gemv_residual<T>(m.x2, m.attn, (const int8_t *)L.o.w, L.o.scale, m.x, H, QD, s,
+                                 m.qkv_attn ? (uint64_t *)m.qkv : nullptr, m.qkv_attn ? (QD + 2 * KD) * (int)sizeof(T) / 8 : 0));
             note(m, "gemv_norm_gateup_swiglu", (double)L.gu.N * H + L.gu.N * eb + 2 * H * eb + F * eb);
             TRY(gemv_norm_swiglu<T>(m.hmid, m.x2, L.norm2, c.eps, (const int8_t *)L.gu.w, L.gu.scale, L.gu.N, H, s));
             note(m, "gemv_down_residual", (double)H * F + H * eb + F * eb + 2 * H * eb);
@@ -574,6 +589,20 @@ static int build(Model &m, void **init, void **state) {
     MYNN_HIP(hipHostMalloc((void **)&m.h_stage, m.stage_bytes, hipHostMallocDefault));
     MYNN_HIP(hipDeviceSynchronize());
 
+    // ---- batch-1 decode: projection and attention in one launch when the shape allows
+    if (m.quant && rows == 1 && !c.quantize_activations && !c.quant_kv_cache && g_fuse_qkv_attention &&
+        attention_fused_supported(c.head_dim, c.n_heads / c.n_kv_heads) &&
+        qkv_attention_supported(H, c.n_heads, c.n_kv_heads, c.head_dim, c.max_seq, c.dtype) && (QD + 2 * KD) * eb % 8 == 0) {
+        bool ok = aligned16(m.qkv) && aligned16(m.x) && aligned16(m.attn);
+        for (const Layer &L : m.layers)
+            ok = ok && aligned16(L.qkv.w) && aligned16(L.norm1) && aligned16(L.k_cache) && aligned16(L.v_cache) && aligned16(L.o.w);
+        if (ok && QD % 8 == 0 && (QD + 1023) / 1024 <= 14) {
+            MYNN_HIP(hipMemset(m.qkv, 0xFF, (size_t)(QD + 2 * KD) * eb));
+            MYNN_HIP(hipDeviceSynchronize());
+            m.qkv_attn = true;
+        }
+    }
+
     // ---- capture the decode step once (one new token per sequence, any batch: every launch reads its
     // positions and lengths from device memory)
     if (c.seq_q == 1) {
@@ -661,6 +690,15 @@ static int upload_inputs(Model &m, const int64_t *ids, const int64_t *pos, int64
     return 0;
 }
 
+// fused projection + attention: a wait that ran out left the error word set (read back after the stream has
+// drained); the hand-over vector is emptied again so that the next step starts clean
+static int qkv_attention_failed(Model &m) {
+    const mynn_model_config &c = m.cfg;
+    (void)hipMemset(m.qkv, 0xFF, (size_t)(c.n_heads + 2 * c.n_kv_heads) * c.head_dim * dtype_size(c.dtype));
+    (void)hipMemset(m.d_past + 3, 0, 4);
+    return fail(MYNN_ERR_STATE, "decode step: the attention waited too long for the q|k|v projection (is the device shared?)");
+}
+
 static int run_once(Model &m) {
     if (m.use_graph && !m.profiling) {
         MYNN_HIP(hipGraphLaunch(m.graph_exec, m.stream));
@@ -724,6 +762,11 @@ extern "C" void *model_init(void **initializer, void **session_state) {
 }
 
 extern "C" void model_destroy(void *state) { destroy((Model *)state); }
+extern "C" int mynn_set_fuse_qkv_attention(int on) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    g_fuse_qkv_attention = on != 0;
+    return 0;
+}
 extern "C" void model_device_sync(void) { (void)hipDeviceSynchronize(); }
 extern "C" int model_memcpy(void *dst, const void *src, size_t n, int kind) {
     return (int)hipMemcpy(dst, src, n, (hipMemcpyKind)kind);
@@ -744,12 +787,20 @@ extern "C" int mynn_model_step(void *state, const int64_t *input_ids, const int6
     TRY(upload_inputs(m, input_ids, position_id, past_len, active_seq_kv));
     TRY(run_once(m));
     const mynn_model_config &c = m.cfg;
-    if (next_token) MYNN_HIP(hipMemcpyAsync(m.h_stage + m.stage_bytes - m.next_stage, m.d_next, (size_t)c.batch * 4, hipMemcpyDeviceToHost, m.stream));
+    char *h_next = m.h_stage + m.stage_bytes - m.next_stage;
+    // (fused projection + attention: the error word travels in the same copy, d_past[3] .. d_next[0])
+    if (m.qkv_attn) MYNN_HIP(hipMemcpyAsync(h_next, m.d_past + 3, 24, hipMemcpyDeviceToHost, m.stream));
+    else if (next_token) MYNN_HIP(hipMemcpyAsync(h_next, m.d_next, (size_t)c.batch * 4, hipMemcpyDeviceToHost, m.stream));
     if (logits_host)
         MYNN_HIP(hipMemcpyAsync(logits_host, m.logits, (size_t)c.batch * c.seq_q * c.vocab * dtype_size(c.dtype),
                                 hipMemcpyDeviceToHost, m.stream));
     MYNN_HIP(hipStreamSynchronize(m.stream));
-    if (next_token) memcpy(next_token, m.h_stage + m.stage_bytes - m.next_stage, (size_t)c.batch * 4);
+    if (m.qkv_attn) {
+        if (*(const int32_t *)h_next) return qkv_attention_failed(m);
+        if (next_token) memcpy(next_token, h_next + 20, 4);
+        return 0;
+    }
+    if (next_token) memcpy(next_token, h_next, (size_t)c.batch * 4);
     return 0;
 }
 
@@ -801,7 +852,10 @@ extern "C" int mynn_model_decode_loop(void *state, int32_t token, int64_t past_l
     TRY(upload_inputs(m, &id, &pos, past_len, past_len + 1));
     for (int i = 0; i < n_steps; i++) TRY(run_once(m));
     MYNN_HIP(hipMemcpyAsync(m.h_stage, m.d_tokens, (size_t)n_steps * 4, hipMemcpyDeviceToHost, m.stream));
+    char *h_err = m.h_stage + m.stage_bytes - m.next_stage;
+    if (m.qkv_attn) MYNN_HIP(hipMemcpyAsync(h_err, m.d_past + 3, 4, hipMemcpyDeviceToHost, m.stream));
     MYNN_HIP(hipStreamSynchronize(m.stream));
+    if (m.qkv_attn && *(const int32_t *)h_err) return qkv_attention_failed(m);
     memcpy(out_tokens, m.h_stage, (size_t)n_steps * 4);
     return 0;
 }

@@ -11,7 +11,7 @@ int gemv_norm(void *out, const void *x, const void *norm_w, float eps, const int
               int N, int K, hipStream_t s);
 template <typename T>
 int gemv_residual(void *out, const void *act, const int8_t *wq, const void *scale, const void *residual,
-                  int N, int K, hipStream_t s);
+                  int N, int K, hipStream_t s, uint64_t *fill = nullptr, int fill_words = 0);
 template <typename T>
 int gemv_norm_swiglu(void *out, const void *x, const void *norm_w, float eps, const int8_t *wq,
                      const void *scale, int N, int K, hipStream_t s);
@@ -69,6 +69,28 @@ int dequant_gemm_mfma(void *out, const void *act, const int8_t *wq, const void *
 
 // elementwise.hip
 // device-side loop state of a batch-1 decode model; a null `ids` means "no bookkeeping"
+// q|k|v projection + decode attention in one launch (qkv_attention.hip), batch 1
+struct QkvAttnParams {
+    const void *x, *norm_w;  // the residual stream row [K] and the RMSNorm weights
+    float eps;
+    const int8_t *wq;        // [N, K] int8, rows of q, k, v
+    const void *scale;       // [N]
+    int N, K;
+    uint64_t *qkv;           // hand-over vector of N 16-bit elements: all 0xFFFF ("empty") on entry
+    int gemv_blocks, groups; // filled in by the launcher
+    void *out;               // [Hq * D]
+    void *k_cache, *v_cache; // [Hkv, max_seq, D]
+    const void *cos_t, *sin_t;
+    const int64_t *d_pos;
+    const int32_t *d_active;
+    int Hq, Hkv, max_seq;
+    float softmax_scale;
+    int *err;                // set to 1 by a wait that ran out
+    int spin_limit;
+};
+bool qkv_attention_supported(int H, int Hq, int Hkv, int D, int max_seq, int dtype);
+int qkv_attention_launch(QkvAttnParams p, int D, int dtype, hipStream_t s);
+
 struct AdvanceState {
     int64_t *ids, *pos;
     int32_t *past, *active, *tokens, *step;

@@ -1,0 +1,227 @@
+// Batch-1 decode: RMSNorm + q|k|v projection AND RoPE + KV append + attention in ONE launch.
+//
+// As two launches the attention starts 3.5-4 us after the projection's last store (the cost of a dependent
+// dispatch on this part), with nothing of its own in flight.  Here the grid holds both: the first workgroups are
+// the projection (the row-pair GEMV of gemv.hip, operation for operation), the last Hq workgroups are the attention
+// of one query head each (attn_short_body).  The attention workgroups request their K / V cache rows at once and
+// then wait for the three projection slices they need (q of the head, k and v of its kv head), which arrive
+// through memory with the data as its own flag: the projection writes 16-bit elements with agent-scope atomic
+// stores into a vector that holds 0xFFFF ("empty": a NaN no conversion here produces) and the consumers poll their
+// words until no element is empty.  Producers never wait, consumers are dispatched after them, every wait is
+// bounded by a spin limit that raises an error word -- the launch always drains.  The vector is emptied again by
+// the launch that follows (the o projection).
+//
+// Reference ops: rms_norm.cuh:9-59, dequant_gemv.cuh:12-59, rope.cuh, kvcache.cuh, attention.cuh:495-513.
+#include "kernels.h"
+#include "attention_short.h"
+
+namespace mynn {
+
+constexpr int kQaThreads = 512, kQaWaves = kQaThreads / 64;
+constexpr int kQaStageThreads = 256;  // the activation is staged, and its RMSNorm summed, as the 256-thread GEMV does
+
+__device__ inline void qa_put16(void *vec, int idx, uint32_t bits) {
+    if (bits == 0xFFFFu) bits = 0xFFFEu;  // (an all-ones NaN stays a NaN and stops meaning "empty")
+    __hip_atomic_store((uint16_t *)vec + idx, (uint16_t)bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// true when one of the four 16-bit elements of w is still empty
+__device__ inline bool qa_some_empty(uint64_t w) {
+    const uint64_t t = ~w;  // an empty element is a zero element of t
+    return ((t - 0x0001000100010001ull) & ~t & 0x8000800080008000ull) != 0;
+}
+__device__ inline uint64_t qa_wait(const uint64_t *p, int limit, int *err) {
+    uint64_t v = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int spins = 0; qa_some_empty(v); spins++) {
+        if (spins > limit) {
+            __hip_atomic_store(err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+        v = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return v;
+}
+template <typename T> __device__ inline uint32_t qa_bits(float v);
+template <> __device__ inline uint32_t qa_bits<f16_t>(float v) { return __builtin_bit_cast(uint16_t, f32_to_f16(v)); }
+template <> __device__ inline uint32_t qa_bits<bf16_t>(float v) { return f32_to_bf16_bits(v); }
+
+template <typename T, int D, int NC>
+__global__ __launch_bounds__(kQaThreads, 2) void qkv_attention_kernel(QkvAttnParams p) {
+    extern __shared__ float act_lds[];  // [K], projection workgroups
+    __shared__ float red[kQaStageThreads / 64];
+    __shared__ float part_s[kShortWaves][D + 2];
+    __shared__ __align__(16) T qkv_l[3 * D];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+    if ((int)blockIdx.x < p.gemv_blocks) {
+        // ---- projection: wave g takes the row pairs g, g + total_waves, ..
+        constexpr int R = 2;
+        const int K = p.K, N = p.N, nchunks = K >> 4;
+        const int total_waves = p.gemv_blocks * kQaWaves;
+        int g = blockIdx.x * kQaWaves + wave;
+        struct Group {
+            U4 w[R][NC];
+            float sc;
+        };
+        const T *scale = (const T *)p.scale;
+        auto load_group = [&](int gg, Group &G) {
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const int row = gg * R + r < N ? gg * R + r : N - 1;
+                const U4 *wrow = (const U4 *)(p.wq + (size_t)row * K);
+#pragma unroll
+                for (int j = 0; j < NC; j++) {
+                    const int c = lane + j * kWave;
+                    if (c < nchunks) G.w[r][j] = __builtin_nontemporal_load(&wrow[c]);
+                    else G.w[r][j] = U4{0u, 0u, 0u, 0u};
+                }
+            }
+            G.sc = Elem<T>::ld(scale, min(gg * R + min(lane, R - 1), N - 1));
+        };
+        Group ga;
+        if (g < p.groups) load_group(g, ga);  // in flight while the activation is staged
+
+        // stage + RMSNorm: thread t < 256 owns the 8-element pieces t, t + 256, ..
+        {
+            const U4 *ap = (const U4 *)p.x;
+            const int npieces = K >> 3;
+            constexpr int PMAX = (NC * 1024 / 8 + kQaStageThreads - 1) / kQaStageThreads;
+            float f[PMAX][8];
+            U4 nwv[PMAX];
+            float ss = 0.f;
+            if (tid < kQaStageThreads) {
+#pragma unroll
+                for (int q = 0; q < PMAX; q++) {
+                    const int pc = tid + q * kQaStageThreads;
+                    if (pc < npieces) {
+                        nwv[q] = ((const U4 *)p.norm_w)[pc];
+                        widen8<T>(ap[pc], f[q]);
+#pragma unroll
+                        for (int i = 0; i < 8; i++) ss = fmaf(f[q][i], f[q][i], ss);
+                    }
+                }
+                ss = wave_sum(ss);
+                if (lane == 0) red[wave] = ss;
+            }
+            __syncthreads();
+            if (tid < kQaStageThreads) {
+                float tot = 0.f;
+#pragma unroll
+                for (int i = 0; i < kQaStageThreads / 64; i++) tot += red[i];
+                const float inv = 1.0f / sqrtf(tot / (float)K + p.eps);
+#pragma unroll
+                for (int q = 0; q < PMAX; q++) {
+                    const int pc = tid + q * kQaStageThreads;
+                    if (pc < npieces) {
+                        float nw[8];
+                        widen8<T>(nwv[q], nw);
+#pragma unroll
+                        for (int i = 0; i < 8; i++) f[q][i] = Elem<T>::rnd((f[q][i] * inv) * nw[i]);
+                        float4 *dst = (float4 *)(act_lds + pc * 8);
+                        dst[0] = float4{f[q][0], f[q][1], f[q][2], f[q][3]};
+                        dst[1] = float4{f[q][4], f[q][5], f[q][6], f[q][7]};
+                    }
+                }
+            }
+        }
+        __syncthreads();
+
+        bool loaded = true;
+        for (; g < p.groups; g += total_waves) {
+            if (!loaded) load_group(g, ga);
+            loaded = false;
+            float acc[R];
+#pragma unroll
+            for (int r = 0; r < R; r++) acc[r] = 0.f;
+#pragma unroll
+            for (int j = 0; j < NC; j++) {
+                const int c = lane + j * kWave;
+                if (c < nchunks) {
+                    float a[16];
+                    const float4 *ap = (const float4 *)(act_lds + c * 16);
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        float4 t = ap[q];
+                        a[4 * q] = t.x; a[4 * q + 1] = t.y; a[4 * q + 2] = t.z; a[4 * q + 3] = t.w;
+                    }
+#pragma unroll
+                    for (int r = 0; r < R; r++) {
+                        float wf[16];
+                        pin(ga.w[r][j]);
+                        widen16_i8(ga.w[r][j], wf);
+#pragma unroll
+                        for (int i = 0; i < 16; i++) acc[r] = fmaf(a[i], wf[i], acc[r]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < R; r++) acc[r] = wave_sum(acc[r]);
+            const int row = g * R + lane;
+            if (lane < R && row < N) qa_put16(p.qkv, row, qa_bits<T>((lane == 0 ? acc[0] : acc[1]) * ga.sc));
+        }
+        return;
+    }
+
+    // ---- attention: one workgroup per query head
+    const int h = blockIdx.x - p.gemv_blocks, Gt = p.Hq / p.Hkv, hkv = h / Gt;
+    const int active = *p.d_active;
+    const int64_t pos = *p.d_pos;
+    const size_t kv_base = (size_t)hkv * p.max_seq * D;
+    constexpr int WPH = D / 4;  // 8-byte words per head slice
+    auto ready = [&] {
+        if (tid < 3 * WPH) {
+            const int part = tid / WPH, w = tid % WPH;
+            const int head = part == 0 ? h : part == 1 ? p.Hq + hkv : p.Hq + p.Hkv + hkv;
+            ((uint64_t *)qkv_l)[tid] = qa_wait(p.qkv + head * WPH + w, p.spin_limit, p.err);
+        }
+        __syncthreads();
+    };
+    float r = 0.f;
+    if (attn_short_body<T, D>(qkv_l, qkv_l + D, qkv_l + 2 * D, (T *)p.k_cache + kv_base, (T *)p.v_cache + kv_base,
+                              min(active, p.max_seq), active - 1, h % Gt == 0, (const T *)p.cos_t + pos * D,
+                              (const T *)p.sin_t + pos * D, p.softmax_scale, part_s, tid, r, ready))
+        Elem<T>::st((T *)p.out, (size_t)h * D + tid, r);
+}
+
+bool qkv_attention_supported(int H, int Hq, int Hkv, int D, int max_seq, int dtype) {
+    if (dtype != MYNN_F16 && dtype != MYNN_BF16) return false;
+    if (D != 64 && D != 128) return false;
+    const int kpp = kShortWaves * (64 / (D / 8));
+    if (max_seq > kShortPasses * kpp) return false;
+    const int N = (Hq + 2 * Hkv) * D;
+    if (H % 16 || H > 4096 || N % 4 || Hq % Hkv || Hq > 1024) return false;
+    return (size_t)H * sizeof(float) <= 48 * 1024;
+}
+
+int qkv_attention_launch(QkvAttnParams p, int D, int dtype, hipStream_t s) {
+    MYNN_REQUIRE(aligned16(p.x) && aligned16(p.norm_w) && aligned16(p.wq) && aligned16(p.qkv) && aligned16(p.k_cache) &&
+                     aligned16(p.v_cache) && aligned16(p.cos_t) && aligned16(p.sin_t),
+                 MYNN_ERR_INVALID, "qkv + attention: operands must be 16-byte aligned");
+    p.groups = p.N / 2;
+    const int max_waves = 256 * 16;
+    const int passes = (p.groups + max_waves - 1) / max_waves;
+    const int waves = (p.groups + passes - 1) / passes;
+    p.gemv_blocks = (waves + kQaWaves - 1) / kQaWaves;
+    const int nc = (p.K + 1023) / 1024;
+    const size_t lds = (size_t)p.K * sizeof(float);
+    const dim3 grid(p.gemv_blocks + p.Hq), block(kQaThreads);
+    return dispatch_dtype16(dtype, [&](auto *t) {
+        using T = std::remove_pointer_t<decltype(t)>;
+#define MYNN_QA(D_, NC_)                                                           \
+    do {                                                                           \
+        MYNN_LAUNCH((qkv_attention_kernel<T, D_, NC_>), grid, block, lds, s, p);   \
+        return launch_status("qkv_attention_kernel");                              \
+    } while (0)
+        if (D == 64) {
+            if (nc <= 1) MYNN_QA(64, 1);
+            if (nc <= 2) MYNN_QA(64, 2);
+            MYNN_QA(64, 4);
+        }
+        if (nc <= 1) MYNN_QA(128, 1);
+        if (nc <= 2) MYNN_QA(128, 2);
+        MYNN_QA(128, 4);
+#undef MYNN_QA
+    });
+}
+
+}  // namespace mynn
