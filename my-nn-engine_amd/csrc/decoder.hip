@@ -247,12 +247,14 @@ static int enqueue_step(Model &m) {
         bool roped = false;
         if (fused && m.qkv_attn) {
             // RMSNorm + q|k|v projection, RoPE, both cache appends and the attention in one launch
-            note(m, "qkv_attention", (double)L.qkv.N * H + L.qkv.N * eb + 2 * H * eb + 2.0 * KD * eb + QD * eb);
+            note(m, "qkv_attention_o", (double)L.qkv.N * H + L.qkv.N * eb + 2 * H * eb + 2.0 * KD * eb + (double)H * QD + H * eb + 2 * H * eb);
             QkvAttnParams p{};
             p.x = m.x; p.norm_w = L.norm1; p.eps = c.eps; p.wq = (const int8_t *)L.qkv.w; p.scale = L.qkv.scale;
             p.N = L.qkv.N; p.K = H; p.qkv = (uint64_t *)m.qkv; p.out = m.attn; p.k_cache = L.k_cache; p.v_cache = L.v_cache;
             p.cos_t = m.cos_t; p.sin_t = m.sin_t; p.d_pos = m.d_pos; p.d_active = m.d_active; p.Hq = Hq; p.Hkv = Hkv;
             p.max_seq = c.max_seq; p.softmax_scale = softmax_scale; p.err = m.d_past + 3; p.spin_limit = 400000;
+            // ... and the o projection + residual behind it: x2 = T(T(Wo . attn) + x)
+            p.o_wq = (const int8_t *)L.o.w; p.o_scale = L.o.scale; p.o_out = m.x2; p.attn_words = (uint64_t *)m.attn;
             TRY(qkv_attention_launch(p, D, c.dtype, s));
         } else if (fused) {
             note(m, "gemv_norm_qkv", (double)L.qkv.N * H + L.qkv.N * eb + 2 * H * eb + L.qkv.N * eb);
@@ -306,12 +308,16 @@ static int enqueue_step(Model &m) {
             }
         }
         if (fused) {
-            note(m, "gemv_o_residual", (double)H * QD + H * eb + QD * eb + 2 * H * eb);
-            // (the o projection also empties the hand-over vector of the fused launch before its next use)
-            TRY(gemv_residual<T>(m.x2, m.attn, (const int8_t *)L.o.w, L.o.scale, m.x, H, QD, s,
-                                 m.qkv_attn ? (uint64_t *)m.qkv : nullptr, m.qkv_attn ? (QD + 2 * KD) * (int)sizeof(T) / 8 : 0));
+            if (!m.qkv_attn) {
+                note(m, "gemv_o_residual", (double)H * QD + H * eb + QD * eb + 2 * H * eb);
+                TRY(gemv_residual<T>(m.x2, m.attn, (const int8_t *)L.o.w, L.o.scale, m.x, H, QD, s));
+            }
             note(m, "gemv_norm_gateup_swiglu", (double)L.gu.N * H + L.gu.N * eb + 2 * H * eb + F * eb);
-            TRY(gemv_norm_swiglu<T>(m.hmid, m.x2, L.norm2, c.eps, (const int8_t *)L.gu.w, L.gu.scale, L.gu.N, H, s));
+            // (after a fused launch the gate/up launch also empties its two hand-over vectors, m.qkv .. m.attn,
+            // before their next use)
+            uint64_t *fill = m.qkv_attn ? (uint64_t *)m.qkv : nullptr;
+            const int fill_words = m.qkv_attn ? (int)(((char *)m.attn + (size_t)QD * sizeof(T) - (char *)m.qkv) / 8) : 0;
+            TRY(gemv_norm_swiglu<T>(m.hmid, m.x2, L.norm2, c.eps, (const int8_t *)L.gu.w, L.gu.scale, L.gu.N, H, s, fill, fill_words));
             note(m, "gemv_down_residual", (double)H * F + H * eb + F * eb + 2 * H * eb);
             TRY(gemv_residual<T>(m.x, m.hmid, (const int8_t *)L.down.w, L.down.scale, m.x2, H, F, s));
         } else if (m.skinny) {
@@ -595,9 +601,9 @@ static int build(Model &m, void **init, void **state) {
         qkv_attention_supported(H, c.n_heads, c.n_kv_heads, c.head_dim, c.max_seq, c.dtype) && (QD + 2 * KD) * eb % 8 == 0) {
         bool ok = aligned16(m.qkv) && aligned16(m.x) && aligned16(m.attn);
         for (const Layer &L : m.layers)
-            ok = ok && aligned16(L.qkv.w) && aligned16(L.norm1) && aligned16(L.k_cache) && aligned16(L.v_cache) && aligned16(L.o.w);
-        if (ok && QD % 8 == 0 && (QD + 1023) / 1024 <= 14) {
-            MYNN_HIP(hipMemset(m.qkv, 0xFF, (size_t)(QD + 2 * KD) * eb));
+            ok = ok && aligned16(L.qkv.w) && aligned16(L.norm1) && aligned16(L.norm2) && aligned16(L.k_cache) && aligned16(L.v_cache) && aligned16(L.o.w);
+        if (ok && (char *)m.attn > (char *)m.qkv && ((char *)m.attn + (size_t)QD * eb - (char *)m.qkv) % 8 == 0) {
+            MYNN_HIP(hipMemset(m.qkv, 0xFF, (size_t)((char *)m.attn + (size_t)QD * eb - (char *)m.qkv)));
             MYNN_HIP(hipDeviceSynchronize());
             m.qkv_attn = true;
         }
@@ -694,7 +700,7 @@ static int upload_inputs(Model &m, const int64_t *ids, const int64_t *pos, int64
 // drained); the hand-over vector is emptied again so that the next step starts clean
 static int qkv_attention_failed(Model &m) {
     const mynn_model_config &c = m.cfg;
-    (void)hipMemset(m.qkv, 0xFF, (size_t)(c.n_heads + 2 * c.n_kv_heads) * c.head_dim * dtype_size(c.dtype));
+    (void)hipMemset(m.qkv, 0xFF, (size_t)((char *)m.attn + (size_t)c.n_heads * c.head_dim * dtype_size(c.dtype) - (char *)m.qkv));
     (void)hipMemset(m.d_past + 3, 0, 4);
     return fail(MYNN_ERR_STATE, "decode step: the attention waited too long for the q|k|v projection (is the device shared?)");
 }

@@ -454,10 +454,13 @@ int gemv_residual(void *out, const void *act, const int8_t *wq, const void *scal
 // wq/scale hold gate and up rows interleaved (row 2i = gate_i, row 2i+1 = up_i); N = 2*ffn
 template <typename T>
 int gemv_norm_swiglu(void *out, const void *x, const void *norm_w, float eps, const int8_t *wq,
-                     const void *scale, int N, int K, hipStream_t s) {
+                     const void *scale, int N, int K, hipStream_t s, uint64_t *fill, int fill_words) {
     GemvParams p{};
     p.out = out; p.act = x; p.wq = wq; p.scale = scale; p.norm_w = norm_w; p.eps = eps; p.N = N; p.K = K;
     p.act_stride = K; p.out_stride = N / 2;
+    p.fill = fill; p.fill_words = fill_words;
+    MYNN_REQUIRE(!fill || (aligned16(x) && aligned16(norm_w) && K % 8 == 0 && (K + 1023) / 1024 <= 14), MYNN_ERR_UNSUPPORTED,
+                 "gemv_norm_swiglu: the fill rides on the decode kernel only");
     MYNN_REQUIRE(N % 2 == 0, MYNN_ERR_INVALID, "gate/up rows must come in pairs (N=%d)", N);
     int rc = check_gemv(p, 1);
     if (rc) return rc;
@@ -468,8 +471,8 @@ template int gemv_norm<bf16_t>(void *, const void *, const void *, float, const 
 template int gemv_norm<f16_t>(void *, const void *, const void *, float, const int8_t *, const void *, int, int, hipStream_t);
 template int gemv_residual<bf16_t>(void *, const void *, const int8_t *, const void *, const void *, int, int, hipStream_t, uint64_t *, int);
 template int gemv_residual<f16_t>(void *, const void *, const int8_t *, const void *, const void *, int, int, hipStream_t, uint64_t *, int);
-template int gemv_norm_swiglu<bf16_t>(void *, const void *, const void *, float, const int8_t *, const void *, int, int, hipStream_t);
-template int gemv_norm_swiglu<f16_t>(void *, const void *, const void *, float, const int8_t *, const void *, int, int, hipStream_t);
+template int gemv_norm_swiglu<bf16_t>(void *, const void *, const void *, float, const int8_t *, const void *, int, int, hipStream_t, uint64_t *, int);
+template int gemv_norm_swiglu<f16_t>(void *, const void *, const void *, float, const int8_t *, const void *, int, int, hipStream_t, uint64_t *, int);
 
 }  // namespace mynn
 

@@ -14,7 +14,7 @@ int gemv_residual(void *out, const void *act, const int8_t *wq, const void *scal
                   int N, int K, hipStream_t s, uint64_t *fill = nullptr, int fill_words = 0);
 template <typename T>
 int gemv_norm_swiglu(void *out, const void *x, const void *norm_w, float eps, const int8_t *wq,
-                     const void *scale, int N, int K, hipStream_t s);
+                     const void *scale, int N, int K, hipStream_t s, uint64_t *fill = nullptr, int fill_words = 0);
 int dequant_gemv_dispatch(void *out, const void *act, const int8_t *wq, const void *scale, int M, int N, int K,
                           int act_dtype, int out_dtype, hipStream_t s);
 
@@ -87,6 +87,13 @@ struct QkvAttnParams {
     float softmax_scale;
     int *err;                // set to 1 by a wait that ran out
     int spin_limit;
+    // optional third stage, the o projection + residual: x2 = T(T(o_wq . attn * o_scale) + x).  The attention
+    // output then travels through attn_words (Hq * D 16-bit elements, all 0xFFFF on entry) instead of `out`.
+    const int8_t *o_wq;      // [K, Hq * D] int8 (null: the launch ends with the attention)
+    const void *o_scale;     // [K]
+    void *o_out;             // [K]
+    uint64_t *attn_words;
+    int o_blocks;            // filled in by the launcher
 };
 bool qkv_attention_supported(int H, int Hq, int Hkv, int D, int max_seq, int dtype);
 int qkv_attention_launch(QkvAttnParams p, int D, int dtype, hipStream_t s);

@@ -45,120 +45,175 @@ template <typename T> __device__ inline uint32_t qa_bits(float v);
 template <> __device__ inline uint32_t qa_bits<f16_t>(float v) { return __builtin_bit_cast(uint16_t, f32_to_f16(v)); }
 template <> __device__ inline uint32_t qa_bits<bf16_t>(float v) { return f32_to_bf16_bits(v); }
 
-template <typename T, int D, int NC>
-__global__ __launch_bounds__(kQaThreads, 2) void qkv_attention_kernel(QkvAttnParams p) {
-    extern __shared__ float act_lds[];  // [K], projection workgroups
-    __shared__ float red[kQaStageThreads / 64];
-    __shared__ float part_s[kShortWaves][D + 2];
-    __shared__ __align__(16) T qkv_l[3 * D];
+// One GEMV role of the launch: row pairs of wq [N, K] against an activation vector, as dequant_gemv1_kernel
+// does it (same staging partition for the RMSNorm sums, same row sums).  Wave w of role block `blk` takes the
+// row pairs blk * 8 + w, + total waves, ..; its first pair is requested before the activation is staged.
+//   NORM: the activation is read from memory and RMS-normalised (256 staging threads, as the 256-thread kernel)
+//   POLL: the activation arrives through a hand-over vector and is waited for
+//   RESID: out = T(T(sum * scale) + residual), stored plainly; else out is a hand-over vector, written element-wise
+struct QaGemv {
+    const void *act;       // NORM: [K] values; POLL: hand-over words
+    const void *norm_w;
+    float eps;
+    const int8_t *wq;
+    const void *scale, *residual;
+    void *out;
+    int N, K;
+};
+
+template <typename T, int NC, bool NORM, bool POLL, bool RESID>
+__device__ __forceinline__ void qa_gemv(const QaGemv &a, float *act_lds, float *red, int blk, int nblk, int limit, int *err) {
+    constexpr int R = 2;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-
-    if ((int)blockIdx.x < p.gemv_blocks) {
-        // ---- projection: wave g takes the row pairs g, g + total_waves, ..
-        constexpr int R = 2;
-        const int K = p.K, N = p.N, nchunks = K >> 4;
-        const int total_waves = p.gemv_blocks * kQaWaves;
-        int g = blockIdx.x * kQaWaves + wave;
-        struct Group {
-            U4 w[R][NC];
-            float sc;
-        };
-        const T *scale = (const T *)p.scale;
-        auto load_group = [&](int gg, Group &G) {
+    const int K = a.K, N = a.N, nchunks = K >> 4, groups = (N + R - 1) / R;
+    const int total_waves = nblk * kQaWaves;
+    int g = blk * kQaWaves + wave;
+    struct Group {
+        U4 w[R][NC];
+        float sc, res;
+    };
+    const T *scale = (const T *)a.scale;
+    auto load_group = [&](int gg, Group &G) {
 #pragma unroll
-            for (int r = 0; r < R; r++) {
-                const int row = gg * R + r < N ? gg * R + r : N - 1;
-                const U4 *wrow = (const U4 *)(p.wq + (size_t)row * K);
+        for (int r = 0; r < R; r++) {
+            const int row = gg * R + r < N ? gg * R + r : N - 1;
+            const U4 *wrow = (const U4 *)(a.wq + (size_t)row * K);
 #pragma unroll
-                for (int j = 0; j < NC; j++) {
-                    const int c = lane + j * kWave;
-                    if (c < nchunks) G.w[r][j] = __builtin_nontemporal_load(&wrow[c]);
-                    else G.w[r][j] = U4{0u, 0u, 0u, 0u};
-                }
+            for (int j = 0; j < NC; j++) {
+                const int c = lane + j * kWave;
+                if (c < nchunks) G.w[r][j] = __builtin_nontemporal_load(&wrow[c]);
+                else G.w[r][j] = U4{0u, 0u, 0u, 0u};
             }
-            G.sc = Elem<T>::ld(scale, min(gg * R + min(lane, R - 1), N - 1));
-        };
-        Group ga;
-        if (g < p.groups) load_group(g, ga);  // in flight while the activation is staged
+        }
+        const int row = min(gg * R + min(lane, R - 1), N - 1);
+        G.sc = Elem<T>::ld(scale, row);
+        G.res = RESID ? Elem<T>::ld((const T *)a.residual, row) : 0.f;
+    };
+    Group ga;
+    if (g < groups) load_group(g, ga);  // in flight while the activation is staged
 
-        // stage + RMSNorm: thread t < 256 owns the 8-element pieces t, t + 256, ..
-        {
-            const U4 *ap = (const U4 *)p.x;
-            const int npieces = K >> 3;
-            constexpr int PMAX = (NC * 1024 / 8 + kQaStageThreads - 1) / kQaStageThreads;
-            float f[PMAX][8];
-            U4 nwv[PMAX];
-            float ss = 0.f;
-            if (tid < kQaStageThreads) {
+    {
+        const int npieces = K >> 3;
+        constexpr int NT = NORM ? kQaStageThreads : kQaThreads;  // thread t < NT owns the 8-element pieces t, t + NT, ..
+        constexpr int PMAX = (NC * 1024 / 8 + NT - 1) / NT;
+        float f[PMAX][8];
+        U4 nwv[NORM ? PMAX : 1];
+        float ss = 0.f;
+        if (tid < NT) {
 #pragma unroll
-                for (int q = 0; q < PMAX; q++) {
-                    const int pc = tid + q * kQaStageThreads;
-                    if (pc < npieces) {
-                        nwv[q] = ((const U4 *)p.norm_w)[pc];
-                        widen8<T>(ap[pc], f[q]);
+            for (int q = 0; q < PMAX; q++) {
+                const int pc = tid + q * NT;
+                if (pc < npieces) {
+                    U4 raw;
+                    if constexpr (POLL) {
+                        const uint64_t *wp = (const uint64_t *)a.act + 2 * pc;
+                        uint64_t w0 = __hip_atomic_load(wp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        uint64_t w1 = __hip_atomic_load(wp + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if (qa_some_empty(w0)) w0 = qa_wait(wp, limit, err);
+                        if (qa_some_empty(w1)) w1 = qa_wait(wp + 1, limit, err);
+                        raw = U4{(uint32_t)w0, (uint32_t)(w0 >> 32), (uint32_t)w1, (uint32_t)(w1 >> 32)};
+                    } else {
+                        raw = ((const U4 *)a.act)[pc];
+                    }
+                    if constexpr (NORM) nwv[q] = ((const U4 *)a.norm_w)[pc];
+                    widen8<T>(raw, f[q]);
+                    if constexpr (NORM) {
 #pragma unroll
                         for (int i = 0; i < 8; i++) ss = fmaf(f[q][i], f[q][i], ss);
                     }
                 }
+            }
+            if constexpr (NORM) {
                 ss = wave_sum(ss);
                 if (lane == 0) red[wave] = ss;
             }
+        }
+        float inv = 1.f;
+        if constexpr (NORM) {
             __syncthreads();
-            if (tid < kQaStageThreads) {
-                float tot = 0.f;
+            float tot = 0.f;
 #pragma unroll
-                for (int i = 0; i < kQaStageThreads / 64; i++) tot += red[i];
-                const float inv = 1.0f / sqrtf(tot / (float)K + p.eps);
+            for (int i = 0; i < kQaStageThreads / 64; i++) tot += red[i];
+            inv = 1.0f / sqrtf(tot / (float)K + a.eps);
+        }
+        if (tid < NT) {
 #pragma unroll
-                for (int q = 0; q < PMAX; q++) {
-                    const int pc = tid + q * kQaStageThreads;
-                    if (pc < npieces) {
+            for (int q = 0; q < PMAX; q++) {
+                const int pc = tid + q * NT;
+                if (pc < npieces) {
+                    if constexpr (NORM) {
                         float nw[8];
                         widen8<T>(nwv[q], nw);
 #pragma unroll
                         for (int i = 0; i < 8; i++) f[q][i] = Elem<T>::rnd((f[q][i] * inv) * nw[i]);
-                        float4 *dst = (float4 *)(act_lds + pc * 8);
-                        dst[0] = float4{f[q][0], f[q][1], f[q][2], f[q][3]};
-                        dst[1] = float4{f[q][4], f[q][5], f[q][6], f[q][7]};
                     }
+                    float4 *dst = (float4 *)(act_lds + pc * 8);
+                    dst[0] = float4{f[q][0], f[q][1], f[q][2], f[q][3]};
+                    dst[1] = float4{f[q][4], f[q][5], f[q][6], f[q][7]};
                 }
             }
         }
-        __syncthreads();
+    }
+    __syncthreads();
 
-        bool loaded = true;
-        for (; g < p.groups; g += total_waves) {
-            if (!loaded) load_group(g, ga);
-            loaded = false;
-            float acc[R];
+    bool loaded = true;
+    for (; g < groups; g += total_waves) {
+        if (!loaded) load_group(g, ga);
+        loaded = false;
+        float acc[R];
 #pragma unroll
-            for (int r = 0; r < R; r++) acc[r] = 0.f;
+        for (int r = 0; r < R; r++) acc[r] = 0.f;
 #pragma unroll
-            for (int j = 0; j < NC; j++) {
-                const int c = lane + j * kWave;
-                if (c < nchunks) {
-                    float a[16];
-                    const float4 *ap = (const float4 *)(act_lds + c * 16);
+        for (int j = 0; j < NC; j++) {
+            const int c = lane + j * kWave;
+            if (c < nchunks) {
+                float av[16];
+                const float4 *ap = (const float4 *)(act_lds + c * 16);
 #pragma unroll
-                    for (int q = 0; q < 4; q++) {
-                        float4 t = ap[q];
-                        a[4 * q] = t.x; a[4 * q + 1] = t.y; a[4 * q + 2] = t.z; a[4 * q + 3] = t.w;
-                    }
+                for (int q = 0; q < 4; q++) {
+                    float4 t = ap[q];
+                    av[4 * q] = t.x; av[4 * q + 1] = t.y; av[4 * q + 2] = t.z; av[4 * q + 3] = t.w;
+                }
 #pragma unroll
-                    for (int r = 0; r < R; r++) {
-                        float wf[16];
-                        pin(ga.w[r][j]);
-                        widen16_i8(ga.w[r][j], wf);
+                for (int r = 0; r < R; r++) {
+                    float wf[16];
+                    pin(ga.w[r][j]);
+                    widen16_i8(ga.w[r][j], wf);
 #pragma unroll
-                        for (int i = 0; i < 16; i++) acc[r] = fmaf(a[i], wf[i], acc[r]);
-                    }
+                    for (int i = 0; i < 16; i++) acc[r] = fmaf(av[i], wf[i], acc[r]);
                 }
             }
-#pragma unroll
-            for (int r = 0; r < R; r++) acc[r] = wave_sum(acc[r]);
-            const int row = g * R + lane;
-            if (lane < R && row < N) qa_put16(p.qkv, row, qa_bits<T>((lane == 0 ? acc[0] : acc[1]) * ga.sc));
         }
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] = wave_sum(acc[r]);
+        const int row = g * R + lane;
+        if (lane < R && row < N) {
+            float y = (lane == 0 ? acc[0] : acc[1]) * ga.sc;
+            if constexpr (RESID) Elem<T>::st((T *)a.out, row, Elem<T>::rnd(y) + ga.res);
+            else qa_put16(a.out, row, qa_bits<T>(y));
+        }
+    }
+}
+
+template <typename T, int D, int NC>
+__global__ __launch_bounds__(kQaThreads, 2) void qkv_attention_kernel(QkvAttnParams p) {
+    extern __shared__ float act_lds[];  // [K], GEMV workgroups
+    __shared__ float red[kQaStageThreads / 64];
+    __shared__ float part_s[kShortWaves][D + 2];
+    __shared__ __align__(16) T qkv_l[3 * D];
+    const int tid = threadIdx.x;
+    const int QD = p.Hq * D;
+
+    if ((int)blockIdx.x < p.gemv_blocks) {
+        // ---- RMSNorm + q|k|v projection into the hand-over vector
+        const QaGemv a{p.x, p.norm_w, p.eps, p.wq, p.scale, nullptr, p.qkv, p.N, p.K};
+        qa_gemv<T, NC, true, false, false>(a, act_lds, red, blockIdx.x, p.gemv_blocks, p.spin_limit, p.err);
+        return;
+    }
+    if ((int)blockIdx.x >= p.gemv_blocks + p.Hq) {
+        // ---- o projection + residual: waits for the attention's output vector
+        const QaGemv a{p.attn_words, nullptr, 0.f, p.o_wq, p.o_scale, p.x, p.o_out, p.K, QD};
+        qa_gemv<T, NC, false, true, true>(a, act_lds, red, blockIdx.x - p.gemv_blocks - p.Hq, p.o_blocks, p.spin_limit, p.err);
         return;
     }
 
@@ -179,8 +234,10 @@ __global__ __launch_bounds__(kQaThreads, 2) void qkv_attention_kernel(QkvAttnPar
     float r = 0.f;
     if (attn_short_body<T, D>(qkv_l, qkv_l + D, qkv_l + 2 * D, (T *)p.k_cache + kv_base, (T *)p.v_cache + kv_base,
                               min(active, p.max_seq), active - 1, h % Gt == 0, (const T *)p.cos_t + pos * D,
-                              (const T *)p.sin_t + pos * D, p.softmax_scale, part_s, tid, r, ready))
-        Elem<T>::st((T *)p.out, (size_t)h * D + tid, r);
+                              (const T *)p.sin_t + pos * D, p.softmax_scale, part_s, tid, r, ready)) {
+        if (p.o_blocks) qa_put16(p.attn_words, h * D + tid, qa_bits<T>(r));
+        else Elem<T>::st((T *)p.out, (size_t)h * D + tid, r);
+    }
 }
 
 bool qkv_attention_supported(int H, int Hq, int Hkv, int D, int max_seq, int dtype) {
@@ -202,9 +259,17 @@ int qkv_attention_launch(QkvAttnParams p, int D, int dtype, hipStream_t s) {
     const int passes = (p.groups + max_waves - 1) / max_waves;
     const int waves = (p.groups + passes - 1) / passes;
     p.gemv_blocks = (waves + kQaWaves - 1) / kQaWaves;
+    p.o_blocks = 0;
+    if (p.o_wq) {
+        // the o projection rides along: K rows of [K, Hq * D] (hidden == heads x head_dim in this decoder)
+        MYNN_REQUIRE(p.o_scale && p.o_out && p.attn_words && aligned16(p.o_wq) && aligned16(p.attn_words), MYNN_ERR_INVALID,
+                     "qkv + attention + o: bad operand");
+        const int ogroups = (p.K + 1) / 2;
+        p.o_blocks = (ogroups < max_waves ? ogroups : max_waves) / kQaWaves + ((ogroups < max_waves ? ogroups : max_waves) % kQaWaves != 0);
+    }
     const int nc = (p.K + 1023) / 1024;
     const size_t lds = (size_t)p.K * sizeof(float);
-    const dim3 grid(p.gemv_blocks + p.Hq), block(kQaThreads);
+    const dim3 grid(p.gemv_blocks + p.Hq + p.o_blocks), block(kQaThreads);
     return dispatch_dtype16(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
 #define MYNN_QA(D_, NC_)                                                           \
