@@ -31,8 +31,8 @@ struct GemvParams {
     int N, K;
     int act_stride;        // elements between activation rows
     int out_stride;        // elements between output rows
-    uint64_t *fill;        // optional: fill_words words that this launch sets to ~0 (the hand-over vector of the
-    int fill_words;        // fused q|k|v + attention launch, emptied between two of its uses)
+    uint64_t *fill;        // optional: fill_words words that this launch sets to ~0 (the hand-over vectors of the
+    int fill_words;        // fused q|k|v + attention + o launch, emptied between two of its uses)
 };
 
 constexpr int kGemvWaves = 4;
@@ -440,13 +440,10 @@ int gemv_norm(void *out, const void *x, const void *norm_w, float eps, const int
 }
 template <typename T>
 int gemv_residual(void *out, const void *act, const int8_t *wq, const void *scale, const void *residual,
-                  int N, int K, hipStream_t s, uint64_t *fill, int fill_words) {
+                  int N, int K, hipStream_t s) {
     GemvParams p{};
     p.out = out; p.act = act; p.wq = wq; p.scale = scale; p.residual = residual; p.N = N; p.K = K;
     p.act_stride = K; p.out_stride = N;
-    p.fill = fill; p.fill_words = fill_words;
-    MYNN_REQUIRE(!fill || (aligned16(act) && K % 8 == 0 && (K + 1023) / 1024 <= 14), MYNN_ERR_UNSUPPORTED,
-                 "gemv_residual: the fill rides on the decode kernel only");
     int rc = check_gemv(p, 1);
     if (rc) return rc;
     return gemv1_dispatch<T, EPI_RESIDUAL, false>(p, s);
@@ -469,8 +466,8 @@ int gemv_norm_swiglu(void *out, const void *x, const void *norm_w, float eps, co
 
 template int gemv_norm<bf16_t>(void *, const void *, const void *, float, const int8_t *, const void *, int, int, hipStream_t);
 template int gemv_norm<f16_t>(void *, const void *, const void *, float, const int8_t *, const void *, int, int, hipStream_t);
-template int gemv_residual<bf16_t>(void *, const void *, const int8_t *, const void *, const void *, int, int, hipStream_t, uint64_t *, int);
-template int gemv_residual<f16_t>(void *, const void *, const int8_t *, const void *, const void *, int, int, hipStream_t, uint64_t *, int);
+template int gemv_residual<bf16_t>(void *, const void *, const int8_t *, const void *, const void *, int, int, hipStream_t);
+template int gemv_residual<f16_t>(void *, const void *, const int8_t *, const void *, const void *, int, int, hipStream_t);
 template int gemv_norm_swiglu<bf16_t>(void *, const void *, const void *, float, const int8_t *, const void *, int, int, hipStream_t, uint64_t *, int);
 template int gemv_norm_swiglu<f16_t>(void *, const void *, const void *, float, const int8_t *, const void *, int, int, hipStream_t, uint64_t *, int);
 

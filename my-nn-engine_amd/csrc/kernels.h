@@ -11,7 +11,7 @@ int gemv_norm(void *out, const void *x, const void *norm_w, float eps, const int
               int N, int K, hipStream_t s);
 template <typename T>
 int gemv_residual(void *out, const void *act, const int8_t *wq, const void *scale, const void *residual,
-                  int N, int K, hipStream_t s, uint64_t *fill = nullptr, int fill_words = 0);
+                  int N, int K, hipStream_t s);
 template <typename T>
 int gemv_norm_swiglu(void *out, const void *x, const void *norm_w, float eps, const int8_t *wq,
                      const void *scale, int N, int K, hipStream_t s, uint64_t *fill = nullptr, int fill_words = 0);
