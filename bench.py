@@ -439,7 +439,10 @@ def main():
                    "hipgraph": stats["graph"], "seed": args.seed,
                    "host_roundtrip_tok_s": round(host_tok_s, 1),
                    "step_algorithmic_bytes": step_bytes,
-                   "step_hbm_frac": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
+                   "step_hbm_frac": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                   # average duration of every launch of the step (HIP events, eager steps): the fused
+                   # q|k|v + attention + o launch is the longest, the gate/up GEMV moves the most bytes
+                   "per_launch_us": {k: round(v[1] / v[0] * 1e3, 2) for k, v in sorted(agg.items(), key=lambda kv: -kv[1][1])}},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": GATEUP_GEMV_TRAFFIC_BYTES if dom == "gemv_norm_gateup_swiglu" else None,
