@@ -1,15 +1,18 @@
-// Batch-1 decode: RMSNorm + q|k|v projection AND RoPE + KV append + attention in ONE launch.
+// Batch-1 decode: RMSNorm + q|k|v projection, RoPE + KV append + attention, and o projection + residual in ONE launch.
 //
-// As two launches the attention starts 3.5-4 us after the projection's last store (the cost of a dependent
-// dispatch on this part), with nothing of its own in flight.  Here the grid holds both: the first workgroups are
-// the projection (the row-pair GEMV of gemv.hip, operation for operation), the last Hq workgroups are the attention
-// of one query head each (attn_short_body).  The attention workgroups request their K / V cache rows at once and
-// then wait for the three projection slices they need (q of the head, k and v of its kv head), which arrive
-// through memory with the data as its own flag: the projection writes 16-bit elements with agent-scope atomic
-// stores into a vector that holds 0xFFFF ("empty": a NaN no conversion here produces) and the consumers poll their
-// words until no element is empty.  Producers never wait, consumers are dispatched after them, every wait is
-// bounded by a spin limit that raises an error word -- the launch always drains.  The vector is emptied again by
-// the launch that follows (the o projection).
+// As separate launches each of them starts 3.5-4 us after its producer's last store (the cost of a dependent
+// dispatch on this part) with nothing of its own in flight.  Here one grid holds all three as ROLES in block order:
+// the first workgroups are the q|k|v projection (the row-pair GEMV of gemv.hip, operation for operation), the next Hq
+// workgroups are the attention of one query head each (attn_short_body), the last ones the o projection.  A consumer
+// requests at once everything that does not depend on its input (K / V cache rows; weight rows, scales, residual)
+// and then waits for the input, which arrives through memory with the data as its own flag: producers write 16-bit
+// elements with agent-scope atomic stores into a vector that holds 0xFFFF ("empty": a NaN no conversion here
+// produces) and consumers poll their words until no element is empty (the attention: q of its head, k and v of its
+// kv head; the o projection: the whole attention output).  Workgroups are dispatched in block order, so a producer
+// is resident or finished before any of its consumers is placed, and the first role never waits; every wait is
+// bounded by a spin limit that raises an error word -- the launch always drains.  The vectors are emptied again by
+// the launch that follows (the gate/up GEMV).  This pays because the weight streams in flight while the consumers
+// poll are small (5 MB and 4 MB): the same construction behind the 23 MB gate/up stream made the layer slower.
 //
 // Reference ops: rms_norm.cuh:9-59, dequant_gemv.cuh:12-59, rope.cuh, kvcache.cuh, attention.cuh:495-513.
 #include "kernels.h"
