@@ -299,7 +299,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_short_kernel(AttnPar
 bool attention_short_supported(const AttnParams &p, int D, int dtype) {
     if (dtype == MYNN_F32 || (D != 64 && D != 128) || p.Sq != 1 || !p.qkv) return false;
     const int kpp = kAttnWaves * (64 / (D / 8));
-    return p.cache_len <= kShortPasses * kpp && (long)p.B * p.Hq <= 65535;
+    return p.cache_len <= kShortRounds * kShortPasses * kpp && (long)p.B * p.Hq <= 65535;
 }
 
 // LDS the kernel may use per workgroup for the V slice, the scores and the v scales
@@ -407,12 +407,14 @@ int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *s
     const int kv_len = p.d_active ? p.cache_len : (p.active < p.cache_len ? p.active : p.cache_len);
     if (!fuse && attn_stream_eligible(p.B, p.Sq, p.Hq, p.Hkv, D, dtype, kv_int8, kv_len, p.cache_len))
         return attention_stream_launch(p, D, dtype, kv_int8, s);
+    bool whole = false;  // the launch wrote the finished output: nothing to merge whatever the plan's split count
     int rc = dispatch_dtype(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
         if constexpr (sizeof(T) == 2) {
             if (fuse) {
                 if (kv_int8) return fail(MYNN_ERR_UNSUPPORTED, "fused decode attention: int8 KV");
                 if (attention_short_supported(p, D, dtype)) {
+                    whole = true;
                     if (D == 64) MYNN_LAUNCH((attn_decode_short_kernel<T, 64>), dim3(p.B * p.Hq), dim3(kAttnThreads), 0, s, p);
                     else MYNN_LAUNCH((attn_decode_short_kernel<T, 128>), dim3(p.B * p.Hq), dim3(kAttnThreads), 0, s, p);
                     return launch_status("attn_decode_short_kernel");
@@ -424,7 +426,7 @@ int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *s
         }
         return kv_int8 ? launch_d<T, true, false>(p, D, s) : launch_d<T, false, false>(p, D, s);
     });
-    if (rc || p.nsplit == 1) return rc;
+    if (rc || p.nsplit == 1 || whole) return rc;
     return attention_merge_launch(p, D, dtype, s);
 }
 

@@ -1,5 +1,5 @@
-// Decode attention for a cache that one workgroup covers in registers (cache_len <= 8 passes of
-// 64 / (D/8) keys per wave and 8 waves): one workgroup of 512 threads per query head, and everything
+// Decode attention for a cache that one workgroup covers in a few rounds of registers (a round is 8 passes of
+// 64 / (D/8) keys per wave and 8 waves; cache_len <= kShortRounds rounds): one workgroup of 512 threads per query head, and everything
 // between the loads and the final merge stays inside a wave -- a group of D/8 lanes owns a key per
 // pass, keeps an online softmax (m, l) and the 8 output dims of its lane over its keys, groups meet by
 // shuffles, waves through one LDS exchange.  No V parking, one barrier.  RoPE of the query and of the new
@@ -11,7 +11,8 @@
 
 namespace mynn {
 
-constexpr int kShortPasses = 8;
+constexpr int kShortPasses = 8;  // keys per lane group held in registers at a time
+constexpr int kShortRounds = 4;  // rounds of kShortPasses passes: the cache may be 4 x 512 rows at D = 64, 4 x 256 at D = 128
 constexpr int kShortWaves = 8;
 
 // qsrc / ksrc / vsrc: the D raw projection values of this query head, of its kv head's new key and new value
@@ -29,17 +30,20 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
     const int dc = lane % LPK, grp = lane / LPK;
     const T *Kc = Kcache + dc * 8, *Vc = Vcache + dc * 8;
 
-    // ---- all K / V loads of this lane
+    // ---- all K / V loads of this lane for a round of kShortPasses passes (the first round before anything else)
     U4 kreg[kShortPasses], vreg[kShortPasses];
+    auto load_round = [&](int base) {
 #pragma unroll
-    for (int i = 0; i < kShortPasses; i++) {
-        const int key = i * KPP + wave * GPW + grp;
-        kreg[i] = vreg[i] = U4{0u, 0u, 0u, 0u};
-        if (key < bound && key != new_row) {
-            kreg[i] = *(const U4 *)(Kc + (size_t)key * D);
-            vreg[i] = *(const U4 *)(Vc + (size_t)key * D);
+        for (int i = 0; i < kShortPasses; i++) {
+            const int key = base + i * KPP + wave * GPW + grp;
+            kreg[i] = vreg[i] = U4{0u, 0u, 0u, 0u};
+            if (key < bound && key != new_row) {
+                kreg[i] = *(const U4 *)(Kc + (size_t)key * D);
+                vreg[i] = *(const U4 *)(Vc + (size_t)key * D);
+            }
         }
-    }
+    };
+    load_round(0);
 
     ready();
     // ---- this lane's 8 dims of the rotated query, of the rotated new key and of the new value
@@ -71,10 +75,12 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
     float m = -INFINITY, l = 0.f, o[8];
 #pragma unroll
     for (int e = 0; e < 8; e++) o[e] = 0.f;
+    for (int base = 0; base < bound; base += kShortPasses * KPP) {
+    if (base > 0) load_round(base);  // (a cache beyond one round: its loads are not overlapped with the round before)
 #pragma unroll
     for (int i = 0; i < kShortPasses; i++) {
-        if (i * KPP >= bound) break;  // no wave has keys in this pass or a later one
-        const int key = i * KPP + wave * GPW + grp;
+        if (base + i * KPP >= bound) break;  // no wave has keys in this pass or a later one
+        const int key = base + i * KPP + wave * GPW + grp;
         float kf[8], vf[8];
         widen8<T>(kreg[i], kf);
         widen8<T>(vreg[i], vf);
@@ -97,6 +103,7 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
             for (int e = 0; e < 8; e++) o[e] = o[e] * corr + pe * vf[e];
             m = mn;
         }
+    }
     }
     // ---- lane groups of the wave meet (lanes of equal dc), then the waves through LDS
     auto merge = [&](float m2, float l2, const float *o2) {

@@ -247,7 +247,7 @@ bool qkv_attention_supported(int H, int Hq, int Hkv, int D, int max_seq, int dty
     if (dtype != MYNN_F16 && dtype != MYNN_BF16) return false;
     if (D != 64 && D != 128) return false;
     const int kpp = kShortWaves * (64 / (D / 8));
-    if (max_seq > kShortPasses * kpp) return false;
+    if (max_seq > kShortRounds * kShortPasses * kpp) return false;
     const int N = (Hq + 2 * Hkv) * D;
     if (H % 16 || H > 4096 || N % 4 || Hq % Hkv || Hq > 1024) return false;
     return (size_t)H * sizeof(float) <= 48 * 1024;

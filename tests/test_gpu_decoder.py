@@ -74,15 +74,22 @@ SHORT_CACHE = {
     64: dict(SMALL, n_layers=2, hidden=256, n_heads=4, n_kv_heads=2, head_dim=64, max_seq=512),
     128: dict(SMALL, n_layers=2, hidden=256, n_heads=2, n_kv_heads=1, head_dim=128, max_seq=256),
 }
+# the same form walks a longer cache in rounds of 512 / 256 rows (up to four)
+LONGER_CACHE = {
+    64: dict(SHORT_CACHE[64], max_seq=1300),
+    128: dict(SHORT_CACHE[128], max_seq=1024),
+}
 
 
 @pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
 @pytest.mark.parametrize("D", [64, 128])
-def test_decode_attention_short_cache_every_pass_vs_oracle(g, dt, D):
-    """Head dims 64 and 128 with a cache one workgroup covers (512 / 256 rows): the decode step's attention
-    keeps every key in registers, a lane group per key and pass.  Token by token through most of the cache,
-    so that every pass and every wave gets keys, and the rows the kernel appends, against the oracle."""
-    cfg, w = llm_weights.synthetic_int8(SHORT_CACHE[D], dt, seed=13 + D)
+@pytest.mark.parametrize("rounds", [1, 4], ids=["one_round", "several_rounds"])
+def test_decode_attention_short_cache_every_pass_vs_oracle(g, dt, D, rounds):
+    """Head dims 64 and 128 with a cache one workgroup covers (512 / 256 rows a round, up to four rounds): the
+    decode step's attention keeps a round's keys in registers, a lane group per key and pass.  Token by token
+    through most of the cache, so that every round, pass and wave gets keys, and the rows the kernel appends,
+    against the oracle."""
+    cfg, w = llm_weights.synthetic_int8((SHORT_CACHE if rounds == 1 else LONGER_CACHE)[D], dt, seed=13 + D)
     ref = orc.Model(cfg, w)
     dec = g.mynn.Decoder(cfg, dev_weights(g, w, dt))
     n = cfg["max_seq"] - 5

@@ -1,5 +1,5 @@
-"""The decode step with the q|k|v projection and the attention of a layer in one launch, against the same step
-with two launches: the same arithmetic operation for operation, so logits, tokens and KV rows must be
+"""The decode step with the q|k|v projection, the attention and the o projection of a layer in one launch, against the
+same step with three launches: the same arithmetic operation for operation, so logits, tokens and KV rows must be
 bit-identical (the two-launch form is what the other tests hold against the oracle)."""
 import numpy as np
 import pytest
@@ -33,11 +33,10 @@ def pair(g, cfg, weights):
 
 
 @pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
-@pytest.mark.parametrize("D", [64, 128])
-def test_fused_step_bit_identical_to_two_launches(g, dt, D):
-    cfg, w = llm_weights.synthetic_int8(SHORT_CACHE[D], dt, seed=31 + D)
+@pytest.mark.parametrize("D,max_seq,n", [(64, 512, 140), (128, 256, 140), (64, 2048, 1100), (128, 1024, 600)])
+def test_fused_step_bit_identical_to_two_launches(g, dt, D, max_seq, n):
+    cfg, w = llm_weights.synthetic_int8(dict(SHORT_CACHE[D], max_seq=max_seq), dt, seed=31 + D)
     one, two = pair(g, cfg, dev_weights(g, w, dt))
-    n = 140
     toks = np.random.default_rng(D + dt).integers(0, cfg["vocab"], n)
     for i, t in enumerate(toks):
         a, la = one.step([t], [i], i, i + 1, want_logits=True)
