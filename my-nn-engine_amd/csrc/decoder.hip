@@ -232,7 +232,9 @@ static int enqueue_step(Model &m) {
     m.events.clear();
 
     // embed: DequantizeLinear(table) -> Gather(ids), one row per token
-    if (m.quant) {
+    // (batch-1 decode with the fused launch: the first layer's launch makes the row itself)
+    if (m.quant && rows == 1 && m.qkv_attn && !w8a8 && !kv8) {
+    } else if (m.quant) {
         note(m, "embed_dequant", (double)rows * (H + eb + H * eb));
         TRY(embed_dequant<T>(m.x, (const int8_t *)m.embed.w, m.embed.scale, m.d_ids, rows, V, H, s));
     } else {
@@ -247,12 +249,15 @@ static int enqueue_step(Model &m) {
         bool roped = false;
         if (fused && m.qkv_attn) {
             // RMSNorm + q|k|v projection, RoPE, both cache appends and the attention in one launch
-            note(m, "qkv_attention_o", (double)L.qkv.N * H + L.qkv.N * eb + 2 * H * eb + 2.0 * KD * eb + (double)H * QD + H * eb + 2 * H * eb);
+            note(m, li == 0 ? "embed_qkv_attention_o" : "qkv_attention_o", (double)L.qkv.N * H + L.qkv.N * eb + 2 * H * eb + 2.0 * KD * eb + (double)H * QD + H * eb + 2 * H * eb);
             QkvAttnParams p{};
             p.x = m.x; p.norm_w = L.norm1; p.eps = c.eps; p.wq = (const int8_t *)L.qkv.w; p.scale = L.qkv.scale;
             p.N = L.qkv.N; p.K = H; p.qkv = (uint64_t *)m.qkv; p.out = m.attn; p.k_cache = L.k_cache; p.v_cache = L.v_cache;
             p.cos_t = m.cos_t; p.sin_t = m.sin_t; p.d_pos = m.d_pos; p.d_active = m.d_active; p.Hq = Hq; p.Hkv = Hkv;
             p.max_seq = c.max_seq; p.softmax_scale = softmax_scale; p.err = m.d_past + 3; p.spin_limit = 400000;
+            if (li == 0) {  // the input row of the first layer: the token's embedding
+                p.embed_w = (const int8_t *)m.embed.w; p.embed_s = m.embed.scale; p.d_ids = m.d_ids; p.vocab = V;
+            }
             // ... and the o projection + residual behind it: x2 = T(T(Wo . attn) + x)
             p.o_wq = (const int8_t *)L.o.w; p.o_scale = L.o.scale; p.o_out = m.x2; p.attn_words = (uint64_t *)m.attn;
             TRY(qkv_attention_launch(p, D, c.dtype, s));
@@ -599,7 +604,7 @@ static int build(Model &m, void **init, void **state) {
     if (m.quant && rows == 1 && !c.quantize_activations && !c.quant_kv_cache && g_fuse_qkv_attention &&
         attention_fused_supported(c.head_dim, c.n_heads / c.n_kv_heads) &&
         qkv_attention_supported(H, c.n_heads, c.n_kv_heads, c.head_dim, c.max_seq, c.dtype) && (QD + 2 * KD) * eb % 8 == 0) {
-        bool ok = aligned16(m.qkv) && aligned16(m.x) && aligned16(m.attn);
+        bool ok = aligned16(m.qkv) && aligned16(m.x) && aligned16(m.attn) && aligned16(m.embed.w);
         for (const Layer &L : m.layers)
             ok = ok && aligned16(L.qkv.w) && aligned16(L.norm1) && aligned16(L.norm2) && aligned16(L.k_cache) && aligned16(L.v_cache) && aligned16(L.o.w);
         if (ok && (char *)m.attn > (char *)m.qkv && ((char *)m.attn + (size_t)QD * eb - (char *)m.qkv) % 8 == 0) {

@@ -94,6 +94,12 @@ struct QkvAttnParams {
     void *o_out;             // [K]
     uint64_t *attn_words;
     int o_blocks;            // filled in by the launcher
+    // optional: the input row is not `x` but row *d_ids of the int8 embedding table times its scale, rounded to
+    // the storage type (the first layer of a step; x is then not read)
+    const int8_t *embed_w;   // [vocab, K]
+    const void *embed_s;     // [vocab]
+    const int64_t *d_ids;
+    int vocab;
 };
 bool qkv_attention_supported(int H, int Hq, int Hkv, int D, int max_seq, int dtype);
 int qkv_attention_launch(QkvAttnParams p, int D, int dtype, hipStream_t s);

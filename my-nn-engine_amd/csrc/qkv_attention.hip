@@ -62,9 +62,13 @@ struct QaGemv {
     const void *scale, *residual;
     void *out;
     int N, K;
+    // EMBED: the activation (NORM role) / the residual (RESID role) is row `erow` of the int8 embedding table times
+    // its scale, rounded to T -- what embed_dequant_kernel would have written
+    const int8_t *erow;
+    float escale;
 };
 
-template <typename T, int NC, bool NORM, bool POLL, bool RESID>
+template <typename T, int NC, bool NORM, bool POLL, bool RESID, bool EMBED>
 __device__ __forceinline__ void qa_gemv(const QaGemv &a, float *act_lds, float *red, int blk, int nblk, int limit, int *err) {
     constexpr int R = 2;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -90,7 +94,11 @@ __device__ __forceinline__ void qa_gemv(const QaGemv &a, float *act_lds, float *
         }
         const int row = min(gg * R + min(lane, R - 1), N - 1);
         G.sc = Elem<T>::ld(scale, row);
-        G.res = RESID ? Elem<T>::ld((const T *)a.residual, row) : 0.f;
+        G.res = 0.f;
+        if constexpr (RESID) {
+            if constexpr (EMBED) G.res = Elem<T>::rnd((float)a.erow[row] * a.escale);
+            else G.res = Elem<T>::ld((const T *)a.residual, row);
+        }
     };
     Group ga;
     if (g < groups) load_group(g, ga);  // in flight while the activation is staged
@@ -116,7 +124,16 @@ __device__ __forceinline__ void qa_gemv(const QaGemv &a, float *act_lds, float *
                         if (qa_some_empty(w1)) w1 = qa_wait(wp + 1, limit, err);
                         raw = U4{(uint32_t)w0, (uint32_t)(w0 >> 32), (uint32_t)w1, (uint32_t)(w1 >> 32)};
                     } else {
-                        raw = ((const U4 *)a.act)[pc];
+                        if constexpr (EMBED) {
+                            const uint2 w = *(const uint2 *)(a.erow + (size_t)pc * 8);
+                            const uint32_t ww[2] = {w.x, w.y};
+                            uint32_t b[8];
+#pragma unroll
+                            for (int i = 0; i < 8; i++) b[i] = qa_bits<T>((float)(int8_t)((ww[i >> 2] >> (8 * (i & 3))) & 0xFF) * a.escale);
+                            raw = U4{b[0] | (b[1] << 16), b[2] | (b[3] << 16), b[4] | (b[5] << 16), b[6] | (b[7] << 16)};
+                        } else {
+                            raw = ((const U4 *)a.act)[pc];
+                        }
                     }
                     if constexpr (NORM) nwv[q] = ((const U4 *)a.norm_w)[pc];
                     widen8<T>(raw, f[q]);
@@ -198,7 +215,8 @@ __device__ __forceinline__ void qa_gemv(const QaGemv &a, float *act_lds, float *
     }
 }
 
-template <typename T, int D, int NC>
+// EMBED: the layer's input row is the embedding row of token *p.d_ids (first layer of a step)
+template <typename T, int D, int NC, bool EMBED>
 __global__ __launch_bounds__(kQaThreads, 2) void qkv_attention_kernel(QkvAttnParams p) {
     extern __shared__ float act_lds[];  // [K], GEMV workgroups
     __shared__ float red[kQaStageThreads / 64];
@@ -207,16 +225,26 @@ __global__ __launch_bounds__(kQaThreads, 2) void qkv_attention_kernel(QkvAttnPar
     const int tid = threadIdx.x;
     const int QD = p.Hq * D;
 
+    const int8_t *erow = nullptr;
+    float escale = 0.f;
+    if constexpr (EMBED) {
+        if ((int)blockIdx.x < p.gemv_blocks || (int)blockIdx.x >= p.gemv_blocks + p.Hq) {
+            int64_t tok = p.d_ids[0];
+            if (tok < 0) tok += p.vocab;
+            erow = p.embed_w + (size_t)tok * p.K;
+            escale = Elem<T>::ld((const T *)p.embed_s, (size_t)tok);
+        }
+    }
     if ((int)blockIdx.x < p.gemv_blocks) {
         // ---- RMSNorm + q|k|v projection into the hand-over vector
-        const QaGemv a{p.x, p.norm_w, p.eps, p.wq, p.scale, nullptr, p.qkv, p.N, p.K};
-        qa_gemv<T, NC, true, false, false>(a, act_lds, red, blockIdx.x, p.gemv_blocks, p.spin_limit, p.err);
+        const QaGemv a{p.x, p.norm_w, p.eps, p.wq, p.scale, nullptr, p.qkv, p.N, p.K, erow, escale};
+        qa_gemv<T, NC, true, false, false, EMBED>(a, act_lds, red, blockIdx.x, p.gemv_blocks, p.spin_limit, p.err);
         return;
     }
     if ((int)blockIdx.x >= p.gemv_blocks + p.Hq) {
         // ---- o projection + residual: waits for the attention's output vector
-        const QaGemv a{p.attn_words, nullptr, 0.f, p.o_wq, p.o_scale, p.x, p.o_out, p.K, QD};
-        qa_gemv<T, NC, false, true, true>(a, act_lds, red, blockIdx.x - p.gemv_blocks - p.Hq, p.o_blocks, p.spin_limit, p.err);
+        const QaGemv a{p.attn_words, nullptr, 0.f, p.o_wq, p.o_scale, p.x, p.o_out, p.K, QD, erow, escale};
+        qa_gemv<T, NC, false, true, true, EMBED>(a, act_lds, red, blockIdx.x - p.gemv_blocks - p.Hq, p.o_blocks, p.spin_limit, p.err);
         return;
     }
 
@@ -254,7 +282,7 @@ bool qkv_attention_supported(int H, int Hq, int Hkv, int D, int max_seq, int dty
 }
 
 int qkv_attention_launch(QkvAttnParams p, int D, int dtype, hipStream_t s) {
-    MYNN_REQUIRE(aligned16(p.x) && aligned16(p.norm_w) && aligned16(p.wq) && aligned16(p.qkv) && aligned16(p.k_cache) &&
+    MYNN_REQUIRE((p.embed_w || aligned16(p.x)) && aligned16(p.norm_w) && aligned16(p.wq) && aligned16(p.qkv) && aligned16(p.k_cache) &&
                      aligned16(p.v_cache) && aligned16(p.cos_t) && aligned16(p.sin_t),
                  MYNN_ERR_INVALID, "qkv + attention: operands must be 16-byte aligned");
     p.groups = p.N / 2;
@@ -273,12 +301,16 @@ int qkv_attention_launch(QkvAttnParams p, int D, int dtype, hipStream_t s) {
     const int nc = (p.K + 1023) / 1024;
     const size_t lds = (size_t)p.K * sizeof(float);
     const dim3 grid(p.gemv_blocks + p.Hq + p.o_blocks), block(kQaThreads);
+    const bool embed = p.embed_w != nullptr;
+    MYNN_REQUIRE(!embed || (p.embed_s && p.d_ids && p.vocab > 0 && p.o_wq && ((uintptr_t)p.embed_w & 7) == 0 && p.K % 8 == 0),
+                 MYNN_ERR_INVALID, "qkv + attention + o: bad embedding operand");
     return dispatch_dtype16(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
-#define MYNN_QA(D_, NC_)                                                           \
-    do {                                                                           \
-        MYNN_LAUNCH((qkv_attention_kernel<T, D_, NC_>), grid, block, lds, s, p);   \
-        return launch_status("qkv_attention_kernel");                              \
+#define MYNN_QA(D_, NC_)                                                                          \
+    do {                                                                                          \
+        if (embed) MYNN_LAUNCH((qkv_attention_kernel<T, D_, NC_, true>), grid, block, lds, s, p);  \
+        else MYNN_LAUNCH((qkv_attention_kernel<T, D_, NC_, false>), grid, block, lds, s, p);       \
+        return launch_status("qkv_attention_kernel");                                             \
     } while (0)
         if (D == 64) {
             if (nc <= 1) MYNN_QA(64, 1);
