@@ -103,6 +103,8 @@ struct Model {
     // batch-1 decode: projection and attention share a launch; m.qkv is then the hand-over vector between them
     // (all 0xFFFF between uses) and d_past[3] the error word of its bounded waits
     bool qkv_attn = false;
+    bool lm_argmax = false;       // ... and the lm_head launch finds the greedy token and moves the loop state on
+    uint64_t *lm_cand = nullptr;  // its candidate words (all ~0 between launches)
     // per-launch record of the last enqueue (names + algorithmic bytes), events when profiling
     std::vector<Launch> record;
     bool profiling = false;
@@ -374,7 +376,15 @@ static int enqueue_step(Model &m) {
             TRY(mynn_add(m.x, m.x2, m.proj, (size_t)rows * H, c.dtype, s));
         }
     }
-    if (fused) {
+    if (fused && m.lm_argmax) {
+        note(m, "gemv_norm_lm_head_argmax", (double)V * H + V * eb + 2 * H * eb + V * eb);
+        TRY(gemv_norm_argmax<T>(m.logits, m.x, m.final_norm, c.eps, (const int8_t *)m.lm_head.w, m.lm_head.scale, V, H, m.lm_cand,
+                                m.d_next, AdvanceState{m.d_ids, m.d_pos, m.d_past, m.d_active, m.d_tokens, m.d_step, m.token_cap},
+                                m.d_past + 3, 400000, s));
+        launch_timer() = LaunchTimer{};
+        m.launches = (int)m.record.size();
+        return 0;
+    } else if (fused) {
         note(m, "gemv_norm_lm_head", (double)V * H + V * eb + 2 * H * eb + V * eb);
         TRY(gemv_norm<T>(m.logits, m.x, m.final_norm, c.eps, (const int8_t *)m.lm_head.w, m.lm_head.scale, V, H, s));
     } else if (m.w8a8_fused) {
@@ -582,6 +592,7 @@ static int build(Model &m, void **init, void **state) {
     size_t o_ids = plan.take((size_t)rows * 8), o_pos = plan.take((size_t)c.seq_q * 8);
     size_t o_sc = plan.take(32 + (size_t)c.batch * 4), o_tok = plan.take((size_t)m.token_cap * 4);
     size_t o_as = plan.take(attn_scratch_bytes(c.batch, c.n_heads, c.seq_q, c.head_dim, m.nsplit));
+    size_t o_cand = plan.take(rows == 1 ? (size_t)kGemvArgmaxWords * 8 : 0);
     m.arena_bytes = plan.off;
     MYNN_HIP(hipMalloc((void **)&m.arena, m.arena_bytes));
     MYNN_HIP(hipMemset(m.arena, 0, m.arena_bytes));
@@ -595,6 +606,7 @@ static int build(Model &m, void **init, void **state) {
     m.d_next = m.d_past + 8;  // one token per sequence after the scalars
     m.d_tokens = (int32_t *)(m.arena + o_tok);
     m.attn_scratch = m.arena + o_as;
+    m.lm_cand = (uint64_t *)(m.arena + o_cand);
     m.next_stage = align_up((size_t)c.batch * 4, 256);  // the sequences' next tokens live in the tail of the staging buffer
     m.stage_bytes = align_up((size_t)rows * 8 + (size_t)c.seq_q * 8 + 64 + (size_t)m.token_cap * 4, 256) + 256 + m.next_stage;
     MYNN_HIP(hipHostMalloc((void **)&m.h_stage, m.stage_bytes, hipHostMallocDefault));
@@ -609,6 +621,8 @@ static int build(Model &m, void **init, void **state) {
             ok = ok && aligned16(L.qkv.w) && aligned16(L.norm1) && aligned16(L.norm2) && aligned16(L.k_cache) && aligned16(L.v_cache) && aligned16(L.o.w);
         if (ok && (char *)m.attn > (char *)m.qkv && ((char *)m.attn + (size_t)QD * eb - (char *)m.qkv) % 8 == 0) {
             MYNN_HIP(hipMemset(m.qkv, 0xFF, (size_t)((char *)m.attn + (size_t)QD * eb - (char *)m.qkv)));
+            m.lm_argmax = gemv_norm_argmax_supported(m.x, m.final_norm, (const int8_t *)m.lm_head.w, V, H);
+            if (m.lm_argmax) MYNN_HIP(hipMemset(m.lm_cand, 0xFF, (size_t)kGemvArgmaxWords * 8));
             MYNN_HIP(hipDeviceSynchronize());
             m.qkv_attn = true;
         }
@@ -706,8 +720,9 @@ static int upload_inputs(Model &m, const int64_t *ids, const int64_t *pos, int64
 static int qkv_attention_failed(Model &m) {
     const mynn_model_config &c = m.cfg;
     (void)hipMemset(m.qkv, 0xFF, (size_t)((char *)m.attn + (size_t)c.n_heads * c.head_dim * dtype_size(c.dtype) - (char *)m.qkv));
+    (void)hipMemset(m.lm_cand, 0xFF, (size_t)kGemvArgmaxWords * 8);
     (void)hipMemset(m.d_past + 3, 0, 4);
-    return fail(MYNN_ERR_STATE, "decode step: the attention waited too long for the q|k|v projection (is the device shared?)");
+    return fail(MYNN_ERR_STATE, "decode step: a stage of a fused launch waited too long for the stage before it (is the device shared?)");
 }
 
 static int run_once(Model &m) {

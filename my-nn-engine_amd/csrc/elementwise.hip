@@ -375,9 +375,6 @@ int interleave_row_groups(void *dst, const void *src, size_t rows, size_t row_by
 
 // ---- greedy argmax, last maximum wins (reference crates/llm/src/session.rs:683-690) -----------
 // one workgroup of 1024 threads per row, 16-byte loads; (value, index) ordered by value, then index
-__device__ inline void argmax_take(float &bv, int &bi, float v, int i) {
-    if (bi < 0 || v > bv || (v == bv && i > bi)) { bv = v; bi = i; }
-}
 template <typename T>
 __global__ __launch_bounds__(1024) void argmax_last_kernel(int32_t *out, const T *logits, int n, AdvanceState adv) {
     __shared__ float sv[16];

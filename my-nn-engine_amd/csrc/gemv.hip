@@ -14,7 +14,7 @@
 //             semantics: y = (x * (1/sqrt(mean(x^2)+eps))) * w, rounded to T like the stored tensor)
 //   RESIDUAL  out = T(T(acc*scale) + residual[n])            (the Add that follows o/down proj)
 //   SWIGLU    rows interleaved gate,up: out[i] = T(silu(T(g)) * T(u))  (Swish+Mul group)
-#include "mynn_common.h"
+#include "kernels.h"
 
 namespace mynn {
 
@@ -31,6 +31,15 @@ struct GemvParams {
     int N, K;
     int act_stride;        // elements between activation rows
     int out_stride;        // elements between output rows
+    // ARGMAX (the decode step's lm_head): the greedy token is found by the same launch.  Every GEMV workgroup leaves
+    // its best (value, row) in cand[block] (one 8-byte word, row low / value bits high, ~0 = "empty" between launches);
+    // one more workgroup waits for them (bounded spin, error word), takes the best, moves the loop state on and empties
+    // the words again.
+    uint64_t *cand;
+    int32_t *next;
+    AdvanceState adv;
+    int *err;
+    int spin_limit;
     uint64_t *fill;        // optional: fill_words words that this launch sets to ~0 (the hand-over vectors of the
     int fill_words;        // fused q|k|v + attention + o launch, emptied between two of its uses)
 };
@@ -158,11 +167,69 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv_kernel(GemvParams p
 // (group g, g + total_waves, ...).  For a group every lane issues all R x NC 16-byte weight loads
 // before the first multiply, dequantises in registers (int8 -> f32 convert + FMA) and the partial
 // sums meet in a wave64 butterfly; the scale is applied after the sum.  NC = ceil(K / 1024).
-template <typename T, int R, int NC, int EPI, bool NORM>
+template <typename T, int R, int NC, int EPI, bool NORM, bool ARGMAX = false>
 __global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(GemvParams p, int groups, int total_waves) {
     extern __shared__ float act_lds[];  // [K]
     __shared__ float red[kGemvWaves];
+    __shared__ float best_v[kGemvWaves];
+    __shared__ int best_i[kGemvWaves];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float bv = -INFINITY;  // ARGMAX: this thread's best stored value and its row
+    int bi = -1;
+    auto meet = [&]() {  // best of the workgroup in thread 0
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ov = __shfl_xor(bv, off, kWave);
+            const int oi = __shfl_xor(bi, off, kWave);
+            if (oi >= 0) argmax_take(bv, bi, ov, oi);
+        }
+        if (lane == 0) { best_v[wave] = bv; best_i[wave] = bi; }
+        __syncthreads();
+        if (tid == 0)
+            for (int w = 1; w < kGemvWaves; w++)
+                if (best_i[w] >= 0) argmax_take(bv, bi, best_v[w], best_i[w]);
+    };
+    if constexpr (ARGMAX) {
+        if (blockIdx.x == gridDim.x - 1) {
+            // ---- the extra workgroup: every GEMV workgroup's candidate -> the token, the loop state moves on
+            const int nb = gridDim.x - 1;
+            int st_step = 0, st_past = 0, st_active = 0;
+            int64_t st_pos = 0;
+            if (p.adv.ids && tid == 0) {
+                st_step = *p.adv.step;
+                st_pos = p.adv.pos[0];
+                st_past = *p.adv.past;
+                st_active = *p.adv.active;
+            }
+            for (int i = tid; i < nb; i += kGemvThreads) {
+                uint64_t w = __hip_atomic_load(p.cand + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                for (int spins = 0; w == ~0ull; spins++) {
+                    if (spins > p.spin_limit) {
+                        __hip_atomic_store(p.err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(1);
+                    w = __hip_atomic_load(p.cand + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                const int oi = (int)(uint32_t)w;
+                if (w != ~0ull && oi >= 0) argmax_take(bv, bi, __builtin_bit_cast(float, (uint32_t)(w >> 32)), oi);
+                p.cand[i] = ~0ull;  // empty again for the next launch
+            }
+            meet();
+            if (tid == 0) {
+                p.next[0] = bi;
+                if (p.adv.ids) {
+                    if (st_step < p.adv.cap) p.adv.tokens[st_step] = bi;
+                    *p.adv.step = st_step + 1;
+                    p.adv.ids[0] = bi;
+                    p.adv.pos[0] = st_pos + 1;
+                    *p.adv.past = st_past + 1;
+                    *p.adv.active = st_active + 1;
+                }
+            }
+            return;
+        }
+    }
     const int K = p.K, N = p.N;
     const int nchunks = K >> 4;
     int g = blockIdx.x * kGemvWaves + wave;
@@ -290,6 +357,7 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(GemvParams 
                     float y = acc[r] * G.sc;
                     if constexpr (EPI == EPI_RESIDUAL) y = Elem<T>::rnd(y) + G.res;
                     Elem<T>::st(out, row0 + r, y);
+                    if constexpr (ARGMAX) argmax_take(bv, bi, Elem<T>::rnd(y), row0 + r);  // (the value as stored)
                 }
             }
         }
@@ -300,8 +368,16 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(GemvParams 
         loaded = false;
         compute(g, ga);
     }
+    if constexpr (ARGMAX) {
+        meet();
+        if (tid == 0) {
+            // (a workgroup without rows leaves index -1: not ~0 as a word, since -inf's bits sit in the high half)
+            const uint64_t word = (uint64_t)(uint32_t)bi | ((uint64_t)__builtin_bit_cast(uint32_t, bv) << 32);
+            __hip_atomic_store(p.cand + blockIdx.x, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
 }
-template <typename T, int R, int NC, int EPI, bool NORM>
+template <typename T, int R, int NC, int EPI, bool NORM, bool ARGMAX = false>
 static int launch_gemv1(const GemvParams &p, hipStream_t s) {
     const int groups = (p.N + R - 1) / R;
     const int max_waves = 256 * 16;  // four resident waves per SIMD (measured best of 8/16/24/32 per CU)
@@ -309,7 +385,7 @@ static int launch_gemv1(const GemvParams &p, hipStream_t s) {
     int waves = (groups + passes - 1) / passes;
     const int blocks = (waves + kGemvWaves - 1) / kGemvWaves;
     waves = blocks * kGemvWaves;
-    MYNN_LAUNCH((dequant_gemv1_kernel<T, R, NC, EPI, NORM>), dim3(blocks), dim3(kGemvThreads),
+    MYNN_LAUNCH((dequant_gemv1_kernel<T, R, NC, EPI, NORM, ARGMAX>), dim3(blocks + (ARGMAX ? 1 : 0)), dim3(kGemvThreads),
                        (size_t)p.K * sizeof(float), s, p, groups, waves);
     return launch_status("dequant_gemv1_kernel");
 }
@@ -438,6 +514,34 @@ int gemv_norm(void *out, const void *x, const void *norm_w, float eps, const int
     if (rc) return rc;
     return gemv1_dispatch<T, EPI_PLAIN, true>(p, s);
 }
+// the decode step's lm_head: RMSNorm + GEMV + greedy token + loop state in one launch (cand: (N / 2 + 3) / 4 + 1
+// words at most, all ~0 on entry and again on exit)
+bool gemv_norm_argmax_supported(const void *x, const void *norm_w, const int8_t *wq, int N, int K) {
+    return aligned16(x) && aligned16(norm_w) && aligned16(wq) && K % 16 == 0 && (K + 1023) / 1024 <= 14 && N > 0 &&
+           (size_t)K * sizeof(float) <= 64 * 1024;
+}
+template <typename T>
+int gemv_norm_argmax(void *out, const void *x, const void *norm_w, float eps, const int8_t *wq, const void *scale, int N, int K,
+                     uint64_t *cand, int32_t *next, AdvanceState adv, int *err, int spin_limit, hipStream_t s) {
+    GemvParams p{};
+    p.out = out; p.act = x; p.wq = wq; p.scale = scale; p.norm_w = norm_w; p.eps = eps; p.N = N; p.K = K;
+    p.act_stride = K; p.out_stride = N;
+    p.cand = cand; p.next = next; p.adv = adv; p.err = err; p.spin_limit = spin_limit;
+    MYNN_REQUIRE(cand && next && err && gemv_norm_argmax_supported(x, norm_w, wq, N, K), MYNN_ERR_UNSUPPORTED,
+                 "gemv_norm_argmax: N=%d K=%d", N, K);
+    const int nc = (K + 1023) / 1024;
+    if (nc <= 1) return launch_gemv1<T, 2, 1, EPI_PLAIN, true, true>(p, s);
+    if (nc <= 2) return launch_gemv1<T, 2, 2, EPI_PLAIN, true, true>(p, s);
+    if (nc <= 4) return launch_gemv1<T, 2, 4, EPI_PLAIN, true, true>(p, s);
+    if (nc <= 6) return launch_gemv1<T, 2, 6, EPI_PLAIN, true, true>(p, s);
+    if (nc <= 8) return launch_gemv1<T, 2, 8, EPI_PLAIN, true, true>(p, s);
+    return launch_gemv1<T, 2, 14, EPI_PLAIN, true, true>(p, s);
+}
+template int gemv_norm_argmax<bf16_t>(void *, const void *, const void *, float, const int8_t *, const void *, int, int, uint64_t *,
+                                      int32_t *, AdvanceState, int *, int, hipStream_t);
+template int gemv_norm_argmax<f16_t>(void *, const void *, const void *, float, const int8_t *, const void *, int, int, uint64_t *,
+                                     int32_t *, AdvanceState, int *, int, hipStream_t);
+
 template <typename T>
 int gemv_residual(void *out, const void *act, const int8_t *wq, const void *scale, const void *residual,
                   int N, int K, hipStream_t s) {

@@ -109,6 +109,14 @@ struct AdvanceState {
     int32_t *past, *active, *tokens, *step;
     int cap;
 };
+
+// gemv.hip -- the decode step's lm_head with the greedy token and the loop state in the same launch
+bool gemv_norm_argmax_supported(const void *x, const void *norm_w, const int8_t *wq, int N, int K);
+constexpr int kGemvArgmaxWords = 4096 / 4 + 1;  // candidate words a launch may use
+template <typename T>
+int gemv_norm_argmax(void *out, const void *x, const void *norm_w, float eps, const int8_t *wq, const void *scale, int N, int K,
+                     uint64_t *cand, int32_t *next, AdvanceState adv, int *err, int spin_limit, hipStream_t s);
+
 // out[r] = index of the LAST maximum of logits row r; when adv.ids != nullptr the launch also
 // records the token and moves the decode loop on by one position
 template <typename T>

@@ -118,6 +118,12 @@ template <int width> __device__ inline float group_sum(float v) {
     return v;
 }
 
+// greedy-token candidates: (value, index) ordered by value, then index -- of equal maxima the LATER one wins
+// (the reference's max_by over the logits, crates/llm/src/session.rs:683-690); index < 0 = no candidate yet
+__device__ inline void argmax_take(float &bv, int &bi, float v, int i) {
+    if (bi < 0 || v > bv || (v == bv && i > bi)) { bv = v; bi = i; }
+}
+
 // exp for softmax / SiLU: one definition for every kernel
 __device__ inline float fast_exp(float x) { return __expf(x); }
 
