@@ -615,8 +615,9 @@ def set_gemm_tile(which):
 
 
 def set_fuse_qkv_attention(on):
-    """Batch-1 decode executors built after this call run a layer's q|k|v projection and attention in one
-    launch (True, the default, when the shape allows) or in two (False)."""
+    """Batch-1 decode executors built after this call share launches between dependent ops (True, the default,
+    when the shape allows: q|k|v projection + attention + o projection of a layer, the embedding row, lm_head +
+    greedy token) or run every op as a launch of its own (False).  Same results bit for bit."""
     check(lib().mynn_set_fuse_qkv_attention(1 if on else 0))
 
 
