@@ -44,14 +44,16 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
         }
     };
     load_round(0);
+    // (the RoPE table rows too: they depend on the position only, not on the projection)
+    constexpr int half = D / 2;
+    const int d0 = dc * 8, dp = d0 < half ? d0 + half : d0 - half;
+    const U4 c_raw = *(const U4 *)(cs + d0), s_raw = *(const U4 *)(snp + d0);
 
     ready();
     // ---- this lane's 8 dims of the rotated query, of the rotated new key and of the new value
-    constexpr int half = D / 2;
-    const int d0 = dc * 8, dp = d0 < half ? d0 + half : d0 - half;
     float c[8], sn[8], q[8], kn[8], vn[8];
-    widen8<T>(*(const U4 *)(cs + d0), c);
-    widen8<T>(*(const U4 *)(snp + d0), sn);
+    widen8<T>(c_raw, c);
+    widen8<T>(s_raw, sn);
     const U4 v_new = *(const U4 *)(vsrc + d0);
     widen8<T>(v_new, vn);
     {
