@@ -32,6 +32,11 @@ GATEUP_GEMV_TRAFFIC_BYTES = 23447552
 # batched-decode gate/up few-row GEMM (Llama-3-8B shape, 32 rows): 61689.4 KiB * 2 + 896.3 KiB
 PREFILL_GATEUP_GEMM_TRAFFIC_BYTES = 680706867
 BATCHED_GATEUP_GEMM_TRAFFIC_BYTES = 127257702
+# share of SIMD clocks in which the matrix pipe is busy during the prefill gate/up GEMM, from rocprofv3 --pmc
+# SQ_VALU_MFMA_BUSY_CYCLES / (GRBM_GUI_ACTIVE / 8 XCDs * 1024 SIMDs); the shader clock under that load is 1.87 GHz
+# (2.06 GHz with int8 activations), which is why it exceeds flop / time / peak-at-2.4-GHz
+# (profiles/prefill_tinyllama_int8_8x1024_pmc_mfma_utilisation.md)
+PREFILL_GATEUP_MFMA_BUSY_FRAC = {"f16": 0.513, "w8a8": 0.382}
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16/fp16 matrix rate
 INT8_PEAK_TOPS = 5000.0    # MI355X published dense int8 matrix rate
 PREFILL_BATCH, PREFILL_LEN = 8, 1024
@@ -156,6 +161,8 @@ def prefill_main(args, mynn, cfg):
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 1), "peak": peak,
                      "unit": unit, "frac": round(achieved / peak, 4),
                      "traffic": PREFILL_GATEUP_GEMM_TRAFFIC_BYTES if dom == "linear_gateup_swiglu" and args.dtype == "f16" else None,
+                     "mfma_busy_frac_pmc": (PREFILL_GATEUP_MFMA_BUSY_FRAC["w8a8" if args.w8a8 else "f16"]
+                                            if dom == "linear_gateup_swiglu" and args.dtype == "f16" else None),
                      "flops_per_launch": fl_tot / calls, "avg_launch_us": round(ms_tot / calls * 1e3, 2),
                      "all_linear_TFLOPs": round(lin_tflops, 1)},
     }
