@@ -73,39 +73,55 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
         *(U4 *)(Vcache + (size_t)new_row * D + d0) = v_new;
     }
 
-    // ---- online softmax over this lane group's keys
+    // ---- softmax over this lane group's keys: the scores of a round are independent of each other (all dot
+    //      products, then one maximum, then one exponential per key); only rounds are chained through (m, l, o)
     float m = -INFINITY, l = 0.f, o[8];
 #pragma unroll
     for (int e = 0; e < 8; e++) o[e] = 0.f;
     for (int base = 0; base < bound; base += kShortPasses * KPP) {
-    if (base > 0) load_round(base);  // (a cache beyond one round: its loads are not overlapped with the round before)
+        if (base > 0) load_round(base);  // (a cache beyond one round: its loads are not overlapped with the round before)
+        float sc[kShortPasses];
+        float mr = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < kShortPasses; i++) {
-        if (base + i * KPP >= bound) break;  // no wave has keys in this pass or a later one
-        const int key = base + i * KPP + wave * GPW + grp;
-        float kf[8], vf[8];
-        widen8<T>(kreg[i], kf);
-        widen8<T>(vreg[i], vf);
-        if (key == new_row) {
+        for (int i = 0; i < kShortPasses; i++) {
+            sc[i] = -INFINITY;
+            if (base + i * KPP >= bound) continue;  // no wave has keys in this pass
+            const int key = base + i * KPP + wave * GPW + grp;
+            float kf[8];
+            widen8<T>(kreg[i], kf);
+            if (key == new_row) {
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-                kf[e] = kn[e];
-                vf[e] = vn[e];
+                for (int e = 0; e < 8; e++) kf[e] = kn[e];
             }
-        }
-        float sc = 0.f;
+            float d = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; e++) sc = fmaf(q[e], kf[e], sc);
-        sc = group_sum<LPK>(sc) * scale;
-        if (key < bound) {
-            const float mn = fmaxf(m, sc);
-            const float corr = fast_exp(m - mn), pe = fast_exp(sc - mn);
-            l = l * corr + pe;
-#pragma unroll
-            for (int e = 0; e < 8; e++) o[e] = o[e] * corr + pe * vf[e];
-            m = mn;
+            for (int e = 0; e < 8; e++) d = fmaf(q[e], kf[e], d);
+            d = group_sum<LPK>(d) * scale;
+            if (key < bound) sc[i] = d;
+            mr = fmaxf(mr, sc[i]);
         }
-    }
+        if (mr == -INFINITY) continue;  // this lane group has no key in the round
+        const float mn = fmaxf(m, mr);
+        const float corr = fast_exp(m - mn);  // (m = -inf: 0)
+        l *= corr;
+#pragma unroll
+        for (int e = 0; e < 8; e++) o[e] *= corr;
+#pragma unroll
+        for (int i = 0; i < kShortPasses; i++) {
+            if (base + i * KPP >= bound) continue;
+            const int key = base + i * KPP + wave * GPW + grp;
+            float vf[8];
+            widen8<T>(vreg[i], vf);
+            if (key == new_row) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) vf[e] = vn[e];
+            }
+            const float pe = fast_exp(sc[i] - mn);  // (no key: exp(-inf) = 0)
+            l += pe;
+#pragma unroll
+            for (int e = 0; e < 8; e++) o[e] = fmaf(pe, vf[e], o[e]);
+        }
+        m = mn;
     }
     // ---- lane groups of the wave meet (lanes of equal dc), then the waves through LDS
     auto merge = [&](float m2, float l2, const float *o2) {
