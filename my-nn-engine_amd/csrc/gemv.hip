@@ -167,8 +167,12 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv_kernel(GemvParams p
 // (group g, g + total_waves, ...).  For a group every lane issues all R x NC 16-byte weight loads
 // before the first multiply, dequantises in registers (int8 -> f32 convert + FMA) and the partial
 // sums meet in a wave64 butterfly; the scale is applied after the sum.  NC = ceil(K / 1024).
+// What the first loads need (pointers, sizes) are leading scalar arguments: they arrive preloaded in SGPRs with
+// the wave (-amdgpu-kernarg-preload-count) instead of through a scalar load from the kernarg segment.
 template <typename T, int R, int NC, int EPI, bool NORM, bool ARGMAX = false>
-__global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(GemvParams p, int groups, int total_waves) {
+__global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(const int8_t *wq, const void *act, const void *scale_p, const void *norm_w,
+                                                                       const void *residual, int N, int K, int groups,
+                                                                       int total_waves, GemvParams p) {
     extern __shared__ float act_lds[];  // [K]
     __shared__ float red[kGemvWaves];
     __shared__ float best_v[kGemvWaves];
@@ -230,53 +234,55 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(GemvParams 
             return;
         }
     }
-    const int K = p.K, N = p.N;
     const int nchunks = K >> 4;
     int g = blockIdx.x * kGemvWaves + wave;
-    if (p.fill && blockIdx.x == gridDim.x - 1)
-        for (int i = tid; i < p.fill_words; i += kGemvThreads) p.fill[i] = ~0ull;
 
     // one row group's operands: R x NC weight chunks per lane, plus, in lane r < R, what the store of row r
     // needs (scale, the next row's scale for SwiGLU, the residual) -- fetched with the weights, not after the sum
     struct Group {
         U4 w[R][NC];
-        float sc, sc1, res;
+        T sc, sc1, res;  // as loaded: widening them here would make the wave wait for every load above
     };
-    const T *scale = (const T *)p.scale;
+    const T *scale = (const T *)scale_p;
     auto load_group = [&](int gg, Group &G) {
 #pragma unroll
         for (int r = 0; r < R; r++) {
             const int row = gg * R + r < N ? gg * R + r : N - 1;
-            const U4 *wrow = (const U4 *)(p.wq + (size_t)row * K);
+            const U4 *wrow = (const U4 *)(wq + (size_t)row * K);
 #pragma unroll
-            for (int j = 0; j < NC; j++) {
-                const int c = lane + j * kWave;
-                if (c < nchunks) G.w[r][j] = __builtin_nontemporal_load(&wrow[c]);
-                else G.w[r][j] = U4{0u, 0u, 0u, 0u};
-            }
+            for (int j = 0; j < NC; j++)  // (unconditional: the wait for the activation can then be counted exactly;
+                G.w[r][j] = __builtin_nontemporal_load(&wrow[min(lane + j * kWave, nchunks - 1)]);  // chunks past K are not used)
         }
         const int row = min(gg * R + min(lane, R - 1), N - 1);
-        G.sc = Elem<T>::ld(scale, row);
-        G.sc1 = EPI == EPI_SWIGLU ? Elem<T>::ld(scale, min(row + 1, N - 1)) : 0.f;
-        G.res = EPI == EPI_RESIDUAL ? Elem<T>::ld((const T *)p.residual, row) : 0.f;
+        G.sc = scale[row];
+        if constexpr (EPI == EPI_SWIGLU) G.sc1 = scale[min(row + 1, N - 1)];
+        if constexpr (EPI == EPI_RESIDUAL) G.res = ((const T *)residual)[row];
     };
+    // the activation pieces (and their norm weights) are requested FIRST: loads return in order, so a wave that asked
+    // for its weights before them would sit out the whole weight fetch before it could stage anything
+    const int npieces = K >> 3;
+    constexpr int PMAX = (NC * 1024 / 8 + kGemvThreads - 1) / kGemvThreads;  // pieces per thread
+    U4 apv[PMAX], nwv[NORM ? PMAX : 1];
+#pragma unroll
+    for (int q = 0; q < PMAX; q++) {
+        const int pc = tid + q * kGemvThreads;
+        if (pc < npieces) {
+            apv[q] = ((const U4 *)act)[pc];
+            if constexpr (NORM) nwv[q] = ((const U4 *)norm_w)[pc];
+        }
+    }
     Group ga;
-    if (g < groups) load_group(g, ga);  // in flight while the activation is staged
+    load_group(min(g, groups - 1), ga);  // in flight while the activation is staged
 
     // ---- stage: thread t owns the 8-element pieces t, t + 256, ... of the row
     {
-        const U4 *ap = (const U4 *)p.act;
-        const int npieces = K >> 3;
-        constexpr int PMAX = (NC * 1024 / 8 + kGemvThreads - 1) / kGemvThreads;  // pieces per thread
         float f[PMAX][8];
-        U4 nwv[NORM ? PMAX : 1];  // the norm weights of this thread's pieces, fetched with the activation
         float ss = 0.f;
 #pragma unroll
         for (int q = 0; q < PMAX; q++) {
             const int pc = tid + q * kGemvThreads;
             if (pc < npieces) {
-                if constexpr (NORM) nwv[q] = ((const U4 *)p.norm_w)[pc];
-                widen8<T>(ap[pc], f[q]);
+                widen8<T>(apv[q], f[q]);
                 if constexpr (NORM) {
 #pragma unroll
                     for (int i = 0; i < 8; i++) ss = fmaf(f[q][i], f[q][i], ss);
@@ -344,8 +350,8 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(GemvParams 
 #pragma unroll
             for (int r = 0; r < R; r += 2) {
                 if (lane == r && row0 + r + 1 < N) {
-                    float gt = Elem<T>::rnd(acc[r] * G.sc);
-                    float up = Elem<T>::rnd(acc[r + 1] * G.sc1);
+                    float gt = Elem<T>::rnd(acc[r] * Elem<T>::ld(&G.sc, 0));
+                    float up = Elem<T>::rnd(acc[r + 1] * Elem<T>::ld(&G.sc1, 0));
                     float sig = 1.0f / (1.0f + expf(-gt));
                     Elem<T>::st(out, (size_t)((row0 + r) >> 1), (gt * sig) * up);
                 }
@@ -354,8 +360,8 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(GemvParams 
 #pragma unroll
             for (int r = 0; r < R; r++) {
                 if (lane == r && row0 + r < N) {
-                    float y = acc[r] * G.sc;
-                    if constexpr (EPI == EPI_RESIDUAL) y = Elem<T>::rnd(y) + G.res;
+                    float y = acc[r] * Elem<T>::ld(&G.sc, 0);
+                    if constexpr (EPI == EPI_RESIDUAL) y = Elem<T>::rnd(y) + Elem<T>::ld(&G.res, 0);
                     Elem<T>::st(out, row0 + r, y);
                     if constexpr (ARGMAX) argmax_take(bv, bi, Elem<T>::rnd(y), row0 + r);  // (the value as stored)
                 }
@@ -368,6 +374,8 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(GemvParams 
         loaded = false;
         compute(g, ga);
     }
+    if (p.fill && blockIdx.x == gridDim.x - 1)
+        for (int i = tid; i < p.fill_words; i += kGemvThreads) p.fill[i] = ~0ull;
     if constexpr (ARGMAX) {
         meet();
         if (tid == 0) {
@@ -386,7 +394,7 @@ static int launch_gemv1(const GemvParams &p, hipStream_t s) {
     const int blocks = (waves + kGemvWaves - 1) / kGemvWaves;
     waves = blocks * kGemvWaves;
     MYNN_LAUNCH((dequant_gemv1_kernel<T, R, NC, EPI, NORM, ARGMAX>), dim3(blocks + (ARGMAX ? 1 : 0)), dim3(kGemvThreads),
-                       (size_t)p.K * sizeof(float), s, p, groups, waves);
+                       (size_t)p.K * sizeof(float), s, p.wq, p.act, p.scale, p.norm_w, p.residual, p.N, p.K, groups, waves, p);
     return launch_status("dequant_gemv1_kernel");
 }
 

@@ -77,7 +77,8 @@ __device__ __forceinline__ void qa_gemv(const QaGemv &a, float *act_lds, float *
     int g = blk * kQaWaves + wave;
     struct Group {
         U4 w[R][NC];
-        float sc, res;
+        T sc, res;        // as loaded: widening them here would make the wave wait for every load above
+        int8_t eres;      // EMBED: the residual's table entry
     };
     const T *scale = (const T *)a.scale;
     auto load_group = [&](int gg, Group &G) {
@@ -86,29 +87,44 @@ __device__ __forceinline__ void qa_gemv(const QaGemv &a, float *act_lds, float *
             const int row = gg * R + r < N ? gg * R + r : N - 1;
             const U4 *wrow = (const U4 *)(a.wq + (size_t)row * K);
 #pragma unroll
-            for (int j = 0; j < NC; j++) {
-                const int c = lane + j * kWave;
-                if (c < nchunks) G.w[r][j] = __builtin_nontemporal_load(&wrow[c]);
-                else G.w[r][j] = U4{0u, 0u, 0u, 0u};
-            }
+            for (int j = 0; j < NC; j++)  // (unconditional, so that waits on earlier loads can be counted; chunks past K are not used)
+                G.w[r][j] = __builtin_nontemporal_load(&wrow[min(lane + j * kWave, nchunks - 1)]);
         }
         const int row = min(gg * R + min(lane, R - 1), N - 1);
-        G.sc = Elem<T>::ld(scale, row);
-        G.res = 0.f;
+        G.sc = scale[row];
         if constexpr (RESID) {
-            if constexpr (EMBED) G.res = Elem<T>::rnd((float)a.erow[row] * a.escale);
-            else G.res = Elem<T>::ld((const T *)a.residual, row);
+            if constexpr (EMBED) G.eres = a.erow[row];
+            else G.res = ((const T *)a.residual)[row];
         }
     };
+    // An activation that is read from memory (and its norm weights) is requested BEFORE the weights: loads return in
+    // order, so a wave that asked for its weights first would sit out the whole weight fetch before it could stage.
+    const int npieces = K >> 3;
+    constexpr int NT = NORM ? kQaStageThreads : kQaThreads;  // thread t < NT owns the 8-element pieces t, t + NT, ..
+    constexpr int PMAX = (NC * 1024 / 8 + NT - 1) / NT;
+    U4 apv[PMAX], nwv[NORM ? PMAX : 1];
+    if constexpr (!POLL) {
+        if (tid < NT) {
+#pragma unroll
+            for (int q = 0; q < PMAX; q++) {
+                const int pc = tid + q * NT;
+                if (pc < npieces) {
+                    if constexpr (EMBED) {
+                        const uint2 w = *(const uint2 *)(a.erow + (size_t)pc * 8);
+                        apv[q] = U4{w.x, w.y, 0u, 0u};
+                    } else {
+                        apv[q] = ((const U4 *)a.act)[pc];
+                    }
+                    if constexpr (NORM) nwv[q] = ((const U4 *)a.norm_w)[pc];
+                }
+            }
+        }
+    }
     Group ga;
-    if (g < groups) load_group(g, ga);  // in flight while the activation is staged
+    load_group(min(g, groups - 1), ga);  // in flight while the activation is staged
 
     {
-        const int npieces = K >> 3;
-        constexpr int NT = NORM ? kQaStageThreads : kQaThreads;  // thread t < NT owns the 8-element pieces t, t + NT, ..
-        constexpr int PMAX = (NC * 1024 / 8 + NT - 1) / NT;
         float f[PMAX][8];
-        U4 nwv[NORM ? PMAX : 1];
         float ss = 0.f;
         if (tid < NT) {
 #pragma unroll
@@ -125,17 +141,15 @@ __device__ __forceinline__ void qa_gemv(const QaGemv &a, float *act_lds, float *
                         raw = U4{(uint32_t)w0, (uint32_t)(w0 >> 32), (uint32_t)w1, (uint32_t)(w1 >> 32)};
                     } else {
                         if constexpr (EMBED) {
-                            const uint2 w = *(const uint2 *)(a.erow + (size_t)pc * 8);
-                            const uint32_t ww[2] = {w.x, w.y};
+                            const uint32_t ww[2] = {apv[q].x, apv[q].y};
                             uint32_t b[8];
 #pragma unroll
                             for (int i = 0; i < 8; i++) b[i] = qa_bits<T>((float)(int8_t)((ww[i >> 2] >> (8 * (i & 3))) & 0xFF) * a.escale);
                             raw = U4{b[0] | (b[1] << 16), b[2] | (b[3] << 16), b[4] | (b[5] << 16), b[6] | (b[7] << 16)};
                         } else {
-                            raw = ((const U4 *)a.act)[pc];
+                            raw = apv[q];
                         }
                     }
-                    if constexpr (NORM) nwv[q] = ((const U4 *)a.norm_w)[pc];
                     widen8<T>(raw, f[q]);
                     if constexpr (NORM) {
 #pragma unroll
@@ -208,56 +222,63 @@ __device__ __forceinline__ void qa_gemv(const QaGemv &a, float *act_lds, float *
         for (int r = 0; r < R; r++) acc[r] = wave_sum(acc[r]);
         const int row = g * R + lane;
         if (lane < R && row < N) {
-            float y = (lane == 0 ? acc[0] : acc[1]) * ga.sc;
-            if constexpr (RESID) Elem<T>::st((T *)a.out, row, Elem<T>::rnd(y) + ga.res);
+            float y = (lane == 0 ? acc[0] : acc[1]) * Elem<T>::ld(&ga.sc, 0);
+            if constexpr (RESID) {
+                const float res = EMBED ? Elem<T>::rnd((float)ga.eres * a.escale) : Elem<T>::ld(&ga.res, 0);
+                Elem<T>::st((T *)a.out, row, Elem<T>::rnd(y) + res);
+            }
             else qa_put16(a.out, row, qa_bits<T>(y));
         }
     }
 }
 
 // EMBED: the layer's input row is the embedding row of token *p.d_ids (first layer of a step)
+// What a workgroup's first loads need are leading scalar arguments (copies of the fields of p): they arrive
+// preloaded in SGPRs with the wave instead of through a scalar load from the kernarg segment.
 template <typename T, int D, int NC, bool EMBED>
-__global__ __launch_bounds__(kQaThreads, 2) void qkv_attention_kernel(QkvAttnParams p) {
+__global__ __launch_bounds__(kQaThreads, 2) void qkv_attention_kernel(const void *x, const void *norm_w, const int8_t *wq,
+                                                                          const int32_t *d_active, const int64_t *d_pos,
+                                                                          int gemv_blocks, int N, int K, int Hq, QkvAttnParams p) {
     extern __shared__ float act_lds[];  // [K], GEMV workgroups
     __shared__ float red[kQaStageThreads / 64];
     __shared__ float part_s[kShortWaves][D + 2];
     __shared__ __align__(16) T qkv_l[3 * D];
     const int tid = threadIdx.x;
-    const int QD = p.Hq * D;
+    const int QD = Hq * D;
 
     const int8_t *erow = nullptr;
     float escale = 0.f;
     if constexpr (EMBED) {
-        if ((int)blockIdx.x < p.gemv_blocks || (int)blockIdx.x >= p.gemv_blocks + p.Hq) {
+        if ((int)blockIdx.x < gemv_blocks || (int)blockIdx.x >= gemv_blocks + Hq) {
             int64_t tok = p.d_ids[0];
             if (tok < 0) tok += p.vocab;
-            erow = p.embed_w + (size_t)tok * p.K;
+            erow = p.embed_w + (size_t)tok * K;
             escale = Elem<T>::ld((const T *)p.embed_s, (size_t)tok);
         }
     }
-    if ((int)blockIdx.x < p.gemv_blocks) {
+    if ((int)blockIdx.x < gemv_blocks) {
         // ---- RMSNorm + q|k|v projection into the hand-over vector
-        const QaGemv a{p.x, p.norm_w, p.eps, p.wq, p.scale, nullptr, p.qkv, p.N, p.K, erow, escale};
-        qa_gemv<T, NC, true, false, false, EMBED>(a, act_lds, red, blockIdx.x, p.gemv_blocks, p.spin_limit, p.err);
+        const QaGemv a{x, norm_w, p.eps, wq, p.scale, nullptr, p.qkv, N, K, erow, escale};
+        qa_gemv<T, NC, true, false, false, EMBED>(a, act_lds, red, blockIdx.x, gemv_blocks, p.spin_limit, p.err);
         return;
     }
-    if ((int)blockIdx.x >= p.gemv_blocks + p.Hq) {
+    if ((int)blockIdx.x >= gemv_blocks + Hq) {
         // ---- o projection + residual: waits for the attention's output vector
-        const QaGemv a{p.attn_words, nullptr, 0.f, p.o_wq, p.o_scale, p.x, p.o_out, p.K, QD, erow, escale};
-        qa_gemv<T, NC, false, true, true, EMBED>(a, act_lds, red, blockIdx.x - p.gemv_blocks - p.Hq, p.o_blocks, p.spin_limit, p.err);
+        const QaGemv a{p.attn_words, nullptr, 0.f, p.o_wq, p.o_scale, x, p.o_out, K, QD, erow, escale};
+        qa_gemv<T, NC, false, true, true, EMBED>(a, act_lds, red, blockIdx.x - gemv_blocks - Hq, p.o_blocks, p.spin_limit, p.err);
         return;
     }
 
     // ---- attention: one workgroup per query head
-    const int h = blockIdx.x - p.gemv_blocks, Gt = p.Hq / p.Hkv, hkv = h / Gt;
-    const int active = *p.d_active;
-    const int64_t pos = *p.d_pos;
+    const int h = blockIdx.x - gemv_blocks, Gt = Hq / p.Hkv, hkv = h / Gt;
+    const int active = *d_active;
+    const int64_t pos = *d_pos;
     const size_t kv_base = (size_t)hkv * p.max_seq * D;
     constexpr int WPH = D / 4;  // 8-byte words per head slice
     auto ready = [&] {
         if (tid < 3 * WPH) {
             const int part = tid / WPH, w = tid % WPH;
-            const int head = part == 0 ? h : part == 1 ? p.Hq + hkv : p.Hq + p.Hkv + hkv;
+            const int head = part == 0 ? h : part == 1 ? Hq + hkv : Hq + p.Hkv + hkv;
             ((uint64_t *)qkv_l)[tid] = qa_wait(p.qkv + head * WPH + w, p.spin_limit, p.err);
         }
         __syncthreads();
@@ -308,8 +329,8 @@ int qkv_attention_launch(QkvAttnParams p, int D, int dtype, hipStream_t s) {
         using T = std::remove_pointer_t<decltype(t)>;
 #define MYNN_QA(D_, NC_)                                                                          \
     do {                                                                                          \
-        if (embed) MYNN_LAUNCH((qkv_attention_kernel<T, D_, NC_, true>), grid, block, lds, s, p);  \
-        else MYNN_LAUNCH((qkv_attention_kernel<T, D_, NC_, false>), grid, block, lds, s, p);       \
+        if (embed) MYNN_LAUNCH((qkv_attention_kernel<T, D_, NC_, true>), grid, block, lds, s, p.x, p.norm_w, p.wq, p.d_active, p.d_pos, p.gemv_blocks, p.N, p.K, p.Hq, p);  \
+        else MYNN_LAUNCH((qkv_attention_kernel<T, D_, NC_, false>), grid, block, lds, s, p.x, p.norm_w, p.wq, p.d_active, p.d_pos, p.gemv_blocks, p.N, p.K, p.Hq, p);       \
         return launch_status("qkv_attention_kernel");                                             \
     } while (0)
         if (D == 64) {
