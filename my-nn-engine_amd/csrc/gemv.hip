@@ -368,7 +368,7 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(const int8_
             }
         }
     };
-    bool loaded = true;
+    bool loaded = true;  // (requesting the next group into a second register set before these sums: measured, no gain)
     for (; g < groups; g += total_waves) {
         if (!loaded) load_group(g, ga);
         loaded = false;
@@ -388,13 +388,13 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(const int8_
 template <typename T, int R, int NC, int EPI, bool NORM, bool ARGMAX = false>
 static int launch_gemv1(const GemvParams &p, hipStream_t s) {
     const int groups = (p.N + R - 1) / R;
-    const int max_waves = 256 * 16;  // four resident waves per SIMD (measured best of 8/16/24/32 per CU)
+    const int max_waves = 256 * 16;  // four resident waves per SIMD (measured best of 8/12/16/20/24/32 per CU)
     const int passes = (groups + max_waves - 1) / max_waves;
     int waves = (groups + passes - 1) / passes;
     const int blocks = (waves + kGemvWaves - 1) / kGemvWaves;
     waves = blocks * kGemvWaves;
     MYNN_LAUNCH((dequant_gemv1_kernel<T, R, NC, EPI, NORM, ARGMAX>), dim3(blocks + (ARGMAX ? 1 : 0)), dim3(kGemvThreads),
-                       (size_t)p.K * sizeof(float), s, p.wq, p.act, p.scale, p.norm_w, p.residual, p.N, p.K, groups, waves, p);
+                (size_t)p.K * sizeof(float), s, p.wq, p.act, p.scale, p.norm_w, p.residual, p.N, p.K, groups, waves, p);
     return launch_status("dequant_gemv1_kernel");
 }
 
@@ -493,7 +493,9 @@ int dequant_gemv_dispatch(void *out, const void *act, const int8_t *wq, const vo
 template <typename T, int EPI, bool NORM>
 static int gemv1_dispatch(const GemvParams &p, hipStream_t s) {
     const int nc = (p.K + 1023) / 1024;
-    const bool wide = false;  // two rows per wave measured as fast or faster than four at every shape
+    // four rows per wave: faster for short rows (gate/up at K = 2048: 6.1 against 6.35 us), slower for long ones
+    // (down at K = 5632: 6.0 against 4.6 us, the wave holds 24 chunks per lane)
+    const bool wide = nc <= 2;
     if (!aligned16(p.act) || (NORM && !aligned16(p.norm_w)) || p.K % 8 != 0 || nc > 14) {
         if (wide) return launch_gemv<T, T, 4, 1, EPI, NORM>(p, s);  // the looping kernel
         return launch_gemv<T, T, 2, 1, EPI, NORM>(p, s);
