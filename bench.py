@@ -24,9 +24,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes per launch of the gate/up GEMV (TinyLlama shape, 16-bit activations) from rocprofv3
-# --pmc FETCH_SIZE (x2.000, scaled by a 256 MiB copy) + WRITE_SIZE (x1.000): 11420.5 KiB * 2 + 57.0 KiB.
+# --pmc FETCH_SIZE (x2.000, scaled by a 256 MiB copy) + WRITE_SIZE (x1.000): 11396.4 KiB * 2 + 35.0 KiB.
 # Counters cannot be read from inside this process; the figure is carried here from that profile run.
-GATEUP_GEMV_TRAFFIC_BYTES = 23447552
+GATEUP_GEMV_TRAFFIC_BYTES = 23375749
 # the same for the dominant kernels of the other workloads (profiles/prefill_and_batched_decode_pmc_hbm_traffic.md):
 # prefill gate/up GEMM + SwiGLU (f16, 8192 x 11264 x 2048): 287320.4 KiB * 2 + 90112.0 KiB;
 # batched-decode gate/up few-row GEMM (Llama-3-8B shape, 32 rows): 61689.4 KiB * 2 + 896.3 KiB
