@@ -541,7 +541,7 @@ int gemv_norm_argmax(void *out, const void *x, const void *norm_w, float eps, co
                  "gemv_norm_argmax: N=%d K=%d", N, K);
     const int nc = (K + 1023) / 1024;
     if (nc <= 1) return launch_gemv1<T, 2, 1, EPI_PLAIN, true, true>(p, s);
-    if (nc <= 2) return launch_gemv1<T, 2, 2, EPI_PLAIN, true, true>(p, s);
+    if (nc <= 2) return launch_gemv1<T, 4, 2, EPI_PLAIN, true, true>(p, s);  // (short rows: four per wave, as gemv1_dispatch)
     if (nc <= 4) return launch_gemv1<T, 2, 4, EPI_PLAIN, true, true>(p, s);
     if (nc <= 6) return launch_gemv1<T, 2, 6, EPI_PLAIN, true, true>(p, s);
     if (nc <= 8) return launch_gemv1<T, 2, 8, EPI_PLAIN, true, true>(p, s);
