@@ -82,6 +82,7 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
         if (base > 0) load_round(base);  // (a cache beyond one round: its loads are not overlapped with the round before)
         float sc[kShortPasses];
         float mr = -INFINITY;
+        const int i_new = new_row >= base ? (new_row - base) / KPP : -1;  // the pass of this round that meets the new row
 #pragma unroll
         for (int i = 0; i < kShortPasses; i++) {
             sc[i] = -INFINITY;
@@ -89,9 +90,9 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
             const int key = base + i * KPP + wave * GPW + grp;
             float kf[8];
             widen8<T>(kreg[i], kf);
-            if (key == new_row) {
+            if (i == i_new) {  // (uniform: only this pass can hold the new row, in one lane group)
 #pragma unroll
-                for (int e = 0; e < 8; e++) kf[e] = kn[e];
+                for (int e = 0; e < 8; e++) kf[e] = key == new_row ? kn[e] : kf[e];
             }
             float d = 0.f;
 #pragma unroll
@@ -112,9 +113,9 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
             const int key = base + i * KPP + wave * GPW + grp;
             float vf[8];
             widen8<T>(vreg[i], vf);
-            if (key == new_row) {
+            if (i == i_new) {
 #pragma unroll
-                for (int e = 0; e < 8; e++) vf[e] = vn[e];
+                for (int e = 0; e < 8; e++) vf[e] = key == new_row ? vn[e] : vf[e];
             }
             const float pe = fast_exp(sc[i] - mn);  // (no key: exp(-inf) = 0)
             l += pe;
@@ -135,9 +136,16 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
 #pragma unroll
     for (int off = LPK; off < 64; off <<= 1) {
         float o2[8];
-        const float m2 = __shfl_xor(m, off, 64), l2 = __shfl_xor(l, off, 64);
+        float m2, l2;
+        if (off == 8) {  // (lane ^ 8 sits in the same row of 16)
+            m2 = dpp_get<kDppRor8>(m), l2 = dpp_get<kDppRor8>(l);
 #pragma unroll
-        for (int e = 0; e < 8; e++) o2[e] = __shfl_xor(o[e], off, 64);
+            for (int e = 0; e < 8; e++) o2[e] = dpp_get<kDppRor8>(o[e]);
+        } else {
+            m2 = __shfl_xor(m, off, 64), l2 = __shfl_xor(l, off, 64);
+#pragma unroll
+            for (int e = 0; e < 8; e++) o2[e] = __shfl_xor(o[e], off, 64);
+        }
         merge(m2, l2, o2);
     }
     if (grp == 0) {

@@ -112,10 +112,26 @@ __device__ inline float wave_max(float v) {
     return v;
 }
 // sum over the lanes of an aligned group of `width` lanes (power of two <= 64)
+// (value of another lane of the same row of 16 through the data-parallel-primitive path: no LDS instruction, no wait)
+template <int CTRL> __device__ inline float dpp_get(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+constexpr int kDppXor1 = 0xB1, kDppXor2 = 0x4E;     // quad_perm [1,0,3,2] / [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141, kDppMirror = 0x140, kDppRor8 = 0x128;  // lane i <- 7-i (per 8) / 15-i / i^8
 template <int width> __device__ inline float group_sum(float v) {
+    if constexpr (width <= 16) {
+        // the same pairs as the xor butterfly: after the steps inside a quad every lane of a quad holds the quad's
+        // sum, so the mirrored lane of the other quad (half row) stands for lane ^ 4 (lane ^ 8)
+        if constexpr (width >= 2) v += dpp_get<kDppXor1>(v);
+        if constexpr (width >= 4) v += dpp_get<kDppXor2>(v);
+        if constexpr (width >= 8) v += dpp_get<kDppHalfMirror>(v);
+        if constexpr (width >= 16) v += dpp_get<kDppMirror>(v);
+        return v;
+    } else {
 #pragma unroll
-    for (int off = width / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
+        for (int off = width / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+        return v;
+    }
 }
 
 // greedy-token candidates: (value, index) ordered by value, then index -- of equal maxima the LATER one wins
