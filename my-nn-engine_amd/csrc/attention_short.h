@@ -8,8 +8,11 @@
 #pragma once
 #include "mynn_common.h"
 #include "mfma.h"
+#include <type_traits>
 
 namespace mynn {
+
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
 
 constexpr int kShortPasses = 8;  // keys per lane group held in registers at a time
 constexpr int kShortRounds = 4;  // rounds of kShortPasses passes: the cache may be 4 x 512 rows at D = 64, 4 x 256 at D = 128
@@ -67,9 +70,10 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
 #pragma unroll
         for (int e = 0; e < 8; e++) kn[e] = Elem<T>::rnd(d0 < half ? own[e] * c[e] - oth[e] * sn[e] : own[e] * c[e] + oth[e] * sn[e]);
     }
+    const U4 kn_packed = U4{pack2<T>(kn[0], kn[1]), pack2<T>(kn[2], kn[3]), pack2<T>(kn[4], kn[5]), pack2<T>(kn[6], kn[7])};
+    const U4 q_packed = U4{pack2<T>(q[0], q[1]), pack2<T>(q[2], q[3]), pack2<T>(q[4], q[5]), pack2<T>(q[6], q[7])};
     if (append && wave == 0 && grp == 0) {  // one lane group appends the new row
-        *(U4 *)(Kcache + (size_t)new_row * D + d0) =
-            U4{pack2<T>(kn[0], kn[1]), pack2<T>(kn[2], kn[3]), pack2<T>(kn[4], kn[5]), pack2<T>(kn[6], kn[7])};
+        *(U4 *)(Kcache + (size_t)new_row * D + d0) = kn_packed;
         *(U4 *)(Vcache + (size_t)new_row * D + d0) = v_new;
     }
 
@@ -88,15 +92,25 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
             sc[i] = -INFINITY;
             if (base + i * KPP >= bound) continue;  // no wave has keys in this pass
             const int key = base + i * KPP + wave * GPW + grp;
-            float kf[8];
-            widen8<T>(kreg[i], kf);
-            if (i == i_new) {  // (uniform: only this pass can hold the new row, in one lane group)
-#pragma unroll
-                for (int e = 0; e < 8; e++) kf[e] = key == new_row ? kn[e] : kf[e];
-            }
             float d = 0.f;
+            if constexpr (std::is_same_v<T, f16_t>) {
+                // fp16: query and key stay packed, two products per instruction with f32 accumulation
+                U4 kk = kreg[i];
+                if (i == i_new && key == new_row) kk = kn_packed;  // (i == i_new is uniform: only this pass can hold the new row)
+                const uint32_t kw[4] = {kk.x, kk.y, kk.z, kk.w}, qw[4] = {q_packed.x, q_packed.y, q_packed.z, q_packed.w};
 #pragma unroll
-            for (int e = 0; e < 8; e++) d = fmaf(q[e], kf[e], d);
+                for (int e = 0; e < 4; e++)
+                    d = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, qw[e]), __builtin_bit_cast(h2_t, kw[e]), d, false);
+            } else {
+                float kf[8];
+                widen8<T>(kreg[i], kf);
+                if (i == i_new) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) kf[e] = key == new_row ? kn[e] : kf[e];
+                }
+#pragma unroll
+                for (int e = 0; e < 8; e++) d = fmaf(q[e], kf[e], d);
+            }
             d = group_sum<LPK>(d) * scale;
             if (key < bound) sc[i] = d;
             mr = fmaxf(mr, sc[i]);
@@ -111,16 +125,25 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
         for (int i = 0; i < kShortPasses; i++) {
             if (base + i * KPP >= bound) continue;
             const int key = base + i * KPP + wave * GPW + grp;
-            float vf[8];
-            widen8<T>(vreg[i], vf);
-            if (i == i_new) {
-#pragma unroll
-                for (int e = 0; e < 8; e++) vf[e] = key == new_row ? vn[e] : vf[e];
-            }
             const float pe = fast_exp(sc[i] - mn);  // (no key: exp(-inf) = 0)
             l += pe;
+            U4 vv = vreg[i];
+            if (i == i_new && key == new_row) vv = v_new;
+            if constexpr (std::is_same_v<T, f16_t>) {
+                // (the widening of a half operand rides on the multiply-add: v_fma_mix_f32)
+                const uint32_t vw[4] = {vv.x, vv.y, vv.z, vv.w};
 #pragma unroll
-            for (int e = 0; e < 8; e++) o[e] = fmaf(pe, vf[e], o[e]);
+                for (int e = 0; e < 4; e++) {
+                    const h2_t hv = __builtin_bit_cast(h2_t, vw[e]);
+                    o[2 * e] = fmaf(pe, (float)hv[0], o[2 * e]);
+                    o[2 * e + 1] = fmaf(pe, (float)hv[1], o[2 * e + 1]);
+                }
+            } else {
+                float vf[8];
+                widen8<T>(vv, vf);
+#pragma unroll
+                for (int e = 0; e < 8; e++) o[e] = fmaf(pe, vf[e], o[e]);
+            }
         }
         m = mn;
     }
