@@ -63,12 +63,21 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
         float own[8], oth[8];
         widen8<T>(*(const U4 *)(qsrc + d0), own);
         widen8<T>(*(const U4 *)(qsrc + dp), oth);
+        // the first half of the dims subtracts the partner's product, the second adds it: the sign goes into the sine once
 #pragma unroll
-        for (int e = 0; e < 8; e++) q[e] = Elem<T>::rnd(d0 < half ? own[e] * c[e] - oth[e] * sn[e] : own[e] * c[e] + oth[e] * sn[e]);
-        widen8<T>(*(const U4 *)(ksrc + d0), own);
-        widen8<T>(*(const U4 *)(ksrc + dp), oth);
+        for (int e = 0; e < 8; e++) sn[e] = d0 < half ? -sn[e] : sn[e];
 #pragma unroll
-        for (int e = 0; e < 8; e++) kn[e] = Elem<T>::rnd(d0 < half ? own[e] * c[e] - oth[e] * sn[e] : own[e] * c[e] + oth[e] * sn[e]);
+        for (int e = 0; e < 8; e++) q[e] = Elem<T>::rnd(own[e] * c[e] + oth[e] * sn[e]);
+        // the rotated new key is needed where its row is met (one wave) and where it is appended
+        if (wave == (new_row % KPP) / GPW || (append && wave == 0)) {
+            widen8<T>(*(const U4 *)(ksrc + d0), own);
+            widen8<T>(*(const U4 *)(ksrc + dp), oth);
+#pragma unroll
+            for (int e = 0; e < 8; e++) kn[e] = Elem<T>::rnd(own[e] * c[e] + oth[e] * sn[e]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) kn[e] = 0.f;
+        }
     }
     const U4 kn_packed = U4{pack2<T>(kn[0], kn[1]), pack2<T>(kn[2], kn[3]), pack2<T>(kn[4], kn[5]), pack2<T>(kn[6], kn[7])};
     const U4 q_packed = U4{pack2<T>(q[0], q[1]), pack2<T>(q[2], q[3]), pack2<T>(q[4], q[5]), pack2<T>(q[6], q[7])};
