@@ -156,29 +156,24 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
         }
         m = mn;
     }
-    // ---- lane groups of the wave meet (lanes of equal dc), then the waves through LDS
-    auto merge = [&](float m2, float l2, const float *o2) {
-        const float mn = fmaxf(m, m2);
-        const float a = m == -INFINITY ? 0.f : fast_exp(m - mn), bb = m2 == -INFINITY ? 0.f : fast_exp(m2 - mn);
-        l = l * a + l2 * bb;
+    // ---- lane groups of the wave meet (lanes of equal dc), then the waves through LDS.  First the wave's maximum,
+    //      then every group rescales its (l, o) to it once, and the groups' values are plain sums.
+    auto other = [&](float v, int off) { return off == 8 ? dpp_get<kDppRor8>(v) : __shfl_xor(v, off, 64); };  // (lane ^ 8: same row of 16)
+    float mw = m;
 #pragma unroll
-        for (int e = 0; e < 8; e++) o[e] = o[e] * a + o2[e] * bb;
-        m = mn;
-    };
+    for (int off = LPK; off < 64; off <<= 1) mw = fmaxf(mw, other(mw, off));
+    {
+        const float a = m == -INFINITY ? 0.f : fast_exp(m - mw);  // (a wave without keys: everything stays 0, mw = -inf)
+        l *= a;
+#pragma unroll
+        for (int e = 0; e < 8; e++) o[e] *= a;
+        m = mw;
+    }
 #pragma unroll
     for (int off = LPK; off < 64; off <<= 1) {
-        float o2[8];
-        float m2, l2;
-        if (off == 8) {  // (lane ^ 8 sits in the same row of 16)
-            m2 = dpp_get<kDppRor8>(m), l2 = dpp_get<kDppRor8>(l);
+        l += other(l, off);
 #pragma unroll
-            for (int e = 0; e < 8; e++) o2[e] = dpp_get<kDppRor8>(o[e]);
-        } else {
-            m2 = __shfl_xor(m, off, 64), l2 = __shfl_xor(l, off, 64);
-#pragma unroll
-            for (int e = 0; e < 8; e++) o2[e] = __shfl_xor(o[e], off, 64);
-        }
-        merge(m2, l2, o2);
+        for (int e = 0; e < 8; e++) o[e] += other(o[e], off);
     }
     if (grp == 0) {
 #pragma unroll
