@@ -54,7 +54,8 @@ class ModelConfig(C.Structure):
     _fields_ = [("n_layers", _i), ("hidden", _i), ("n_heads", _i), ("n_kv_heads", _i), ("head_dim", _i),
                 ("ffn", _i), ("vocab", _i), ("max_seq", _i), ("eps", _f), ("rope_theta", _f), ("dtype", _i),
                 ("seq_q", _i), ("batch", _i), ("weights_int8", _i), ("quant_kv_cache", _i),
-                ("quantize_activations", _i)]
+                ("quantize_activations", _i), ("streaming_kv", _i), ("gemm_tile", _i), ("unfused_decode", _i),
+                ("handover_spin_limit", _i)]
 
 
 class KernelTime(C.Structure):
@@ -71,11 +72,17 @@ SIGNATURES = {
     "mynn_dequantize_linear": (_i, [_vp, _vp, _vp, _sz, _sz, _i, _vp]),
     "mynn_dequant_gemv": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mynn_dequant_matmul": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
-    "mynn_set_gemm_tile": (_i, [_i]),
-    "mynn_set_fuse_qkv_attention": (_i, [_i]),
+    "mynn_dequant_matmul_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
+    "mynn_dequant_matmul_ws": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _sz, _i, _vp]),
+    "mynn_dequant_weight_bytes": (_sz, [_i, _i]),
+    "mynn_dequant_weight_prepare": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "mynn_dequant_matmul_prepared": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "mynn_quantized_matmul": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mynn_dynamic_quantize_linear": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mynn_attention": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "mynn_attention_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i, _i, _i]),
+    "mynn_attention_ws": (_i, [_vp, _vp, _vp, _vp, _vp, C.c_long, C.c_long, _vp, _vp, _f, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i,
+                                _i, _vp, _sz, _vp]),
     "mynn_kvcache_update": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "mynn_kvcache_update_streaming": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "mynn_quantizing_kvcache_update_streaming": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
@@ -88,6 +95,7 @@ SIGNATURES = {
     "mynn_add": (_i, [_vp, _vp, _vp, _sz, _i, _vp]),
     "mynn_argmax_last": (_i, [_vp, _vp, _i, _i, _vp]),
     "mynn_model_configure": (_i, [C.POINTER(ModelConfig)]),
+    "mynn_model_create": (_vp, [C.POINTER(ModelConfig), C.POINTER(_vp), C.POINTER(_vp)]),
     "model_init": (_vp, [C.POINTER(_vp), C.POINTER(_vp)]),
     "model": (None, [_vp, C.POINTER(_vp), C.POINTER(_vp)]),
     "model_destroy": (None, [_vp]),
@@ -96,6 +104,9 @@ SIGNATURES = {
     "alloc_pinned": (_vp, [_sz]),
     "free_pinned": (None, [_vp]),
     "mynn_model_step": (_i, [_vp, _vp, _vp, _i64, _i64, _vp, _vp]),
+    "mynn_model_step_streaming": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp]),
+    "mynn_model_handover_failures": (_i, [_vp]),
+    "mynn_model_last_status": (_i, [_vp]),
     "mynn_model_argmax_row": (_i, [_vp, _i, C.POINTER(C.c_int32)]),
     "mynn_model_logits_device": (_vp, [_vp]),
     "mynn_model_stats": (_i, [_vp, C.POINTER(_sz), C.POINTER(_i), C.POINTER(_i)]),
@@ -120,6 +131,7 @@ SIGNATURES = {
     "mynn_llm_reset": (None, [_vp]),
     "mynn_llm_past_len": (_i64, [_vp]),
     "mynn_llm_set_past_len": (None, [_vp, _i64]),
+    "mynn_llm_set_streaming": (_i, [_vp, _i, _i]),
     "mynn_llm_generate_ids": (_i, [_vp, _vp, _sz, _sz, _vp]),
     "mynn_llm_create_with_step": (_vp, [STEP_FN, _vp, _i, _i64]),
 }
@@ -203,6 +215,40 @@ def dequant_matmul(act, wq, scale):
     return out
 
 
+def dequant_matmul_ws(act, wq, scale, gemm_tile=0):
+    """mynn_dequant_matmul_ws: the caller's workspace (a torch tensor here), optional forced GEMM tile."""
+    import torch
+
+    N, K = wq.shape
+    M = act.numel() // K
+    out = torch.empty(tuple(act.shape[:-1]) + (N,), dtype=scale.dtype, device=wq.device)
+    need = lib().mynn_dequant_matmul_workspace_bytes(M, N, K, _dt(act), _dt(scale))
+    ws = torch.empty((max(need, 16),), dtype=torch.uint8, device=wq.device)
+    check(lib().mynn_dequant_matmul_ws(_ptr(out), _ptr(act), _ptr(wq), _ptr(scale), M, N, K, _dt(act), _dt(scale), _ptr(ws), need,
+                                       int(gemm_tile), _stream()))
+    return out
+
+
+def dequant_weight_prepare(wq, scale):
+    """W dequantised once to the scale's type (mynn_dequant_weight_prepare); returns the opaque prepared buffer."""
+    import torch
+
+    N, K = wq.shape
+    wt = torch.empty((lib().mynn_dequant_weight_bytes(N, K),), dtype=torch.uint8, device=wq.device)
+    check(lib().mynn_dequant_weight_prepare(_ptr(wt), _ptr(wq), _ptr(scale), N, K, _dt(scale), _stream()))
+    return wt
+
+
+def dequant_matmul_prepared(act, wt, N, gemm_tile=0):
+    import torch
+
+    K = act.shape[-1]
+    M = act.numel() // K
+    out = torch.empty(tuple(act.shape[:-1]) + (N,), dtype=act.dtype, device=act.device)
+    check(lib().mynn_dequant_matmul_prepared(_ptr(out), _ptr(act), _ptr(wt), M, N, K, _dt(act), int(gemm_tile), _stream()))
+    return out
+
+
 def quantized_matmul(lhs, lhs_scale, rhs, rhs_scale, want_acc=True):
     import torch
 
@@ -242,6 +288,37 @@ def attention(q, k, v, scale, is_causal=False, active=None, d_active=None, q_pos
     check(lib().mynn_attention(_ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(k_scale), _ptr(v_scale), float(scale),
                                int(is_causal), B, Sq, int(active), _ptr(d_active), cache_len, int(q_pos_offset),
                                Hq, Hkv, D, _dt(q), int(k.dtype == torch.int8), _stream()))
+    return out
+
+
+def attention_ws(q, k, v, scale, is_causal=False, active=None, d_active=None, q_pos_offset=None, k_scale=None, v_scale=None,
+                 mask=None):
+    """mynn_attention_ws: caller-owned workspace, optional additive mask [..., Sq or 1, cache_len] broadcast over the
+    leading (batch x head) dimensions when they multiply to 1 (operator slot 3)."""
+    import torch
+
+    B, Hq, Sq, D = q.shape
+    Hkv, cache_len = k.shape[1], k.shape[2]
+    if active is None:
+        active = cache_len
+    if q_pos_offset is None:
+        q_pos_offset = 0 if Sq == cache_len else active - Sq
+    out = torch.empty_like(q)
+    kv8 = int(k.dtype == torch.int8)
+    need = lib().mynn_attention_workspace_bytes(B, Sq, cache_len, Hq, Hkv, D, _dt(q), kv8)
+    ws = torch.empty((max(need, 16),), dtype=torch.uint8, device=q.device)
+    m_os = m_rs = 0
+    if mask is not None:
+        # the strides the reference derives from the mask's dims (src/codegen/cuda.rs:1297-1323)
+        rows = mask.shape[-2] if mask.dim() >= 2 else 1
+        cols = mask.shape[-1]
+        assert cols == cache_len
+        outer = mask.numel() // (rows * cols)
+        m_rs = cols if rows > 1 else 0
+        m_os = rows * cols if outer > 1 else 0
+    check(lib().mynn_attention_ws(_ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(mask), m_os, m_rs, _ptr(k_scale), _ptr(v_scale),
+                                  float(scale), int(is_causal), B, Sq, int(active), _ptr(d_active), cache_len, int(q_pos_offset),
+                                  Hq, Hkv, D, _dt(q), kv8, _ptr(ws), need, _stream()))
     return out
 
 
@@ -428,7 +505,8 @@ class Decoder:
       prefill and a decode model can share them (PersistentBuffers in the reference).
     """
 
-    def __init__(self, cfg, weights, seq_q=1, batch=1, kv=None, quant_kv_cache=False, quantize_activations=False):
+    def __init__(self, cfg, weights, seq_q=1, batch=1, kv=None, quant_kv_cache=False, quantize_activations=False,
+                 streaming_kv=False, gemm_tile=0, unfused_decode=False, handover_spin_limit=0, reference_abi=False):
         import torch
 
         tdt = {F16: torch.float16, BF16: torch.bfloat16}[cfg["dtype"]]
@@ -436,7 +514,8 @@ class Decoder:
         quant = True if from_file else isinstance(weights["embed"], tuple)
         self.cfg = ModelConfig(cfg["n_layers"], cfg["hidden"], cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"],
                                cfg["ffn"], cfg["vocab"], cfg["max_seq"], float(cfg["eps"]), float(cfg["rope_theta"]),
-                               cfg["dtype"], seq_q, batch, int(quant), int(quant_kv_cache), int(quantize_activations))
+                               cfg["dtype"], seq_q, batch, int(quant), int(quant_kv_cache), int(quantize_activations),
+                               int(streaming_kv), int(gemm_tile), int(unfused_decode), int(handover_spin_limit))
         self.weights = weights  # keep the tensors alive
         if kv is None:
             shape = (batch, cfg["n_kv_heads"], cfg["max_seq"], cfg["head_dim"])
@@ -457,10 +536,7 @@ class Decoder:
             src = weights if isinstance(weights, Weights) else Weights(weights)
             self.weights = DeviceWeights(src, self.cfg)
             self.cfg.weights_int8 = int(self.weights.int8)
-            check(lib().mynn_model_configure(C.byref(self.cfg)))
-            self.handle = lib().model_init(self.weights.initializer, self._state)
-            if not self.handle:
-                raise MynnError("model_init failed: %s" % lib().mynn_last_error().decode())
+            self.handle = self._create(self.weights.initializer, reference_abi)
             return
         init = []
 
@@ -481,11 +557,20 @@ class Decoder:
         init.append(_ptr(weights["final_norm"]))
         lin(weights["lm_head"])
         self._init = (_vp * len(init))(*init)
-        check(lib().mynn_model_configure(C.byref(self.cfg)))
         torch.cuda.synchronize()
-        self.handle = lib().model_init(self._init, self._state)
-        if not self.handle:
+        self.handle = self._create(self._init, reference_abi)
+
+    def _create(self, init, reference_abi):
+        """reference_abi: mynn_model_configure + model_init (the symbols SessionCUDA binds) instead of the one call
+        that touches nothing process-wide."""
+        if reference_abi:
+            check(lib().mynn_model_configure(C.byref(self.cfg)))
+            handle = lib().model_init(init, self._state)
+        else:
+            handle = lib().mynn_model_create(C.byref(self.cfg), init, self._state)
+        if not handle:
             raise MynnError("model_init failed: %s" % lib().mynn_last_error().decode())
+        return handle
 
     def close(self):
         if getattr(self, "handle", None) and _lib is not None:
@@ -516,8 +601,26 @@ class Decoder:
                                     int(past_len), int(active), nxt, lp))
         return list(nxt), logits
 
-    def model(self, ids, positions, past_len, active):
-        """The reference ABI call `model(state, output, input)` with host pointers."""
+    def step_streaming(self, ids, positions, past_len, active, sink, window, start, kv_position, want_logits=False):
+        """One run of a streaming_kv model: the four ring inputs of the reference's streaming session."""
+        import numpy as np
+
+        ids = np.ascontiguousarray(np.asarray(ids, np.int64).ravel())
+        positions = np.ascontiguousarray(np.asarray(positions, np.int64).ravel())
+        kvp = np.ascontiguousarray(np.asarray(kv_position, np.int64).ravel())
+        assert ids.size == self.cfg.batch * self.cfg.seq_q and positions.size == self.cfg.seq_q and kvp.size == self.cfg.max_seq
+        nxt = (C.c_int32 * self.cfg.batch)()
+        logits, lp = None, None
+        if want_logits:
+            logits = np.empty((self.cfg.batch * self.cfg.seq_q, self.cfg.vocab), np.uint16)
+            lp = logits.ctypes.data_as(_vp)
+        check(lib().mynn_model_step_streaming(self.handle, ids.ctypes.data_as(_vp), positions.ctypes.data_as(_vp), int(past_len),
+                                              int(active), int(sink), int(window), int(start), kvp.ctypes.data_as(_vp), nxt, lp))
+        return list(nxt), logits
+
+    def model(self, ids, positions, past_len, active, ring=None):
+        """The reference ABI call `model(state, output, input)` with host pointers; ring = (sink, window, start,
+        kv_position) for a streaming_kv model.  Raises when the state's status after the void call is not 0."""
         import numpy as np
 
         ids = np.ascontiguousarray(np.asarray(ids, np.int64).ravel())
@@ -525,10 +628,21 @@ class Decoder:
         pl = np.array([past_len], np.int64)
         ac = np.array([active], np.int64)
         logits = np.empty((self.cfg.batch * self.cfg.seq_q, self.cfg.vocab), np.uint16)
-        inp = (_vp * 4)(ids.ctypes.data, positions.ctypes.data, pl.ctypes.data, ac.ctypes.data)
+        ptrs = [ids.ctypes.data, positions.ctypes.data, pl.ctypes.data, ac.ctypes.data]
+        keep = []
+        if ring is not None:
+            keep = [np.array([ring[0]], np.int64), np.array([ring[1]], np.int64), np.array([ring[2]], np.int64),
+                    np.ascontiguousarray(np.asarray(ring[3], np.int64))]
+            ptrs += [a.ctypes.data for a in keep]
+        inp = (_vp * len(ptrs))(*ptrs)
         out = (_vp * 1)(logits.ctypes.data)
         lib().model(self.handle, out, inp)
+        check(lib().mynn_model_last_status(self.handle))
         return logits
+
+    @property
+    def handover_failures(self):
+        return lib().mynn_model_handover_failures(self.handle)
 
     def decode_loop(self, token, past_len, n_steps):
         out = (C.c_int32 * n_steps)()
@@ -566,13 +680,16 @@ class Decoder:
 class LlmSession:
     """crates/llm LlmSession: decode model + optional prefill model over shared weights and KV."""
 
-    def __init__(self, decoder, prefill=None, eos=-1):
+    def __init__(self, decoder, prefill=None, eos=-1, streaming=None):
+        """streaming = (sink, window): DecodeKind::LlamaStreaming; the models must have been built with streaming_kv."""
         self.decoder, self.prefill = decoder, prefill
         pl = prefill.cfg.seq_q if prefill is not None else 0
         self.handle = lib().mynn_llm_create(decoder.handle, prefill.handle if prefill is not None else None, pl,
                                             decoder.cfg.max_seq, int(eos))
         if not self.handle:
             raise MynnError(lib().mynn_last_error().decode())
+        if streaming is not None:
+            check(lib().mynn_llm_set_streaming(self.handle, int(streaming[0]), int(streaming[1])))
 
     def close(self):
         if getattr(self, "handle", None) and _lib is not None:
@@ -606,19 +723,6 @@ class LlmSession:
         if n < 0:
             raise MynnError("generate_ids error %d: %s" % (n, lib().mynn_last_error().decode()))
         return [int(t) for t in out[:n]]
-
-
-def set_gemm_tile(which):
-    """Workgroup tile of the matrix-core GEMM: 0 = per-shape choice, 1 = 256x128, 2 = 256x256 with
-    operands staged through registers, 3 = 256x256 and 4 = 256x320 with operands loaded straight into LDS."""
-    check(lib().mynn_set_gemm_tile(int(which)))
-
-
-def set_fuse_qkv_attention(on):
-    """Batch-1 decode executors built after this call share launches between dependent ops (True, the default,
-    when the shape allows: q|k|v projection + attention + o projection of a layer, the embedding row, lm_head +
-    greedy token) or run every op as a launch of its own (False).  Same results bit for bit."""
-    check(lib().mynn_set_fuse_qkv_attention(1 if on else 0))
 
 
 def quantize_per_channel(w_f32, scale_dt):

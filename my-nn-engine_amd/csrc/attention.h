@@ -20,6 +20,10 @@ struct AttnParams {
     // K and V then are the caches the new row is appended to
     const void *qkv, *cos_t, *sin_t;
     const int64_t *d_pos;
+    // additive mask (operator slot 3), storage type: element (b * Hq + h) * mask_os + sq * mask_rs + key
+    const void *mask;
+    long mask_os, mask_rs;
+    const int32_t *d_past;    // fused decode form: cache row the new token is appended to (KVCacheUpdate's offset)
     float *part_o;            // [B*Hq*Sq, nsplit, D]
     float *part_ml;           // [B*Hq*Sq, nsplit, 2]
     // element strides of Q and out: batch, head, row.  Reference layout [B,Hq,Sq,D] is

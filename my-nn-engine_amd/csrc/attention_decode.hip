@@ -20,6 +20,9 @@
 // key bound); the matrix-core prefill kernel lives in attention_prefill.hip.
 #include <type_traits>
 
+#include <map>
+#include <mutex>
+
 #include "attention.h"
 #include "mfma.h"
 #include "attention_short.h"
@@ -70,7 +73,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
     const int k0 = split * nmax;
     const int k1 = min(bound, k0 + nmax);
     const int n = max(k1 - k0, 0);
-    const int new_row = FUSE ? active - 1 : -1;  // cache row of the token being decoded
+    const int new_row = FUSE ? *p.d_past : -1;  // cache row of the token being decoded (KVCacheUpdate's offset = past_len)
 
     TKV *v_s = (TKV *)smem;                                        // [nmax][D]
     float *sc = (float *)(smem + (size_t)nmax * D * sizeof(TKV));  // [G][nmax]
@@ -202,7 +205,12 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
                 for (int e = 0; e < EPL; e++) part = fmaf(q[g][e], kf[e], part);
                 part = group_sum<LPK>(part);
                 if constexpr (KVI8) part *= ksc;
-                if (dc == g % LPK) sc[(size_t)g * nmax + (key - k0)] = part * p.scale;
+                if (dc == g % LPK) {
+                    float val = part * p.scale;
+                    if (!FUSE && p.mask)
+                        val += Elem<T>::ld((const T *)p.mask, (size_t)(b * p.Hq + head0 + g) * p.mask_os + (size_t)sq * p.mask_rs + key);
+                    sc[(size_t)g * nmax + (key - k0)] = val;
+                }
             }
         }
     }
@@ -214,9 +222,10 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
         float m = -INFINITY;
         for (int k = lane; k < n; k += 64) m = fmaxf(m, row[k]);
         m = wave_max(m);
+        const float mm = m == -INFINITY ? 0.f : m;  // (every key masked out: all weights 0, not exp(-inf + inf))
         float l = 0.f;
         for (int k = lane; k < n; k += 64) {
-            const float e = fast_exp(row[k] - m);
+            const float e = fast_exp(row[k] - mm);
             l += e;
             row[k] = KVI8 ? e * vsc_s[k] : e;
         }
@@ -291,7 +300,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_short_kernel(AttnPar
     const size_t tab = (size_t)(*p.d_pos) * D;
     float r;
     if (attn_short_body<T, D>(row + (size_t)h * D, row + (size_t)(p.Hq + hkv) * D, row + (size_t)(p.Hq + p.Hkv + hkv) * D,
-                              (T *)p.k + kv_base * D, (T *)p.v + kv_base * D, bound, active - 1, h % Gt == 0,
+                              (T *)p.k + kv_base * D, (T *)p.v + kv_base * D, bound, *p.d_past, h % Gt == 0,
                               (const T *)p.cos_t + tab, (const T *)p.sin_t + tab, p.scale, part_s, tid, r, [] {}))
         Elem<T>::st((T *)p.out, (size_t)b * p.o_bs + (size_t)h * p.o_hs + tid, r);
 }
@@ -403,9 +412,11 @@ int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *s
         p.part_ml = p.part_o + rows * p.nsplit * D;
     }
     const bool fuse = p.qkv != nullptr;
+    MYNN_REQUIRE(!fuse || (p.d_past && p.d_pos && p.d_active && p.cos_t && p.sin_t), MYNN_ERR_INVALID,
+                 "fused decode attention: position, past_len and active length must be device scalars");
     // the plan (attn_plan, with the same kv_len) was made for the streaming kernel when it is eligible
     const int kv_len = p.d_active ? p.cache_len : (p.active < p.cache_len ? p.active : p.cache_len);
-    if (!fuse && attn_stream_eligible(p.B, p.Sq, p.Hq, p.Hkv, D, dtype, kv_int8, kv_len, p.cache_len))
+    if (!fuse && !p.mask && attn_stream_eligible(p.B, p.Sq, p.Hq, p.Hkv, D, dtype, kv_int8, kv_len, p.cache_len))
         return attention_stream_launch(p, D, dtype, kv_int8, s);
     bool whole = false;  // the launch wrote the finished output: nothing to merge whatever the plan's split count
     int rc = dispatch_dtype(dtype, [&](auto *t) {
@@ -430,14 +441,16 @@ int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *s
     return attention_merge_launch(p, D, dtype, s);
 }
 
-// ---- library-owned scratch for the op-level entry point: grown on demand
+// ---- library-owned scratch, grown on demand (the streaming-KV operators below; one set for all streams)
 struct Grown {
     void *ptr = nullptr;
     size_t bytes = 0;
 };
-static Grown g_scratch;
 static int ensure(Grown &g, size_t bytes, bool zero, hipStream_t s) {
     if (bytes <= g.bytes) return 0;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone)
+        return fail(MYNN_ERR_STATE, "the library's scratch memory cannot grow while the stream is being captured");
     MYNN_HIP(hipStreamSynchronize(s));
     if (g.ptr) MYNN_HIP(hipFree(g.ptr));
     g.ptr = nullptr;
@@ -447,15 +460,23 @@ static int ensure(Grown &g, size_t bytes, bool zero, hipStream_t s) {
     g.bytes = bytes;
     return 0;
 }
+// mynn_attention: the partial results of a cache split over workgroups, one block per stream
+static std::mutex g_scratch_mu;
+static std::map<hipStream_t, Grown> g_scratch;
 
-}  // namespace mynn
+enum { WS_LIBRARY = 0, WS_CALLER = 1 };
 
-using namespace mynn;
+// bytes of partial results the launch plan of this call needs (0: no key range is split)
+static size_t plan_scratch_bytes(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, int cache_len, bool masked) {
+    int slice = 0, nsplit = 1, hpw = 1;
+    attn_plan(B, Sq, Hq, Hkv, D, dtype, kv_int8, kv_len, cache_len, masked, &slice, &nsplit, &hpw);
+    return nsplit > 1 ? attn_scratch_bytes(B, Hq, Sq, D, nsplit) : 0;
+}
 
-extern "C" int mynn_attention(void *out, const void *Q, const void *K, const void *V, const void *k_scale,
-                              const void *v_scale, float scale, int is_causal, int B, int Sq, int active_seq_kv,
-                              const int32_t *d_active, int cache_seq_len, int q_pos_offset, int num_q_heads,
-                              int num_kv_heads, int head_dim, int dtype, int kv_int8, mynn_stream s) {
+static int attention_entry(void *out, const void *Q, const void *K, const void *V, const void *mask, long mask_os, long mask_rs,
+                           const void *k_scale, const void *v_scale, float scale, int is_causal, int B, int Sq, int active_seq_kv,
+                           const int32_t *d_active, int cache_seq_len, int q_pos_offset, int num_q_heads, int num_kv_heads,
+                           int head_dim, int dtype, int kv_int8, int ws_mode, void *workspace, size_t workspace_bytes, hipStream_t st) {
     MYNN_REQUIRE(out && Q && K && V, MYNN_ERR_INVALID, "attention: null operand");
     MYNN_REQUIRE(B > 0 && Sq > 0 && cache_seq_len > 0 && num_q_heads > 0 && num_kv_heads > 0, MYNN_ERR_INVALID,
                  "attention: B=%d Sq=%d cache=%d Hq=%d Hkv=%d", B, Sq, cache_seq_len, num_q_heads, num_kv_heads);
@@ -466,23 +487,67 @@ extern "C" int mynn_attention(void *out, const void *Q, const void *K, const voi
     MYNN_REQUIRE(aligned16(K) && aligned16(V), MYNN_ERR_INVALID, "attention: K and V must be 16-byte aligned");
     MYNN_REQUIRE(dtype_ok(dtype), MYNN_ERR_INVALID, "attention: dtype %d", dtype);
     MYNN_REQUIRE(Sq <= 65535, MYNN_ERR_UNSUPPORTED, "attention: Sq=%d too large for the per-row kernel", Sq);
+    MYNN_REQUIRE(!mask || (mask_os >= 0 && mask_rs >= 0), MYNN_ERR_INVALID, "attention: negative mask stride");
     AttnParams p{};
     p.out = out; p.q = Q; p.k = K; p.v = V; p.k_scale = k_scale; p.v_scale = v_scale; p.scale = scale;
     p.is_causal = is_causal; p.B = B; p.Sq = Sq; p.Hq = num_q_heads; p.Hkv = num_kv_heads;
     p.cache_len = cache_seq_len; p.active = active_seq_kv; p.d_active = d_active; p.q_pos_offset = q_pos_offset;
+    p.mask = mask; p.mask_os = mask_os; p.mask_rs = mask_rs;
     attn_reference_layout(p, head_dim);
-    hipStream_t st = as_stream(s);
-    if (Sq > 1 && attention_prefill_supported(p, head_dim, dtype, kv_int8))
+    if (!mask && Sq > 1 && attention_prefill_supported(p, head_dim, dtype, kv_int8))
         return attention_prefill_launch(p, head_dim, dtype, st);
     int kv_len = d_active ? cache_seq_len : (active_seq_kv < cache_seq_len ? active_seq_kv : cache_seq_len);
-    attn_plan(B, Sq, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, kv_len, cache_seq_len, false, &p.slice, &p.nsplit,
+    attn_plan(B, Sq, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, kv_len, cache_seq_len, mask != nullptr, &p.slice, &p.nsplit,
               &p.heads_per_wg);
     MYNN_REQUIRE(p.nsplit <= 65535, MYNN_ERR_UNSUPPORTED, "attention: cache of %d rows needs too many slices", kv_len);
+    void *scr = nullptr;
     if (p.nsplit > 1) {
-        int rc = ensure(g_scratch, attn_scratch_bytes(B, num_q_heads, Sq, head_dim, p.nsplit), false, st);
-        if (rc) return rc;
+        const size_t need = attn_scratch_bytes(B, num_q_heads, Sq, head_dim, p.nsplit);
+        if (ws_mode == WS_CALLER) {
+            MYNN_REQUIRE(workspace && aligned16(workspace) && workspace_bytes >= need, MYNN_ERR_INVALID,
+                         "attention: the workspace must hold %zu bytes (mynn_attention_workspace_bytes), 16-byte aligned", need);
+            scr = workspace;
+        } else {
+            std::lock_guard<std::mutex> lk(g_scratch_mu);
+            Grown &g = g_scratch[st];
+            int rc = ensure(g, need, false, st);
+            if (rc) return rc;
+            scr = g.ptr;
+        }
     }
-    return attention_decode_launch(p, head_dim, dtype, kv_int8, g_scratch.ptr, st);
+    return attention_decode_launch(p, head_dim, dtype, kv_int8, scr, st);
+}
+
+}  // namespace mynn
+
+using namespace mynn;
+
+extern "C" int mynn_attention(void *out, const void *Q, const void *K, const void *V, const void *k_scale,
+                              const void *v_scale, float scale, int is_causal, int B, int Sq, int active_seq_kv,
+                              const int32_t *d_active, int cache_seq_len, int q_pos_offset, int num_q_heads,
+                              int num_kv_heads, int head_dim, int dtype, int kv_int8, mynn_stream s) {
+    return attention_entry(out, Q, K, V, nullptr, 0, 0, k_scale, v_scale, scale, is_causal, B, Sq, active_seq_kv, d_active,
+                           cache_seq_len, q_pos_offset, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, WS_LIBRARY, nullptr, 0,
+                           as_stream(s));
+}
+
+extern "C" size_t mynn_attention_workspace_bytes(int B, int Sq, int cache_seq_len, int num_q_heads, int num_kv_heads, int head_dim,
+                                                 int dtype, int kv_int8) {
+    if (B <= 0 || Sq <= 0 || cache_seq_len <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads) return 0;
+    // the longest key range a call can have, with and without a mask (a mask keeps the call off the streaming kernel)
+    const size_t a = plan_scratch_bytes(B, Sq, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, cache_seq_len, cache_seq_len, false);
+    const size_t b = plan_scratch_bytes(B, Sq, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, cache_seq_len, cache_seq_len, true);
+    return a > b ? a : b;
+}
+
+extern "C" int mynn_attention_ws(void *out, const void *Q, const void *K, const void *V, const void *mask, long mask_outer_stride,
+                                 long mask_row_stride, const void *k_scale, const void *v_scale, float scale, int is_causal, int B,
+                                 int Sq, int active_seq_kv, const int32_t *d_active, int cache_seq_len, int q_pos_offset,
+                                 int num_q_heads, int num_kv_heads, int head_dim, int dtype, int kv_int8, void *workspace,
+                                 size_t workspace_bytes, mynn_stream s) {
+    return attention_entry(out, Q, K, V, mask, mask_outer_stride, mask_row_stride, k_scale, v_scale, scale, is_causal, B, Sq,
+                           active_seq_kv, d_active, cache_seq_len, q_pos_offset, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8,
+                           WS_CALLER, workspace, workspace_bytes, as_stream(s));
 }
 
 // ---- streaming KV (sink + ring cache): the slot map of the reference's kernels and the two operators that

@@ -10,6 +10,7 @@
 //   everything else (prefill rows, un-quantised checkpoints): op-by-op launches in the
 //     reference's order, with the reference's kernel choice per op.
 // One stream, one arena allocated at init; weights and KV buffers stay caller-owned.
+#include <algorithm>
 #include <cstdio>
 #include <cstring>
 #include <map>
@@ -40,6 +41,36 @@ __global__ void swiglu_rows_kernel(T *out, const T *gate, const T *up, size_t n)
     float g = Elem<T>::ld(gate, i);
     float sig = 1.0f / (1.0f + expf(-g));
     Elem<T>::st(out, i, (g * sig) * Elem<T>::ld(up, i));
+}
+
+// Streaming-KV graph (crates/llm/src/decoder.rs:281-347): q is rotated by the token's position, k and v leave
+// un-rotated, all three in the operators' [heads, S, D] layout.  qkv [S, (Hq + 2 Hkv) D] token-major.
+template <typename T>
+__global__ __launch_bounds__(64) void stream_split_kernel(T *q_ref, T *k_new, T *v_new, const T *qkv, const T *cos_t, const T *sin_t,
+                                                         const int64_t *position, int S, int Hq, int Hkv, int D) {
+    const int s = blockIdx.x, head = blockIdx.y, half = D / 2;
+    const T *src = qkv + ((size_t)s * (Hq + 2 * Hkv) + head) * D;
+    if (head < Hq) {
+        T *dst = q_ref + ((size_t)head * S + s) * D;
+        const size_t tab = (size_t)position[s] * D;
+        for (int j = threadIdx.x; j < half; j += blockDim.x) {
+            const float xl = Elem<T>::ld(src, j), xh = Elem<T>::ld(src, j + half);
+            Elem<T>::st(dst, j, xl * Elem<T>::ld(cos_t, tab + j) - xh * Elem<T>::ld(sin_t, tab + j));
+            Elem<T>::st(dst, j + half, xh * Elem<T>::ld(cos_t, tab + j + half) + xl * Elem<T>::ld(sin_t, tab + j + half));
+        }
+        return;
+    }
+    const bool is_k = head < Hq + Hkv;
+    T *dst = (is_k ? k_new : v_new) + ((size_t)(is_k ? head - Hq : head - Hq - Hkv) * S + s) * D;
+    for (int j = threadIdx.x; j < D; j += blockDim.x) dst[j] = src[j];
+}
+// [H, S, D] -> [S, H * D]
+template <typename T>
+__global__ void heads_to_tokens_kernel(T *out, const T *in, int H, int S, int D) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)H * S * D) return;
+    const int d = (int)(i % D), h = (int)((i / D) % H), s = (int)(i / ((size_t)D * H));
+    out[i] = in[((size_t)h * S + s) * D + d];
 }
 
 struct Lin {
@@ -105,6 +136,15 @@ struct Model {
     bool qkv_attn = false;
     bool lm_argmax = false;       // ... and the lm_head launch finds the greedy token and moves the loop state on
     uint64_t *lm_cand = nullptr;  // its candidate words (all ~0 between launches)
+    int spin_limit = 400000;      // polls a consumer role makes before it gives up and raises the error word
+    int handover_failures = 0;    // steps whose hand-over gave up; the executor then rebuilt itself with one op per launch
+    // streaming_kv: the ring inputs of the step in flight (host copies: the operators take them at launch time, as the
+    // reference's kernels do), kv_position on the device, and the operators' [heads, S, D] tensors
+    int ring_sink = 0, ring_window = 0, ring_start = 0, h_past = 0, h_active = 0;
+    int64_t *d_kvpos = nullptr;
+    void *q_ref = nullptr, *k_new = nullptr, *v_new = nullptr, *attn_ref = nullptr, *k_rot = nullptr;
+    int last_status = 0;          // of the last model() call on this state
+    void *ws = nullptr;           // executors that dequantise a weight per call (M >= 16, no resident copy): their own workspace
     // per-launch record of the last enqueue (names + algorithmic bytes), events when profiling
     std::vector<Launch> record;
     bool profiling = false;
@@ -113,8 +153,6 @@ struct Model {
 
 static mynn_model_config g_cfg{};
 static bool g_cfg_set = false;
-static int g_weights_quantized = 1;
-static int g_fuse_qkv_attention = 1;  // batch-1 decode executors built from now on share a launch between q|k|v and attention
 static std::mutex g_mu;
 
 static size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -152,7 +190,7 @@ static int gemm_rows(Model &m, void *out, const void *act, const void *wt, const
                      const char *name) {
     const double eb = 2.0, n_out = epi == GEMM_SWIGLU ? N / 2 : N;
     note(m, name, ((double)N * K + (double)M * K + (double)M * n_out * (epi == GEMM_RESIDUAL ? 2 : 1)) * eb, 2.0 * M * N * K);
-    return gemm_nt_mfma(out, act, wt, res, M, N, K, m.cfg.dtype, epi, m.stream);
+    return gemm_nt_mfma(out, act, wt, res, M, N, K, m.cfg.dtype, epi, m.stream, m.cfg.gemm_tile);
 }
 
 template <typename T>
@@ -161,10 +199,11 @@ static int linear_rows(Model &m, void *out, const void *act, const Lin &l, int M
     if (l.scale) {
         if (M >= 16 && l.K % 8 == 0) {
             // W_T = T(wq * scale) into the workspace, then the matrix-core product (two launches, two records)
+            MYNN_REQUIRE(m.ws, MYNN_ERR_STATE, "decoder: no weight workspace for %s", name);
             note(m, "dequant_weight", (double)l.N * l.K * (1 + eb) + l.N * eb);
-            TRY(dequant_weight_to_workspace((const int8_t *)l.w, l.scale, l.N, l.K, m.cfg.dtype, m.stream));
+            TRY(dequant_weight_rows(m.ws, (const int8_t *)l.w, l.scale, l.N, l.K, m.cfg.dtype, 0, 0, m.stream));
             note(m, name, ((double)l.N * l.K + (double)M * l.K + (double)M * l.N) * eb, 2.0 * M * l.N * l.K);
-            return gemm_from_workspace(out, act, M, l.N, l.K, m.cfg.dtype, m.stream);
+            return gemm_nt_mfma(out, act, m.ws, nullptr, M, l.N, l.K, m.cfg.dtype, GEMM_PLAIN, m.stream, m.cfg.gemm_tile);
         }
         note(m, name, (double)l.N * l.K + l.N * eb + (double)M * l.K * eb + (double)M * l.N * eb, 2.0 * M * l.N * l.K);
         return dequant_gemv_dispatch(out, act, (const int8_t *)l.w, l.scale, M, l.N, l.K, m.cfg.dtype, m.cfg.dtype,
@@ -219,6 +258,53 @@ static int qlinear_fused(Model &m, void *out, const void *act, const void *norm_
     return qgemm_dma(out, nullptr, m.a8, m.a8_scale, (const int8_t *)w, scale, res, M, N, K, m.cfg.dtype, epi, m.stream);
 }
 
+// The attention block of the streaming-KV graph, op for op (decoder.rs:281-347, 472-487): RoPE(q); k and v un-rotated
+// into the caches through the sink + ring slot map; 16-bit KV: Rope over the whole K cache by kv_position, then
+// Attention with the ring inputs; int8 KV: Attention rotates the dequantised keys itself (slots 10-12).
+template <typename T>
+static int streaming_attention(Model &m, Layer &L, float softmax_scale) {
+    const mynn_model_config &c = m.cfg;
+    const int S = c.seq_q, Hq = c.n_heads, Hkv = c.n_kv_heads, D = c.head_dim;
+    const double eb = sizeof(T);
+    hipStream_t s = m.stream;
+    note(m, "streaming_rope_q_split", (double)S * (Hq + 2 * Hkv) * D * 2 * eb);
+    MYNN_LAUNCH(stream_split_kernel<T>, dim3(S, Hq + 2 * Hkv), dim3(64), 0, s, (T *)m.q_ref, (T *)m.k_new, (T *)m.v_new,
+                (const T *)m.qkv, (const T *)m.cos_t, (const T *)m.sin_t, m.d_pos, S, Hq, Hkv, D);
+    TRY(launch_status("stream_split_kernel"));
+    void *attn_out = S == 1 ? m.attn : m.attn_ref;  // (one row: [heads, 1, D] is the token-major row)
+    if (c.quant_kv_cache) {
+        note(m, "quantizing_kvcache_update_streaming", (double)S * 2 * Hkv * D * (eb + 1));
+        TRY(mynn_quantizing_kvcache_update_streaming((int8_t *)L.k_cache, L.k_scale, m.k_new, m.h_past, Hkv, S, c.max_seq, D,
+                                                     m.ring_sink, m.ring_window, m.ring_start, c.dtype, s));
+        TRY(mynn_quantizing_kvcache_update_streaming((int8_t *)L.v_cache, L.v_scale, m.v_new, m.h_past, Hkv, S, c.max_seq, D,
+                                                     m.ring_sink, m.ring_window, m.ring_start, c.dtype, s));
+        note(m, "attention_streaming_rope", (double)S * 2.0 * Hq * D * eb);
+        TRY(mynn_attention_streaming(attn_out, m.q_ref, L.k_cache, L.v_cache, L.k_scale, L.v_scale, softmax_scale, S > 1, 1, S,
+                                     m.h_active, c.max_seq, m.h_active - S, Hq, Hkv, D, c.dtype, 1, m.ring_sink, m.ring_window,
+                                     m.ring_start, m.cos_t, m.sin_t, m.d_kvpos, s));
+    } else {
+        note(m, "kvcache_update_streaming", (double)S * 4 * Hkv * D * eb);
+        TRY(mynn_kvcache_update_streaming(L.k_cache, m.k_new, m.h_past, Hkv, S, c.max_seq, D, m.ring_sink, m.ring_window,
+                                          m.ring_start, c.dtype, s));
+        TRY(mynn_kvcache_update_streaming(L.v_cache, m.v_new, m.h_past, Hkv, S, c.max_seq, D, m.ring_sink, m.ring_window,
+                                          m.ring_start, c.dtype, s));
+        note(m, "rope_k_cache", 2.0 * Hkv * c.max_seq * D * eb);
+        TRY(mynn_rope(m.k_rot, L.k_cache, m.cos_t, m.sin_t, m.d_kvpos, Hkv, c.max_seq, D, c.dtype, s));
+        note(m, "attention_streaming", (double)S * 2.0 * Hq * D * eb);
+        TRY(mynn_attention_streaming(attn_out, m.q_ref, m.k_rot, L.v_cache, nullptr, nullptr, softmax_scale, S > 1, 1, S,
+                                     m.h_active, c.max_seq, m.h_active - S, Hq, Hkv, D, c.dtype, 0, m.ring_sink, m.ring_window,
+                                     m.ring_start, nullptr, nullptr, nullptr, s));
+    }
+    if (S > 1) {
+        const size_t n = (size_t)Hq * S * D;
+        note(m, "heads_to_tokens", 2.0 * n * eb);
+        MYNN_LAUNCH(heads_to_tokens_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (T *)m.attn, (const T *)m.attn_ref,
+                    Hq, S, D);
+        TRY(launch_status("heads_to_tokens_kernel"));
+    }
+    return 0;
+}
+
 template <typename T>
 static int enqueue_step(Model &m) {
     const mynn_model_config &c = m.cfg;
@@ -227,7 +313,8 @@ static int enqueue_step(Model &m) {
     const int QD = Hq * D, KD = Hkv * D;
     const double eb = sizeof(T);
     const bool w8a8 = c.quantize_activations != 0, kv8 = c.quant_kv_cache != 0;
-    const bool fused = m.quant && rows == 1 && !w8a8 && !kv8;
+    const bool streaming = c.streaming_kv != 0;
+    const bool fused = m.quant && rows == 1 && !w8a8 && !kv8 && !streaming;
     hipStream_t s = m.stream;
     m.record.clear();
     for (hipEvent_t e : m.events) hipEventDestroy(e);
@@ -255,8 +342,8 @@ static int enqueue_step(Model &m) {
             QkvAttnParams p{};
             p.x = m.x; p.norm_w = L.norm1; p.eps = c.eps; p.wq = (const int8_t *)L.qkv.w; p.scale = L.qkv.scale;
             p.N = L.qkv.N; p.K = H; p.qkv = (uint64_t *)m.qkv; p.out = m.attn; p.k_cache = L.k_cache; p.v_cache = L.v_cache;
-            p.cos_t = m.cos_t; p.sin_t = m.sin_t; p.d_pos = m.d_pos; p.d_active = m.d_active; p.Hq = Hq; p.Hkv = Hkv;
-            p.max_seq = c.max_seq; p.softmax_scale = softmax_scale; p.err = m.d_past + 3; p.spin_limit = 400000;
+            p.cos_t = m.cos_t; p.sin_t = m.sin_t; p.d_pos = m.d_pos; p.d_active = m.d_active; p.d_past = m.d_past; p.Hq = Hq; p.Hkv = Hkv;
+            p.max_seq = c.max_seq; p.softmax_scale = softmax_scale; p.err = m.d_past + 3; p.spin_limit = m.spin_limit;
             if (li == 0) {  // the input row of the first layer: the token's embedding
                 p.embed_w = (const int8_t *)m.embed.w; p.embed_s = m.embed.scale; p.d_ids = m.d_ids; p.vocab = V;
             }
@@ -278,13 +365,15 @@ static int enqueue_step(Model &m) {
                 // (16-bit KV cache) RoPE and both cache appends ride on the launch that sums the projection's K ranges
                 const SkinnyRope rp{m.q, L.k_cache, L.v_cache, m.cos_t, m.sin_t, m.d_pos, m.d_past, S, Hq, Hkv, D, c.max_seq};
                 TRY(skinny_rows(m, m.qkv, m.nrm, L.qkv, L.pk_qkv, nullptr, rows, GEMM_PLAIN, "linear_qkv", nullptr, nullptr,
-                                kv8 ? nullptr : &rp, &roped));
+                                kv8 || streaming ? nullptr : &rp, &roped));
             }
             else if (w8a8) TRY(linear_w8a8(m, m.qkv, m.nrm, L.qkv, rows, true, "qlinear_qkv"));
             else if (m.resident16) TRY(gemm_rows(m, m.qkv, m.nrm, L.wt_qkv, nullptr, rows, L.qkv.N, H, GEMM_PLAIN, "linear_qkv"));
             else TRY(linear_rows<T>(m, m.qkv, m.nrm, L.qkv, rows, "linear_qkv"));
         }
-        if (!(fused && m.qkv_attn)) {
+        if (streaming) {
+            TRY(streaming_attention<T>(m, L, softmax_scale));
+        } else if (!(fused && m.qkv_attn)) {
             AttnParams p{};
             p.out = m.attn; p.q = m.q; p.k = L.k_cache; p.v = L.v_cache; p.scale = softmax_scale;
             p.k_scale = L.k_scale; p.v_scale = L.v_scale;
@@ -294,7 +383,7 @@ static int enqueue_step(Model &m) {
             const bool fuse_attn = fused && attention_fused_supported(D, Hq / Hkv);
             if (fuse_attn) {
                 // RoPE(q), RoPE(k), both cache appends and the attention in one launch
-                p.qkv = m.qkv; p.cos_t = m.cos_t; p.sin_t = m.sin_t; p.d_pos = m.d_pos;
+                p.qkv = m.qkv; p.cos_t = m.cos_t; p.sin_t = m.sin_t; p.d_pos = m.d_pos; p.d_past = m.d_past;
                 note(m, "attention_rope_append", (double)(QD + 2 * KD) * eb + 2.0 * KD * eb + QD * eb);
                 TRY(attention_decode_launch(p, D, c.dtype, 0, m.attn_scratch, s));
             } else {
@@ -380,7 +469,7 @@ static int enqueue_step(Model &m) {
         note(m, "gemv_norm_lm_head_argmax", (double)V * H + V * eb + 2 * H * eb + V * eb);
         TRY(gemv_norm_argmax<T>(m.logits, m.x, m.final_norm, c.eps, (const int8_t *)m.lm_head.w, m.lm_head.scale, V, H, m.lm_cand,
                                 m.d_next, AdvanceState{m.d_ids, m.d_pos, m.d_past, m.d_active, m.d_tokens, m.d_step, m.token_cap},
-                                m.d_past + 3, 400000, s));
+                                m.d_past + 3, m.spin_limit, s));
         launch_timer() = LaunchTimer{};
         m.launches = (int)m.record.size();
         return 0;
@@ -443,6 +532,7 @@ static int interleave_rows(void **out, const void *a, const void *b, size_t rows
 }
 
 static int host_rope_tables(Model &m);
+static int capture_step(Model &m);
 
 static int build(Model &m, void **init, void **state) {
     const mynn_model_config &c = m.cfg;
@@ -542,6 +632,16 @@ static int build(Model &m, void **init, void **state) {
         m.resident16 = true;
     }
 
+    if (m.quant && !m.skinny && !m.resident16 && !c.quantize_activations && c.batch * c.seq_q >= 16) {
+        // a weight is dequantised per call: the executor's own workspace, sized for its largest linear (never shared
+        // with another model or stream, never grown afterwards)
+        size_t need = 0;
+        auto grow = [&](const Lin &l) { if (l.K % 8 == 0) need = std::max(need, gemm_weight_bytes(l.N, l.K)); };
+        for (Layer &L : m.layers) { grow(L.qkv); grow(L.o); grow(L.gate); grow(L.up); grow(L.down); }
+        grow(m.lm_head);
+        if (need) MYNN_HIP(hipMalloc(&m.ws, need));
+    }
+
     // ---- W8A8 prefill executors: every linear is large enough for the 256-row int8 tiles; gate and up become one
     // product whose store applies SwiGLU, so their rows (and scales) are interleaved in groups of 32 once
     {
@@ -593,6 +693,11 @@ static int build(Model &m, void **init, void **state) {
     size_t o_sc = plan.take(32 + (size_t)c.batch * 4), o_tok = plan.take((size_t)m.token_cap * 4);
     size_t o_as = plan.take(attn_scratch_bytes(c.batch, c.n_heads, c.seq_q, c.head_dim, m.nsplit));
     size_t o_cand = plan.take(rows == 1 ? (size_t)kGemvArgmaxWords * 8 : 0);
+    const bool strm = c.streaming_kv != 0;
+    size_t o_kvpos = plan.take(strm ? (size_t)c.max_seq * 8 : 0);
+    size_t o_qref = plan.take(strm ? (size_t)rows * QD * eb : 0), o_knew = plan.take(strm ? (size_t)rows * KD * eb : 0);
+    size_t o_vnew = plan.take(strm ? (size_t)rows * KD * eb : 0), o_aref = plan.take(strm ? (size_t)rows * QD * eb : 0);
+    size_t o_krot = plan.take(strm && !c.quant_kv_cache ? (size_t)KD * c.max_seq * eb : 0);
     m.arena_bytes = plan.off;
     MYNN_HIP(hipMalloc((void **)&m.arena, m.arena_bytes));
     MYNN_HIP(hipMemset(m.arena, 0, m.arena_bytes));
@@ -607,13 +712,18 @@ static int build(Model &m, void **init, void **state) {
     m.d_tokens = (int32_t *)(m.arena + o_tok);
     m.attn_scratch = m.arena + o_as;
     m.lm_cand = (uint64_t *)(m.arena + o_cand);
+    m.d_kvpos = (int64_t *)(m.arena + o_kvpos);
+    m.q_ref = m.arena + o_qref; m.k_new = m.arena + o_knew; m.v_new = m.arena + o_vnew; m.attn_ref = m.arena + o_aref;
+    m.k_rot = m.arena + o_krot;
     m.next_stage = align_up((size_t)c.batch * 4, 256);  // the sequences' next tokens live in the tail of the staging buffer
-    m.stage_bytes = align_up((size_t)rows * 8 + (size_t)c.seq_q * 8 + 64 + (size_t)m.token_cap * 4, 256) + 256 + m.next_stage;
+    m.stage_bytes = align_up((size_t)rows * 8 + (size_t)c.seq_q * 8 + 64 + (size_t)m.token_cap * 4 + (strm ? (size_t)c.max_seq * 8 : 0), 256) +
+                    256 + m.next_stage;
     MYNN_HIP(hipHostMalloc((void **)&m.h_stage, m.stage_bytes, hipHostMallocDefault));
     MYNN_HIP(hipDeviceSynchronize());
 
     // ---- batch-1 decode: projection and attention in one launch when the shape allows
-    if (m.quant && rows == 1 && !c.quantize_activations && !c.quant_kv_cache && g_fuse_qkv_attention &&
+    m.spin_limit = c.handover_spin_limit > 0 ? c.handover_spin_limit : c.handover_spin_limit < 0 ? 0 : 400000;
+    if (m.quant && rows == 1 && !c.quantize_activations && !c.quant_kv_cache && !c.unfused_decode &&
         attention_fused_supported(c.head_dim, c.n_heads / c.n_kv_heads) &&
         qkv_attention_supported(H, c.n_heads, c.n_kv_heads, c.head_dim, c.max_seq, c.dtype) && (QD + 2 * KD) * eb % 8 == 0) {
         bool ok = aligned16(m.qkv) && aligned16(m.x) && aligned16(m.attn) && aligned16(m.embed.w);
@@ -628,21 +738,29 @@ static int build(Model &m, void **init, void **state) {
         }
     }
 
-    // ---- capture the decode step once (one new token per sequence, any batch: every launch reads its
-    // positions and lengths from device memory)
-    if (c.seq_q == 1) {
-        hipError_t e = hipStreamBeginCapture(m.stream, hipStreamCaptureModeThreadLocal);
-        if (e == hipSuccess) {
-            int rc = enqueue(m);
-            hipError_t e2 = hipStreamEndCapture(m.stream, &m.graph);
-            if (rc == 0 && e2 == hipSuccess && hipGraphInstantiate(&m.graph_exec, m.graph, nullptr, nullptr, 0) == hipSuccess)
-                m.use_graph = true;
-            else {
-                (void)hipGetLastError();
-                if (rc) return rc;
-            }
-        } else (void)hipGetLastError();
-    }
+    return capture_step(m);
+}
+
+// Captures the decode step once (one new token per sequence, any batch: every launch reads its positions and
+// lengths from device memory).  Called again when the executor changes its launch plan.
+static int capture_step(Model &m) {
+    if (m.graph_exec) (void)hipGraphExecDestroy(m.graph_exec);
+    if (m.graph) (void)hipGraphDestroy(m.graph);
+    m.graph_exec = nullptr;
+    m.graph = nullptr;
+    m.use_graph = false;
+    if (m.cfg.seq_q != 1 || m.cfg.streaming_kv) return 0;  // (the streaming operators take host scalars at launch time)
+    hipError_t e = hipStreamBeginCapture(m.stream, hipStreamCaptureModeThreadLocal);
+    if (e == hipSuccess) {
+        int rc = enqueue(m);
+        hipError_t e2 = hipStreamEndCapture(m.stream, &m.graph);
+        if (rc == 0 && e2 == hipSuccess && hipGraphInstantiate(&m.graph_exec, m.graph, nullptr, nullptr, 0) == hipSuccess)
+            m.use_graph = true;
+        else {
+            (void)hipGetLastError();
+            if (rc) return rc;
+        }
+    } else (void)hipGetLastError();
     return 0;
 }
 
@@ -680,6 +798,7 @@ static void destroy(Model *m) {
         if (L.pk_gu) hipFree(L.pk_gu);
         if (L.pk_down) hipFree(L.pk_down);
     }
+    if (m->ws) hipFree(m->ws);
     if (m->wt_lm_head) hipFree(m->wt_lm_head);
     if (m->pk_lm_head) hipFree(m->pk_lm_head);
     if (m->cos_t) hipFree(m->cos_t);
@@ -709,20 +828,30 @@ static int upload_inputs(Model &m, const int64_t *ids, const int64_t *pos, int64
     memcpy(h_ids, ids, (size_t)rows * 8);
     memcpy(h_pos, pos, (size_t)c.seq_q * 8);
     h_sc[0] = (int32_t)past; h_sc[1] = (int32_t)active; h_sc[2] = 0;
+    m.h_past = (int)past;
+    m.h_active = (int)active;
     MYNN_HIP(hipMemcpyAsync(m.d_ids, h_ids, (size_t)rows * 8, hipMemcpyHostToDevice, m.stream));
     MYNN_HIP(hipMemcpyAsync(m.d_pos, h_pos, (size_t)c.seq_q * 8, hipMemcpyHostToDevice, m.stream));
     MYNN_HIP(hipMemcpyAsync(m.d_past, h_sc, 12, hipMemcpyHostToDevice, m.stream));
     return 0;
 }
 
-// fused projection + attention: a wait that ran out left the error word set (read back after the stream has
-// drained); the hand-over vector is emptied again so that the next step starts clean
-static int qkv_attention_failed(Model &m) {
+// A wait inside a fused launch ran out (the error word is set; read back after the stream has drained): the step's
+// results -- logits, token, loop state, the KV row it appended -- are undefined.  The executor empties the hand-over
+// vectors, gives up sharing launches for good (every op becomes a launch of its own: same arithmetic, bit-identical
+// results, no workgroup ever waits for another) and captures its step again; the caller then repeats the step from
+// its host-side inputs, which overwrites the KV row.
+static int handover_recover(Model &m) {
     const mynn_model_config &c = m.cfg;
-    (void)hipMemset(m.qkv, 0xFF, (size_t)((char *)m.attn + (size_t)c.n_heads * c.head_dim * dtype_size(c.dtype) - (char *)m.qkv));
-    (void)hipMemset(m.lm_cand, 0xFF, (size_t)kGemvArgmaxWords * 8);
-    (void)hipMemset(m.d_past + 3, 0, 4);
-    return fail(MYNN_ERR_STATE, "decode step: a stage of a fused launch waited too long for the stage before it (is the device shared?)");
+    MYNN_HIP(hipMemset(m.qkv, 0xFF, (size_t)((char *)m.attn + (size_t)c.n_heads * c.head_dim * dtype_size(c.dtype) - (char *)m.qkv)));
+    MYNN_HIP(hipMemset(m.lm_cand, 0xFF, (size_t)kGemvArgmaxWords * 8));
+    MYNN_HIP(hipMemset(m.d_past + 3, 0, 4));
+    m.handover_failures++;
+    m.qkv_attn = false;
+    m.lm_argmax = false;
+    set_error("decode step: a stage of a fused launch waited too long for the stage before it (is the device shared?); "
+              "the executor now runs one op per launch");
+    return capture_step(m);
 }
 
 static int run_once(Model &m) {
@@ -737,7 +866,7 @@ static int run_once(Model &m) {
 
 using namespace mynn;
 
-extern "C" int mynn_model_configure(const mynn_model_config *cfg) {
+static int check_config(const mynn_model_config *cfg) {
     MYNN_REQUIRE(cfg, MYNN_ERR_INVALID, "model_configure: null config");
     MYNN_REQUIRE(cfg->n_layers > 0 && cfg->hidden > 0 && cfg->n_heads > 0 && cfg->n_kv_heads > 0 && cfg->head_dim > 0 &&
                      cfg->ffn > 0 && cfg->vocab > 0 && cfg->max_seq > 0 && cfg->seq_q > 0 && cfg->batch > 0,
@@ -753,16 +882,38 @@ extern "C" int mynn_model_configure(const mynn_model_config *cfg) {
                  "model_configure: quant_kv_cache needs an even head_dim <= 128 (got %d)", cfg->head_dim);
     MYNN_REQUIRE(cfg->seq_q <= cfg->max_seq, MYNN_ERR_INVALID, "model_configure: prefill_len %d > max_seq %d", cfg->seq_q,
                  cfg->max_seq);
+    MYNN_REQUIRE(cfg->gemm_tile >= 0 && cfg->gemm_tile <= 4, MYNN_ERR_INVALID, "model_configure: gemm_tile %d (0..4)", cfg->gemm_tile);
+    MYNN_REQUIRE(!cfg->streaming_kv || (cfg->batch == 1 && cfg->head_dim % 2 == 0), MYNN_ERR_UNSUPPORTED,
+                 "model_configure: streaming_kv is a batch-1 graph (crates/llm) with an even head_dim");
+    return 0;
+}
+
+extern "C" int mynn_model_configure(const mynn_model_config *cfg) {
+    TRY(check_config(cfg));
     std::lock_guard<std::mutex> lk(g_mu);
     g_cfg = *cfg;
     g_cfg_set = true;
-    g_weights_quantized = cfg->weights_int8;
     return 0;
+}
+
+extern "C" void *mynn_model_create(const mynn_model_config *cfg, void **initializer, void **session_state) {
+    if (check_config(cfg)) return nullptr;
+    if (!initializer || !session_state) {
+        fail(MYNN_ERR_INVALID, "model_create: null initializer / session_state array");
+        return nullptr;
+    }
+    Model *m = new Model;
+    m->cfg = *cfg;
+    m->quant = cfg->weights_int8 != 0;
+    if (build(*m, initializer, session_state)) {
+        destroy(m);
+        return nullptr;
+    }
+    return m;
 }
 
 extern "C" void *model_init(void **initializer, void **session_state) {
     mynn_model_config cfg;
-    int quant;
     {
         std::lock_guard<std::mutex> lk(g_mu);
         if (!g_cfg_set) {
@@ -770,29 +921,11 @@ extern "C" void *model_init(void **initializer, void **session_state) {
             return nullptr;
         }
         cfg = g_cfg;
-        quant = g_weights_quantized;
     }
-    if (!initializer || !session_state) {
-        fail(MYNN_ERR_INVALID, "model_init: null initializer / session_state array");
-        return nullptr;
-    }
-    Model *m = new Model;
-    m->cfg = cfg;
-    m->quant = quant != 0;
-    int rc = build(*m, initializer, session_state);
-    if (rc) {
-        destroy(m);
-        return nullptr;
-    }
-    return m;
+    return mynn_model_create(&cfg, initializer, session_state);
 }
 
 extern "C" void model_destroy(void *state) { destroy((Model *)state); }
-extern "C" int mynn_set_fuse_qkv_attention(int on) {
-    std::lock_guard<std::mutex> lk(g_mu);
-    g_fuse_qkv_attention = on != 0;
-    return 0;
-}
 extern "C" void model_device_sync(void) { (void)hipDeviceSynchronize(); }
 extern "C" int model_memcpy(void *dst, const void *src, size_t n, int kind) {
     return (int)hipMemcpy(dst, src, n, (hipMemcpyKind)kind);
@@ -806,10 +939,10 @@ extern "C" void free_pinned(void *p) {
     if (p) (void)hipHostFree(p);
 }
 
-extern "C" int mynn_model_step(void *state, const int64_t *input_ids, const int64_t *position_id, int64_t past_len,
-                               int64_t active_seq_kv, int32_t *next_token, void *logits_host) {
-    MYNN_REQUIRE(state && input_ids && position_id, MYNN_ERR_INVALID, "model_step: null argument");
-    Model &m = *(Model *)state;
+// one step; *handover_failed is set when a fused launch gave up (results undefined, error word still set)
+static int step_once(Model &m, const int64_t *input_ids, const int64_t *position_id, int64_t past_len, int64_t active_seq_kv,
+                     int32_t *next_token, void *logits_host, bool *handover_failed) {
+    *handover_failed = false;
     TRY(upload_inputs(m, input_ids, position_id, past_len, active_seq_kv));
     TRY(run_once(m));
     const mynn_model_config &c = m.cfg;
@@ -822,7 +955,10 @@ extern "C" int mynn_model_step(void *state, const int64_t *input_ids, const int6
                                 hipMemcpyDeviceToHost, m.stream));
     MYNN_HIP(hipStreamSynchronize(m.stream));
     if (m.qkv_attn) {
-        if (*(const int32_t *)h_next) return qkv_attention_failed(m);
+        if (*(const int32_t *)h_next) {
+            *handover_failed = true;
+            return 0;
+        }
         if (next_token) memcpy(next_token, h_next + 20, 4);
         return 0;
     }
@@ -830,16 +966,71 @@ extern "C" int mynn_model_step(void *state, const int64_t *input_ids, const int6
     return 0;
 }
 
-// Reference ABI: void, host pointers, synchronous.  A failure is reported on stderr and through
-// mynn_last_error(); it never exits the process.
+extern "C" int mynn_model_step(void *state, const int64_t *input_ids, const int64_t *position_id, int64_t past_len,
+                               int64_t active_seq_kv, int32_t *next_token, void *logits_host) {
+    MYNN_REQUIRE(state && input_ids && position_id, MYNN_ERR_INVALID, "model_step: null argument");
+    Model &m = *(Model *)state;
+    MYNN_REQUIRE(!m.cfg.streaming_kv, MYNN_ERR_STATE, "model_step: a streaming_kv model takes the ring inputs (mynn_model_step_streaming)");
+    bool failed = false;
+    TRY(step_once(m, input_ids, position_id, past_len, active_seq_kv, next_token, logits_host, &failed));
+    if (!failed) return 0;
+    TRY(handover_recover(m));
+    TRY(step_once(m, input_ids, position_id, past_len, active_seq_kv, next_token, logits_host, &failed));
+    return failed ? fail(MYNN_ERR_STATE, "decode step: hand-over failure after recovery") : 0;
+}
+
+extern "C" int mynn_model_step_streaming(void *state, const int64_t *input_ids, const int64_t *position_id, int64_t past_len,
+                                         int64_t active_seq_kv, int64_t ring_sink, int64_t ring_window, int64_t ring_start,
+                                         const int64_t *kv_position, int32_t *next_token, void *logits_host) {
+    MYNN_REQUIRE(state && input_ids && position_id && kv_position, MYNN_ERR_INVALID, "model_step_streaming: null argument");
+    Model &m = *(Model *)state;
+    const mynn_model_config &c = m.cfg;
+    MYNN_REQUIRE(c.streaming_kv, MYNN_ERR_STATE, "model_step_streaming: the model was not built with streaming_kv");
+    MYNN_REQUIRE(ring_sink >= 0 && ring_window > 0 && ring_sink + ring_window <= c.max_seq && ring_start >= 0 && ring_start < ring_window,
+                 MYNN_ERR_INVALID, "model_step_streaming: ring sink=%lld window=%lld start=%lld (max_seq %d)", (long long)ring_sink,
+                 (long long)ring_window, (long long)ring_start, c.max_seq);
+    // Past sink + window the reference's session (session.rs:572-597) and its kernels' slot map (kvcache_update.cuh:21,
+    // common.cuh:55-60) disagree: the update maps the unbounded position through ring_start a second time, so every
+    // second ring slot is never overwritten again and the rank order the attention enumerates is not the token order.
+    // No fixture pins a value there; nothing is invented here.
+    MYNN_REQUIRE(past_len + c.seq_q <= ring_sink + ring_window, MYNN_ERR_UNSUPPORTED,
+                 "streaming_kv: past_len %lld + %d rows goes past sink + window = %lld, where the reference's session inputs and "
+                 "slot map are not consistent with each other", (long long)past_len, c.seq_q, (long long)(ring_sink + ring_window));
+    for (int r = 0; r < c.max_seq; r++)
+        MYNN_REQUIRE(kv_position[r] >= 0 && kv_position[r] < c.max_seq, MYNN_ERR_INVALID, "kv_position[%d]=%lld outside the RoPE table",
+                     r, (long long)kv_position[r]);
+    m.ring_sink = (int)ring_sink;
+    m.ring_window = (int)ring_window;
+    m.ring_start = (int)ring_start;
+    int64_t *h_kvpos = (int64_t *)(m.h_stage + align_up((size_t)c.batch * c.seq_q * 8 + (size_t)c.seq_q * 8 + 64 + (size_t)m.token_cap * 4, 8));
+    memcpy(h_kvpos, kv_position, (size_t)c.max_seq * 8);
+    MYNN_HIP(hipMemcpyAsync(m.d_kvpos, h_kvpos, (size_t)c.max_seq * 8, hipMemcpyHostToDevice, m.stream));
+    bool failed = false;
+    return step_once(m, input_ids, position_id, past_len, active_seq_kv, next_token, logits_host, &failed);
+}
+
+extern "C" int mynn_model_handover_failures(void *state) { return state ? ((Model *)state)->handover_failures : 0; }
+extern "C" int mynn_model_last_status(void *state) { return state ? ((Model *)state)->last_status : MYNN_ERR_INVALID; }
+
+// Reference ABI: void, host pointers, synchronous.  A failure is reported on stderr, through mynn_last_error()
+// and mynn_model_last_status(); it never exits the process.
 extern "C" void model(void *state, void **output, void **input) {
     if (!state || !output || !input) {
         fail(MYNN_ERR_INVALID, "model: null argument");
         fprintf(stderr, "mynn model(): %s\n", mynn_last_error());
+        if (state) ((Model *)state)->last_status = MYNN_ERR_INVALID;
         return;
     }
-    int rc = mynn_model_step(state, (const int64_t *)input[0], (const int64_t *)input[1], *(const int64_t *)input[2],
+    Model &m = *(Model *)state;
+    int rc;
+    if (m.cfg.streaming_kv)
+        rc = mynn_model_step_streaming(state, (const int64_t *)input[0], (const int64_t *)input[1], *(const int64_t *)input[2],
+                                       *(const int64_t *)input[3], *(const int64_t *)input[4], *(const int64_t *)input[5],
+                                       *(const int64_t *)input[6], (const int64_t *)input[7], nullptr, output[0]);
+    else
+        rc = mynn_model_step(state, (const int64_t *)input[0], (const int64_t *)input[1], *(const int64_t *)input[2],
                              *(const int64_t *)input[3], nullptr, output[0]);
+    m.last_status = rc;
     if (rc) fprintf(stderr, "mynn model(): error %d: %s\n", rc, mynn_last_error());
 }
 
@@ -871,19 +1062,27 @@ extern "C" int mynn_model_decode_loop(void *state, int32_t token, int64_t past_l
     MYNN_REQUIRE(state && out_tokens && n_steps > 0, MYNN_ERR_INVALID, "decode_loop: bad argument");
     Model &m = *(Model *)state;
     const mynn_model_config &c = m.cfg;
-    MYNN_REQUIRE(c.batch * c.seq_q == 1, MYNN_ERR_STATE, "decode_loop: needs a batch-1 decode model");
+    MYNN_REQUIRE(c.batch * c.seq_q == 1 && !c.streaming_kv, MYNN_ERR_STATE, "decode_loop: needs a batch-1 decode model without streaming_kv");
     MYNN_REQUIRE(past_len + n_steps <= c.max_seq && n_steps <= m.token_cap, MYNN_ERR_TOO_LONG,
                  "decode_loop: past_len %lld + %d steps exceeds max_seq %d", (long long)past_len, n_steps, c.max_seq);
-    int64_t id = token, pos = past_len;
-    TRY(upload_inputs(m, &id, &pos, past_len, past_len + 1));
-    for (int i = 0; i < n_steps; i++) TRY(run_once(m));
-    MYNN_HIP(hipMemcpyAsync(m.h_stage, m.d_tokens, (size_t)n_steps * 4, hipMemcpyDeviceToHost, m.stream));
-    char *h_err = m.h_stage + m.stage_bytes - m.next_stage;
-    if (m.qkv_attn) MYNN_HIP(hipMemcpyAsync(h_err, m.d_past + 3, 4, hipMemcpyDeviceToHost, m.stream));
-    MYNN_HIP(hipStreamSynchronize(m.stream));
-    if (m.qkv_attn && *(const int32_t *)h_err) return qkv_attention_failed(m);
-    memcpy(out_tokens, m.h_stage, (size_t)n_steps * 4);
-    return 0;
+    for (int attempt = 0; attempt < 2; attempt++) {
+        int64_t id = token, pos = past_len;
+        TRY(upload_inputs(m, &id, &pos, past_len, past_len + 1));
+        for (int i = 0; i < n_steps; i++) TRY(run_once(m));
+        MYNN_HIP(hipMemcpyAsync(m.h_stage, m.d_tokens, (size_t)n_steps * 4, hipMemcpyDeviceToHost, m.stream));
+        char *h_err = m.h_stage + m.stage_bytes - m.next_stage;
+        if (m.qkv_attn) MYNN_HIP(hipMemcpyAsync(h_err, m.d_past + 3, 4, hipMemcpyDeviceToHost, m.stream));
+        MYNN_HIP(hipStreamSynchronize(m.stream));
+        if (m.qkv_attn && *(const int32_t *)h_err) {
+            // some step's hand-over gave up: every later token is undefined.  Rebuild with one op per launch and run the
+            // whole loop again from the same inputs (the KV rows are overwritten).
+            TRY(handover_recover(m));
+            continue;
+        }
+        memcpy(out_tokens, m.h_stage, (size_t)n_steps * 4);
+        return 0;
+    }
+    return fail(MYNN_ERR_STATE, "decode loop: hand-over failure after recovery");
 }
 
 static int profile_enqueue(Model &m, mynn_kernel_time *out, int cap) {

@@ -14,6 +14,9 @@
 // or 256 x 256, K step 32, operands staged through registers into padded LDS tiles, any K % 8 == 0).
 // The store can add a residual (o_proj, down_proj) or apply SwiGLU to interleaved gate/up columns.
 // The int8 form of gemm_nt_dma_kernel is QuantizedMatMul for large grids (qgemm_dma).
+#include <map>
+#include <mutex>
+
 #include "kernels.h"
 #include "mfma.h"
 
@@ -454,10 +457,6 @@ __global__ __launch_bounds__(G::THREADS) void gemm_nt_dma_kernel(T *C, const voi
     }
 }
 
-// library-owned workspace for the dequantised weight of the call in flight (grown on demand)
-static void *g_ws = nullptr;
-static size_t g_ws_bytes = 0;
-
 static int gemm_kp(int K) { return (K + 2 * BK - 1) / (2 * BK) * (2 * BK); }  // the GEMM walks K in pairs of steps
 
 size_t gemm_weight_bytes(int N, int K) { return (size_t)N * gemm_kp(K) * 2; }
@@ -541,11 +540,10 @@ int qgemm_dma(void *out, int32_t *acc_out, const int8_t *lhs, const void *lhs_sc
     });
 }
 
-static int g_gemm_tile_override = 0;  // 0 = heuristic, 1 = 256x128, 2 = 256x256 via registers, 3 = 256x256 / 4 = 256x320 direct to LDS
-void gemm_set_tile(int which) { g_gemm_tile_override = which; }
-
+// tile: 0 = heuristic, 1 = 256x128, 2 = 256x256 via registers, 3 = 256x256 / 4 = 256x320 direct to LDS
 template <typename T, int EPI>
-static int gemm_launch(void *out, const void *act, const void *wt, const void *res, int M, int N, int K, hipStream_t s) {
+static int gemm_launch(void *out, const void *act, const void *wt, const void *res, int M, int N, int K, int tile, hipStream_t s) {
+    const int g_gemm_tile_override = tile;
     // the large tile needs fewer LDS reads per MFMA (measured 10-25% faster) but runs one workgroup per CU:
     // it is chosen once it fills the 256 CUs at least once (a partly filled second round still wins: the
     // CUs left running clock higher)
@@ -568,7 +566,9 @@ static int gemm_launch(void *out, const void *act, const void *wt, const void *r
 }
 
 int gemm_nt_mfma(void *out, const void *act, const void *wt, const void *res, int M, int N, int K, int dtype, int epi,
-                 hipStream_t s) {
+                 hipStream_t s, int tile) {
+    MYNN_REQUIRE(tile >= 0 && tile <= 4, MYNN_ERR_INVALID,
+                 "gemm tile %d is not 0 (automatic), 1 (256x128), 2 (256x256), 3 (256x256, direct-to-LDS loads) or 4 (256x320, direct-to-LDS loads)", tile);
     MYNN_REQUIRE(out && act && wt, MYNN_ERR_INVALID, "dequant_matmul: null operand");
     MYNN_REQUIRE(M > 0 && N > 0 && K > 0 && K % 8 == 0, MYNN_ERR_INVALID, "dequant_matmul: M=%d N=%d K=%d", M, N, K);
     MYNN_REQUIRE(aligned16(act) && aligned16(wt), MYNN_ERR_INVALID, "dequant_matmul: act must be 16-byte aligned");
@@ -576,54 +576,97 @@ int gemm_nt_mfma(void *out, const void *act, const void *wt, const void *res, in
     MYNN_REQUIRE(epi != GEMM_SWIGLU || N % 64 == 0, MYNN_ERR_INVALID, "dequant_matmul: SwiGLU store needs N %% 64 == 0, N=%d", N);
     return dispatch_dtype16(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
-        if (epi == GEMM_RESIDUAL) return gemm_launch<T, GEMM_RESIDUAL>(out, act, wt, res, M, N, K, s);
-        if (epi == GEMM_SWIGLU) return gemm_launch<T, GEMM_SWIGLU>(out, act, wt, res, M, N, K, s);
-        return gemm_launch<T, GEMM_PLAIN>(out, act, wt, res, M, N, K, s);
+        if (epi == GEMM_RESIDUAL) return gemm_launch<T, GEMM_RESIDUAL>(out, act, wt, res, M, N, K, tile, s);
+        if (epi == GEMM_SWIGLU) return gemm_launch<T, GEMM_SWIGLU>(out, act, wt, res, M, N, K, tile, s);
+        return gemm_launch<T, GEMM_PLAIN>(out, act, wt, res, M, N, K, tile, s);
     });
 }
 
-int dequant_weight_to_workspace(const int8_t *wq, const void *scale, int N, int K, int dtype, hipStream_t s) {
-    MYNN_REQUIRE(N > 0 && K > 0, MYNN_ERR_INVALID, "dequant_matmul: N=%d K=%d", N, K);
-    const size_t need = gemm_weight_bytes(N, K);
-    if (need > g_ws_bytes) {
+// ---- library-owned workspaces of the stand-alone entry point: one per stream, so calls on different streams never
+// share a dequantised weight; the table is guarded by a mutex.  A workspace only ever grows, and growing waits for
+// the stream's earlier work before the old block is released.
+struct StreamWs {
+    void *ptr = nullptr;
+    size_t bytes = 0;
+};
+static std::mutex g_ws_mu;
+static std::map<hipStream_t, StreamWs> g_ws;
+
+static int stream_workspace(hipStream_t s, size_t need, void **out) {
+    std::lock_guard<std::mutex> lk(g_ws_mu);
+    StreamWs &w = g_ws[s];
+    if (need > w.bytes) {
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone)
+            return fail(MYNN_ERR_STATE, "dequant_matmul: the library workspace cannot grow while the stream is being captured; "
+                                        "pass a workspace (mynn_dequant_matmul_ws) or a prepared weight");
         MYNN_HIP(hipStreamSynchronize(s));
-        if (g_ws) MYNN_HIP(hipFree(g_ws));
-        g_ws = nullptr;
-        g_ws_bytes = 0;
-        MYNN_HIP(hipMalloc(&g_ws, need));
-        g_ws_bytes = need;
+        if (w.ptr) MYNN_HIP(hipFree(w.ptr));
+        w = StreamWs{};
+        MYNN_HIP(hipMalloc(&w.ptr, need));
+        w.bytes = need;
     }
-    return dequant_weight_rows(g_ws, wq, scale, N, K, dtype, 0, 0, s);
+    *out = w.ptr;
+    return 0;
 }
 
-int gemm_from_workspace(void *out, const void *act, int M, int N, int K, int dtype, hipStream_t s) {
-    MYNN_REQUIRE(g_ws && g_ws_bytes >= gemm_weight_bytes(N, K), MYNN_ERR_STATE,
-                 "dequant_matmul: the workspace does not hold a [%d, %d] weight", N, K);
-    return gemm_nt_mfma(out, act, g_ws, nullptr, M, N, K, dtype, GEMM_PLAIN, s);
-}
-
-int dequant_gemm_mfma(void *out, const void *act, const int8_t *wq, const void *scale, int M, int N, int K,
-                      int dtype, hipStream_t s) {
-    int rc = dequant_weight_to_workspace(wq, scale, N, K, dtype, s);
+int dequant_gemm_mfma(void *out, const void *act, const int8_t *wq, const void *scale, int M, int N, int K, int dtype, void *ws,
+                      int tile, hipStream_t s) {
+    int rc = dequant_weight_rows(ws, wq, scale, N, K, dtype, 0, 0, s);
     if (rc) return rc;
-    return gemm_from_workspace(out, act, M, N, K, dtype, s);
+    return gemm_nt_mfma(out, act, ws, nullptr, M, N, K, dtype, GEMM_PLAIN, s, tile);
+}
+
+// the reference's kernel choice (cuda.rs:1518-1652): matrix cores for M >= 16 with 16-bit operands
+static bool takes_matrix_cores(const void *act, const int8_t *wq, int M, int K, int act_dtype, int out_dtype) {
+    const bool sixteen = act_dtype != MYNN_F32 && out_dtype != MYNN_F32 && act_dtype == out_dtype;
+    return M >= 16 && sixteen && K % 8 == 0 && aligned16(act) && ((uintptr_t)wq & 7) == 0;
 }
 
 }  // namespace mynn
 
-extern "C" int mynn_set_gemm_tile(int which) {
-    MYNN_REQUIRE(which >= 0 && which <= 4, MYNN_ERR_INVALID,
-                 "set_gemm_tile: %d is not 0 (automatic), 1 (256x128), 2 (256x256), 3 (256x256, direct-to-LDS loads) or 4 (256x320, direct-to-LDS loads)", which);
-    mynn::gemm_set_tile(which);
-    return 0;
+using namespace mynn;
+
+extern "C" size_t mynn_dequant_matmul_workspace_bytes(int M, int N, int K, int act_dtype, int out_dtype) {
+    if (M < 16 || N <= 0 || K <= 0 || K % 8 != 0 || act_dtype == MYNN_F32 || act_dtype != out_dtype) return 0;
+    return gemm_weight_bytes(N, K);
+}
+
+extern "C" int mynn_dequant_matmul_ws(void *out, const void *act, const int8_t *wq, const void *scale, int M, int N, int K,
+                                      int act_dtype, int out_dtype, void *workspace, size_t workspace_bytes, int gemm_tile,
+                                      mynn_stream s) {
+    MYNN_REQUIRE(M >= 1, MYNN_ERR_INVALID, "dequant_matmul: M=%d", M);
+    if (takes_matrix_cores(act, wq, M, K, act_dtype, out_dtype)) {
+        MYNN_REQUIRE(N > 0 && K > 0, MYNN_ERR_INVALID, "dequant_matmul: N=%d K=%d", N, K);
+        MYNN_REQUIRE(workspace && aligned16(workspace) && workspace_bytes >= gemm_weight_bytes(N, K), MYNN_ERR_INVALID,
+                     "dequant_matmul: the workspace must hold %zu bytes (mynn_dequant_matmul_workspace_bytes), 16-byte aligned",
+                     gemm_weight_bytes(N, K));
+        return dequant_gemm_mfma(out, act, wq, scale, M, N, K, out_dtype, workspace, gemm_tile, as_stream(s));
+    }
+    return dequant_gemv_dispatch(out, act, wq, scale, M, N, K, act_dtype, out_dtype, as_stream(s));
 }
 
 extern "C" int mynn_dequant_matmul(void *out, const void *act, const int8_t *wq, const void *scale, int M, int N,
                                    int K, int act_dtype, int out_dtype, mynn_stream s) {
-    using namespace mynn;
     MYNN_REQUIRE(M >= 1, MYNN_ERR_INVALID, "dequant_matmul: M=%d", M);
-    const bool sixteen = act_dtype != MYNN_F32 && out_dtype != MYNN_F32 && act_dtype == out_dtype;
-    if (M >= 16 && sixteen && K % 8 == 0 && aligned16(act) && ((uintptr_t)wq & 7) == 0)
-        return dequant_gemm_mfma(out, act, wq, scale, M, N, K, out_dtype, as_stream(s));
+    if (takes_matrix_cores(act, wq, M, K, act_dtype, out_dtype)) {
+        MYNN_REQUIRE(N > 0 && K > 0, MYNN_ERR_INVALID, "dequant_matmul: N=%d K=%d", N, K);
+        void *ws = nullptr;
+        int rc = stream_workspace(as_stream(s), gemm_weight_bytes(N, K), &ws);
+        if (rc) return rc;
+        return dequant_gemm_mfma(out, act, wq, scale, M, N, K, out_dtype, ws, 0, as_stream(s));
+    }
     return dequant_gemv_dispatch(out, act, wq, scale, M, N, K, act_dtype, out_dtype, as_stream(s));
+}
+
+extern "C" size_t mynn_dequant_weight_bytes(int N, int K) { return N > 0 && K > 0 ? gemm_weight_bytes(N, K) : 0; }
+
+extern "C" int mynn_dequant_weight_prepare(void *wt, const int8_t *wq, const void *scale, int N, int K, int dtype, mynn_stream s) {
+    return dequant_weight_rows(wt, wq, scale, N, K, dtype, 0, 0, as_stream(s));
+}
+
+extern "C" int mynn_dequant_matmul_prepared(void *out, const void *act, const void *wt, int M, int N, int K, int dtype,
+                                            int gemm_tile, mynn_stream s) {
+    MYNN_REQUIRE(M >= 16, MYNN_ERR_UNSUPPORTED, "dequant_matmul_prepared: M=%d (the prepared weight serves the matrix-core path, M >= 16)", M);
+    return gemm_nt_mfma(out, act, wt, nullptr, M, N, K, dtype, GEMM_PLAIN, as_stream(s), gemm_tile);
 }

@@ -58,14 +58,12 @@ int interleave_row_groups(void *dst, const void *src, size_t rows, size_t row_by
 bool qgemm_dma_supported(int M, int N, int K);
 int qgemm_dma(void *out, int32_t *acc_out, const int8_t *lhs, const void *lhs_scale, const int8_t *rhs, const void *rhs_scale,
               const void *res, int M, int N, int K, int dtype, int epi, hipStream_t s);
-void gemm_set_tile(int which);  // 0 heuristic; 1 = 256x128, 2 = 256x256 (register staged); 3 = 256x256, 4 = 256x320 (direct to LDS)
+// tile: 0 heuristic; 1 = 256x128, 2 = 256x256 (register staged); 3 = 256x256, 4 = 256x320 (direct to LDS)
 int gemm_nt_mfma(void *out, const void *act, const void *wt, const void *res, int M, int N, int K, int dtype, int epi,
-                 hipStream_t s);
-// the two halves of dequant_gemm_mfma: W_T = T(wq * scale) into the library workspace, then out = act . W_T^T
-int dequant_weight_to_workspace(const int8_t *wq, const void *scale, int N, int K, int dtype, hipStream_t s);
-int gemm_from_workspace(void *out, const void *act, int M, int N, int K, int dtype, hipStream_t s);
-int dequant_gemm_mfma(void *out, const void *act, const int8_t *wq, const void *scale, int M, int N, int K,
-                      int dtype, hipStream_t s);
+                 hipStream_t s, int tile = 0);
+// W_T = T(wq * scale) into `ws` (gemm_weight_bytes), then out = act . W_T^T
+int dequant_gemm_mfma(void *out, const void *act, const int8_t *wq, const void *scale, int M, int N, int K, int dtype, void *ws,
+                      int tile, hipStream_t s);
 
 // elementwise.hip
 // device-side loop state of a batch-1 decode model; a null `ids` means "no bookkeeping"
@@ -83,6 +81,7 @@ struct QkvAttnParams {
     const void *cos_t, *sin_t;
     const int64_t *d_pos;
     const int32_t *d_active;
+    const int32_t *d_past;   // the cache row the new token is appended to (KVCacheUpdate's offset)
     int Hq, Hkv, max_seq;
     float softmax_scale;
     int *err;                // set to 1 by a wait that ran out

@@ -1,6 +1,7 @@
 // Host side of crates/llm: the greedy generate loop of LlmSession (session.rs:311-537), the
 // per-output-channel int8 weight quantiser (quantize.rs:124-169) and the RoPE tables
 // (builder.rs:359-393).  Plain C++; nothing here touches the device except through the model ABI.
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 #include <vector>
@@ -71,7 +72,37 @@ struct mynn_llm {
     mynn_step_fn step = nullptr;
     void *user = nullptr;
     int last_error = 0;
+    bool streaming = false;  // DecodeKind::LlamaStreaming { sink, window }
+    int sink = 0, window = 0;
 };
+
+// streaming_kv_position (session.rs:604-635): the recency rank of every cache slot -- sink slots keep their position,
+// ring slots are walked in age order from ring_start, slots not written yet keep their own index
+static void streaming_kv_position(std::vector<int64_t> &out, int64_t sink, int64_t window, int64_t stream_pos) {
+    const int64_t max_active = sink + window;
+    const int64_t ring_start = stream_pos < max_active ? 0 : (stream_pos - sink) % window;
+    const int64_t in_ring = std::min<int64_t>(std::max<int64_t>(stream_pos - sink, 0), window);
+    for (int64_t slot = 0; slot < (int64_t)out.size(); slot++) {
+        int64_t v = slot;
+        if (slot >= sink && slot < max_active) {
+            const int64_t rel_age = (slot - sink + window - ring_start) % window;
+            if (rel_age < in_ring) v = sink + rel_age;
+        }
+        out[slot] = v;
+    }
+}
+
+extern "C" int mynn_llm_set_streaming(mynn_llm *l, int sink, int window) {
+    MYNN_REQUIRE(l && !l->step, MYNN_ERR_INVALID, "llm_set_streaming: needs a Llama session");
+    MYNN_REQUIRE(sink >= 0 && window > 0 && sink + window <= l->max_seq, MYNN_ERR_INVALID,
+                 "llm_set_streaming: sink %d + window %d must fit max_seq %d, window > 0", sink, window, l->max_seq);
+    MYNN_REQUIRE(!l->prefill || l->prefill_len <= window, MYNN_ERR_INVALID,
+                 "llm_set_streaming: prefill_len (%d) must be <= window (%d) in streaming KV mode", l->prefill_len, window);
+    l->streaming = true;
+    l->sink = sink;
+    l->window = window;
+    return 0;
+}
 
 extern "C" mynn_llm *mynn_llm_create(void *decode_state, void *prefill_state, int prefill_len, int max_seq,
                                      int64_t eos_token_id) {
@@ -111,7 +142,19 @@ static int decode_step(mynn_llm *l, int64_t token, int64_t *next) {
     } else {
         int32_t t = 0;
         int64_t pos = l->past_len;
-        int rc = mynn_model_step(l->decode, &token, &pos, l->past_len, l->past_len + 1, &t, nullptr);
+        int rc;
+        if (l->streaming) {
+            // streaming_decode_inputs (session.rs:571-597): past_len is the unbounded stream position
+            const int64_t max_active = l->sink + l->window, sp = l->past_len;
+            pos = std::min(sp, max_active - 1);
+            const int64_t ring_start = sp < max_active ? 0 : (sp - l->sink) % l->window;
+            std::vector<int64_t> kvpos((size_t)l->max_seq);
+            streaming_kv_position(kvpos, l->sink, l->window, sp);
+            rc = mynn_model_step_streaming(l->decode, &token, &pos, sp, std::min(sp + 1, max_active), l->sink, l->window, ring_start,
+                                           kvpos.data(), &t, nullptr);
+        } else {
+            rc = mynn_model_step(l->decode, &token, &pos, l->past_len, l->past_len + 1, &t, nullptr);
+        }
         if (rc) return rc;
         *next = t;
     }
@@ -134,14 +177,25 @@ static int run_prefill(mynn_llm *l, const int64_t *ids, size_t n, int64_t *next)
         // the token wanted is that of row chunk-1; the model reports the last row, so the final
         // (possibly padded) chunk reads its logits back
         const bool last = chunk == n;
-        if (last && chunk < P) {
-            // argmax of row chunk-1 on the device: run, then pick from the device logits
-            int rc = mynn_model_step(l->prefill, padded.data(), pos.data(), l->past_len, l->past_len + (int64_t)P, nullptr, nullptr);
-            if (rc) return rc;
-            rc = mynn_model_argmax_row(l->prefill, (int)(chunk - 1), &t);
-            if (rc) return rc;
+        const bool pick_row = last && chunk < P;
+        int rc;
+        if (l->streaming) {
+            // streaming_prefill_inputs (session.rs:539-569)
+            const int64_t max_active = l->sink + l->window, sp = l->past_len, after = sp + (int64_t)P;
+            for (size_t i = 0; i < P; i++) pos[i] = std::min(sp + (int64_t)i, max_active - 1);
+            const int64_t ring_start = after <= max_active ? 0 : (after - l->sink) % l->window;
+            std::vector<int64_t> kvpos((size_t)l->max_seq);
+            streaming_kv_position(kvpos, l->sink, l->window, after);
+            rc = mynn_model_step_streaming(l->prefill, padded.data(), pos.data(), sp, std::min(after, max_active), l->sink, l->window,
+                                           ring_start, kvpos.data(), pick_row ? nullptr : &t, nullptr);
         } else {
-            int rc = mynn_model_step(l->prefill, padded.data(), pos.data(), l->past_len, l->past_len + (int64_t)P, &t, nullptr);
+            rc = mynn_model_step(l->prefill, padded.data(), pos.data(), l->past_len, l->past_len + (int64_t)P, pick_row ? nullptr : &t,
+                                 nullptr);
+        }
+        if (rc) return rc;
+        if (pick_row) {
+            // argmax of row chunk-1 on the device, from the device logits
+            rc = mynn_model_argmax_row(l->prefill, (int)(chunk - 1), &t);
             if (rc) return rc;
         }
         l->past_len += (int64_t)chunk;
@@ -161,11 +215,11 @@ extern "C" int mynn_llm_generate_ids(mynn_llm *l, const int64_t *prompt_ids, siz
     const int64_t needed = prefill_runs
         ? l->past_len + (int64_t)((n_prompt + l->prefill_len - 1) / l->prefill_len * l->prefill_len)
         : l->past_len + (int64_t)n_prompt;
-    MYNN_REQUIRE(l->max_seq >= needed, MYNN_ERR_TOO_LONG, "prompt needs %lld cache rows, max_seq_len is %d (past_len %lld)",
+    MYNN_REQUIRE(l->streaming || l->max_seq >= needed, MYNN_ERR_TOO_LONG, "prompt needs %lld cache rows, max_seq_len is %d (past_len %lld)",
                  (long long)needed, l->max_seq, (long long)l->past_len);
     int n_new = 0;
     for (size_t i = 0; i < max_new_tokens; i++) {
-        if (l->max_seq < l->past_len + 1) break;
+        if (!l->streaming && l->max_seq < l->past_len + 1) break;
         int64_t tok = 0;
         int rc;
         if (i == 0) {

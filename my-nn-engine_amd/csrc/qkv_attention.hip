@@ -285,7 +285,7 @@ __global__ __launch_bounds__(kQaThreads, 2) void qkv_attention_kernel(const void
     };
     float r = 0.f;
     if (attn_short_body<T, D>(qkv_l, qkv_l + D, qkv_l + 2 * D, (T *)p.k_cache + kv_base, (T *)p.v_cache + kv_base,
-                              min(active, p.max_seq), active - 1, h % Gt == 0, (const T *)p.cos_t + pos * D,
+                              min(active, p.max_seq), *p.d_past, h % Gt == 0, (const T *)p.cos_t + pos * D,
                               (const T *)p.sin_t + pos * D, p.softmax_scale, part_s, tid, r, ready)) {
         if (p.o_blocks) qa_put16(p.attn_words, h * D + tid, qa_bits<T>(r));
         else Elem<T>::st((T *)p.out, (size_t)h * D + tid, r);

@@ -37,7 +37,8 @@ def test_attention_golden(g, name, causal, scale, active_slot):
 
 
 @pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
-@pytest.mark.parametrize("B,L", [(1, 512), (4, 2048), (16, 512), (2, 4096), (1, 37), (3, 1)])
+@pytest.mark.parametrize("B,L", [(1, 512), (4, 2048), (16, 512), (2, 4096), (1, 37), (3, 1), (1, 2048), (1, 4096), (4, 512),
+                                 (4, 4096), (16, 2048), (16, 4096)])
 def test_decode_attention_vs_oracle_cfg2_shapes(g, dt, B, L):
     """GQA decode attention op of the second benchmark config: 32 query heads, 4 KV heads,
     head_dim 64, softmax scale 1/8, no mask beyond the cache length."""

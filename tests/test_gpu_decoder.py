@@ -45,7 +45,7 @@ def test_tiny_llama_random_golden_ids_on_gpu(g, dt):
 def test_int8_decoder_step_logits_and_kv_vs_oracle(g, dt):
     cfg, w = llm_weights.synthetic_int8(SMALL, dt, seed=7)
     ref = orc.Model(cfg, w)
-    dec = g.mynn.Decoder(cfg, dev_weights(g, w, dt))
+    dec = g.mynn.Decoder(cfg, dev_weights(g, w, dt), reference_abi=True)  # mynn_model_configure + model_init
     st = dec.stats()
     assert st["graph"], "the decode step must replay a captured hipGraph"
     assert st["launches_per_step"] <= 2 + 6 * cfg["n_layers"] + 3
@@ -157,10 +157,8 @@ def test_generate_bookkeeping_and_errors(g):
 
 
 @pytest.fixture(params=[0, 1, 2, 3, 4], ids=["tile_auto", "tile_256x128", "tile_256x256", "tile_256x256_direct_lds", "tile_256x320_direct_lds"])
-def gemm_tile(g, request):
-    g.mynn.set_gemm_tile(request.param)
-    yield request.param
-    g.mynn.set_gemm_tile(0)
+def gemm_tile(request):
+    return request.param
 
 
 @pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
@@ -172,7 +170,7 @@ def test_prefill_model_logits_and_kv_vs_oracle(g, dt, P, gemm_tile):
     cfg, w = llm_weights.synthetic_int8(SMALL, dt, seed=21)
     ref = orc.Model(cfg, w)
     ref.set_gemm_mode(2)  # the CUDA backend's kernel choice, which the HIP path reproduces
-    dec = g.mynn.Decoder(cfg, dev_weights(g, w, dt), seq_q=P)
+    dec = g.mynn.Decoder(cfg, dev_weights(g, w, dt), seq_q=P, gemm_tile=gemm_tile)
     rng = np.random.default_rng(P)
     past = 0
     for chunk in range(2):

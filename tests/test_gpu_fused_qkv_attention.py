@@ -21,11 +21,7 @@ def g():
 
 def pair(g, cfg, weights):
     """(fused executor, two-launch executor) over the same weights, each with its own KV cache"""
-    g.mynn.set_fuse_qkv_attention(False)
-    try:
-        two = g.mynn.Decoder(cfg, weights)
-    finally:
-        g.mynn.set_fuse_qkv_attention(True)
+    two = g.mynn.Decoder(cfg, weights, unfused_decode=True)
     one = g.mynn.Decoder(cfg, weights)
     assert one.stats()["graph"] and two.stats()["graph"]
     assert one.stats()["launches_per_step"] == two.stats()["launches_per_step"] - 2 * cfg["n_layers"] - 2

@@ -94,13 +94,13 @@ def test_dequant_matmul_every_workgroup_tile(g, dt, M, N, K, tile):
     W = rng.integers(-127, 128, (N, K)).astype(np.int8)
     sc = orc.to_storage(rng.uniform(1e-3, 1e-2, N), dt)
     want = orc.dequant_matmul(act, W, sc, dt, dt, mode=2)
-    g.mynn.set_gemm_tile(tile)
-    try:
-        got = g.to_host(g.mynn.dequant_matmul(g.to_dev(act, dt), g.to_dev(W), g.to_dev(sc, dt)))
-    finally:
-        g.mynn.set_gemm_tile(0)
+    da, dw, ds = g.to_dev(act, dt), g.to_dev(W), g.to_dev(sc, dt)
+    got = g.to_host(g.mynn.dequant_matmul_ws(da, dw, ds, gemm_tile=tile))
     assert max_abs_rel(g.f32(got, dt), g.f32(want, dt)) <= 1e-2
     assert np.mean(got == want) > 0.97
+    # prepare once / multiply many gives the values of the per-call dequantisation
+    wt = g.mynn.dequant_weight_prepare(dw, ds)
+    assert np.array_equal(g.to_host(g.mynn.dequant_matmul_prepared(da, wt, N, gemm_tile=tile)), got)
 
 
 def test_dequant_matmul_linearity_at_prefill_size(g):

@@ -187,7 +187,7 @@ def test_dequantize_linear_golden(g):
     assert np.array_equal(got, y.array)
 
 
-@pytest.mark.parametrize("name", ["gather_negative_indices"])
+@pytest.mark.parametrize("name", ["gather_default_axis", "gather_negative_indices"])
 def test_gather_golden(g, name):
     import torch
 
@@ -223,6 +223,21 @@ def test_dynquant_golden(g, name, sym):
     assert np.array_equal(g.to_host(gz), zp.array)
     ok, md = close_either(g.f32(g.to_host(gs), orc.BF16), s.f32(), 1e-3)
     assert ok, md
+
+
+@pytest.mark.parametrize("name,sym", [("dyn_quantize_linear_sym_per_tensor", True), ("dyn_quantize_linear_asym_per_tensor", False)])
+def test_dynquant_per_tensor_golden(g, name, sym):
+    """The per-tensor fixtures: one quantisation slice over the whole tensor (axis_dim 1)."""
+    (x,), (y, s, zp) = case(name)
+    flat = g.to_dev(x.array.reshape(1, -1), orc.BF16)
+    gy, gs, gz = g.mynn.dynamic_quantize_linear(flat, symmetric=sym)
+    assert np.array_equal(g.to_host(gy).reshape(y.array.shape), y.array)
+    assert int(g.to_host(gz)[0]) == int(np.asarray(zp.array).reshape(-1)[0])
+    ok, md = close_either(g.f32(g.to_host(gs), orc.BF16), s.f32().reshape(1), 1e-3)
+    assert ok, md
+    if sym:
+        wy, ws = orc.dynquant_i8_per_tensor(x.array, orc.BF16)
+        assert np.array_equal(g.to_host(gy).reshape(wy.shape), wy) and np.array_equal(g.to_host(gs).reshape(-1), np.asarray(ws).reshape(-1))
 
 
 @pytest.mark.parametrize("dt", DT)
