@@ -80,6 +80,7 @@ SIGNATURES = {
     "mynn_quantized_matmul": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mynn_dynamic_quantize_linear": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mynn_attention": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "mynn_attention_noalloc": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "mynn_attention_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i, _i, _i]),
     "mynn_attention_ws": (_i, [_vp, _vp, _vp, _vp, _vp, C.c_long, C.c_long, _vp, _vp, _f, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i,
                                 _i, _vp, _sz, _vp]),
@@ -288,6 +289,23 @@ def attention(q, k, v, scale, is_causal=False, active=None, d_active=None, q_pos
     check(lib().mynn_attention(_ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(k_scale), _ptr(v_scale), float(scale),
                                int(is_causal), B, Sq, int(active), _ptr(d_active), cache_len, int(q_pos_offset),
                                Hq, Hkv, D, _dt(q), int(k.dtype == torch.int8), _stream()))
+    return out
+
+
+def attention_noalloc(q, k, v, scale, out, is_causal=False, active=None, d_active=None, q_pos_offset=None, k_scale=None,
+                      v_scale=None):
+    """mynn_attention_noalloc: the caller passes `out`; nothing is allocated on the way (not by this wrapper either)."""
+    import torch
+
+    B, Hq, Sq, D = q.shape
+    Hkv, cache_len = k.shape[1], k.shape[2]
+    if active is None:
+        active = cache_len
+    if q_pos_offset is None:
+        q_pos_offset = 0 if Sq == cache_len else active - Sq
+    check(lib().mynn_attention_noalloc(_ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(k_scale), _ptr(v_scale), float(scale),
+                                       int(is_causal), B, Sq, int(active), _ptr(d_active), cache_len, int(q_pos_offset),
+                                       Hq, Hkv, D, _dt(q), int(k.dtype == torch.int8), _stream()))
     return out
 
 

@@ -464,7 +464,29 @@ static int ensure(Grown &g, size_t bytes, bool zero, hipStream_t s) {
 static std::mutex g_scratch_mu;
 static std::map<hipStream_t, Grown> g_scratch;
 
-enum { WS_LIBRARY = 0, WS_CALLER = 1 };
+// mynn_attention_noalloc: the same partial results in a device array of the library (one copy per GPU, held until the
+// process ends).  The array's name is only a handle on the host: the address kernels get is asked for once per device.
+constexpr size_t kStaticScratchBytes = 8u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+static void *g_static_ptr[kMaxDevices] = {};
+static std::mutex g_static_mu;
+static int static_scratch(void **out) {
+    int dev = 0;
+    MYNN_HIP(hipGetDevice(&dev));
+    MYNN_REQUIRE(dev >= 0 && dev < kMaxDevices, MYNN_ERR_UNSUPPORTED, "attention_noalloc: device %d", dev);
+    std::lock_guard<std::mutex> lk(g_static_mu);
+    if (!g_static_ptr[dev]) {
+        void *ptr = nullptr;
+        MYNN_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        MYNN_REQUIRE(ptr, MYNN_ERR_STATE, "attention_noalloc: the scratch array has no device address");
+        g_static_ptr[dev] = ptr;
+    }
+    *out = g_static_ptr[dev];
+    return 0;
+}
+
+enum { WS_LIBRARY = 0, WS_CALLER = 1, WS_STATIC = 2 };
 
 // bytes of partial results the launch plan of this call needs (0: no key range is split)
 static size_t plan_scratch_bytes(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, int cache_len, bool masked) {
@@ -507,6 +529,12 @@ static int attention_entry(void *out, const void *Q, const void *K, const void *
             MYNN_REQUIRE(workspace && aligned16(workspace) && workspace_bytes >= need, MYNN_ERR_INVALID,
                          "attention: the workspace must hold %zu bytes (mynn_attention_workspace_bytes), 16-byte aligned", need);
             scr = workspace;
+        } else if (ws_mode == WS_STATIC) {
+            MYNN_REQUIRE(need <= kStaticScratchBytes, MYNN_ERR_UNSUPPORTED,
+                         "attention_noalloc: this shape needs %zu bytes of partial results, the library's fixed array holds %zu", need,
+                         kStaticScratchBytes);
+            int rc = static_scratch(&scr);
+            if (rc) return rc;
         } else {
             std::lock_guard<std::mutex> lk(g_scratch_mu);
             Grown &g = g_scratch[st];
@@ -548,6 +576,15 @@ extern "C" int mynn_attention_ws(void *out, const void *Q, const void *K, const 
     return attention_entry(out, Q, K, V, mask, mask_outer_stride, mask_row_stride, k_scale, v_scale, scale, is_causal, B, Sq,
                            active_seq_kv, d_active, cache_seq_len, q_pos_offset, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8,
                            WS_CALLER, workspace, workspace_bytes, as_stream(s));
+}
+
+extern "C" int mynn_attention_noalloc(void *out, const void *Q, const void *K, const void *V, const void *k_scale,
+                                      const void *v_scale, float scale, int is_causal, int B, int Sq, int active_seq_kv,
+                                      const int32_t *d_active, int cache_seq_len, int q_pos_offset, int num_q_heads,
+                                      int num_kv_heads, int head_dim, int dtype, int kv_int8, mynn_stream s) {
+    return attention_entry(out, Q, K, V, nullptr, 0, 0, k_scale, v_scale, scale, is_causal, B, Sq, active_seq_kv, d_active,
+                           cache_seq_len, q_pos_offset, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, WS_STATIC, nullptr, 0,
+                           as_stream(s));
 }
 
 // ---- streaming KV (sink + ring cache): the slot map of the reference's kernels and the two operators that
