@@ -23,23 +23,170 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
-# HBM bytes per launch of the gate/up GEMV (TinyLlama shape, 16-bit activations) from rocprofv3
-# --pmc FETCH_SIZE (x2.000, scaled by a 256 MiB copy) + WRITE_SIZE (x1.000): 11396.4 KiB * 2 + 35.0 KiB.
-# Counters cannot be read from inside this process; the figure is carried here from that profile run.
-GATEUP_GEMV_TRAFFIC_BYTES = 23375749
-# the same for the dominant kernels of the other workloads (profiles/prefill_and_batched_decode_pmc_hbm_traffic.md):
-# prefill gate/up GEMM + SwiGLU (f16, 8192 x 11264 x 2048): 287320.4 KiB * 2 + 90112.0 KiB;
-# batched-decode gate/up few-row GEMM (Llama-3-8B shape, 32 rows): 61689.4 KiB * 2 + 896.3 KiB
-PREFILL_GATEUP_GEMM_TRAFFIC_BYTES = 680706867
-BATCHED_GATEUP_GEMM_TRAFFIC_BYTES = 127257702
-# share of SIMD clocks in which the matrix pipe is busy during the prefill gate/up GEMM, from rocprofv3 --pmc
-# SQ_VALU_MFMA_BUSY_CYCLES / (GRBM_GUI_ACTIVE / 8 XCDs * 1024 SIMDs); the shader clock under that load is 1.87 GHz
-# (2.06 GHz with int8 activations), which is why it exceeds flop / time / peak-at-2.4-GHz
-# (profiles/prefill_tinyllama_int8_8x1024_pmc_mfma_utilisation.md)
-PREFILL_GATEUP_MFMA_BUSY_FRAC = {"f16": 0.513, "w8a8": 0.382}
+# Figures that cannot be measured from inside this process (rocprofv3's own kernel durations, HBM traffic and
+# matrix-pipe counters of a launch) are read from small JSON files under profiles/ that `--summarize-rocprof`
+# writes from rocprofv3 output of this same script; each entry carries the kernel's mangled name, and is used
+# only while the built library still contains that symbol.
+PROFILE_JSON = {"decode": "decode_tinyllama_int8_bs1.json", "prefill": "prefill_tinyllama_int8_8x1024.json",
+                "prefill_w8a8": "prefill_w8a8_tinyllama_8x1024.json", "decode_batch": "decode_llama3_8b_int8_bs32_ctx2048.json",
+                "decode_batch_kv8": "decode_llama3_8b_int8_bs32_ctx2048_kv_int8.json",
+                "attention": "attention_decode_b16_l4096.json"}
+# launch role (the executor's name for a launch) -> pattern of the mangled kernel name
+ROLE_PATTERNS = {
+    "gemv_norm_gateup_swiglu": r"dequant_gemv1_kernelI\w+?Li\d+ELi\d+ELi2ELb1ELb0EE",
+    "gemv_down_residual": r"dequant_gemv1_kernelI\w+?Li\d+ELi\d+ELi1ELb0ELb0EE",
+    "gemv_norm_lm_head_argmax": r"dequant_gemv1_kernelI\w+?Li\d+ELi\d+ELi0ELb1ELb1EE",
+    "qkv_attention_o": r"qkv_attention_kernelI\w+?Li\d+ELi\d+ELb0EE",
+    "embed_qkv_attention_o": r"qkv_attention_kernelI\w+?Li\d+ELi\d+ELb1EE",
+    "linear_gateup_swiglu": r"(gemm_nt_dma_kernelI\w+?Li2ELb0EE|skinny_gemm_kernel)",
+    "qlinear_gateup_swiglu": r"gemm_nt_dma_kernelI\w+?Li2ELb1EE",
+    "attention": r"(attn_stream_kernel|attn_prefill_kernel)",
+}
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16/fp16 matrix rate
 INT8_PEAK_TOPS = 5000.0    # MI355X published dense int8 matrix rate
 PREFILL_BATCH, PREFILL_LEN = 8, 1024
+
+
+
+def source_digest():
+    """sha256 over the kernel sources the library was built from (a profile taken from other sources is stale)."""
+    import glob
+    import hashlib
+
+    h = hashlib.sha256()
+    for f in sorted(glob.glob(os.path.join(ROOT, "my-nn-engine_amd", "csrc", "*"))):
+        if f.endswith((".hip", ".h", "Makefile")):
+            h.update(os.path.basename(f).encode())
+            h.update(open(f, "rb").read())
+    return h.hexdigest()[:16]
+
+
+_lib_bytes = None
+
+
+def library_has_symbol(mangled):
+    global _lib_bytes
+    if _lib_bytes is None:
+        mynn = importlib.import_module("my-nn-engine_amd")
+        _lib_bytes = open(mynn.LIB_PATH, "rb").read()
+    return mangled.encode() in _lib_bytes
+
+
+def load_profile(key):
+    """The tracked rocprofv3 summary for a workload, or None.  Entries whose kernel the library no longer holds
+    are dropped, so that a changed kernel never inherits an old figure."""
+    path = os.path.join(ROOT, "profiles", PROFILE_JSON[key])
+    if not os.path.exists(path):
+        return None
+    prof = json.load(open(path))
+    prof["kernels"] = [k for k in prof.get("kernels", []) if library_has_symbol(k["mangled"])]
+    prof["file"] = "profiles/" + PROFILE_JSON[key]
+    prof["stale"] = prof.get("source_sha256") != source_digest()
+    return prof
+
+
+def profile_entry(prof, role):
+    """The profile's entry for a launch role (matched on the mangled kernel name); None when absent."""
+    import re
+
+    if not prof or role not in ROLE_PATTERNS:
+        return None
+    hits = [k for k in prof["kernels"] if re.search(ROLE_PATTERNS[role], k["mangled"])]
+    if not hits:
+        return None
+    return max(hits, key=lambda k: k["total_ms"])
+
+
+def traffic_bytes(entry):
+    """HBM bytes per launch from the two counter runs, scaled by what the same counters read for a 256 MiB copy."""
+    if not entry or entry.get("fetch_kib") is None or entry.get("write_kib") is None:
+        return None
+    return int(round((entry["fetch_kib"] * entry["fetch_factor"] + entry["write_kib"] * entry["write_factor"]) * 1024))
+
+
+def summarize_rocprof(args):
+    """Reads rocprofv3 output of this script (kernel trace, and optionally the FETCH_SIZE and WRITE_SIZE counter
+    runs, all as csv with mangled kernel names) and writes the JSON that later runs read back, plus the same
+    figures as a markdown table."""
+    import csv
+    import glob
+
+    def rows(d, suffix):
+        files = glob.glob(os.path.join(d, "**", "*" + suffix), recursive=True)
+        if not files:
+            raise SystemExit("no *%s under %s" % (suffix, d))
+        for f in files:
+            with open(f, newline="") as fh:
+                for r in csv.DictReader(fh):
+                    yield r
+
+    def kname(r):  # (mangled names come with the kernel descriptor's suffix)
+        n = r["Kernel_Name"]
+        return n[:-3] if n.endswith(".kd") else n
+
+    kern = {}
+    for r in rows(args.summarize_rocprof, "kernel_trace.csv"):
+        name = kname(r)
+        if "mynn" not in name:
+            continue
+        d = (int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e3
+        k = kern.setdefault(name, {"mangled": name, "calls": 0, "total_us": 0.0, "min_us": 1e30, "max_us": 0.0})
+        k["calls"] += 1
+        k["total_us"] += d
+        k["min_us"] = min(k["min_us"], d)
+        k["max_us"] = max(k["max_us"], d)
+    copy = {}
+    for which, d in (("fetch", args.pmc_fetch), ("write", args.pmc_write)):
+        if not d:
+            continue
+        acc = {}
+        per = 0.0  # counter reading of the one 256 MiB device-to-device copy (262144 KiB read, 262144 written): the largest copy
+        for r in rows(d, "counter_collection.csv"):
+            a = acc.setdefault(kname(r), [0, 0.0])
+            a[0] += 1
+            a[1] += float(r["Counter_Value"])
+            if "copyBuffer" in r["Kernel_Name"]:
+                per = max(per, float(r["Counter_Value"]))
+        if per < 65536:
+            raise SystemExit("%s: no 256 MiB __amd_rocclr_copyBuffer dispatch (run with --traffic-calibration)" % d)
+        copy[which] = per
+        for n, (cnt, tot) in acc.items():
+            if n in kern:
+                kern[n][which + "_kib"] = tot / cnt
+                kern[n][which + "_factor"] = 262144.0 / per
+    if args.pmc_mfma:
+        # SQ_VALU_MFMA_BUSY_CYCLES (summed over the SIMDs) against GRBM_GUI_ACTIVE (summed over the 8 XCDs): the share of
+        # SIMD clocks (1024 SIMDs) in which the matrix pipe is busy
+        acc = {}
+        for r in rows(args.pmc_mfma, "counter_collection.csv"):
+            a = acc.setdefault(r["Kernel_Name"], {})
+            a[r["Counter_Name"]] = a.get(r["Counter_Name"], 0.0) + float(r["Counter_Value"])
+        for n, c in acc.items():
+            if n in kern and c.get("GRBM_GUI_ACTIVE"):
+                kern[n]["mfma_busy_frac"] = round(c.get("SQ_VALU_MFMA_BUSY_CYCLES", 0.0) / (c["GRBM_GUI_ACTIVE"] / 8.0 * 1024.0), 4)
+    out = {"workload": args.workload + ("_w8a8" if args.w8a8 else "") + ("_kv8" if args.kv_int8 else ""),
+           "command": args.profile_command, "commit": args.profile_commit, "source_sha256": source_digest(),
+           "calibration_copy_reading": copy, "kernels": []}
+    for k in sorted(kern.values(), key=lambda k: -k["total_us"]):
+        k["avg_us"] = round(k["total_us"] / k["calls"], 3)
+        k["total_ms"] = round(k.pop("total_us") / 1e3, 3)
+        k["min_us"], k["max_us"] = round(k["min_us"], 3), round(k["max_us"], 3)
+        for f in ("fetch_kib", "write_kib"):
+            if f in k:
+                k[f] = round(k[f], 1)
+        out["kernels"].append(k)
+    with open(args.out, "w") as fh:
+        json.dump(out, fh, indent=1)
+        fh.write("\n")
+    lines = ["| kernel | calls | avg us | min us | max us | total ms | FETCH_SIZE KiB | WRITE_SIZE KiB | HBM bytes per launch |",
+             "|---|---|---|---|---|---|---|---|---|"]
+    for k in out["kernels"]:
+        tb = traffic_bytes(k)
+        lines.append("| `%s` | %d | %.2f | %.2f | %.2f | %.2f | %s | %s | %s |" % (
+            k["mangled"], k["calls"], k["avg_us"], k["min_us"], k["max_us"], k["total_ms"], k.get("fetch_kib", "-"),
+            k.get("write_kib", "-"), tb if tb is not None else "-"))
+    print("\n".join(lines))
+
 
 TINYLLAMA = dict(n_layers=22, hidden=2048, n_heads=32, n_kv_heads=4, head_dim=64, ffn=5632, vocab=32000,
                  max_seq=384, eps=1e-5, rope_theta=10000.0)
@@ -145,6 +292,8 @@ def prefill_main(args, mynn, cfg):
     peak = INT8_PEAK_TOPS if args.w8a8 else MFMA_PEAK_TFLOPS
     unit = "TOP/s" if args.w8a8 else "TFLOP/s"
     lin_tflops = sum(v[3] for v in lin.values()) / (sum(v[1] for v in lin.values()) * 1e-3) / 1e12
+    prof = load_profile("prefill_w8a8" if args.w8a8 else "prefill") if args.dtype == "f16" else None
+    entry = profile_entry(prof, dom)
     out = {
         "metric": "prefill tok/s 8x1024 TinyLlama-shape int8; MFMA utilisation" + (" (W8A8: quantize_activations)" if args.w8a8 else ""),
         "value": round(B * S * K / elapsed, 1), "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
@@ -160,9 +309,9 @@ def prefill_main(args, mynn, cfg):
                    "per_kernel_ms": {k: round(v[1] / 2, 3) for k, v in sorted(agg.items(), key=lambda kv: -kv[1][1])}},
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 1), "peak": peak,
                      "unit": unit, "frac": round(achieved / peak, 4),
-                     "traffic": PREFILL_GATEUP_GEMM_TRAFFIC_BYTES if dom == "linear_gateup_swiglu" and args.dtype == "f16" else None,
-                     "mfma_busy_frac_pmc": (PREFILL_GATEUP_MFMA_BUSY_FRAC["w8a8" if args.w8a8 else "f16"]
-                                            if dom == "linear_gateup_swiglu" and args.dtype == "f16" else None),
+                     "traffic": traffic_bytes(entry), "mfma_busy_frac_pmc": entry.get("mfma_busy_frac") if entry else None,
+                     "avg_launch_us_rocprof": entry["avg_us"] if entry else None,
+                     "profile": {"file": prof["file"], "commit": prof.get("commit"), "stale": prof["stale"]} if prof and entry else None,
                      "flops_per_launch": fl_tot / calls, "avg_launch_us": round(ms_tot / calls * 1e3, 2),
                      "all_linear_TFLOPs": round(lin_tflops, 1)},
     }
@@ -316,6 +465,8 @@ def decode_batch_main(args, mynn):
     dom = max(lin, key=lambda k: lin[k][1])
     calls, ms_tot, bytes_tot = lin[dom]
     achieved = bytes_tot / (ms_tot * 1e-3) / 1e9
+    prof = load_profile("decode_batch_kv8" if args.kv_int8 else "decode_batch") if args.dtype == "f16" else None
+    entry = profile_entry(prof, dom)
     out = {
         "metric": "decode tok/s, batch 32 at context 2048, Llama-3-8B-shape int8 (aggregate over the batch)",
         "value": round(B * K / elapsed, 1), "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
@@ -330,12 +481,47 @@ def decode_batch_main(args, mynn):
                    "per_kernel_ms": {k: round(v[1] / 2, 3) for k, v in sorted(agg.items(), key=lambda kv: -kv[1][1])}},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": BATCHED_GATEUP_GEMM_TRAFFIC_BYTES if dom == "linear_gateup_swiglu" and not args.kv_int8 else None,
+                     "traffic": traffic_bytes(entry), "avg_launch_us_rocprof": entry["avg_us"] if entry else None,
+                     "profile": {"file": prof["file"], "commit": prof.get("commit"), "stale": prof["stale"]} if prof and entry else None,
                      "bytes_per_launch": bytes_tot / calls,
                      "avg_launch_us": round(ms_tot / calls * 1e3, 2)},
     }
     dec.close()
     print(json.dumps(out))
+
+
+def short_prefill(mynn, cfg, weights, seed):
+    """Two passes of the 8 x 1024 prefill (configs[3]) over the same weights, outside any timed decode region: the
+    matrix-core side of the path, for the same JSON line."""
+    import numpy as np
+    import torch
+
+    B, S = PREFILL_BATCH, PREFILL_LEN
+    pcfg = dict(cfg, max_seq=S)
+    pre = mynn.Decoder(pcfg, weights, seq_q=S, batch=B)
+    ids = np.random.default_rng(seed).integers(0, cfg["vocab"], B * S)
+    pos = np.arange(S)
+    pre.step(ids, pos, 0, S)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(2):
+        pre.step(ids, pos, 0, S)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / 2
+    agg = {}
+    for name, kms, _, flops in pre.profile(ids, pos, 0, S):
+        a = agg.setdefault(name, [0.0, 0.0])
+        a[0] += kms
+        a[1] += flops
+    step_flops = sum(v[1] for v in agg.values())
+    gu = agg.get("linear_gateup_swiglu")
+    out = {"workload": "configs[3]: %d x %d prefill, same weights, 2 timed passes" % (B, S), "ms_per_pass": round(ms, 3),
+           "tok_s": round(B * S / (ms * 1e-3), 1), "launches_per_pass": pre.stats()["launches_per_step"],
+           "step_mfma_frac": round(step_flops / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4),
+           "gateup_TFLOPs": round(gu[1] / (gu[0] * 1e-3) / 1e12, 1) if gu and gu[0] > 0 else None}
+    pre.close()
+    torch.cuda.empty_cache()
+    return out
 
 
 def main():
@@ -347,6 +533,7 @@ def main():
     ap.add_argument("--dtype", choices=["f16", "bf16"], default="f16")
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-prefill", action="store_true", help="decode: leave the short prefill run (config.prefill) out")
     ap.add_argument("--cpu-steps", type=int, default=96)
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="first run one 256 MiB device-to-device copy (a kernel of known traffic, for scaling "
@@ -354,10 +541,22 @@ def main():
     ap.add_argument("--w8a8", action="store_true",
                     help="prefill: quantise activations per row and run every linear as int8 x int8 (Options::quantize_activations)")
     ap.add_argument("--kv-int8", action="store_true",
-                    help="decode_batch: int8 KV cache with per-token scales (BuildOptions::quant_kv_cache)")
+                    help="decode / decode_batch: int8 KV cache with per-token scales (BuildOptions::quant_kv_cache)")
+    ap.add_argument("--unfused", action="store_true", help="decode: every op a launch of its own (unfused_decode)")
     ap.add_argument("--check-tokens", type=int, default=0,
-                    help="also compare the first N greedy tokens with the oracle (slow: CPU decode)")
+                    help="also compare the first N generated tokens with the oracle generating freely (slow: CPU decode)")
+    ap.add_argument("--summarize-rocprof", metavar="DIR",
+                    help="no GPU work: read rocprofv3 csv output of this script under DIR (kernel trace, mangled names) and "
+                         "write the profile JSON given by --out")
+    ap.add_argument("--pmc-fetch", metavar="DIR", help="with --summarize-rocprof: the --pmc FETCH_SIZE run")
+    ap.add_argument("--pmc-write", metavar="DIR", help="with --summarize-rocprof: the --pmc WRITE_SIZE run")
+    ap.add_argument("--pmc-mfma", metavar="DIR", help="with --summarize-rocprof: the --pmc SQ_VALU_MFMA_BUSY_CYCLES GRBM_GUI_ACTIVE run")
+    ap.add_argument("--out", help="with --summarize-rocprof: the JSON file to write")
+    ap.add_argument("--profile-command", default="", help="with --summarize-rocprof: the command line that was profiled")
+    ap.add_argument("--profile-commit", default="", help="with --summarize-rocprof: the commit the library was built from")
     args = ap.parse_args()
+    if args.summarize_rocprof:
+        return summarize_rocprof(args)
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives are built)" % args.gpus,
               file=sys.stderr)
@@ -389,7 +588,7 @@ def main():
 
     weights = make_weights(cfg, dt, args.seed)
     torch.cuda.synchronize()
-    dec = mynn.Decoder(cfg, weights)
+    dec = mynn.Decoder(cfg, weights, quant_kv_cache=args.kv_int8, quantize_activations=args.w8a8, unfused_decode=args.unfused)
     stats = dec.stats()
     rng = np.random.default_rng(args.seed)
     prompt = rng.integers(0, cfg["vocab"], PROMPT_LEN).tolist()
@@ -398,90 +597,132 @@ def main():
     # (each of these steps is a host round trip: inputs up, graph replay, token down -- timed for the record)
     first = None
     t_host = None
+    prompt_choice = []  # the greedy token after each prompt position (compared with the CPU baseline's below)
     for i, t in enumerate(prompt):
         if i == 16:
             torch.cuda.synchronize()
             t_host = time.perf_counter()
         first, _ = dec.step([t], [i], i, i + 1)
+        prompt_choice.append(first[0])
     host_tok_s = (PROMPT_LEN - 16) / (time.perf_counter() - t_host)
     first = first[0]
 
+    loop = dec.decode_loop
     if W > 0:
-        dec.decode_loop(first, PROMPT_LEN, W)  # untimed; its KV rows are overwritten below
+        loop(first, PROMPT_LEN, W)  # untimed; its KV rows are overwritten below
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    toks = dec.decode_loop(first, PROMPT_LEN, K)
+    toks = loop(first, PROMPT_LEN, K)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     generated = [first] + toks[:-1]
     ms_per_step = elapsed * 1e3 / K
     tok_s = K / elapsed
 
-    # ---- roofline of the dominant kernel: HIP events around every launch of eager steps at
-    # contexts spread over the timed range, on the executor's own stream
+    # ---- per-launch durations: HIP events tied to every launch of eager steps at contexts spread over the timed
+    # range, on the executor's own stream.  The K / V rows an attention launch reads depend on the context, which the
+    # executor's own byte count leaves out: added here.
+    KD = cfg["n_kv_heads"] * cfg["head_dim"]
     agg = {}
     n_prof = 8
     for j in range(n_prof):
         past = PROMPT_LEN + (j * (K - 1)) // max(n_prof - 1, 1)
         for name, ms, nbytes, _ in dec.profile_step(generated[min(past - PROMPT_LEN, K - 1)], past):
+            if "attention" in name:
+                nbytes += 2.0 * ((KD + cfg["n_kv_heads"] * eb) if args.kv_int8 else KD * eb) * past
             a = agg.setdefault(name, [0, 0.0, 0.0])
             a[0] += 1
             a[1] += ms
             a[2] += nbytes
-    gemv = {k: v for k, v in agg.items() if k.startswith("gemv_")}
-    dom = max(gemv, key=lambda k: gemv[k][1])
-    calls, ms_tot, bytes_tot = gemv[dom]
-    achieved = bytes_tot / (ms_tot * 1e-3) / 1e9
-    all_gemv_gbs = sum(v[2] for v in gemv.values()) / (sum(v[1] for v in gemv.values()) * 1e-3) / 1e9
-    step_bytes = algorithmic_bytes_per_token(cfg, eb, PROMPT_LEN + K // 2)
+    prof = load_profile("decode") if (args.dtype == "f16" and not (args.kv_int8 or args.w8a8 or args.unfused)) else None
 
+    def launch_roofline(role):
+        """Algorithmic bytes per launch over the launch's average duration: by rocprofv3's kernel trace of this
+        script where the tracked profile still matches the built kernel (`achieved`), and by the events of this
+        run (`achieved_events`)."""
+        calls, ms_tot, bytes_tot = agg[role]
+        per_launch, ev_us = bytes_tot / calls, ms_tot / calls * 1e3
+        entry = profile_entry(prof, role)
+        ev_gbs = per_launch / (ev_us * 1e-6) / 1e9
+        r = {"kernel": role, "mangled": entry["mangled"] if entry else None, "bytes_per_launch": round(per_launch),
+             "avg_launch_us_events": round(ev_us, 3), "achieved_events": round(ev_gbs, 1),
+             "frac_events": round(ev_gbs / HBM_PEAK_GBS, 4),
+             "avg_launch_us_rocprof": entry["avg_us"] if entry else None, "traffic": traffic_bytes(entry)}
+        if entry:
+            gbs = per_launch / (entry["avg_us"] * 1e-6) / 1e9
+            r.update({"achieved": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4), "duration_from": "rocprofv3 kernel trace"})
+        else:
+            r.update({"achieved": round(ev_gbs, 1), "frac": round(ev_gbs / HBM_PEAK_GBS, 4),
+                      "duration_from": "hip events (no tracked profile matches the built kernel)"})
+        return r
+
+    dom = max(agg, key=lambda k: agg[k][1])  # the launch with the largest total time in the step
+    gemv = {k: v for k, v in agg.items() if k.startswith("gemv_")}
+    all_gemv_gbs = sum(v[2] for v in gemv.values()) / (sum(v[1] for v in gemv.values()) * 1e-3) / 1e9 if gemv else None
+    step_bytes = algorithmic_bytes_per_token(cfg, eb, PROMPT_LEN + K // 2)
+    roof = {"bound": "hbm", "peak": HBM_PEAK_GBS, "unit": "GB/s"}
+    roof.update(launch_roofline(dom))
+    roof["profile"] = {"file": prof["file"], "commit": prof.get("commit"), "stale": prof["stale"]} if prof else None
+    if "gemv_norm_gateup_swiglu" in agg:  # the dequant GEMV that moves the most bytes, whichever launch dominates
+        roof["gateup_gemv"] = launch_roofline("gemv_norm_gateup_swiglu")
+    if "gemv_down_residual" in agg:
+        roof["down_gemv"] = launch_roofline("gemv_down_residual")
+    roof["all_gemv_GBs"] = round(all_gemv_gbs, 1) if all_gemv_gbs else None
+
+    variant = (", int8 KV cache" if args.kv_int8 else "") + (", int8 activations (W8A8)" if args.w8a8 else "") + \
+              (", one op per launch" if args.unfused else "")
     out = {
         "metric": "decode tok/s bs1 TinyLlama-shape int8; dequant-GEMV HBM GB/s vs peak",
         "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32 accumulate over int8 weights, %s activations/KV" % args.dtype, "data": "synthetic",
         "config": {"workload": "configs[2]: TinyLlama-1.1B-shape int8 decoder, batch 1 greedy decode, 128 prompt tokens "
-                               "fed through the decode path then %d generated (timed: the generated tokens)" % K,
+                               "fed through the decode path then %d generated (timed: the generated tokens)%s" % (K, variant),
                    "prompt_len": PROMPT_LEN, "max_seq": cfg["max_seq"], "launches_per_step": stats["launches_per_step"],
                    "hipgraph": stats["graph"], "seed": args.seed,
                    "host_roundtrip_tok_s": round(host_tok_s, 1),
                    "step_algorithmic_bytes": step_bytes,
                    "step_hbm_frac": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                   # average duration of every launch of the step (HIP events, eager steps): the fused
-                   # q|k|v + attention + o launch is the longest, the gate/up GEMV moves the most bytes
+                   # average duration of every launch of the step (HIP events, eager steps)
                    "per_launch_us": {k: round(v[1] / v[0] * 1e3, 2) for k, v in sorted(agg.items(), key=lambda kv: -kv[1][1])}},
-        "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": GATEUP_GEMV_TRAFFIC_BYTES if dom == "gemv_norm_gateup_swiglu" else None,
-                     "bytes_per_launch": bytes_tot / calls, "avg_launch_us": round(ms_tot / calls * 1e3, 3),
-                     "all_gemv_GBs": round(all_gemv_gbs, 1)},
+        "roofline": roof,
     }
+    dec.close()
+    if not args.no_prefill and not (args.kv_int8 or args.w8a8 or args.unfused):
+        out["config"]["prefill"] = short_prefill(mynn, cfg, weights, args.seed)
 
     if not args.no_cpu_baseline:
         import oracle as orc
 
         hw = to_host_weights(weights)
         ref = orc.Model(dict(cfg), hw)
+        ref.set_options(quant_kv_cache=args.kv_int8, quantize_activations=args.w8a8)
         n_cpu = args.cpu_steps
         ref.past_len = 0
         stream = prompt + generated
         # bounded sample: the first n_cpu decode steps of the same token stream
         t0 = time.perf_counter()
-        last = None
+        cpu_choice = []
         for i in range(n_cpu):
-            last = ref.decode_step(stream[i])
+            cpu_choice.append(int(ref.decode_step(stream[i])))
         cpu_elapsed = time.perf_counter() - t0
         out["cpu_baseline"] = {"value": round(n_cpu / cpu_elapsed, 3), "unit": "tok/s", "cores": orc.get_threads(),
                                "kind": "port",
                                "sample": "first %d decode steps (contexts 0..%d) of the same model and token stream, "
                                          "C port of the reference CPU backend, OpenMP over N" % (n_cpu, n_cpu - 1)}
+        # the same steps ran on the GPU: the greedy choice after each of them, both sides on the same context
+        gpu_choice = (prompt_choice + generated[1:])[:n_cpu]
+        same = sum(int(a == b) for a, b in zip(cpu_choice, gpu_choice))
+        out["config"]["tokens_identical_to_oracle"] = same == n_cpu
+        out["config"]["tokens_checked"] = {"steps": n_cpu, "identical": same,
+                                           "what": "greedy choice after each of the first %d positions of the stream, oracle and "
+                                                   "GPU on the same context" % n_cpu}
         if args.check_tokens:
             n = min(args.check_tokens, K)
             ref2 = orc.Model(dict(cfg), hw)
             want = ref2.generate(prompt, n)
-            out["config"]["tokens_identical_to_oracle"] = (want == generated[:n])
-            out["config"]["tokens_checked"] = n
-    dec.close()
+            out["config"]["generated_identical_to_free_running_oracle"] = {"tokens": n, "identical_prefix": next(
+                (i for i in range(n) if want[i] != generated[i]), n)}
     print(json.dumps(out))
 
 
