@@ -33,8 +33,10 @@ struct Json {
     }
 };
 struct JsonParser {
-    const char *p, *end;
+    const char *p, *end;  // [p, end) is followed by a NUL (parse_json copies the text), so strtod cannot run past it
     bool ok = true;
+    int depth = 0;
+    static constexpr int kMaxDepth = 32;  // a safetensors header nests 3 deep
     void ws() {
         while (p < end && (*p == ' ' || *p == '\n' || *p == '\t' || *p == '\r')) p++;
     }
@@ -77,10 +79,17 @@ struct JsonParser {
             ok = false;
             return j;
         }
+        if ((*p == '{' || *p == '[') && ++depth > kMaxDepth) {
+            ok = false;
+            return j;
+        }
         if (*p == '{') {
             p++;
             j.kind = Json::OBJ;
-            if (eat('}')) return j;
+            if (eat('}')) {
+                depth--;
+                return j;
+            }
             do {
                 std::string k = string();
                 if (!ok || !eat(':')) {
@@ -91,19 +100,24 @@ struct JsonParser {
                 if (!ok) return j;
             } while (eat(','));
             if (!eat('}')) ok = false;
+            depth--;
         } else if (*p == '[') {
             p++;
             j.kind = Json::ARR;
-            if (eat(']')) return j;
+            if (eat(']')) {
+                depth--;
+                return j;
+            }
             do {
                 j.arr.push_back(value());
                 if (!ok) return j;
             } while (eat(','));
             if (!eat(']')) ok = false;
+            depth--;
         } else if (*p == '"') {
             j.kind = Json::STR;
             j.str = string();
-        } else if (!strncmp(p, "true", 4) || !strncmp(p, "false", 5) || !strncmp(p, "null", 4)) {
+        } else if ((end - p >= 4 && (!strncmp(p, "true", 4) || !strncmp(p, "null", 4))) || (end - p >= 5 && !strncmp(p, "false", 5))) {
             j.kind = *p == 'n' ? Json::NUL : Json::BOOL;
             j.num = *p == 't';
             p += *p == 'f' ? 5 : 4;
@@ -111,16 +125,24 @@ struct JsonParser {
             char *q = nullptr;
             j.kind = Json::NUM;
             j.num = strtod(p, &q);
-            if (q == p) ok = false;
+            if (q == p || q > end) ok = false;
             p = q;
         }
         return j;
     }
 };
 static bool parse_json(const char *data, size_t n, Json &out) {
-    JsonParser ps{data, data + n};
+    const std::string text(data, n);  // NUL-terminated copy: the mapped header may end exactly at the end of the file
+    JsonParser ps{text.c_str(), text.c_str() + n};
     out = ps.value();
     return ps.ok;
+}
+
+// a JSON number that must be a non-negative integer below 2^53 (offsets, extents): false otherwise
+static bool as_size(const Json &j, size_t *out) {
+    if (j.kind != Json::NUM || !(j.num >= 0.0) || j.num > 9007199254740992.0 || j.num != (double)(uint64_t)j.num) return false;
+    *out = (size_t)j.num;
+    return true;
 }
 
 // ---- shards ---------------------------------------------------------------------------------------
@@ -200,15 +222,22 @@ static int add_shard(mynn_weights &w, const std::string &path) {
         e.dtype = dtype_of(dt->str);
         MYNN_REQUIRE(e.dtype >= 0, MYNN_ERR_UNSUPPORTED, "weights: %s: dtype %s of %s", path.c_str(), dt->str.c_str(),
                      kv.first.c_str());
-        size_t count = 1;
+        MYNN_REQUIRE(dt->kind == Json::STR && shp->kind == Json::ARR && off->kind == Json::ARR && shp->arr.size() <= 8, MYNN_ERR_INVALID,
+                     "weights: %s: malformed entry %s", path.c_str(), kv.first.c_str());
+        // every extent and offset is a checked unsigned integer; products and sums cannot wrap
+        size_t count = 1, off0 = 0, off1 = 0;
+        bool sane = as_size(off->arr[0], &off0) && as_size(off->arr[1], &off1) && off0 <= off1 && off1 <= sh->bytes - data_start;
         for (auto &d : shp->arr) {
-            e.shape.push_back((int64_t)d.num);
-            count *= (size_t)d.num;
+            size_t ext = 0;
+            sane = sane && as_size(d, &ext) && (ext == 0 || count <= sh->bytes / ext);  // (count * ext stays within the file size)
+            if (!sane) break;
+            count *= ext;
+            e.shape.push_back((int64_t)ext);
         }
-        e.offset = data_start + (size_t)off->arr[0].num;
-        e.length = (size_t)(off->arr[1].num - off->arr[0].num);
-        MYNN_REQUIRE(e.offset + e.length <= sh->bytes && e.length == count * dtype_bytes(e.dtype), MYNN_ERR_INVALID,
-                     "weights: %s: %s has inconsistent offsets", path.c_str(), kv.first.c_str());
+        MYNN_REQUIRE(sane && count <= (off1 - off0) && off1 - off0 == count * dtype_bytes(e.dtype), MYNN_ERR_INVALID,
+                     "weights: %s: %s has inconsistent shape or offsets", path.c_str(), kv.first.c_str());
+        e.offset = data_start + off0;
+        e.length = off1 - off0;
         if (!w.entries.count(kv.first)) w.order.push_back(kv.first);
         w.entries[kv.first] = std::move(e);
     }
@@ -231,7 +260,11 @@ static int shards_of_index(const std::string &index_path, std::vector<std::strin
     MYNN_REQUIRE(wm && wm->kind == Json::OBJ, MYNN_ERR_INVALID, "weights: %s: missing weight_map", index_path.c_str());
     const std::string dir = index_path.substr(0, index_path.find_last_of('/') + 1);
     for (auto &kv : wm->obj) {
-        std::string p = dir + kv.second.str;
+        const std::string &name = kv.second.str;
+        MYNN_REQUIRE(kv.second.kind == Json::STR && !name.empty() && name.find('/') == std::string::npos &&
+                         name.find('\\') == std::string::npos && name != "." && name != "..",
+                     MYNN_ERR_INVALID, "weights: %s: shard name '%s' is not a plain file name", index_path.c_str(), name.c_str());
+        std::string p = dir + name;
         bool seen = false;
         for (auto &s : files) seen |= s == p;
         if (!seen) files.push_back(p);
@@ -328,7 +361,7 @@ static int write_safetensors(const std::string &dst, const std::vector<OutTensor
 
 using namespace mynn;
 
-extern "C" mynn_weights *mynn_weights_open(const char *path) {
+static mynn_weights *weights_open_impl(const char *path) {
     if (!path) {
         set_error("weights_open: null path");
         return nullptr;
@@ -361,7 +394,7 @@ extern "C" int mynn_weights_find(const mynn_weights *w, const char *name, int *d
 }
 
 // quantize.rs:313-337 (and copy_view :170-188: an f16 tensor that is not quantised is stored as bf16)
-extern "C" int mynn_quantize_safetensors_int8(const char *src, const char *dst, int *quantized, int *passthrough) {
+static int quantize_safetensors_int8_impl(const char *src, const char *dst, int *quantized, int *passthrough) {
     MYNN_REQUIRE(src && dst, MYNN_ERR_INVALID, "quantize_safetensors_int8: null path");
     std::vector<std::string> files;
     int rc = source_files(src, false, files);
@@ -458,7 +491,7 @@ static int upload_linear(mynn_device_weights &dw, const mynn_weights &w, const s
     return upload_float(dw, w, name + ".scale", dt, N);
 }
 
-extern "C" mynn_device_weights *mynn_weights_upload(const mynn_weights *w, const mynn_model_config *c) {
+static mynn_device_weights *weights_upload_impl(const mynn_weights *w, const mynn_model_config *c) {
     if (!w || !c) {
         set_error("weights_upload: null argument");
         return nullptr;
@@ -501,4 +534,26 @@ extern "C" void mynn_device_weights_free(mynn_device_weights *dw) {
     if (!dw) return;
     for (void *p : dw->owned) (void)hipFree(p);
     delete dw;
+}
+
+// No exception crosses the C boundary: an allocation that fails (a corrupt header can ask for one) becomes an error.
+template <typename R, typename F>
+static R guarded(F &&f, R on_fail) {
+    try {
+        return f();
+    } catch (const std::exception &e) {
+        set_error("weights: %s", e.what());
+    } catch (...) {
+        set_error("weights: unknown failure");
+    }
+    return on_fail;
+}
+extern "C" mynn_weights *mynn_weights_open(const char *path) {
+    return guarded<mynn_weights *>([&] { return weights_open_impl(path); }, nullptr);
+}
+extern "C" int mynn_quantize_safetensors_int8(const char *src, const char *dst, int *quantized, int *passthrough) {
+    return guarded<int>([&] { return quantize_safetensors_int8_impl(src, dst, quantized, passthrough); }, (int)MYNN_ERR_INVALID);
+}
+extern "C" mynn_device_weights *mynn_weights_upload(const mynn_weights *w, const mynn_model_config *c) {
+    return guarded<mynn_device_weights *>([&] { return weights_upload_impl(w, c); }, nullptr);
 }

@@ -136,3 +136,47 @@ def test_int8_checkpoint_upload_matches_tensors_passed_by_hand(tmp_path):
         _, b = by_hand.step([t], [i], i, i + 1, want_logits=True)
         assert np.array_equal(a, b)
     from_file.close(), by_hand.close()
+
+
+def _write_raw(path, header_text, payload=b""):
+    hdr = header_text.encode()
+    with open(path, "wb") as f:
+        f.write(struct.pack("<Q", len(hdr)))
+        f.write(hdr)
+        f.write(payload)
+
+
+@pytest.mark.parametrize("header", [
+    '{"t":{"dtype":"F32","shape":[2],"data_offsets":[0,16]}}',                       # length != count * element size
+    '{"t":{"dtype":"F32","shape":[2],"data_offsets":[-8,0]}}',                       # negative offset
+    '{"t":{"dtype":"F32","shape":[2],"data_offsets":[9223372036854775808,9223372036854775816]}}',  # offsets past 2^63
+    '{"t":{"dtype":"I8","shape":[4294967296,4294967296],"data_offsets":[0,0]}}',     # extents whose product wraps
+    '{"t":{"dtype":"F32","shape":[-2],"data_offsets":[0,8]}}',                       # negative extent
+    '{"t":{"dtype":"F32","shape":[1.5],"data_offsets":[0,8]}}',                      # fractional extent
+    '{"t":{"dtype":"F32","shape":[2],"data_offsets":[8,0]}}',                        # end before begin
+    '{"t":{"dtype":"F32","shape":[4],"data_offsets":[0,16]}}',                       # data beyond the end of the file
+    "[" * 100000,                                                                    # nesting without bound
+    '{"t":{"dtype":"F32","shape":[2],"data_offsets":[0,8]}',                         # truncated
+    '{"t":{"dtype":"F32","shape":"2","data_offsets":[0,8]}}',                        # wrong kinds
+    '{"t":12345',                                                                    # a number that ends the file
+])
+def test_reader_rejects_hostile_headers_with_an_error(tmp_path, header):
+    """A header the `safetensors` crate would refuse is refused here too -- with an error return, never a wild
+    read, a wrapped size or an exception across the C boundary."""
+    p = tmp_path / "bad.safetensors"
+    _write_raw(p, header, b"\0" * 8)
+    with pytest.raises(mynn.MynnError):
+        mynn.Weights(p)
+
+
+def test_reader_accepts_a_header_that_ends_the_file_and_refuses_path_tricks_in_the_index(tmp_path):
+    p = tmp_path / "empty.safetensors"
+    _write_raw(p, '{"t":{"dtype":"F32","shape":[0],"data_offsets":[0,0]}}')  # the header is the last byte of the mapping
+    w = mynn.Weights(p)
+    assert w.names() == ["t"] and w.find("t")[1] == (0,)
+    w.close()
+    d = tmp_path / "model"
+    d.mkdir()
+    (d / "model.safetensors.index.json").write_text(json.dumps({"weight_map": {"t": "../empty.safetensors"}}))
+    with pytest.raises(mynn.MynnError, match="plain file name"):
+        mynn.Weights(d)
