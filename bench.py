@@ -542,6 +542,7 @@ def main():
                     help="prefill: quantise activations per row and run every linear as int8 x int8 (Options::quantize_activations)")
     ap.add_argument("--kv-int8", action="store_true",
                     help="decode / decode_batch: int8 KV cache with per-token scales (BuildOptions::quant_kv_cache)")
+    ap.add_argument("--weight-arena", action="store_true", help="decode: all weights in one allocation in execution order (weight_arena)")
     ap.add_argument("--unfused", action="store_true", help="decode: every op a launch of its own (unfused_decode)")
     ap.add_argument("--check-tokens", type=int, default=0,
                     help="also compare the first N generated tokens with the oracle generating freely (slow: CPU decode)")
@@ -588,7 +589,8 @@ def main():
 
     weights = make_weights(cfg, dt, args.seed)
     torch.cuda.synchronize()
-    dec = mynn.Decoder(cfg, weights, quant_kv_cache=args.kv_int8, quantize_activations=args.w8a8, unfused_decode=args.unfused)
+    dec = mynn.Decoder(cfg, weights, quant_kv_cache=args.kv_int8, quantize_activations=args.w8a8, unfused_decode=args.unfused,
+                       weight_arena=args.weight_arena)
     stats = dec.stats()
     rng = np.random.default_rng(args.seed)
     prompt = rng.integers(0, cfg["vocab"], PROMPT_LEN).tolist()

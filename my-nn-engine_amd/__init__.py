@@ -55,7 +55,7 @@ class ModelConfig(C.Structure):
                 ("ffn", _i), ("vocab", _i), ("max_seq", _i), ("eps", _f), ("rope_theta", _f), ("dtype", _i),
                 ("seq_q", _i), ("batch", _i), ("weights_int8", _i), ("quant_kv_cache", _i),
                 ("quantize_activations", _i), ("streaming_kv", _i), ("gemm_tile", _i), ("unfused_decode", _i),
-                ("handover_spin_limit", _i)]
+                ("handover_spin_limit", _i), ("weight_arena", _i)]
 
 
 class KernelTime(C.Structure):
@@ -524,7 +524,8 @@ class Decoder:
     """
 
     def __init__(self, cfg, weights, seq_q=1, batch=1, kv=None, quant_kv_cache=False, quantize_activations=False,
-                 streaming_kv=False, gemm_tile=0, unfused_decode=False, handover_spin_limit=0, reference_abi=False):
+                 streaming_kv=False, gemm_tile=0, unfused_decode=False, handover_spin_limit=0, weight_arena=False,
+                 reference_abi=False):
         import torch
 
         tdt = {F16: torch.float16, BF16: torch.bfloat16}[cfg["dtype"]]
@@ -533,7 +534,7 @@ class Decoder:
         self.cfg = ModelConfig(cfg["n_layers"], cfg["hidden"], cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"],
                                cfg["ffn"], cfg["vocab"], cfg["max_seq"], float(cfg["eps"]), float(cfg["rope_theta"]),
                                cfg["dtype"], seq_q, batch, int(quant), int(quant_kv_cache), int(quantize_activations),
-                               int(streaming_kv), int(gemm_tile), int(unfused_decode), int(handover_spin_limit))
+                               int(streaming_kv), int(gemm_tile), int(unfused_decode), int(handover_spin_limit), int(weight_arena))
         self.weights = weights  # keep the tensors alive
         if kv is None:
             shape = (batch, cfg["n_kv_heads"], cfg["max_seq"], cfg["head_dim"])

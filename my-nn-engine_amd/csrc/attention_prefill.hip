@@ -2,7 +2,9 @@
 // reference's attention_tc (attention.cuh:45-314: mma.m16n8k16, S and P round-tripping through
 // shared memory, 16 lanes doing the softmax serially).
 //
-// One workgroup = 4 waves = 128 query rows of one (batch, query head); each wave owns 32 rows.
+// One workgroup = 4 waves = 128 query rows of one (batch, query head); each wave owns 32 rows.  Two workgroups
+// per CU (two waves per SIMD, up to 256 registers a lane: at three the kernel spilled into scratch inside the
+// key loop).  Workgroups are dispatched longest first: grid y = query block, last block (most keys) first.
 // Per 64-key tile (staged once in LDS for the four waves, K row-major, V transposed; two 32-key S^T tiles):
 //   S^T = K . Q^T      v_mfma_f32_32x32x16: A = K rows from LDS, B = Q kept in registers
 //   softmax            each lane owns ONE query column and 16 of the 32 keys of each S^T tile, so the
@@ -11,7 +13,10 @@
 //                      contracted in the permuted order 4g+0..3, 8+4g+0..3), so P never leaves
 //                      registers; A = V^T read from LDS with two 8-byte reads
 // The rescale factor of the online softmax is a per-lane scalar because O^T keeps the same query
-// column per lane.  Key tiles past a wave's last causal position are skipped.
+// column per lane; the rescale is skipped when no lane of the wave moved its maximum (most tiles after the
+// first few).  Key tiles past a wave's last causal position are skipped.
+// A thread stages CH neighbouring keys of the same 8 dims, so V^T goes to LDS CH keys at a time (4- or 8-byte
+// writes of values gathered with v_perm) instead of one 2-byte write per value.
 #include <type_traits>
 
 #include "attention.h"
@@ -22,26 +27,27 @@ namespace mynn {
 constexpr int kPfThreads = 256, kPfRows = 128, kPfKeys = 64;
 
 template <typename T, int D>
-__global__ __launch_bounds__(kPfThreads, D == 64 ? 3 : 2) void attn_prefill_kernel(AttnParams p) {
+__global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_kernel(AttnParams p) {
     constexpr int LDK = D + 8;          // K tile row stride (elements): conflict-free 16-byte reads
     constexpr int LDV = kPfKeys + 4;    // V^T tile row stride
     constexpr int KS = D / 16;          // k-steps of the S^T product
     constexpr int DT = D / 32;          // 32-row tiles of O^T
-    constexpr int CH = (kPfKeys * D / 8) / kPfThreads;  // 16-byte chunks per thread and tile (2 or 4)
-    static_assert(CH >= 1, "tile smaller than the workgroup");
+    constexpr int CH = (kPfKeys * D / 8) / kPfThreads;  // 16-byte chunks per thread and tile (2 or 4): neighbouring keys
+    constexpr int NPF = D == 64 ? 2 : 1;                // tiles in flight in registers ahead of the one in LDS
+    static_assert(CH == 2 || CH == 4, "a thread stages 2 or 4 neighbouring keys");
     __shared__ __align__(16) uint16_t Ks[2][kPfKeys * LDK];
     __shared__ __align__(16) uint16_t Vt[2][D * LDV];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, g = lane >> 5;
-    const int bh = blockIdx.y, b = bh / p.Hq, h = bh % p.Hq;
+    const int bh = blockIdx.x, b = bh / p.Hq, h = bh % p.Hq;
     const int G = p.Hq / p.Hkv, hkv = h / G;
     const int Sq = p.Sq;
     const int active = p.d_active ? *p.d_active : p.active;
     const int qoff = p.d_active ? active - Sq : p.q_pos_offset;
     const int kv_bound = min(active, p.cache_len);
 
-    const int q_blk = blockIdx.x * kPfRows;
+    const int q_blk = ((int)gridDim.y - 1 - (int)blockIdx.y) * kPfRows;  // the blocks with the most keys are dispatched first
     const int qrow = q_blk + wave * 32 + col;           // this lane's query row
     const int qrow_c = min(qrow, Sq - 1);
     // keys this lane's query may see, and the furthest any row of the wave / workgroup may see
@@ -60,29 +66,35 @@ __global__ __launch_bounds__(kPfThreads, D == 64 ? 3 : 2) void attn_prefill_kern
 
     const T *Kg = (const T *)p.k + (size_t)(b * p.Hkv + hkv) * p.cache_len * D;
     const T *Vg = (const T *)p.v + (size_t)(b * p.Hkv + hkv) * p.cache_len * D;
-    // a tile travels global -> registers (one iteration ahead of) -> LDS (one iteration ahead of) the MFMAs.
+    // a tile travels global -> registers (NPF iterations ahead of) -> LDS (one iteration ahead of) the MFMAs.
+    // Thread t stages the keys CH * (t / (D/8)) + 0 .. CH-1 of a tile, dims 8 * (t % (D/8)) .. +7.
     // Rows past the end are clamped to the last visible key: whatever they hold is masked out.
-    U4 rk[CH], rv[CH];
-    auto load_tile = [&](int t) {
+    const int key0 = (tid / (D / 8)) * CH, dd = (tid % (D / 8)) * 8;
+    U4 rk[NPF][CH], rv[NPF][CH];
+    auto load_tile = [&](int t, U4 *k_, U4 *v_) {
 #pragma unroll
         for (int c = 0; c < CH; c++) {
-            const int chunk = tid + c * kPfThreads;
-            const int key = min(t * kPfKeys + chunk / (D / 8), blk_bound - 1), dd = (chunk % (D / 8)) * 8;
-            rk[c] = *(const U4 *)(Kg + (size_t)key * D + dd);
-            rv[c] = *(const U4 *)(Vg + (size_t)key * D + dd);
+            const int key = min(t * kPfKeys + key0 + c, blk_bound - 1);
+            k_[c] = *(const U4 *)(Kg + (size_t)key * D + dd);
+            v_[c] = *(const U4 *)(Vg + (size_t)key * D + dd);
         }
     };
-    auto store_tile = [&](int buf) {
+    auto store_tile = [&](int buf, const U4 *k_, const U4 *v_) {
 #pragma unroll
-        for (int c = 0; c < CH; c++) {
-            const int chunk = tid + c * kPfThreads;
-            const int kk = chunk / (D / 8), dd = (chunk % (D / 8)) * 8;
-            *(U4 *)&Ks[buf][kk * LDK + dd] = rk[c];
-            const uint32_t w[4] = {rv[c].x, rv[c].y, rv[c].z, rv[c].w};
+        for (int c = 0; c < CH; c++) *(U4 *)&Ks[buf][(key0 + c) * LDK + dd] = k_[c];
+        // V^T[d][key0 .. key0 + CH - 1] for the 8 dims: dword i of a chunk holds dims 2i (low half) and 2i + 1
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                Vt[buf][(dd + 2 * i) * LDV + kk] = (uint16_t)(w[i] & 0xFFFFu);
-                Vt[buf][(dd + 2 * i + 1) * LDV + kk] = (uint16_t)(w[i] >> 16);
+        for (int i = 0; i < 4; i++) {
+            uint32_t w[CH];
+#pragma unroll
+            for (int c = 0; c < CH; c++) w[c] = i == 0 ? v_[c].x : i == 1 ? v_[c].y : i == 2 ? v_[c].z : v_[c].w;
+            uint16_t *lo = &Vt[buf][(dd + 2 * i) * LDV + key0], *hi = &Vt[buf][(dd + 2 * i + 1) * LDV + key0];
+            if constexpr (CH == 2) {
+                *(uint32_t *)lo = __builtin_amdgcn_perm(w[1], w[0], 0x05040100u);
+                *(uint32_t *)hi = __builtin_amdgcn_perm(w[1], w[0], 0x07060302u);
+            } else {
+                *(uint2 *)lo = uint2{__builtin_amdgcn_perm(w[1], w[0], 0x05040100u), __builtin_amdgcn_perm(w[3], w[2], 0x05040100u)};
+                *(uint2 *)hi = uint2{__builtin_amdgcn_perm(w[1], w[0], 0x07060302u), __builtin_amdgcn_perm(w[3], w[2], 0x07060302u)};
             }
         }
     };
@@ -148,10 +160,13 @@ __global__ __launch_bounds__(kPfThreads, D == 64 ? 3 : 2) void attn_prefill_kern
             l = fmaf(l, corr, ls);
             m = mn;
         }
+        // (a factor of exactly 1 in every lane leaves O^T as it is: the multiplications are skipped)
+        if (__builtin_amdgcn_ballot_w64(corr != 1.f) != 0) {
 #pragma unroll
-        for (int t2 = 0; t2 < DT; t2++)
+            for (int t2 = 0; t2 < DT; t2++)
 #pragma unroll
-            for (int e = 0; e < 16; e++) o[t2][e] *= corr;
+                for (int e = 0; e < 16; e++) o[t2][e] *= corr;
+        }
         // ---- O^T += V^T . P^T, keys contracted in the order the D-layout delivers them
 #pragma unroll
         for (int st = 0; st < 4; st++) {
@@ -167,21 +182,42 @@ __global__ __launch_bounds__(kPfThreads, D == 64 ? 3 : 2) void attn_prefill_kern
             }
         }
     };
+    auto compute = [&](int t) {
+        const int k0 = t * kPfKeys;
+        if (k0 + kPfKeys <= wave_all) tile(t & 1, k0, std::false_type{});
+        else if (k0 < wave_bound) tile(t & 1, k0, std::true_type{});
+    };
 
+    // tile 0 goes straight to LDS; tiles 1 .. NPF wait in registers (slot j holds tile 1 + j, then 1 + j + NPF, ..)
     if (ntiles > 0) {
-        load_tile(0);
-        store_tile(0);
-        if (ntiles > 1) load_tile(1);
+        load_tile(0, rk[0], rv[0]);
+        store_tile(0, rk[0], rv[0]);
+#pragma unroll
+        for (int j = 0; j < NPF; j++) load_tile(min(1 + j, ntiles - 1), rk[j], rv[j]);
     }
     __syncthreads();
-    for (int t = 0; t < ntiles; t++) {
-        const int buf = t & 1;
-        if (t + 1 < ntiles) store_tile(buf ^ 1);  // tile t+1, loaded an iteration ago; its buffer was released by the last barrier
-        if (t + 2 < ntiles) load_tile(t + 2);
-        const int k0 = t * kPfKeys;
-        if (k0 + kPfKeys <= wave_all) tile(buf, k0, std::false_type{});
-        else if (k0 < wave_bound) tile(buf, k0, std::true_type{});
-        __syncthreads();
+    int t = 0;
+    // groups of NPF iterations that all still issue a load (unconditional, so the waits on older loads can be counted)
+    for (; t + 2 * NPF < ntiles; t += NPF) {
+#pragma unroll
+        for (int j = 0; j < NPF; j++) {
+            store_tile((t + j + 1) & 1, rk[j], rv[j]);  // tile t + j + 1, loaded NPF iterations ago; its buffer was released by the last barrier
+            load_tile(t + j + 1 + NPF, rk[j], rv[j]);   // (< ntiles by the loop bound)
+            compute(t + j);
+            __syncthreads();
+        }
+    }
+    // the rest: every tile still missing from LDS is in registers already or on its way
+    for (; t < ntiles; t += NPF) {
+#pragma unroll
+        for (int j = 0; j < NPF; j++) {
+            if (t + j < ntiles) {
+                if (t + j + 1 < ntiles) store_tile((t + j + 1) & 1, rk[j], rv[j]);
+                if (t + j + 1 + NPF < ntiles) load_tile(t + j + 1 + NPF, rk[j], rv[j]);
+                compute(t + j);
+                __syncthreads();
+            }
+        }
     }
 
     // ---- out[query, d] = O^T[d, query] / l
@@ -214,8 +250,8 @@ bool attention_prefill_supported(const AttnParams &p, int D, int dtype, int kv_i
 }
 
 int attention_prefill_launch(const AttnParams &p, int D, int dtype, hipStream_t s) {
-    MYNN_REQUIRE(p.B * p.Hq <= 65535, MYNN_ERR_UNSUPPORTED, "attention: batch*heads = %d exceeds the grid", p.B * p.Hq);
-    dim3 grid((p.Sq + kPfRows - 1) / kPfRows, p.B * p.Hq);
+    MYNN_REQUIRE((p.Sq + kPfRows - 1) / kPfRows <= 65535, MYNN_ERR_UNSUPPORTED, "attention: Sq = %d exceeds the grid", p.Sq);
+    dim3 grid(p.B * p.Hq, (p.Sq + kPfRows - 1) / kPfRows);
     return dispatch_dtype16(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
         if (D == 64) MYNN_LAUNCH((attn_prefill_kernel<T, 64>), grid, dim3(kPfThreads), 0, s, p);

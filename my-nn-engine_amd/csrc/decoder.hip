@@ -144,6 +144,7 @@ struct Model {
     int64_t *d_kvpos = nullptr;
     void *q_ref = nullptr, *k_new = nullptr, *v_new = nullptr, *attn_ref = nullptr, *k_rot = nullptr;
     int last_status = 0;          // of the last model() call on this state
+    void *warena = nullptr;       // weight_arena: every linear weight and scale of the model in one allocation, in execution order
     void *ws = nullptr;           // executors that dequantise a weight per call (M >= 16, no resident copy): their own workspace
     // per-launch record of the last enqueue (names + algorithmic bytes), events when profiling
     std::vector<Launch> record;
@@ -590,6 +591,32 @@ static int build(Model &m, void **init, void **state) {
     MYNN_HIP(hipStreamCreateWithFlags(&m.stream, hipStreamNonBlocking));
     TRY(host_rope_tables(m));
 
+    if (c.weight_arena && m.quant) {
+        // One allocation for every int8 linear weight and its scales, in the order a step reads them (the caller's o / down /
+        // lm_head buffers are copied, like q|k|v and gate/up already are): an explicit repack, done once.
+        struct Piece { const void **slot; size_t bytes; };
+        std::vector<Piece> pieces;
+        auto add = [&](Lin &l) {
+            pieces.push_back({&l.w, (size_t)l.N * l.K});
+            pieces.push_back({&l.scale, (size_t)l.N * eb});
+        };
+        for (Layer &L : m.layers) { add(L.qkv); add(L.o); add(L.gu); add(L.down); }
+        add(m.lm_head);
+        size_t total = 0;
+        for (const Piece &pc : pieces) total += align_up(pc.bytes, 256);
+        MYNN_HIP(hipMalloc(&m.warena, total));
+        size_t off = 0;
+        for (const Piece &pc : pieces) {
+            MYNN_HIP(hipMemcpy((char *)m.warena + off, *pc.slot, pc.bytes, hipMemcpyDeviceToDevice));
+            *pc.slot = (char *)m.warena + off;
+            off += align_up(pc.bytes, 256);
+        }
+        for (Layer &L : m.layers) {  // the separate repacked copies are not needed any more
+            (void)hipFree(L.own_qkv_w); (void)hipFree(L.own_qkv_s); (void)hipFree(L.own_gu_w); (void)hipFree(L.own_gu_s);
+            L.own_qkv_w = L.own_qkv_s = L.own_gu_w = L.own_gu_s = nullptr;
+        }
+    }
+
     // ---- prefill executors keep every linear weight dequantised to the 16-bit type (2 bytes per weight
     // on top of the int8 originals): the matrix-core GEMM reads them directly, and the values are
     // those of the per-call dequantisation, T(wq * scale)
@@ -799,6 +826,7 @@ static void destroy(Model *m) {
         if (L.pk_down) hipFree(L.pk_down);
     }
     if (m->ws) hipFree(m->ws);
+    if (m->warena) hipFree(m->warena);
     if (m->wt_lm_head) hipFree(m->wt_lm_head);
     if (m->pk_lm_head) hipFree(m->pk_lm_head);
     if (m->cos_t) hipFree(m->cos_t);
