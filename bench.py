@@ -155,15 +155,21 @@ def summarize_rocprof(args):
                 kern[n][which + "_kib"] = tot / cnt
                 kern[n][which + "_factor"] = 262144.0 / per
     if args.pmc_mfma:
-        # SQ_VALU_MFMA_BUSY_CYCLES (summed over the SIMDs) against GRBM_GUI_ACTIVE (summed over the 8 XCDs): the share of
-        # SIMD clocks (1024 SIMDs) in which the matrix pipe is busy
+        # SQ_VALU_MFMA_BUSY_CYCLES (summed over the 1024 SIMDs) against GRBM_GUI_ACTIVE (summed over the 8 XCDs): the share
+        # of SIMD clocks in which the matrix pipe is busy; and against the dispatch's own duration at the 2.4 GHz the
+        # published peak is quoted at (the two differ by the clock the kernel actually ran at)
         acc = {}
         for r in rows(args.pmc_mfma, "counter_collection.csv"):
-            a = acc.setdefault(r["Kernel_Name"], {})
+            a = acc.setdefault(kname(r), {"ns": 0.0})
             a[r["Counter_Name"]] = a.get(r["Counter_Name"], 0.0) + float(r["Counter_Value"])
+            if r["Counter_Name"] == "SQ_VALU_MFMA_BUSY_CYCLES":
+                a["ns"] += int(r["End_Timestamp"]) - int(r["Start_Timestamp"])
         for n, c in acc.items():
-            if n in kern and c.get("GRBM_GUI_ACTIVE"):
-                kern[n]["mfma_busy_frac"] = round(c.get("SQ_VALU_MFMA_BUSY_CYCLES", 0.0) / (c["GRBM_GUI_ACTIVE"] / 8.0 * 1024.0), 4)
+            if n in kern and c.get("GRBM_GUI_ACTIVE") and c["ns"] > 0:
+                busy = c.get("SQ_VALU_MFMA_BUSY_CYCLES", 0.0)
+                kern[n]["mfma_busy_frac"] = round(busy / (c["GRBM_GUI_ACTIVE"] / 8.0 * 1024.0), 4)
+                kern[n]["mfma_busy_frac_at_2p4ghz"] = round(busy / 1024.0 / (c["ns"] * 2.4), 4)
+                kern[n]["shader_clock_ghz"] = round(c["GRBM_GUI_ACTIVE"] / 8.0 / c["ns"], 3)
     out = {"workload": args.workload + ("_w8a8" if args.w8a8 else "") + ("_kv8" if args.kv_int8 else ""),
            "command": args.profile_command, "commit": args.profile_commit, "source_sha256": source_digest(),
            "calibration_copy_reading": copy, "kernels": []}
@@ -361,6 +367,8 @@ def attention_main(args, mynn):
     gpu_ms = start.elapsed_time(stop) / K  # launches are queued ahead of the GPU: this is device time per call
     nbytes = 2 * B * Hkv * L * D * 2 + 2 * B * Hq * D * 2
     achieved = nbytes / (gpu_ms * 1e-3) / 1e9
+    prof = load_profile("attention") if args.dtype == "f16" else None
+    entry = profile_entry(prof, "attention")  # (the streaming launch; the merge launch is listed in the profile beside it)
     out = {
         "metric": "GQA decode attention op: achieved HBM GB/s vs peak (configs[1], B=16, L=4096)",
         "value": round(achieved, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
@@ -369,7 +377,9 @@ def attention_main(args, mynn):
         "config": {"workload": "configs[1]: attention op, B=16, Hq=32, Hkv=4, D=64, L=4096, scale 0.125, seq_q=1",
                    "seed": args.seed, "rotating_kv_sets": n, "device_ms_per_call": round(gpu_ms, 4)},
         "roofline": {"bound": "hbm", "kernel": "attn_stream_kernel + attn_merge_kernel", "achieved": round(achieved, 1),
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic_bytes(entry),
+                     "avg_launch_us_rocprof": entry["avg_us"] if entry else None,
+                     "profile": {"file": prof["file"], "commit": prof.get("commit"), "stale": prof["stale"]} if prof and entry else None,
                      "bytes_per_launch": nbytes, "avg_launch_us": round(gpu_ms * 1e3, 2)},
     }
     if not args.no_cpu_baseline:

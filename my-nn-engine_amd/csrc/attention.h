@@ -23,6 +23,7 @@ struct AttnParams {
     // additive mask (operator slot 3), storage type: element (b * Hq + h) * mask_os + sq * mask_rs + key
     const void *mask;
     long mask_os, mask_rs;
+    int rope_q;               // prefill kernel: Q is un-rotated; rotate row sq by table row d_pos[sq] (cos_t, sin_t, d_pos above)
     const int32_t *d_past;    // fused decode form: cache row the new token is appended to (KVCacheUpdate's offset)
     float *part_o;            // [B*Hq*Sq, nsplit, D]
     float *part_ml;           // [B*Hq*Sq, nsplit, 2]

@@ -15,6 +15,8 @@
 // The rescale factor of the online softmax is a per-lane scalar because O^T keeps the same query
 // column per lane; the rescale is skipped when no lane of the wave moved its maximum (most tiles after the
 // first few).  Key tiles past a wave's last causal position are skipped.
+// rope_q: the queries are read un-rotated from the projection's output and rotated in registers (the RoPE launch
+// then only has the keys and values left to do).
 // A thread stages CH neighbouring keys of the same 8 dims, so V^T goes to LDS CH keys at a time (4- or 8-byte
 // writes of values gathered with v_perm) instead of one 2-byte write per value.
 #include <type_traits>
@@ -58,12 +60,6 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_kernel(AttnParams 
     const int blk_bound = p.is_causal ? min(kv_bound, qoff + blk_last + 1) : kv_bound;
     const int ntiles = (blk_bound + kPfKeys - 1) / kPfKeys;
 
-    // Q^T fragments: B operand, lane (query col, g): d = 16*ks + 8*g .. +7
-    const T *Q = (const T *)p.q + (size_t)b * p.q_bs + (size_t)h * p.q_hs + (size_t)qrow_c * p.q_rs;
-    U4 qf[KS];
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) qf[ks] = *(const U4 *)(Q + 16 * ks + 8 * g);
-
     const T *Kg = (const T *)p.k + (size_t)(b * p.Hkv + hkv) * p.cache_len * D;
     const T *Vg = (const T *)p.v + (size_t)(b * p.Hkv + hkv) * p.cache_len * D;
     // a tile travels global -> registers (NPF iterations ahead of) -> LDS (one iteration ahead of) the MFMAs.
@@ -98,6 +94,40 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_kernel(AttnParams 
             }
         }
     };
+
+    // the first tile's loads are on their way before the queries (and their RoPE table rows) are asked for
+    if (ntiles > 0) load_tile(0, rk[0], rv[0]);
+    // Q^T fragments: B operand, lane (query col, g): d = 16*ks + 8*g .. +7
+    const T *Q = (const T *)p.q + (size_t)b * p.q_bs + (size_t)h * p.q_hs + (size_t)qrow_c * p.q_rs;
+    U4 qf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) qf[ks] = *(const U4 *)(Q + 16 * ks + 8 * g);
+    if (p.rope_q) {
+        // the query rows arrive un-rotated (straight from the projection): RoPE by the row's position, the arithmetic of
+        // rope.cuh:18-46 -- lo' = lo*cos[j] - hi*sin[j], hi' = hi*cos[j + D/2] + lo*sin[j + D/2], separate products, one
+        // rounding.  Dims d and d + D/2 sit in fragments ks and ks + KS/2 of the same lane.
+        const size_t tab = (size_t)p.d_pos[qrow_c] * D;
+        const T *cs = (const T *)p.cos_t + tab, *sn = (const T *)p.sin_t + tab;
+#pragma unroll
+        for (int ks = 0; ks < KS / 2; ks++) {
+            const int d0 = 16 * ks + 8 * g;
+            float xl[8], xh[8], cl[8], ch[8], sl[8], sh[8], ol[8], oh[8];
+            widen8<T>(qf[ks], xl);
+            widen8<T>(qf[ks + KS / 2], xh);
+            widen8<T>(*(const U4 *)(cs + d0), cl);
+            widen8<T>(*(const U4 *)(cs + d0 + D / 2), ch);
+            widen8<T>(*(const U4 *)(sn + d0), sl);
+            widen8<T>(*(const U4 *)(sn + d0 + D / 2), sh);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                ol[i] = xl[i] * cl[i] - xh[i] * sl[i];
+                oh[i] = xh[i] * ch[i] + xl[i] * sh[i];
+            }
+            qf[ks] = U4{pack2<T>(ol[0], ol[1]), pack2<T>(ol[2], ol[3]), pack2<T>(ol[4], ol[5]), pack2<T>(ol[6], ol[7])};
+            qf[ks + KS / 2] = U4{pack2<T>(oh[0], oh[1]), pack2<T>(oh[2], oh[3]), pack2<T>(oh[4], oh[5]), pack2<T>(oh[6], oh[7])};
+        }
+    }
+
 
     f16x_t o[DT];
 #pragma unroll
@@ -190,7 +220,6 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_kernel(AttnParams 
 
     // tile 0 goes straight to LDS; tiles 1 .. NPF wait in registers (slot j holds tile 1 + j, then 1 + j + NPF, ..)
     if (ntiles > 0) {
-        load_tile(0, rk[0], rv[0]);
         store_tile(0, rk[0], rv[0]);
 #pragma unroll
         for (int j = 0; j < NPF; j++) load_tile(min(1 + j, ntiles - 1), rk[j], rv[j]);

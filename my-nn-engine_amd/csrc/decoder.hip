@@ -315,7 +315,9 @@ static int enqueue_step(Model &m) {
     const double eb = sizeof(T);
     const bool w8a8 = c.quantize_activations != 0, kv8 = c.quant_kv_cache != 0;
     const bool streaming = c.streaming_kv != 0;
-    const bool fused = m.quant && rows == 1 && !w8a8 && !kv8 && !streaming;
+    // batch-1 decode over int8 weights: the GEMVs carry RMSNorm, residual add and SwiGLU (also with an int8 KV cache, whose
+    // attention block then runs as RoPE + quantising append and the int8-KV attention kernel)
+    const bool fused = m.quant && rows == 1 && !w8a8 && !streaming;
     hipStream_t s = m.stream;
     m.record.clear();
     for (hipEvent_t e : m.events) hipEventDestroy(e);
@@ -381,21 +383,30 @@ static int enqueue_step(Model &m) {
             p.is_causal = S > 1; p.B = B; p.Sq = S; p.Hq = Hq; p.Hkv = Hkv; p.cache_len = c.max_seq;
             p.d_active = m.d_active; p.nsplit = m.nsplit; p.slice = m.slice; p.heads_per_wg = m.heads_per_wg;
             attn_token_major_layout(p, D);
-            const bool fuse_attn = fused && attention_fused_supported(D, Hq / Hkv);
+            const bool fuse_attn = fused && !kv8 && attention_fused_supported(D, Hq / Hkv);
             if (fuse_attn) {
                 // RoPE(q), RoPE(k), both cache appends and the attention in one launch
                 p.qkv = m.qkv; p.cos_t = m.cos_t; p.sin_t = m.sin_t; p.d_pos = m.d_pos; p.d_past = m.d_past;
                 note(m, "attention_rope_append", (double)(QD + 2 * KD) * eb + 2.0 * KD * eb + QD * eb);
                 TRY(attention_decode_launch(p, D, c.dtype, 0, m.attn_scratch, s));
             } else {
-                if (!roped) note(m, kv8 ? "rope_quant_kv_append" : "rope_kv_append", (double)rows * (QD + 2 * KD) * 2 * eb);
+                // prefill on the matrix cores: the attention kernel rotates the queries itself, reading them from the
+                // projection's output; the RoPE launch is left with the keys and the values
+                const bool pf = S > 1 && !kv8 && !roped && attention_prefill_supported(p, D, c.dtype, kv8);
+                const bool q_in_attn = pf && ((size_t)(QD + 2 * KD) * sizeof(T)) % 16 == 0 && aligned16(m.qkv);
+                if (!roped) note(m, kv8 ? "rope_quant_kv_append" : q_in_attn ? "rope_kv_append_k_v" : "rope_kv_append",
+                                 q_in_attn ? (double)rows * 2 * KD * 2 * eb : (double)rows * (QD + 2 * KD) * 2 * eb);
                 if (roped) {
                 } else if (kv8)
                     TRY(rope_quant_kv_append<T>(m.q, (int8_t *)L.k_cache, (int8_t *)L.v_cache, L.k_scale, L.v_scale, m.qkv,
                                                 m.cos_t, m.sin_t, m.d_pos, m.d_past, B, S, Hq, Hkv, D, c.max_seq, s));
                 else
-                    TRY(rope_kv_append<T>(m.q, L.k_cache, L.v_cache, m.qkv, m.cos_t, m.sin_t, m.d_pos, m.d_past, 0, B, S,
+                    TRY(rope_kv_append<T>(q_in_attn ? nullptr : m.q, L.k_cache, L.v_cache, m.qkv, m.cos_t, m.sin_t, m.d_pos, m.d_past, 0, B, S,
                                           Hq, Hkv, D, c.max_seq, s));
+                if (q_in_attn) {
+                    p.q = m.qkv; p.rope_q = 1; p.cos_t = m.cos_t; p.sin_t = m.sin_t; p.d_pos = m.d_pos;
+                    p.q_bs = (long)S * (QD + 2 * KD); p.q_hs = D; p.q_rs = QD + 2 * KD;
+                }
                 // bytes: q in, out; the K/V rows read depend on the context, which the host does not
                 // know under replay -- callers add 2*KD*eb per cached row when they report
                 // flops: the causal half of QK^T and PV over the new rows alone (exact when past_len is 0)

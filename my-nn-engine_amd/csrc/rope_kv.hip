@@ -20,6 +20,7 @@ __global__ void rope_kv_append_kernel(T *q_out, T *k_cache, T *v_cache, const T 
     const size_t row = (size_t)b * S + s;
     const int width = (Hq + 2 * Hkv) * D;
     const T *src = qkv + row * width + (size_t)head * D;
+    if (head < Hq && !q_out) return;
     if (head < Hq + Hkv) {
         T *dst = head < Hq ? q_out + row * (size_t)Hq * D + (size_t)head * D
                            : k_cache + (((size_t)b * Hkv + (head - Hq)) * max_seq + past + s) * D;
@@ -52,7 +53,8 @@ __global__ __launch_bounds__(256) void rope_kv_append_vec_kernel(T *q_out, T *k_
     const int heads = Hq + 2 * Hkv;
     const T *src_row = qkv + row * (size_t)heads * D;
     const size_t tab = (size_t)position[s] * D;
-    for (int u = threadIdx.x; u < heads * upc; u += blockDim.x) {
+    // (q_out == nullptr: the queries are rotated by their consumer; only k and v are done here)
+    for (int u = threadIdx.x + (q_out ? 0 : Hq * upc); u < heads * upc; u += blockDim.x) {
         const int head = u / upc, j = (u % upc) * 8;
         const T *src = src_row + (size_t)head * D;
         const U4 lo = *(const U4 *)(src + j), hi = *(const U4 *)(src + j + half);
@@ -157,9 +159,9 @@ int rope_kv_append(void *q_out, void *k_cache, void *v_cache, const void *qkv, c
                    const int64_t *position, const int32_t *d_past, int past_host, int B, int S, int Hq, int Hkv, int D,
                    int max_seq, hipStream_t s) {
     MYNN_REQUIRE(S <= 65535 * 32 && Hq + 2 * Hkv <= 65535 && B <= 65535, MYNN_ERR_UNSUPPORTED, "rope_kv_append: grid");
-    if (D % 16 == 0 && S <= 65535 * 32 && aligned16(q_out) && aligned16(k_cache) && aligned16(v_cache) && aligned16(qkv) &&
+    if (D % 16 == 0 && S <= 65535 * 32 && (!q_out || aligned16(q_out)) && aligned16(k_cache) && aligned16(v_cache) && aligned16(qkv) &&
         aligned16(cos_t) && aligned16(sin_t)) {
-        const int units = (Hq + 2 * Hkv) * (D / 16);
+        const int units = (q_out ? Hq + 2 * Hkv : 2 * Hkv) * (D / 16);
         const int threads = units >= 256 ? 256 : (units + 63) / 64 * 64;
         MYNN_LAUNCH(rope_kv_append_vec_kernel<T>, dim3(S, B), dim3(threads), 0, s, (T *)q_out, (T *)k_cache,
                            (T *)v_cache, (const T *)qkv, (const T *)cos_t, (const T *)sin_t, position, d_past, past_host,
