@@ -15,6 +15,7 @@
 //   RESIDUAL  out = T(T(acc*scale) + residual[n])            (the Add that follows o/down proj)
 //   SWIGLU    rows interleaved gate,up: out[i] = T(silu(T(g)) * T(u))  (Swish+Mul group)
 #include "kernels.h"
+#include "gemv_dot.h"
 
 namespace mynn {
 
@@ -309,9 +310,7 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(const int8_
 #pragma unroll
                     for (int i = 0; i < 8; i++) f[q][i] = Elem<T>::rnd((f[q][i] * inv) * nw[i]);
                 }
-                float4 *dst = (float4 *)(act_lds + pc * 8);
-                dst[0] = float4{f[q][0], f[q][1], f[q][2], f[q][3]};
-                dst[1] = float4{f[q][4], f[q][5], f[q][6], f[q][7]};
+                gemv_stage_piece<T>(act_lds, K, pc, f[q]);
             }
         }
     }
@@ -320,51 +319,32 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(const int8_
     T *out = (T *)p.out;
     auto compute = [&](int gg, Group &G) {
         float acc[R];
-#pragma unroll
-        for (int r = 0; r < R; r++) acc[r] = 0.f;
-#pragma unroll
-        for (int j = 0; j < NC; j++) {
-            const int c = lane + j * kWave;
-            if (c < nchunks) {
-                float a[16];
-                const float4 *ap = (const float4 *)(act_lds + c * 16);
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    float4 t = ap[q];
-                    a[4 * q] = t.x; a[4 * q + 1] = t.y; a[4 * q + 2] = t.z; a[4 * q + 3] = t.w;
-                }
-#pragma unroll
-                for (int r = 0; r < R; r++) {
-                    float wf[16];
-                    pin(G.w[r][j]);
-                    widen16_i8(G.w[r][j], wf);
-#pragma unroll
-                    for (int i = 0; i < 16; i++) acc[r] = fmaf(a[i], wf[i], acc[r]);
-                }
-            }
-        }
+        gemv_rows_dot<T, R, NC>(act_lds, K, lane, G.w, acc);
 #pragma unroll
         for (int r = 0; r < R; r++) acc[r] = wave_sum(acc[r]);
         const int row0 = gg * R;
-        if constexpr (EPI == EPI_SWIGLU) {
+        // lane r finishes row r (SwiGLU: lane r = 0, 2, .. the pair r, r + 1): one pass for all rows of the group
+        float mine = acc[0], next = R > 1 ? acc[1] : 0.f;
 #pragma unroll
-            for (int r = 0; r < R; r += 2) {
-                if (lane == r && row0 + r + 1 < N) {
-                    float gt = Elem<T>::rnd(acc[r] * Elem<T>::ld(&G.sc, 0));
-                    float up = Elem<T>::rnd(acc[r + 1] * Elem<T>::ld(&G.sc1, 0));
-                    float sig = 1.0f / (1.0f + expf(-gt));
-                    Elem<T>::st(out, (size_t)((row0 + r) >> 1), (gt * sig) * up);
-                }
+        for (int r = 1; r < R; r++) {
+            if (lane == r) {
+                mine = acc[r];
+                if (r + 1 < R) next = acc[r + 1];
+            }
+        }
+        if constexpr (EPI == EPI_SWIGLU) {
+            if (lane < R && (lane & 1) == 0 && row0 + lane + 1 < N) {
+                float gt = Elem<T>::rnd(mine * Elem<T>::ld(&G.sc, 0));
+                float up = Elem<T>::rnd(next * Elem<T>::ld(&G.sc1, 0));
+                float sig = 1.0f / (1.0f + expf(-gt));
+                Elem<T>::st(out, (size_t)((row0 + lane) >> 1), (gt * sig) * up);
             }
         } else {
-#pragma unroll
-            for (int r = 0; r < R; r++) {
-                if (lane == r && row0 + r < N) {
-                    float y = acc[r] * Elem<T>::ld(&G.sc, 0);
-                    if constexpr (EPI == EPI_RESIDUAL) y = Elem<T>::rnd(y) + Elem<T>::ld(&G.res, 0);
-                    Elem<T>::st(out, row0 + r, y);
-                    if constexpr (ARGMAX) argmax_take(bv, bi, Elem<T>::rnd(y), row0 + r);  // (the value as stored)
-                }
+            if (lane < R && row0 + lane < N) {
+                float y = mine * Elem<T>::ld(&G.sc, 0);
+                if constexpr (EPI == EPI_RESIDUAL) y = Elem<T>::rnd(y) + Elem<T>::ld(&G.res, 0);
+                Elem<T>::st(out, row0 + lane, y);
+                if constexpr (ARGMAX) argmax_take(bv, bi, Elem<T>::rnd(y), row0 + lane);  // (the value as stored)
             }
         }
     };

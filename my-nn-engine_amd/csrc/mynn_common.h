@@ -101,23 +101,39 @@ __device__ inline void widen16_i8(const U4 &v, float *f) {
 }
 
 // ---- wave64 reductions ------------------------------------------------------------------------
-__device__ inline float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
-}
-__device__ inline float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
-    return v;
-}
-// sum over the lanes of an aligned group of `width` lanes (power of two <= 64)
-// (value of another lane of the same row of 16 through the data-parallel-primitive path: no LDS instruction, no wait)
+// (value of another lane through the data-parallel-primitive path: no LDS instruction, no wait)
 template <int CTRL> __device__ inline float dpp_get(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
 }
+// the same for the rows of 16 lanes named by ROWS (bit r = row r); the other rows get `other`
+template <int CTRL, int ROWS> __device__ inline float dpp_rows(float v, float other) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, other), __builtin_bit_cast(int, v), CTRL, ROWS, 0xF, false));
+}
 constexpr int kDppXor1 = 0xB1, kDppXor2 = 0x4E;     // quad_perm [1,0,3,2] / [2,3,0,1]
 constexpr int kDppHalfMirror = 0x141, kDppMirror = 0x140, kDppRor8 = 0x128;  // lane i <- 7-i (per 8) / 15-i / i^8
+constexpr int kDppBcast15 = 0x142, kDppBcast31 = 0x143;  // lane 15 of a row to the next row / lane 31 to rows 2 and 3
+// Sum / maximum over the wave, the same value in every lane: a butterfly inside each row of 16 (after the steps
+// inside a quad every lane of a quad holds the quad's sum, so the mirrored lane of the other quad (half row) stands
+// for lane ^ 4 (lane ^ 8)), then row 1 += row 0 and row 3 += row 2, rows 2 and 3 += row 1, and lane 63 is read back.
+__device__ inline float wave_sum(float v) {
+    v += dpp_get<kDppXor1>(v);
+    v += dpp_get<kDppXor2>(v);
+    v += dpp_get<kDppHalfMirror>(v);
+    v += dpp_get<kDppMirror>(v);
+    v += dpp_rows<kDppBcast15, 0xA>(v, 0.f);
+    v += dpp_rows<kDppBcast31, 0xC>(v, 0.f);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+__device__ inline float wave_max(float v) {
+    v = fmaxf(v, dpp_get<kDppXor1>(v));
+    v = fmaxf(v, dpp_get<kDppXor2>(v));
+    v = fmaxf(v, dpp_get<kDppHalfMirror>(v));
+    v = fmaxf(v, dpp_get<kDppMirror>(v));
+    v = fmaxf(v, dpp_rows<kDppBcast15, 0xA>(v, v));
+    v = fmaxf(v, dpp_rows<kDppBcast31, 0xC>(v, v));
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+// sum over the lanes of an aligned group of `width` lanes (power of two <= 64)
 template <int width> __device__ inline float group_sum(float v) {
     if constexpr (width <= 16) {
         // the same pairs as the xor butterfly: after the steps inside a quad every lane of a quad holds the quad's

@@ -16,6 +16,7 @@
 //
 // Reference ops: rms_norm.cuh:9-59, dequant_gemv.cuh:12-59, rope.cuh, kvcache.cuh, attention.cuh:495-513.
 #include "kernels.h"
+#include "gemv_dot.h"
 #include "attention_short.h"
 
 namespace mynn {
@@ -181,9 +182,7 @@ __device__ __forceinline__ void qa_gemv(const QaGemv &a, float *act_lds, float *
 #pragma unroll
                         for (int i = 0; i < 8; i++) f[q][i] = Elem<T>::rnd((f[q][i] * inv) * nw[i]);
                     }
-                    float4 *dst = (float4 *)(act_lds + pc * 8);
-                    dst[0] = float4{f[q][0], f[q][1], f[q][2], f[q][3]};
-                    dst[1] = float4{f[q][4], f[q][5], f[q][6], f[q][7]};
+                    gemv_stage_piece<T>(act_lds, K, pc, f[q]);
                 }
             }
         }
@@ -195,29 +194,7 @@ __device__ __forceinline__ void qa_gemv(const QaGemv &a, float *act_lds, float *
         if (!loaded) load_group(g, ga);
         loaded = false;
         float acc[R];
-#pragma unroll
-        for (int r = 0; r < R; r++) acc[r] = 0.f;
-#pragma unroll
-        for (int j = 0; j < NC; j++) {
-            const int c = lane + j * kWave;
-            if (c < nchunks) {
-                float av[16];
-                const float4 *ap = (const float4 *)(act_lds + c * 16);
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    float4 t = ap[q];
-                    av[4 * q] = t.x; av[4 * q + 1] = t.y; av[4 * q + 2] = t.z; av[4 * q + 3] = t.w;
-                }
-#pragma unroll
-                for (int r = 0; r < R; r++) {
-                    float wf[16];
-                    pin(ga.w[r][j]);
-                    widen16_i8(ga.w[r][j], wf);
-#pragma unroll
-                    for (int i = 0; i < 16; i++) acc[r] = fmaf(av[i], wf[i], acc[r]);
-                }
-            }
-        }
+        gemv_rows_dot<T, R, NC>(act_lds, K, lane, ga.w, acc);
 #pragma unroll
         for (int r = 0; r < R; r++) acc[r] = wave_sum(acc[r]);
         const int row = g * R + lane;

@@ -8,7 +8,8 @@ import oracle as orc
 
 mynn = importlib.import_module("my-nn-engine_amd")
 
-TOL = {orc.F32: 2e-5, orc.BF16: 1e-2, orc.F16: 1e-2}  # max-abs-rel bound for float outputs
+# max-abs-rel bound for float outputs (f32: two summation orders of a few thousand f32 terms; 16-bit: the reference's own bound)
+TOL = {orc.F32: 5e-5, orc.BF16: 1e-2, orc.F16: 1e-2}
 
 
 def torch_dtype(dt):

@@ -48,7 +48,7 @@ def test_dequant_gemv_vs_oracle(g, dt, N, K):
     ulp = {orc.F32: 2.0 ** -23, orc.BF16: 2.0 ** -8, orc.F16: 2.0 ** -10}[dt]
     assert np.all(np.abs(g.f32(got, dt) - exact) <= bound + np.abs(exact) * ulp + 1e-30)
     if dt != orc.F32:  # most elements agree with the oracle bit for bit; the rest are 1 ulp apart
-        assert np.mean(got == want) > 0.97
+        assert np.mean(got == want) > 0.95
 
 
 def test_dequant_gemv_mixed_types_cfg1(g):
