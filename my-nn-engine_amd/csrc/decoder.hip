@@ -107,6 +107,7 @@ struct Model {
     std::vector<Layer> layers;
     void *wt_lm_head = nullptr, *pk_lm_head = nullptr;
     bool w8a8_fused = false;  // W8A8 with the large int8 tiles: norm+quantise, residual and SwiGLU ride on the launches
+    bool qgemv1 = false;      // W8A8 at batch 1: norm, quantiser, int8 GEMV and residual / SwiGLU of a linear in one launch
     bool resident16 = false;  // the wt_* copies exist and the matrix-core path with fused stores is used
     bool skinny = false;      // 16..64 rows: int8 weights streamed once through the few-row matrix-core kernel
     float *skinny_scratch = nullptr;
@@ -318,6 +319,13 @@ static int enqueue_step(Model &m) {
     // batch-1 decode over int8 weights: the GEMVs carry RMSNorm, residual add and SwiGLU (also with an int8 KV cache, whose
     // attention block then runs as RoPE + quantising append and the int8-KV attention kernel)
     const bool fused = m.quant && rows == 1 && !w8a8 && !streaming;
+    // batch-1 decode with quantize_activations: norm + quantiser + int8 GEMV + residual / SwiGLU of a linear in one launch
+    const bool qfused = m.qgemv1 && rows == 1;
+    auto qlinear1 = [&](void *out, const void *act, const void *norm_w, const Lin &l, const void *res, int epi, const char *name) {
+        const int n_out = epi == GEMM_SWIGLU ? l.N / 2 : l.N;
+        note(m, name, (double)l.N * l.K + l.K * eb + l.N * eb + (double)n_out * eb * (res ? 2 : 1) + (norm_w ? l.K * eb : 0.0), 2.0 * l.N * l.K);
+        return qgemv_fused(out, act, norm_w, c.eps, (const int8_t *)l.w, l.scale, res, l.N, l.K, c.dtype, epi, m.stream);
+    };
     hipStream_t s = m.stream;
     m.record.clear();
     for (hipEvent_t e : m.events) hipEventDestroy(e);
@@ -356,6 +364,8 @@ static int enqueue_step(Model &m) {
         } else if (fused) {
             note(m, "gemv_norm_qkv", (double)L.qkv.N * H + L.qkv.N * eb + 2 * H * eb + L.qkv.N * eb);
             TRY(gemv_norm<T>(m.qkv, m.x, L.norm1, c.eps, (const int8_t *)L.qkv.w, L.qkv.scale, L.qkv.N, H, s));
+        } else if (qfused) {
+            TRY(qlinear1(m.qkv, m.x, L.norm1, L.qkv, nullptr, GEMM_PLAIN, "qgemv_norm_quant_qkv"));
         } else if (m.w8a8_fused) {
             TRY(qlinear_fused(m, m.qkv, m.x, L.norm1, L.qkv.w, L.qkv.scale, nullptr, rows, L.qkv.N, H, GEMM_PLAIN, "qlinear_qkv"));
         } else {
@@ -383,7 +393,7 @@ static int enqueue_step(Model &m) {
             p.is_causal = S > 1; p.B = B; p.Sq = S; p.Hq = Hq; p.Hkv = Hkv; p.cache_len = c.max_seq;
             p.d_active = m.d_active; p.nsplit = m.nsplit; p.slice = m.slice; p.heads_per_wg = m.heads_per_wg;
             attn_token_major_layout(p, D);
-            const bool fuse_attn = fused && !kv8 && attention_fused_supported(D, Hq / Hkv);
+            const bool fuse_attn = (fused || qfused) && !kv8 && attention_fused_supported(D, Hq / Hkv);
             if (fuse_attn) {
                 // RoPE(q), RoPE(k), both cache appends and the attention in one launch
                 p.qkv = m.qkv; p.cos_t = m.cos_t; p.sin_t = m.sin_t; p.d_pos = m.d_pos; p.d_past = m.d_past;
@@ -438,6 +448,10 @@ static int enqueue_step(Model &m) {
             TRY(skinny_rows(m, m.hmid, m.nrm, L.gu, L.pk_gu, nullptr, rows, GEMM_SWIGLU, "linear_gateup_swiglu"));
             const void *next_norm = li + 1 < m.layers.size() ? m.layers[li + 1].norm1 : m.final_norm;
             TRY(skinny_rows(m, m.x, m.hmid, L.down, L.pk_down, m.x2, rows, GEMM_RESIDUAL, "linear_down_residual", next_norm, &nrm_ready));
+        } else if (qfused) {
+            TRY(qlinear1(m.x2, m.attn, nullptr, L.o, m.x, GEMM_RESIDUAL, "qgemv_quant_o_residual"));
+            TRY(qlinear1(m.hmid, m.x2, L.norm2, L.gu, nullptr, GEMM_SWIGLU, "qgemv_norm_quant_gateup_swiglu"));
+            TRY(qlinear1(m.x, m.hmid, nullptr, L.down, m.x2, GEMM_RESIDUAL, "qgemv_quant_down_residual"));
         } else if (m.w8a8_fused) {
             TRY(qlinear_fused(m, m.x2, m.attn, nullptr, L.o.w, L.o.scale, m.x, rows, H, QD, GEMM_RESIDUAL, "qlinear_o_residual"));
             TRY(qlinear_fused(m, m.hmid, m.x2, L.norm2, L.q8_gu, L.q8_gu_scale, nullptr, rows, 2 * F, H, GEMM_SWIGLU, "qlinear_gateup_swiglu"));
@@ -488,6 +502,8 @@ static int enqueue_step(Model &m) {
     } else if (fused) {
         note(m, "gemv_norm_lm_head", (double)V * H + V * eb + 2 * H * eb + V * eb);
         TRY(gemv_norm<T>(m.logits, m.x, m.final_norm, c.eps, (const int8_t *)m.lm_head.w, m.lm_head.scale, V, H, s));
+    } else if (qfused) {
+        TRY(qlinear1(m.logits, m.x, m.final_norm, m.lm_head, nullptr, GEMM_PLAIN, "qgemv_norm_quant_lm_head"));
     } else if (m.w8a8_fused) {
         TRY(qlinear_fused(m, m.logits, m.x, m.final_norm, m.lm_head.w, m.lm_head.scale, nullptr, rows, V, H, GEMM_PLAIN, "qlinear_lm_head"));
     } else {
@@ -774,6 +790,18 @@ static int build(Model &m, void **init, void **state) {
             MYNN_HIP(hipDeviceSynchronize());
             m.qkv_attn = true;
         }
+    }
+
+    // ---- batch-1 decode with quantize_activations: one launch per linear (norm, quantiser, int8 GEMV, residual / SwiGLU)
+    if (m.quant && rows == 1 && c.quantize_activations && !c.streaming_kv && !c.unfused_decode && c.dtype != MYNN_F32) {
+        bool ok = qgemv_fused_supported(m.x, m.final_norm, (const int8_t *)m.lm_head.w, V, H) && aligned16(m.x2) && aligned16(m.attn) &&
+                  aligned16(m.hmid);
+        for (const Layer &L : m.layers)
+            ok = ok && qgemv_fused_supported(m.x, L.norm1, (const int8_t *)L.qkv.w, L.qkv.N, H) &&
+                 qgemv_fused_supported(m.attn, nullptr, (const int8_t *)L.o.w, H, QD) &&
+                 qgemv_fused_supported(m.x2, L.norm2, (const int8_t *)L.gu.w, 2 * F, H) &&
+                 qgemv_fused_supported(m.hmid, nullptr, (const int8_t *)L.down.w, H, F);
+        m.qgemv1 = ok;
     }
 
     return capture_step(m);

@@ -101,6 +101,12 @@ struct QkvAttnParams {
     int vocab;
 };
 bool qkv_attention_supported(int H, int Hq, int Hkv, int D, int max_seq, int dtype);
+
+// Batch-1 W8A8 linear in one launch (qgemv_fused.hip): (RMSNorm ->) per-row quantisation -> int8 x int8 GEMV ->
+// plain / residual / SwiGLU store.  norm_w null: no normalisation; epi: GEMM_PLAIN / GEMM_RESIDUAL / GEMM_SWIGLU
+bool qgemv_fused_supported(const void *act, const void *norm_w, const int8_t *wq, int N, int K);
+int qgemv_fused(void *out, const void *act, const void *norm_w, float eps, const int8_t *wq, const void *scale, const void *residual,
+                int N, int K, int dtype, int epi, hipStream_t s);
 int qkv_attention_launch(QkvAttnParams p, int D, int dtype, hipStream_t s);
 
 struct AdvanceState {

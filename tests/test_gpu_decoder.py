@@ -239,6 +239,10 @@ def test_int8_kv_cache_and_w8a8_executor_vs_oracle(g, dt, kv8, w8a8):
     ref.set_gemm_mode(2)
     dw = dev_weights(g, w, dt)
     dec = g.mynn.Decoder(cfg, dw, quant_kv_cache=kv8, quantize_activations=w8a8)
+    if w8a8:
+        # batch-1 decode: norm, quantiser, int8 GEMV and residual / SwiGLU of a linear are one launch (qkv, o, gate/up,
+        # down), the attention block one (16-bit cache) or two (int8 cache) more; embedding, lm_head, greedy token
+        assert dec.stats()["launches_per_step"] == (6 if kv8 else 5) * cfg["n_layers"] + 3, dec.stats()
     pre = g.mynn.Decoder(cfg, dw, seq_q=16, kv=dec.kv, quant_kv_cache=kv8, quantize_activations=w8a8)
     rng = np.random.default_rng(3)
     ids = rng.integers(0, cfg["vocab"], 16)
@@ -267,6 +271,32 @@ def test_int8_kv_cache_and_w8a8_executor_vs_oracle(g, dt, kv8, w8a8):
             assert max_abs_rel(g.f32(ks_gpu[:, :past], dt), g.f32(ks_ref[:, :past], dt)) <= 2e-2
             assert max_abs_rel(g.f32(vs_gpu[:, :past], dt), g.f32(vs_ref[:, :past], dt)) <= 2e-2
     pre.close(), dec.close()
+
+
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+def test_w8a8_batch1_one_launch_per_linear_vs_one_op_per_launch(g, dt):
+    """Options::quantize_activations at batch 1: the executor's default (a linear with its norm, quantiser and store in
+    one launch) against unfused_decode (RMSNorm, DynamicQuantizeLinear, QuantizedMatMul, Add / SwiGLU as launches of
+    their own) and against the oracle.  The two forms sum the squares of a row in different orders, so a normalised
+    value may differ by a spacing of T and with it an int8 code: they agree within the path's quantisation noise, not
+    bit for bit."""
+    cfg, w = llm_weights.synthetic_int8(SMALL, dt, seed=43)
+    ref = orc.Model(cfg, w)
+    ref.set_options(quant_kv_cache=False, quantize_activations=True)
+    dw = dev_weights(g, w, dt)
+    a = g.mynn.Decoder(cfg, dw, quantize_activations=True)
+    b = g.mynn.Decoder(cfg, dw, quantize_activations=True, unfused_decode=True)
+    assert a.stats()["launches_per_step"] == 5 * cfg["n_layers"] + 3
+    assert b.stats()["launches_per_step"] > 3 * a.stats()["launches_per_step"] - 10
+    for i, t in enumerate([11, 402, 77, 3, 950, 640, 12, 8]):
+        want = ref.forward([t], [i], i, i + 1, False)
+        na, la = a.step([t], [i], i, i + 1, want_logits=True)
+        nb, lb = b.step([t], [i], i, i + 1, want_logits=True)
+        assert max_err_rel_to_max(g.f32(la, dt), g.f32(want, dt)) <= 2e-2, i
+        assert max_err_rel_to_max(g.f32(lb, dt), g.f32(want, dt)) <= 2e-2, i
+        assert max_err_rel_to_max(g.f32(la, dt), g.f32(lb, dt)) <= 2e-2, i
+        assert na[0] == orc.argmax_last(la[0], dt) and nb[0] == orc.argmax_last(lb[0], dt)
+    a.close(), b.close()
 
 
 W8A8_LARGE = dict(n_layers=1, hidden=2048, n_heads=16, n_kv_heads=4, head_dim=128, ffn=1024, vocab=2048, max_seq=1024,
