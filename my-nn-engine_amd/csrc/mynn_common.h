@@ -115,6 +115,7 @@ constexpr int kDppBcast15 = 0x142, kDppBcast31 = 0x143;  // lane 15 of a row to 
 // Sum / maximum over the wave, the same value in every lane: a butterfly inside each row of 16 (after the steps
 // inside a quad every lane of a quad holds the quad's sum, so the mirrored lane of the other quad (half row) stands
 // for lane ^ 4 (lane ^ 8)), then row 1 += row 0 and row 3 += row 2, rows 2 and 3 += row 1, and lane 63 is read back.
+// Every lane of the wave must be active at the call (a DPP read of an inactive lane returns zero, and lane 63 is read).
 __device__ inline float wave_sum(float v) {
     v += dpp_get<kDppXor1>(v);
     v += dpp_get<kDppXor2>(v);

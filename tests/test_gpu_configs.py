@@ -171,6 +171,43 @@ def test_config4_llama3_8b_widths_batch32_decode_vs_per_sequence_oracles(g, benc
     torch.cuda.empty_cache()
 
 
+@pytest.mark.parametrize("variant", ["default", "kv_int8", "w8a8", "unfused"])
+def test_llama3_8b_widths_batch1_decode_vs_oracle(g, bench, variant):
+    """The Llama-3-8B widths at batch 1 (two layers; max_seq 512 so that the D = 128 short attention covers the cache):
+    the shared-launch decode step at hidden 4096 / ffn 14336 / vocab 128256 -- four 1024-element chunks per lane in the
+    projection roles, fourteen in the down projection, 16 k candidate words in the lm_head launch -- and the same model
+    with the int8 KV cache, with int8 activations and as one op per launch, each against the oracle with the same
+    options, 12 steps."""
+    import torch
+
+    dt = orc.F16
+    cfg = dict(LLAMA3_WIDTHS, dtype=dt, max_seq=512)
+    weights = bench.make_weights(cfg, dt, 777)
+    torch.cuda.synchronize()
+    host = bench.to_host_weights(weights)
+    kw = dict(default={}, kv_int8=dict(quant_kv_cache=True), w8a8=dict(quantize_activations=True), unfused=dict(unfused_decode=True))[variant]
+    dec = g.mynn.Decoder(cfg, weights, **kw)
+    L = cfg["n_layers"]
+    want_launches = dict(default=3 * L + 1, kv_int8=6 * L + 3, w8a8=5 * L + 3, unfused=5 * L + 3)[variant]
+    assert dec.stats()["graph"] and dec.stats()["launches_per_step"] == want_launches, dec.stats()
+    ref = orc.Model(dict(cfg), host)
+    ref.set_options(quant_kv_cache=variant == "kv_int8", quantize_activations=variant == "w8a8")
+    tol = 2e-2 if variant in ("kv_int8", "w8a8") else 1e-2
+    tok = 12345
+    for step in range(12):
+        want = ref.forward([tok], [step], step, step + 1, False)
+        nxt, got = dec.step([tok], [step], step, step + 1, want_logits=True)
+        assert max_err_rel_to_max(g.f32(got, dt), g.f32(want, dt)) <= tol, step
+        assert nxt[0] == orc.argmax_last(got[0], dt), step
+        tok = int(nxt[0])
+    # the device-resident loop continues the same stream
+    more = dec.decode_loop(tok, 12, 4)
+    assert len(more) == 4
+    dec.close()
+    del weights
+    torch.cuda.empty_cache()
+
+
 def test_config4_streaming_decode_attention_at_batch32_context_2048(g):
     """The attention of configs[4] at the benchmarked size: 32 sequences, 32 / 8 heads of 128 dims, 2048 cached
     keys of a 2304-row cache, fp16 and int8 caches, against the oracle and f64."""
