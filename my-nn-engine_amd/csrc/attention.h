@@ -46,6 +46,7 @@ inline void attn_token_major_layout(AttnParams &p, int D) {
 void attn_plan(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, int cache_len, bool fused,
                int *slice, int *nsplit, int *heads_per_wg);
 bool attention_fused_supported(int D, int G);
+bool attention_fused_kv8_supported(int D, int cache_len);
 size_t attn_scratch_bytes(int B, int Hq, int Sq, int D, int nsplit);
 int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *scratch, hipStream_t s);
 int attention_prefill_launch(const AttnParams &p, int D, int dtype, hipStream_t s);

@@ -286,7 +286,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnParams p)
 
 // ---- FUSE form for a cache that one workgroup covers in registers: one workgroup per query head, the
 // body is attn_short_body (attention_short.h)
-template <typename T, int D>
+template <typename T, int D, bool KV8>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_short_kernel(AttnParams p) {
     static_assert(kAttnWaves == kShortWaves, "the short form is written for 8 waves");
     __shared__ float part_s[kShortWaves][D + 2];
@@ -299,9 +299,11 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_short_kernel(AttnPar
     const T *row = (const T *)p.qkv + (size_t)b * (p.Hq + 2 * p.Hkv) * D;
     const size_t tab = (size_t)(*p.d_pos) * D;
     float r;
-    if (attn_short_body<T, D>(row + (size_t)h * D, row + (size_t)(p.Hq + hkv) * D, row + (size_t)(p.Hq + p.Hkv + hkv) * D,
-                              (T *)p.k + kv_base * D, (T *)p.v + kv_base * D, bound, *p.d_past, h % Gt == 0,
-                              (const T *)p.cos_t + tab, (const T *)p.sin_t + tab, p.scale, part_s, tid, r, [] {}))
+    using TKV = typename std::conditional<KV8, int8_t, T>::type;
+    if (attn_short_body<T, D, KV8>(row + (size_t)h * D, row + (size_t)(p.Hq + hkv) * D, row + (size_t)(p.Hq + p.Hkv + hkv) * D,
+                                   (TKV *)p.k + kv_base * D, (TKV *)p.v + kv_base * D, KV8 ? (T *)p.k_scale + kv_base : nullptr,
+                                   KV8 ? (T *)p.v_scale + kv_base : nullptr, bound, *p.d_past, h % Gt == 0,
+                                   (const T *)p.cos_t + tab, (const T *)p.sin_t + tab, p.scale, part_s, tid, r, [] {}))
         Elem<T>::st((T *)p.out, (size_t)b * p.o_bs + (size_t)h * p.o_hs + tid, r);
 }
 
@@ -378,6 +380,13 @@ bool attention_fused_supported(int D, int G) {
     return (D == 32 || D == 64 || D == 128) && (G == 1 || G == 2 || G == 4 || G == 8);
 }
 
+// the fused form over an int8 cache exists for caches one workgroup covers (attention_short.h)
+bool attention_fused_kv8_supported(int D, int cache_len) {
+    if (D != 64 && D != 128) return false;
+    const int kpp = kAttnWaves * (64 / (D / 8));
+    return cache_len <= kShortRounds * kShortPasses * kpp;
+}
+
 // Slice length, number of slices and query heads per workgroup for a launch.  kv_len = longest key
 // range any row can have.  All heads of a kv head share one workgroup (one K/V read) unless that
 // leaves fewer than ~64 workgroups; then the heads are divided, halving until there are enough.
@@ -423,13 +432,17 @@ int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *s
         using T = std::remove_pointer_t<decltype(t)>;
         if constexpr (sizeof(T) == 2) {
             if (fuse) {
-                if (kv_int8) return fail(MYNN_ERR_UNSUPPORTED, "fused decode attention: int8 KV");
                 if (attention_short_supported(p, D, dtype)) {
                     whole = true;
-                    if (D == 64) MYNN_LAUNCH((attn_decode_short_kernel<T, 64>), dim3(p.B * p.Hq), dim3(kAttnThreads), 0, s, p);
-                    else MYNN_LAUNCH((attn_decode_short_kernel<T, 128>), dim3(p.B * p.Hq), dim3(kAttnThreads), 0, s, p);
+                    MYNN_REQUIRE(!kv_int8 || (p.k_scale && p.v_scale), MYNN_ERR_INVALID, "fused decode attention: int8 KV without scales");
+                    const dim3 grid(p.B * p.Hq), block(kAttnThreads);
+                    if (D == 64 && kv_int8) MYNN_LAUNCH((attn_decode_short_kernel<T, 64, true>), grid, block, 0, s, p);
+                    else if (D == 64) MYNN_LAUNCH((attn_decode_short_kernel<T, 64, false>), grid, block, 0, s, p);
+                    else if (kv_int8) MYNN_LAUNCH((attn_decode_short_kernel<T, 128, true>), grid, block, 0, s, p);
+                    else MYNN_LAUNCH((attn_decode_short_kernel<T, 128, false>), grid, block, 0, s, p);
                     return launch_status("attn_decode_short_kernel");
                 }
+                if (kv_int8) return fail(MYNN_ERR_UNSUPPORTED, "fused decode attention: int8 KV beyond the short form");
                 return launch_d<T, false, true>(p, D, s);
             }
         } else {

@@ -24,25 +24,39 @@ constexpr int kShortWaves = 8;
 // part_s: kShortWaves x (D + 2) floats of LDS.  Every thread of the 512 calls it; threads tid < D get the
 // output dim tid in `result` and return true.  `ready()` runs once the cache loads are on their way and before
 // qsrc / ksrc / vsrc are read: a caller whose projection values arrive late waits for them there.
-template <typename T, int D, typename Ready>
-__device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, const T *vsrc, T *Kcache, T *Vcache, int bound,
-                                                int new_row, bool append, const T *cs, const T *snp, float scale,
+// KV8 (BuildOptions::quant_kv_cache): Kcache / Vcache hold int8 rows and Kscale / Vscale one scale of type T per row
+// (QuantizingKVCacheUpdate, kvcache.cuh): the new key and value are quantised as that operator does it (scale = amax /
+// 127 stored as T, codes rounded half away from zero), appended as codes, and met by the query as the codes times the
+// stored scale -- exactly what a later step reads back; a score is (q . codes) * k_scale * scale and a weight
+// exp(..) * v_scale, as the int8-KV attention operator computes them (attention.cuh:495-513 with its scale slots).
+template <typename T, int D, bool KV8 = false, typename Ready>
+__device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, const T *vsrc, void *Kcache_v, void *Vcache_v, T *Kscale,
+                                                T *Vscale, int bound, int new_row, bool append, const T *cs, const T *snp, float scale,
                                                 float (*part_s)[D + 2], int tid, float &result, Ready ready) {
     constexpr int LPK = D / 8, GPW = 64 / LPK, KPP = kShortWaves * GPW;  // lanes per key, keys per wave / workgroup and pass
     const int lane = tid & 63, wave = tid >> 6;
     const int dc = lane % LPK, grp = lane / LPK;
-    const T *Kc = Kcache + dc * 8, *Vc = Vcache + dc * 8;
+    using TKV = typename std::conditional<KV8, int8_t, T>::type;
+    using Chunk = typename std::conditional<KV8, uint2, U4>::type;  // this lane's 8 dims of a row
+    TKV *Kcache = (TKV *)Kcache_v, *Vcache = (TKV *)Vcache_v;
+    const TKV *Kc = Kcache + dc * 8, *Vc = Vcache + dc * 8;
 
     // ---- all K / V loads of this lane for a round of kShortPasses passes (the first round before anything else)
-    U4 kreg[kShortPasses], vreg[kShortPasses];
+    Chunk kreg[kShortPasses], vreg[kShortPasses];
+    T ksc[KV8 ? kShortPasses : 1], vsc[KV8 ? kShortPasses : 1];  // as loaded
     auto load_round = [&](int base) {
 #pragma unroll
         for (int i = 0; i < kShortPasses; i++) {
             const int key = base + i * KPP + wave * GPW + grp;
-            kreg[i] = vreg[i] = U4{0u, 0u, 0u, 0u};
+            kreg[i] = vreg[i] = Chunk{};
+            if constexpr (KV8) ksc[i] = vsc[i] = T{};
             if (key < bound && key != new_row) {
-                kreg[i] = *(const U4 *)(Kc + (size_t)key * D);
-                vreg[i] = *(const U4 *)(Vc + (size_t)key * D);
+                kreg[i] = *(const Chunk *)(Kc + (size_t)key * D);
+                vreg[i] = *(const Chunk *)(Vc + (size_t)key * D);
+                if constexpr (KV8) {
+                    ksc[i] = Kscale[key];
+                    vsc[i] = Vscale[key];
+                }
             }
         }
     };
@@ -81,9 +95,42 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
     }
     const U4 kn_packed = U4{pack2<T>(kn[0], kn[1]), pack2<T>(kn[2], kn[3]), pack2<T>(kn[4], kn[5]), pack2<T>(kn[6], kn[7])};
     const U4 q_packed = U4{pack2<T>(q[0], q[1]), pack2<T>(q[2], q[3]), pack2<T>(q[4], q[5]), pack2<T>(q[6], q[7])};
-    if (append && wave == 0 && grp == 0) {  // one lane group appends the new row
-        *(U4 *)(Kcache + (size_t)new_row * D + d0) = kn_packed;
-        *(U4 *)(Vcache + (size_t)new_row * D + d0) = v_new;
+    Chunk kn_q{}, vn_q{};       // KV8: the new row's codes (this lane's 8 dims)
+    float kn_sc = 0.f, vn_sc = 0.f;  // ... and its scales as stored
+    if constexpr (KV8) {
+        // per-row symmetric quantisation over the D values of the row (the lanes of this group)
+        auto quantise = [&](const float *x, Chunk &codes, float &stored_scale) {
+            float amax = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(x[e]));
+            amax = group_max<LPK>(amax);
+            const float inv = amax == 0.f ? 0.f : 127.0f / amax;
+            stored_scale = Elem<T>::rnd(amax * (1.0f / 127.0f));
+            uint32_t b[2] = {0u, 0u};
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float a = x[e] * inv;
+                int c = (int)(a + (a >= 0.f ? 0.5f : -0.5f));
+                c = c < -128 ? -128 : (c > 127 ? 127 : c);
+                b[e >> 2] |= ((uint32_t)c & 0xFFu) << (8 * (e & 3));
+            }
+            codes = Chunk{b[0], b[1]};
+        };
+        quantise(kn, kn_q, kn_sc);
+        quantise(vn, vn_q, vn_sc);
+        if (append && wave == 0 && grp == 0) {
+            *(Chunk *)(Kcache + (size_t)new_row * D + d0) = kn_q;
+            *(Chunk *)(Vcache + (size_t)new_row * D + d0) = vn_q;
+            if (dc == 0) {
+                Elem<T>::st(Kscale, new_row, kn_sc);
+                Elem<T>::st(Vscale, new_row, vn_sc);
+            }
+        }
+    } else {
+        if (append && wave == 0 && grp == 0) {  // one lane group appends the new row
+            *(U4 *)(Kcache + (size_t)new_row * D + d0) = kn_packed;
+            *(U4 *)(Vcache + (size_t)new_row * D + d0) = v_new;
+        }
     }
 
     // ---- softmax over this lane group's keys: the scores of a round are independent of each other (all dot
@@ -102,7 +149,18 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
             if (base + i * KPP >= bound) continue;  // no wave has keys in this pass
             const int key = base + i * KPP + wave * GPW + grp;
             float d = 0.f;
-            if constexpr (std::is_same_v<T, f16_t>) {
+            float k_scale_i = 1.f;
+            if constexpr (KV8) {
+                Chunk kk = kreg[i];
+                k_scale_i = Elem<T>::ld(&ksc[i], 0);
+                if (i == i_new && key == new_row) {
+                    kk = kn_q;
+                    k_scale_i = kn_sc;
+                }
+                const uint32_t kw[2] = {kk.x, kk.y};
+#pragma unroll
+                for (int e = 0; e < 8; e++) d = fmaf(q[e], (float)(int8_t)((kw[e >> 2] >> (8 * (e & 3))) & 0xFF), d);
+            } else if constexpr (std::is_same_v<T, f16_t>) {
                 // fp16: query and key stay packed, two products per instruction with f32 accumulation
                 U4 kk = kreg[i];
                 if (i == i_new && key == new_row) kk = kn_packed;  // (i == i_new is uniform: only this pass can hold the new row)
@@ -120,7 +178,9 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
 #pragma unroll
                 for (int e = 0; e < 8; e++) d = fmaf(q[e], kf[e], d);
             }
-            d = group_sum<LPK>(d) * scale;
+            d = group_sum<LPK>(d);
+            if constexpr (KV8) d *= k_scale_i;
+            d *= scale;
             if (key < bound) sc[i] = d;
             mr = fmaxf(mr, sc[i]);
         }
@@ -136,7 +196,21 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
             const int key = base + i * KPP + wave * GPW + grp;
             const float pe = fast_exp(sc[i] - mn);  // (no key: exp(-inf) = 0)
             l += pe;
-            U4 vv = vreg[i];
+            if constexpr (KV8) {
+                Chunk vv = vreg[i];
+                float v_scale_i = Elem<T>::ld(&vsc[i], 0);
+                if (i == i_new && key == new_row) {
+                    vv = vn_q;
+                    v_scale_i = vn_sc;
+                }
+                const float pv = pe * v_scale_i;
+                const uint32_t vw[2] = {vv.x, vv.y};
+#pragma unroll
+                for (int e = 0; e < 8; e++) o[e] = fmaf(pv, (float)(int8_t)((vw[e >> 2] >> (8 * (e & 3))) & 0xFF), o[e]);
+                continue;
+            }
+            U4 vv;
+            if constexpr (!KV8) vv = vreg[i];
             if (i == i_new && key == new_row) vv = v_new;
             if constexpr (std::is_same_v<T, f16_t>) {
                 // (the widening of a half operand rides on the multiply-add: v_fma_mix_f32)

@@ -333,7 +333,7 @@ static int enqueue_step(Model &m) {
 
     // embed: DequantizeLinear(table) -> Gather(ids), one row per token
     // (batch-1 decode with the fused launch: the first layer's launch makes the row itself)
-    if (m.quant && rows == 1 && m.qkv_attn && !w8a8 && !kv8) {
+    if (m.quant && rows == 1 && m.qkv_attn && !w8a8) {
     } else if (m.quant) {
         note(m, "embed_dequant", (double)rows * (H + eb + H * eb));
         TRY(embed_dequant<T>(m.x, (const int8_t *)m.embed.w, m.embed.scale, m.d_ids, rows, V, H, s));
@@ -353,6 +353,7 @@ static int enqueue_step(Model &m) {
             QkvAttnParams p{};
             p.x = m.x; p.norm_w = L.norm1; p.eps = c.eps; p.wq = (const int8_t *)L.qkv.w; p.scale = L.qkv.scale;
             p.N = L.qkv.N; p.K = H; p.qkv = (uint64_t *)m.qkv; p.out = m.attn; p.k_cache = L.k_cache; p.v_cache = L.v_cache;
+            p.k_scale = kv8 ? L.k_scale : nullptr; p.v_scale = kv8 ? L.v_scale : nullptr;
             p.cos_t = m.cos_t; p.sin_t = m.sin_t; p.d_pos = m.d_pos; p.d_active = m.d_active; p.d_past = m.d_past; p.Hq = Hq; p.Hkv = Hkv;
             p.max_seq = c.max_seq; p.softmax_scale = softmax_scale; p.err = m.d_past + 3; p.spin_limit = m.spin_limit;
             if (li == 0) {  // the input row of the first layer: the token's embedding
@@ -393,12 +394,14 @@ static int enqueue_step(Model &m) {
             p.is_causal = S > 1; p.B = B; p.Sq = S; p.Hq = Hq; p.Hkv = Hkv; p.cache_len = c.max_seq;
             p.d_active = m.d_active; p.nsplit = m.nsplit; p.slice = m.slice; p.heads_per_wg = m.heads_per_wg;
             attn_token_major_layout(p, D);
-            const bool fuse_attn = (fused || qfused) && !kv8 && attention_fused_supported(D, Hq / Hkv);
+            // (an int8 cache: the form for a cache one workgroup covers quantises the new row itself)
+            const bool fuse_attn = (fused || qfused) &&
+                                   (kv8 ? attention_fused_kv8_supported(D, c.max_seq) : attention_fused_supported(D, Hq / Hkv));
             if (fuse_attn) {
                 // RoPE(q), RoPE(k), both cache appends and the attention in one launch
                 p.qkv = m.qkv; p.cos_t = m.cos_t; p.sin_t = m.sin_t; p.d_pos = m.d_pos; p.d_past = m.d_past;
-                note(m, "attention_rope_append", (double)(QD + 2 * KD) * eb + 2.0 * KD * eb + QD * eb);
-                TRY(attention_decode_launch(p, D, c.dtype, 0, m.attn_scratch, s));
+                note(m, kv8 ? "attention_rope_quant_append" : "attention_rope_append", (double)(QD + 2 * KD) * eb + 2.0 * KD * (kv8 ? 1 + eb / D : eb) + QD * eb);
+                TRY(attention_decode_launch(p, D, c.dtype, kv8 ? 1 : 0, m.attn_scratch, s));
             } else {
                 // prefill on the matrix cores: the attention kernel rotates the queries itself, reading them from the
                 // projection's output; the RoPE launch is left with the keys and the values
@@ -777,8 +780,9 @@ static int build(Model &m, void **init, void **state) {
 
     // ---- batch-1 decode: projection and attention in one launch when the shape allows
     m.spin_limit = c.handover_spin_limit > 0 ? c.handover_spin_limit : c.handover_spin_limit < 0 ? 0 : 400000;
-    if (m.quant && rows == 1 && !c.quantize_activations && !c.quant_kv_cache && !c.unfused_decode &&
+    if (m.quant && rows == 1 && !c.quantize_activations && !c.unfused_decode &&
         attention_fused_supported(c.head_dim, c.n_heads / c.n_kv_heads) &&
+        (!c.quant_kv_cache || attention_fused_kv8_supported(c.head_dim, c.max_seq)) &&
         qkv_attention_supported(H, c.n_heads, c.n_kv_heads, c.head_dim, c.max_seq, c.dtype) && (QD + 2 * KD) * eb % 8 == 0) {
         bool ok = aligned16(m.qkv) && aligned16(m.x) && aligned16(m.attn) && aligned16(m.embed.w);
         for (const Layer &L : m.layers)

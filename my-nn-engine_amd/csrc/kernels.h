@@ -78,6 +78,7 @@ struct QkvAttnParams {
     int gemv_blocks, groups; // filled in by the launcher
     void *out;               // [Hq * D]
     void *k_cache, *v_cache; // [Hkv, max_seq, D]
+    void *k_scale, *v_scale; // int8 cache (BuildOptions::quant_kv_cache): [Hkv, max_seq] row scales; null: 16-bit cache
     const void *cos_t, *sin_t;
     const int64_t *d_pos;
     const int32_t *d_active;

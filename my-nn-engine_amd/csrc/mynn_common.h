@@ -151,6 +151,16 @@ template <int width> __device__ inline float group_sum(float v) {
     }
 }
 
+// maximum over the lanes of an aligned group of `width` lanes (power of two <= 16)
+template <int width> __device__ inline float group_max(float v) {
+    static_assert(width <= 16, "inside a row of 16 lanes");
+    if constexpr (width >= 2) v = fmaxf(v, dpp_get<kDppXor1>(v));
+    if constexpr (width >= 4) v = fmaxf(v, dpp_get<kDppXor2>(v));
+    if constexpr (width >= 8) v = fmaxf(v, dpp_get<kDppHalfMirror>(v));
+    if constexpr (width >= 16) v = fmaxf(v, dpp_get<kDppMirror>(v));
+    return v;
+}
+
 // greedy-token candidates: (value, index) ordered by value, then index -- of equal maxima the LATER one wins
 // (the reference's max_by over the logits, crates/llm/src/session.rs:683-690); index < 0 = no candidate yet
 __device__ inline void argmax_take(float &bv, int &bi, float v, int i) {

@@ -225,35 +225,48 @@ def test_prefill_then_decode_shares_kv_and_matches_decode_only(g, dt):
     b.close(), dec.close(), pre.close(), dec2.close()
 
 
+SMALL_D64 = dict(SMALL, n_heads=4, n_kv_heads=2, head_dim=64)
+
+
 @pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+@pytest.mark.parametrize("shape", ["d32", "d64"])
 @pytest.mark.parametrize("kv8,w8a8", [(True, False), (False, True), (True, True)])
-def test_int8_kv_cache_and_w8a8_executor_vs_oracle(g, dt, kv8, w8a8):
+def test_int8_kv_cache_and_w8a8_executor_vs_oracle(g, dt, kv8, w8a8, shape):
     """BuildOptions::quant_kv_cache (int8 caches + per-token scales, QuantizingKVCacheUpdate, attention
     scale slots; crates/llm/src/decoder.rs:405-470) and Options::quantize_activations
     (DynamicQuantizeLinear + QuantizedMatMul for every int8 linear; quantize_activations.rs) in the
     executor: a 16-token prefill chunk, then decode steps over the same caches, against the oracle
     with the same options."""
-    cfg, w = llm_weights.synthetic_int8(SMALL, dt, seed=41)
+    cfg, w = llm_weights.synthetic_int8(SMALL if shape == "d32" else SMALL_D64, dt, seed=41)
     ref = orc.Model(cfg, w)
     ref.set_options(quant_kv_cache=kv8, quantize_activations=w8a8)
     ref.set_gemm_mode(2)
     dw = dev_weights(g, w, dt)
     dec = g.mynn.Decoder(cfg, dw, quant_kv_cache=kv8, quantize_activations=w8a8)
-    if w8a8:
-        # batch-1 decode: norm, quantiser, int8 GEMV and residual / SwiGLU of a linear are one launch (qkv, o, gate/up,
-        # down), the attention block one (16-bit cache) or two (int8 cache) more; embedding, lm_head, greedy token
-        assert dec.stats()["launches_per_step"] == (6 if kv8 else 5) * cfg["n_layers"] + 3, dec.stats()
+    # batch-1 decode: a linear with its norm (quantiser) and store is one launch (qkv, o, gate/up, down); the attention
+    # block is one more (RoPE, append -- quantising for an int8 cache at head_dim 64 / 128 -- and attention) or, for an
+    # int8 cache at head_dim 32, two; embedding, lm_head, greedy token
+    nl = cfg["n_layers"]
+    if not w8a8:  # (int8 cache, 16-bit activations: the layer's attention block is one launch as with a 16-bit cache)
+        want_launches = 6 * nl + 3 if shape == "d32" else 3 * nl + 1
+    else:
+        want_launches = (6 if kv8 and shape == "d32" else 5) * nl + 3
+    assert dec.stats()["launches_per_step"] == want_launches, dec.stats()
     pre = g.mynn.Decoder(cfg, dw, seq_q=16, kv=dec.kv, quant_kv_cache=kv8, quantize_activations=w8a8)
     rng = np.random.default_rng(3)
     ids = rng.integers(0, cfg["vocab"], 16)
     want = ref.forward(ids, np.arange(16), 0, 16, True)
     _, got = pre.step(ids, np.arange(16), 0, 16, want_logits=True)
-    assert max_err_rel_to_max(g.f32(got, dt), g.f32(want, dt)) <= 2e-2
+    # (int8 activations at the wider heads: measured up to 2.7e-2 in the prefill chunk and 2.2e-2 in the decode steps,
+    # the latter the same to the last bit whether a linear is one launch or four -- an activation's code that lands on
+    # the other side of a rounding moves every output of the row)
+    tol = 3e-2 if w8a8 and shape == "d64" else 2e-2
+    assert max_err_rel_to_max(g.f32(got, dt), g.f32(want, dt)) <= tol
     past = 16
     for t in [7, 500, 31, 999, 2, 640]:
         want = ref.forward([t], [past], past, past + 1, False)
         nxt, got = dec.step([t], [past], past, past + 1, want_logits=True)
-        assert max_err_rel_to_max(g.f32(got, dt), g.f32(want, dt)) <= 2e-2, past
+        assert max_err_rel_to_max(g.f32(got, dt), g.f32(want, dt)) <= tol, past
         assert nxt[0] == orc.argmax_last(got[0], dt)
         past += 1
     if kv8:
