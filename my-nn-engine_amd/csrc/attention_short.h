@@ -232,10 +232,12 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
     }
     // ---- lane groups of the wave meet (lanes of equal dc), then the waves through LDS.  First the wave's maximum,
     //      then every group rescales its (l, o) to it once, and the groups' values are plain sums.
-    auto other = [&](float v, int off) { return off == 8 ? dpp_get<kDppRor8>(v) : __shfl_xor(v, off, 64); };  // (lane ^ 8: same row of 16)
+    // (lane ^ 8 is in the same row of 16: DPP; lane ^ 16 and lane ^ 32 through the row swaps; the same pairs either way)
+    auto meet_sum = [&](float v, int off) { return off == 8 ? v + dpp_get<kDppRor8>(v) : off == 16 ? xor16_sum(v) : xor32_sum(v); };
+    auto meet_max = [&](float v, int off) { return off == 8 ? fmaxf(v, dpp_get<kDppRor8>(v)) : off == 16 ? xor16_max(v) : xor32_max(v); };
     float mw = m;
 #pragma unroll
-    for (int off = LPK; off < 64; off <<= 1) mw = fmaxf(mw, other(mw, off));
+    for (int off = LPK; off < 64; off <<= 1) mw = meet_max(mw, off);
     {
         const float a = m == -INFINITY ? 0.f : fast_exp(m - mw);  // (a wave without keys: everything stays 0, mw = -inf)
         l *= a;
@@ -245,9 +247,9 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
     }
 #pragma unroll
     for (int off = LPK; off < 64; off <<= 1) {
-        l += other(l, off);
+        l = meet_sum(l, off);
 #pragma unroll
-        for (int e = 0; e < 8; e++) o[e] += other(o[e], off);
+        for (int e = 0; e < 8; e++) o[e] = meet_sum(o[e], off);
     }
     if (grp == 0) {
 #pragma unroll

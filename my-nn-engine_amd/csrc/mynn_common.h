@@ -134,6 +134,29 @@ __device__ inline float wave_max(float v) {
     v = fmaxf(v, dpp_rows<kDppBcast31, 0xC>(v, v));
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
+// Exchange across rows of 16 lanes without the LDS crossbar: v_permlane16_swap / v_permlane32_swap swap the odd rows
+// (the upper half) of one register with the even rows (the lower half) of another.  Applied to two copies of v, one
+// copy ends up holding the even-row (lower-half) values in both rows of a pair and the other the odd-row (upper-half)
+// values, so their sum / maximum is v[lane] combined with v[lane ^ 16] (v[lane ^ 32]) in every lane.  (Inline
+// assembly: the compiler's builtin for these instructions returns the first result twice when both operands hold
+// the same value.  The s_nop covers the wait states between a vector write and the swap that reads it.)
+__device__ inline void permlane16_swap(float &a, float &b) { asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
+__device__ inline void permlane32_swap(float &a, float &b) { asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
+__device__ inline float xor16_sum(float v) { float a = v, b = v; permlane16_swap(a, b); return a + b; }
+__device__ inline float xor32_sum(float v) { float a = v, b = v; permlane32_swap(a, b); return a + b; }
+__device__ inline float xor16_max(float v) { float a = v, b = v; permlane16_swap(a, b); return fmaxf(a, b); }
+__device__ inline float xor32_max(float v) { float a = v, b = v; permlane32_swap(a, b); return fmaxf(a, b); }
+// exact integer sum over the wave, the same value in every lane
+__device__ inline int wave_sum_i32(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, kDppXor1, 0xF, 0xF, false);
+    v += __builtin_amdgcn_update_dpp(0, v, kDppXor2, 0xF, 0xF, false);
+    v += __builtin_amdgcn_update_dpp(0, v, kDppHalfMirror, 0xF, 0xF, false);
+    v += __builtin_amdgcn_update_dpp(0, v, kDppMirror, 0xF, 0xF, false);
+    v += __builtin_amdgcn_update_dpp(0, v, kDppBcast15, 0xA, 0xF, false);
+    v += __builtin_amdgcn_update_dpp(0, v, kDppBcast31, 0xC, 0xF, false);
+    return __builtin_amdgcn_readlane(v, 63);
+}
+
 // sum over the lanes of an aligned group of `width` lanes (power of two <= 64)
 template <int width> __device__ inline float group_sum(float v) {
     if constexpr (width <= 16) {
@@ -145,8 +168,9 @@ template <int width> __device__ inline float group_sum(float v) {
         if constexpr (width >= 16) v += dpp_get<kDppMirror>(v);
         return v;
     } else {
-#pragma unroll
-        for (int off = width / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+        v = group_sum<16>(v);
+        v = xor16_sum(v);
+        if constexpr (width >= 64) v = xor32_sum(v);
         return v;
     }
 }

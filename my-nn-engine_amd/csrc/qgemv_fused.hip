@@ -18,19 +18,6 @@ namespace mynn {
 
 constexpr int kQgThreads = 256, kQgWaves = kQgThreads / 64;
 
-template <int CTRL> __device__ inline int dpp_i(int v) { return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, false); }
-template <int CTRL, int ROWS> __device__ inline int dpp_rows_i(int v) { return __builtin_amdgcn_update_dpp(0, v, CTRL, ROWS, 0xF, false); }
-// exact, so any order will do: the butterfly of wave_sum
-__device__ inline int wave_sum_i(int v) {
-    v += dpp_i<kDppXor1>(v);
-    v += dpp_i<kDppXor2>(v);
-    v += dpp_i<kDppHalfMirror>(v);
-    v += dpp_i<kDppMirror>(v);
-    v += dpp_rows_i<kDppBcast15, 0xA>(v);
-    v += dpp_rows_i<kDppBcast31, 0xC>(v);
-    return __builtin_amdgcn_readlane(v, 63);
-}
-
 struct QGemvParams {
     void *out;
     float eps;
@@ -170,7 +157,7 @@ __global__ __launch_bounds__(kQgThreads) void qgemv1_kernel(const int8_t *wq, co
             }
         }
 #pragma unroll
-        for (int r = 0; r < R; r++) acc[r] = wave_sum_i(acc[r]);
+        for (int r = 0; r < R; r++) acc[r] = wave_sum_i32(acc[r]);
         const int row0 = g * R;
         // lane r finishes row r (SwiGLU: lane r = 0, 2, .. the pair r, r + 1)
         int mine = acc[0], next = R > 1 ? acc[1] : 0;

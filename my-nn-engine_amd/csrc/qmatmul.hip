@@ -15,11 +15,7 @@ namespace mynn {
 typedef int i4x_t __attribute__((ext_vector_type(4)));
 typedef int i16x_t __attribute__((ext_vector_type(16)));
 
-__device__ inline int wave_sum_i32(int v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
-}
+
 
 // ---- small M: one wave per (R rows of rhs) x (MB rows of lhs)
 template <typename T, int R, int MB>
