@@ -36,8 +36,8 @@ ROLE_PATTERNS = {
     "gemv_norm_gateup_swiglu": r"dequant_gemv1_kernelI\w+?Li\d+ELi\d+ELi2ELb1ELb0EE",
     "gemv_down_residual": r"dequant_gemv1_kernelI\w+?Li\d+ELi\d+ELi1ELb0ELb0EE",
     "gemv_norm_lm_head_argmax": r"dequant_gemv1_kernelI\w+?Li\d+ELi\d+ELi0ELb1ELb1EE",
-    "qkv_attention_o": r"qkv_attention_kernelI\w+?Li\d+ELi\d+ELb0EE",
-    "embed_qkv_attention_o": r"qkv_attention_kernelI\w+?Li\d+ELi\d+ELb1EE",
+    "qkv_attention_o": r"qkv_attention_kernelI\w+?Li\d+ELi\d+ELb0ELb0EE",        # <T, D, NC, EMBED = false, KV8 = false>
+    "embed_qkv_attention_o": r"qkv_attention_kernelI\w+?Li\d+ELi\d+ELb1ELb0EE",
     "linear_gateup_swiglu": r"(gemm_nt_dma_kernelI\w+?Li2ELb0EE|skinny_gemm_kernel)",
     "qlinear_gateup_swiglu": r"gemm_nt_dma_kernelI\w+?Li2ELb1EE",
     "attention": r"(attn_stream_kernel|attn_prefill_kernel)",
