@@ -56,15 +56,16 @@ def test_decode_step_appends_at_past_len_whatever_active_says(g, kind):
 
 
 # ------------------------------------------------------------------ hand-over give-up and recovery
+@pytest.mark.parametrize("kv8", [False, True], ids=["kv16", "kv_int8"])
 @pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
-def test_handover_give_up_falls_back_to_one_op_per_launch(g, dt):
+def test_handover_give_up_falls_back_to_one_op_per_launch(g, dt, kv8):
     """A consumer role that gives up at once (handover_spin_limit = -1) raises the error word; every kernel still
     exits normally.  The executor then discards the step, rebuilds itself with one op per launch and repeats the
     step: the caller sees the results of the un-fused executor, bit for bit, and a failure count of 1."""
     cfg, w = llm_weights.synthetic_int8(SHORT_CACHE[64], dt, seed=71)
     dw = dev_weights(g, w, dt)
-    plain = g.mynn.Decoder(cfg, dw, unfused_decode=True)
-    quick = g.mynn.Decoder(cfg, dw, handover_spin_limit=-1)
+    plain = g.mynn.Decoder(cfg, dw, unfused_decode=True, quant_kv_cache=kv8)
+    quick = g.mynn.Decoder(cfg, dw, handover_spin_limit=-1, quant_kv_cache=kv8)
     assert quick.stats()["launches_per_step"] == 3 * cfg["n_layers"] + 1 and quick.handover_failures == 0
     toks = np.random.default_rng(1).integers(0, cfg["vocab"], 12)
     for i, t in enumerate(toks):
@@ -74,16 +75,16 @@ def test_handover_give_up_falls_back_to_one_op_per_launch(g, dt):
     assert quick.handover_failures == 1, "producers cannot have finished before the consumers' first look"
     assert quick.stats()["launches_per_step"] == plain.stats()["launches_per_step"] and quick.stats()["graph"]
     for l in range(cfg["n_layers"]):
-        for j in range(2):
+        for j in range(len(plain.kv[l])):  # (int8 KV: codes and per-row scales)
             assert np.array_equal(g.to_host(quick.kv[l][j]), g.to_host(plain.kv[l][j]))
     quick.close()
     # the same inside the device-resident loop: the whole loop is repeated after the rebuild
-    loop = g.mynn.Decoder(cfg, dw, handover_spin_limit=-1)
+    loop = g.mynn.Decoder(cfg, dw, handover_spin_limit=-1, quant_kv_cache=kv8)
     n = len(toks)
     for i, t in enumerate(toks):
         first, _ = plain.step([t], [i], i, i + 1)  # (plain's cache already holds these rows: same values again)
     for l in range(cfg["n_layers"]):
-        for j in range(2):
+        for j in range(len(plain.kv[l])):
             loop.kv[l][j].copy_(plain.kv[l][j])
     assert loop.decode_loop(first[0], n, 20) == plain.decode_loop(first[0], n, 20)
     assert loop.handover_failures == 1
