@@ -55,7 +55,7 @@ class ModelConfig(C.Structure):
                 ("ffn", _i), ("vocab", _i), ("max_seq", _i), ("eps", _f), ("rope_theta", _f), ("dtype", _i),
                 ("seq_q", _i), ("batch", _i), ("weights_int8", _i), ("quant_kv_cache", _i),
                 ("quantize_activations", _i), ("streaming_kv", _i), ("gemm_tile", _i), ("unfused_decode", _i),
-                ("handover_spin_limit", _i), ("weight_arena", _i)]
+                ("handover_spin_limit", _i), ("weight_arena", _i), ("kv_page_rows", _i)]
 
 
 class KernelTime(C.Structure):
@@ -84,6 +84,20 @@ SIGNATURES = {
     "mynn_attention_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i, _i, _i]),
     "mynn_attention_ws": (_i, [_vp, _vp, _vp, _vp, _vp, C.c_long, C.c_long, _vp, _vp, _f, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i,
                                 _i, _vp, _sz, _vp]),
+    "mynn_attention_paged_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i, _i]),
+    "mynn_attention_paged": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
+    "mynn_kvcache_update_paged": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _i, _i, _vp]),
+    "mynn_kv_pool_create": (_vp, [_i, _i]),
+    "mynn_kv_pool_free_pages": (_i, [_vp]),
+    "mynn_kv_pool_destroy": (_i, [_vp]),
+    "mynn_kv_pages_create": (_vp, [_vp, _i, _i]),
+    "mynn_kv_pages_reserve": (_i, [_vp, _i64]),
+    "mynn_kv_pages_release": (_i, [_vp]),
+    "mynn_kv_pages_mapped_rows": (_i, [_vp]),
+    "mynn_kv_pages_per_seq": (_i, [_vp]),
+    "mynn_kv_pages_table": (_vp, [_vp]),
+    "mynn_kv_pages_table_host": (_i, [_vp, _vp]),
+    "mynn_kv_pages_destroy": (_i, [_vp]),
     "mynn_kvcache_update": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "mynn_kvcache_update_streaming": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "mynn_quantizing_kvcache_update_streaming": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
@@ -347,6 +361,101 @@ def kvcache_update(cache, new_kv, offset):
     return cache
 
 
+class KvPool:
+    """Free list of the page numbers of a paged KV cache (mynn_kv_pool); the pool buffers themselves are the
+    caller's: `buffers(...)` makes one K and one V tensor [n_pages, Hkv, page_rows, D] per layer."""
+
+    def __init__(self, n_pages, page_rows):
+        self.n_pages, self.page_rows = int(n_pages), int(page_rows)
+        self.handle = lib().mynn_kv_pool_create(self.n_pages, self.page_rows)
+        if not self.handle:
+            raise MynnError("kv_pool_create failed: %s" % lib().mynn_last_error().decode())
+
+    @property
+    def free_pages(self):
+        return lib().mynn_kv_pool_free_pages(self.handle)
+
+    def buffers(self, n_layers, n_kv_heads, head_dim, dtype, fill=None):
+        import torch
+
+        shape = (self.n_pages, n_kv_heads, self.page_rows, head_dim)
+        make = (lambda: torch.zeros(shape, dtype=dtype, device="cuda")) if fill is None else \
+            (lambda: torch.full(shape, fill, dtype=dtype, device="cuda"))
+        return [(make(), make()) for _ in range(n_layers)]
+
+    def close(self):
+        if getattr(self, "handle", None) and _lib is not None:
+            check(_lib.mynn_kv_pool_destroy(self.handle))
+            self.handle = None
+
+
+class KvPages:
+    """Page table of the `batch` sequences of one session over a KvPool (mynn_kv_pages)."""
+
+    def __init__(self, pool, batch, max_seq):
+        self.pool, self.batch, self.max_seq = pool, int(batch), int(max_seq)
+        self.handle = lib().mynn_kv_pages_create(pool.handle, self.batch, self.max_seq)
+        if not self.handle:
+            raise MynnError("kv_pages_create failed: %s" % lib().mynn_last_error().decode())
+
+    def reserve(self, rows):
+        check(lib().mynn_kv_pages_reserve(self.handle, int(rows)))
+
+    def release(self):
+        check(lib().mynn_kv_pages_release(self.handle))
+
+    @property
+    def mapped_rows(self):
+        return lib().mynn_kv_pages_mapped_rows(self.handle)
+
+    @property
+    def pages_per_seq(self):
+        return lib().mynn_kv_pages_per_seq(self.handle)
+
+    @property
+    def table_ptr(self):
+        return lib().mynn_kv_pages_table(self.handle)
+
+    def table(self):
+        """numpy int32 [batch, pages_per_seq]; -1 = not mapped"""
+        import numpy as np
+
+        out = np.empty((self.batch, self.pages_per_seq), np.int32)
+        check(lib().mynn_kv_pages_table_host(self.handle, out.ctypes.data_as(_vp)))
+        return out
+
+    def close(self):
+        if getattr(self, "handle", None) and _lib is not None:
+            check(_lib.mynn_kv_pages_destroy(self.handle))
+            self.handle = None
+
+
+def attention_paged(q, k_pool, v_pool, table, page_rows, scale, is_causal, active, q_pos_offset=0, d_active=None,
+                    k_scale_pool=None, v_scale_pool=None):
+    """mynn_attention_paged: q [B,Hq,Sq,D]; pools [n_pages,Hkv,page_rows,D]; table: cuda int32 [B, pages_per_seq]."""
+    import torch
+
+    B, Hq, Sq, D = q.shape
+    Hkv = k_pool.shape[1]
+    pps = table.shape[1]
+    assert table.dtype == torch.int32 and table.shape[0] == B and k_pool.shape[2] == page_rows
+    out = torch.empty_like(q)
+    need = lib().mynn_attention_paged_workspace_bytes(B, Sq, pps, int(page_rows), Hq, Hkv, D)
+    ws = torch.empty((max(need, 16),), dtype=torch.uint8, device=q.device)
+    check(lib().mynn_attention_paged(_ptr(out), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(k_scale_pool), _ptr(v_scale_pool),
+                                     _ptr(table), pps, int(page_rows), float(scale), int(is_causal), B, Sq, int(active), _ptr(d_active),
+                                     int(q_pos_offset), Hq, Hkv, D, _dt(q), int(k_pool.dtype == torch.int8), _ptr(ws), need, _stream()))
+    return out
+
+
+def kvcache_update_paged(pool, new_kv, offset, table, page_rows):
+    """mynn_kvcache_update_paged: new_kv [B,Hkv,S_new,D] into pool [n_pages,Hkv,page_rows,D] through table [B,pages_per_seq]."""
+    B, Hkv, S_new, D = new_kv.shape
+    check(lib().mynn_kvcache_update_paged(_ptr(pool), _ptr(new_kv), int(offset), B, Hkv, S_new, D, _dt(new_kv), _ptr(table),
+                                          table.shape[1], int(page_rows), _stream()))
+    return pool
+
+
 def kvcache_update_streaming(cache, new_kv, offset, ring_sink, ring_window, ring_start):
     """KVCacheUpdate through the sink + ring slot map (the reference's streaming-KV graph)."""
     import torch
@@ -525,7 +634,7 @@ class Decoder:
 
     def __init__(self, cfg, weights, seq_q=1, batch=1, kv=None, quant_kv_cache=False, quantize_activations=False,
                  streaming_kv=False, gemm_tile=0, unfused_decode=False, handover_spin_limit=0, weight_arena=False,
-                 reference_abi=False):
+                 reference_abi=False, kv_pages=None):
         import torch
 
         tdt = {F16: torch.float16, BF16: torch.bfloat16}[cfg["dtype"]]
@@ -534,8 +643,13 @@ class Decoder:
         self.cfg = ModelConfig(cfg["n_layers"], cfg["hidden"], cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"],
                                cfg["ffn"], cfg["vocab"], cfg["max_seq"], float(cfg["eps"]), float(cfg["rope_theta"]),
                                cfg["dtype"], seq_q, batch, int(quant), int(quant_kv_cache), int(quantize_activations),
-                               int(streaming_kv), int(gemm_tile), int(unfused_decode), int(handover_spin_limit), int(weight_arena))
+                               int(streaming_kv), int(gemm_tile), int(unfused_decode), int(handover_spin_limit), int(weight_arena),
+                               kv_pages.pool.page_rows if kv_pages is not None else 0)
         self.weights = weights  # keep the tensors alive
+        self.kv_pages = kv_pages
+        if kv_pages is not None:
+            # paged cache: kv = the pool buffers (KvPool.buffers), one (K pool, V pool) per layer, shared by every session of the pool
+            assert kv is not None, "a paged decoder takes the pool's buffers as kv"
         if kv is None:
             shape = (batch, cfg["n_kv_heads"], cfg["max_seq"], cfg["head_dim"])
             if quant_kv_cache:  # (k i8, v i8, k_scale, v_scale) per layer
@@ -549,6 +663,8 @@ class Decoder:
         state = []
         for bufs in kv:
             state.extend([_ptr(t) for t in bufs])
+        if kv_pages is not None:
+            state.append(kv_pages.handle)
         self._state = (_vp * len(state))(*state)
         if from_file:
             # a checkpoint: read, convert and upload by the library (names as the reference's ModelSpec)

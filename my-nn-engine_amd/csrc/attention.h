@@ -25,6 +25,12 @@ struct AttnParams {
     long mask_os, mask_rs;
     int rope_q;               // prefill kernel: Q is un-rotated; rotate row sq by table row d_pos[sq] (cos_t, sin_t, d_pos above)
     const int32_t *d_past;    // fused decode form: cache row the new token is appended to (KVCacheUpdate's offset)
+    // paged K/V (page_table != nullptr; streaming decode and prefill kernels): k and v are pools [n_pages, Hkv, P, D] with
+    // P = 1 << page_shift rows per page (an int8 cache: scale pools [n_pages, Hkv, P]); row r of sequence b lives in pool
+    // page page_table[b * pages_per_seq + (r >> page_shift)], row r % P of it; cache_len is pages_per_seq * P.  Entries of
+    // pages no row below the active length falls into are never read.
+    const int32_t *page_table;
+    int page_shift, pages_per_seq;
     float *part_o;            // [B*Hq*Sq, nsplit, D]
     float *part_ml;           // [B*Hq*Sq, nsplit, 2]
     // element strides of Q and out: batch, head, row.  Reference layout [B,Hq,Sq,D] is
@@ -55,6 +61,8 @@ bool attention_prefill_supported(const AttnParams &p, int D, int dtype, int kv_i
 bool attn_stream_eligible(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, int cache_len);
 void attn_stream_plan(int B, int Hkv, int kv_len, int *slice, int *nsplit);
 int attention_stream_launch(const AttnParams &p, int D, int dtype, int kv_int8, hipStream_t s);
+// paged K/V: the streaming kernel takes every decode shape it has a form for, whatever the sizes
+bool attn_stream_paged_supported(int Sq, int Hq, int Hkv, int D, int dtype, int page_rows);
 // out = merge of the nsplit partial results in p.part_o / p.part_ml (its own launch)
 int attention_merge_launch(const AttnParams &p, int D, int dtype, hipStream_t s);
 

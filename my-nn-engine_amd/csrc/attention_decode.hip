@@ -427,6 +427,10 @@ int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *s
     const int kv_len = p.d_active ? p.cache_len : (p.active < p.cache_len ? p.active : p.cache_len);
     if (!fuse && !p.mask && attn_stream_eligible(p.B, p.Sq, p.Hq, p.Hkv, D, dtype, kv_int8, kv_len, p.cache_len))
         return attention_stream_launch(p, D, dtype, kv_int8, s);
+    if (p.page_table) {  // (the plan is the streaming kernel's: that kernel has the paged form)
+        MYNN_REQUIRE(!fuse && !p.mask, MYNN_ERR_UNSUPPORTED, "paged attention: neither the fused decode form nor a mask");
+        return attention_stream_launch(p, D, dtype, kv_int8, s);
+    }
     bool whole = false;  // the launch wrote the finished output: nothing to merge whatever the plan's split count
     int rc = dispatch_dtype(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
@@ -598,6 +602,62 @@ extern "C" int mynn_attention_noalloc(void *out, const void *Q, const void *K, c
     return attention_entry(out, Q, K, V, nullptr, 0, 0, k_scale, v_scale, scale, is_causal, B, Sq, active_seq_kv, d_active,
                            cache_seq_len, q_pos_offset, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, WS_STATIC, nullptr, 0,
                            as_stream(s));
+}
+
+// ---- paged K/V: the same operator over pools and a page table
+static void paged_plan(int B, int Sq, int Hkv, int kv_len, int *slice, int *nsplit) {
+    *slice = 0;
+    *nsplit = 1;
+    if (Sq == 1) attn_stream_plan(B, Hkv, kv_len, slice, nsplit);
+}
+
+extern "C" size_t mynn_attention_paged_workspace_bytes(int B, int Sq, int pages_per_seq, int page_rows, int num_q_heads,
+                                                       int num_kv_heads, int head_dim) {
+    if (B <= 0 || Sq <= 0 || pages_per_seq <= 0 || page_rows <= 0 || num_q_heads <= 0 || num_kv_heads <= 0) return 0;
+    int slice, nsplit;
+    paged_plan(B, Sq, num_kv_heads, pages_per_seq * page_rows, &slice, &nsplit);
+    return nsplit > 1 ? attn_scratch_bytes(B, num_q_heads, Sq, head_dim, nsplit) : 0;
+}
+
+extern "C" int mynn_attention_paged(void *out, const void *Q, const void *K_pool, const void *V_pool, const void *k_scale_pool,
+                                    const void *v_scale_pool, const int32_t *page_table, int pages_per_seq, int page_rows,
+                                    float scale, int is_causal, int B, int Sq, int active_seq_kv, const int32_t *d_active,
+                                    int q_pos_offset, int num_q_heads, int num_kv_heads, int head_dim, int dtype, int kv_int8,
+                                    void *workspace, size_t workspace_bytes, mynn_stream s) {
+    MYNN_REQUIRE(out && Q && K_pool && V_pool && page_table, MYNN_ERR_INVALID, "attention_paged: null operand");
+    MYNN_REQUIRE(B > 0 && Sq > 0 && pages_per_seq > 0 && num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0,
+                 MYNN_ERR_INVALID, "attention_paged: B=%d Sq=%d pages=%d Hq=%d Hkv=%d", B, Sq, pages_per_seq, num_q_heads, num_kv_heads);
+    MYNN_REQUIRE(page_rows >= 32 && page_rows <= (1 << 20) && (page_rows & (page_rows - 1)) == 0, MYNN_ERR_INVALID,
+                 "attention_paged: %d rows per page (a power of two, 32 or more)", page_rows);
+    MYNN_REQUIRE((long)pages_per_seq * page_rows <= INT32_MAX, MYNN_ERR_INVALID, "attention_paged: %d pages of %d rows", pages_per_seq, page_rows);
+    MYNN_REQUIRE(!kv_int8 || (k_scale_pool && v_scale_pool), MYNN_ERR_INVALID, "attention_paged: int8 KV needs the scale pools");
+    MYNN_REQUIRE(d_active || (active_seq_kv >= 1), MYNN_ERR_INVALID, "attention_paged: active_seq_kv=%d", active_seq_kv);
+    MYNN_REQUIRE(dtype == MYNN_F16 || dtype == MYNN_BF16, MYNN_ERR_UNSUPPORTED, "attention_paged: dtype %d (fp16 or bf16)", dtype);
+    AttnParams p{};
+    p.out = out; p.q = Q; p.k = K_pool; p.v = V_pool; p.k_scale = k_scale_pool; p.v_scale = v_scale_pool; p.scale = scale;
+    p.is_causal = is_causal; p.B = B; p.Sq = Sq; p.Hq = num_q_heads; p.Hkv = num_kv_heads;
+    p.cache_len = pages_per_seq * page_rows; p.active = active_seq_kv; p.d_active = d_active; p.q_pos_offset = q_pos_offset;
+    p.page_table = page_table; p.pages_per_seq = pages_per_seq;
+    while ((1 << p.page_shift) < page_rows) p.page_shift++;
+    attn_reference_layout(p, head_dim);
+    if (Sq > 1) {
+        MYNN_REQUIRE(!kv_int8 && (head_dim == 64 || head_dim == 128) && scale > 0.f && aligned16(Q) && aligned16(out) && aligned16(K_pool) &&
+                         aligned16(V_pool),
+                     MYNN_ERR_UNSUPPORTED, "attention_paged: several query rows need a 16-bit cache, head_dim 64 or 128, a positive scale and 16-byte aligned operands");
+        return attention_prefill_launch(p, head_dim, dtype, as_stream(s));
+    }
+    const int kv_len = d_active ? p.cache_len : (active_seq_kv < p.cache_len ? active_seq_kv : p.cache_len);
+    paged_plan(B, Sq, num_kv_heads, kv_len, &p.slice, &p.nsplit);
+    p.heads_per_wg = num_q_heads / num_kv_heads;
+    if (p.nsplit > 1) {
+        const size_t need = attn_scratch_bytes(B, num_q_heads, Sq, head_dim, p.nsplit);
+        MYNN_REQUIRE(workspace && aligned16(workspace) && workspace_bytes >= need, MYNN_ERR_INVALID,
+                     "attention_paged: the workspace must hold %zu bytes (mynn_attention_paged_workspace_bytes), 16-byte aligned", need);
+        const size_t rows = (size_t)B * num_q_heads * Sq;
+        p.part_o = (float *)workspace;
+        p.part_ml = p.part_o + rows * p.nsplit * head_dim;
+    }
+    return attention_stream_launch(p, head_dim, dtype, kv_int8, as_stream(s));
 }
 
 // ---- streaming KV (sink + ring cache): the slot map of the reference's kernels and the two operators that

@@ -28,7 +28,10 @@ namespace mynn {
 
 constexpr int kPfThreads = 256, kPfRows = 128, kPfKeys = 64;
 
-template <typename T, int D>
+// PAGED: K/V rows are found through a page table (AttnParams::page_table) of at most 64 pages per sequence, each a
+// power of two >= 64 rows: a 64-key tile lies in one page, and the sequence's table row sits in one register (lane i =
+// page i) from which a tile picks its entry with v_readlane.
+template <typename T, int D, bool PAGED>
 __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_kernel(AttnParams p) {
     constexpr int LDK = D + 8;          // K tile row stride (elements): conflict-free 16-byte reads
     constexpr int LDV = kPfKeys + 4;    // V^T tile row stride
@@ -60,19 +63,30 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_kernel(AttnParams 
     const int blk_bound = p.is_causal ? min(kv_bound, qoff + blk_last + 1) : kv_bound;
     const int ntiles = (blk_bound + kPfKeys - 1) / kPfKeys;
 
-    const T *Kg = (const T *)p.k + (size_t)(b * p.Hkv + hkv) * p.cache_len * D;
-    const T *Vg = (const T *)p.v + (size_t)(b * p.Hkv + hkv) * p.cache_len * D;
+    const T *Kg = (const T *)p.k + (PAGED ? 0 : (size_t)(b * p.Hkv + hkv) * p.cache_len * D);
+    const T *Vg = (const T *)p.v + (PAGED ? 0 : (size_t)(b * p.Hkv + hkv) * p.cache_len * D);
+    const int psh = p.page_shift, pmask = (1 << psh) - 1;
+    int pg_reg = 0;
+    if constexpr (PAGED) {
+        if (lane < p.pages_per_seq) pg_reg = p.page_table[(size_t)b * p.pages_per_seq + lane];
+    }
     // a tile travels global -> registers (NPF iterations ahead of) -> LDS (one iteration ahead of) the MFMAs.
     // Thread t stages the keys CH * (t / (D/8)) + 0 .. CH-1 of a tile, dims 8 * (t % (D/8)) .. +7.
     // Rows past the end are clamped to the last visible key: whatever they hold is masked out.
     const int key0 = (tid / (D / 8)) * CH, dd = (tid % (D / 8)) * 8;
     U4 rk[NPF][CH], rv[NPF][CH];
     auto load_tile = [&](int t, U4 *k_, U4 *v_) {
+        size_t po = 0;  // PAGED: first row of the tile's page, in rows of one head of the pool
+        if constexpr (PAGED) {
+            const int pg = __builtin_amdgcn_readlane(pg_reg, __builtin_amdgcn_readfirstlane((t * kPfKeys) >> psh));
+            po = ((size_t)pg * p.Hkv + hkv) << psh;
+        }
 #pragma unroll
         for (int c = 0; c < CH; c++) {
             const int key = min(t * kPfKeys + key0 + c, blk_bound - 1);
-            k_[c] = *(const U4 *)(Kg + (size_t)key * D + dd);
-            v_[c] = *(const U4 *)(Vg + (size_t)key * D + dd);
+            const size_t row = PAGED ? po + (size_t)(key & pmask) : (size_t)key;
+            k_[c] = *(const U4 *)(Kg + row * D + dd);
+            v_[c] = *(const U4 *)(Vg + row * D + dd);
         }
     };
     auto store_tile = [&](int buf, const U4 *k_, const U4 *v_) {
@@ -280,11 +294,22 @@ bool attention_prefill_supported(const AttnParams &p, int D, int dtype, int kv_i
 
 int attention_prefill_launch(const AttnParams &p, int D, int dtype, hipStream_t s) {
     MYNN_REQUIRE((p.Sq + kPfRows - 1) / kPfRows <= 65535, MYNN_ERR_UNSUPPORTED, "attention: Sq = %d exceeds the grid", p.Sq);
+    if (p.page_table) {
+        const int P = 1 << p.page_shift;
+        MYNN_REQUIRE(P >= kPfKeys && p.pages_per_seq <= 64 && p.cache_len == p.pages_per_seq << p.page_shift, MYNN_ERR_UNSUPPORTED,
+                     "paged prefill attention: %d pages of %d rows per sequence (at most 64 pages of 2^n >= %d rows)",
+                     p.pages_per_seq, P, kPfKeys);
+    }
     dim3 grid(p.B * p.Hq, (p.Sq + kPfRows - 1) / kPfRows);
     return dispatch_dtype16(dtype, [&](auto *t) {
         using T = std::remove_pointer_t<decltype(t)>;
-        if (D == 64) MYNN_LAUNCH((attn_prefill_kernel<T, 64>), grid, dim3(kPfThreads), 0, s, p);
-        else MYNN_LAUNCH((attn_prefill_kernel<T, 128>), grid, dim3(kPfThreads), 0, s, p);
+        if (p.page_table) {
+            if (D == 64) MYNN_LAUNCH((attn_prefill_kernel<T, 64, true>), grid, dim3(kPfThreads), 0, s, p);
+            else MYNN_LAUNCH((attn_prefill_kernel<T, 128, true>), grid, dim3(kPfThreads), 0, s, p);
+        } else {
+            if (D == 64) MYNN_LAUNCH((attn_prefill_kernel<T, 64, false>), grid, dim3(kPfThreads), 0, s, p);
+            else MYNN_LAUNCH((attn_prefill_kernel<T, 128, false>), grid, dim3(kPfThreads), 0, s, p);
+        }
         return launch_status("attn_prefill_kernel");
     });
 }

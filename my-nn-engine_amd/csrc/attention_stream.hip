@@ -40,7 +40,11 @@ constexpr int kStreamWaves = 4, kStreamThreads = kStreamWaves * 64, kStreamTile 
 
 // KVI8: int8 caches with one scale per token row (QuantizingKVCacheUpdate): K and V are widened exactly to
 // the 16-bit type in registers, the key's k scale multiplies its score and its v scale its p.
-template <typename T, int D, int G, bool KVI8>
+// PAGED: K/V rows are found through a page table (AttnParams::page_table).  A tile of 32 keys never crosses a page
+// (pages hold a power of two >= 32 rows, tiles start at multiples of 32), so the page is a wave-uniform value per
+// tile: the workgroup's part of the table sits in one register (lane i = the i-th page of its key range, at most 64)
+// and a tile picks its entry with v_readlane -- no dependent load in the key loop.
+template <typename T, int D, int G, bool KVI8, bool PAGED>
 __global__ __launch_bounds__(kStreamThreads) void attn_stream_kernel(AttnParams p) {
     constexpr int KB = D / 32;              // 32-dim blocks of a key row
     constexpr int LPK = D / 8;              // lanes per key row when a tile is loaded 16 bytes per lane
@@ -66,11 +70,21 @@ __global__ __launch_bounds__(kStreamThreads) void attn_stream_kernel(AttnParams 
     const int active = p.d_active ? *p.d_active : p.active;
     const int bound = min(active, p.cache_len);
     const int k0 = split * p.slice, k1 = min(bound, k0 + p.slice);
-    const size_t kv_base = (size_t)bhkv * p.cache_len;
+    const size_t kv_base = PAGED ? 0 : (size_t)bhkv * p.cache_len;
     using TKV = typename std::conditional<KVI8, int8_t, T>::type;
     using Chunk = typename std::conditional<KVI8, uint2, U4>::type;  // 8 elements of a cached row
     const TKV *Kp = (const TKV *)p.k + kv_base * D, *Vp = (const TKV *)p.v + kv_base * D;
     const T *ksc = (const T *)p.k_scale + kv_base, *vsc = (const T *)p.v_scale + kv_base;  // KVI8 only
+    // PAGED: pool row (in units of rows of one head) of row `r` of the tile starting at t0 = page's first row + r % P
+    const int psh = p.page_shift, pmask = (1 << psh) - 1, pg0 = k0 >> psh;
+    int pg_reg = 0;
+    if constexpr (PAGED) {
+        if (pg0 + lane < p.pages_per_seq) pg_reg = p.page_table[(size_t)b * p.pages_per_seq + pg0 + lane];
+    }
+    auto page_rows0 = [&](int t0) -> size_t {
+        const int pg = __builtin_amdgcn_readlane(pg_reg, __builtin_amdgcn_readfirstlane((t0 >> psh) - pg0));
+        return ((size_t)pg * p.Hkv + hkv) << psh;
+    };
     auto operand = [](const Chunk &c) -> U4 {
         if constexpr (KVI8) return i8x8_to_operand<T>(c.x, c.y);
         else return c;
@@ -101,11 +115,17 @@ __global__ __launch_bounds__(kStreamThreads) void attn_stream_kernel(AttnParams 
     // (KVI8: the scales of the lane's 2 x 4 score keys travel with the tile, 8 bytes per load; the cache
     // length is a multiple of 32 there, so a tile never reaches past its row of scales)
     auto load_tile = [&](int t0, Chunk (*kr)[KB], Chunk *vr, uint2 *sr) {
+        size_t po = 0;
+        if constexpr (PAGED) po = page_rows0(t0);
+        auto at = [&](int row) -> size_t {
+            if constexpr (PAGED) return po + (size_t)(row & pmask);
+            else return (size_t)row;
+        };
         if constexpr (KVI8) {
 #pragma unroll
             for (int a = 0; a < 2; a++) {
-                sr[a] = *(const uint2 *)(ksc + t0 + a * 16 + quad * 4);
-                sr[2 + a] = *(const uint2 *)(vsc + t0 + a * 16 + quad * 4);
+                sr[a] = *(const uint2 *)(ksc + at(t0 + a * 16 + quad * 4));
+                sr[2 + a] = *(const uint2 *)(vsc + at(t0 + a * 16 + quad * 4));
             }
         }
         // rows past the range re-read the last valid row; their scores are masked below
@@ -113,12 +133,12 @@ __global__ __launch_bounds__(kStreamThreads) void attn_stream_kernel(AttnParams 
         for (int a = 0; a < 2; a++) {
             const int krow = min(t0 + a * 16 + col, k1 - 1);
 #pragma unroll
-            for (int j = 0; j < KB; j++) kr[a][j] = *(const Chunk *)(Kp + (size_t)krow * D + j * 32 + quad * 8);
+            for (int j = 0; j < KB; j++) kr[a][j] = *(const Chunk *)(Kp + at(krow) * D + j * 32 + quad * 8);
         }
 #pragma unroll
         for (int q = 0; q < NP; q++) {
             const int vrow = min(t0 + q * KPP + vk, k1 - 1);
-            vr[q] = *(const Chunk *)(Vp + (size_t)vrow * D + vd);
+            vr[q] = *(const Chunk *)(Vp + at(vrow) * D + vd);
         }
     };
 
@@ -217,7 +237,9 @@ __global__ __launch_bounds__(kStreamThreads) void attn_stream_kernel(AttnParams 
     Chunk kA[2][KB], vA[NP], kB[2][KB], vB[NP];
     uint2 sA[4], sB[4];
     const int tstep = kStreamWaves * kStreamTile;
-    const int last_tile = max(p.cache_len - kStreamTile, 0);  // start of the last whole tile (0 for a cache shorter than a tile)
+    // start of the last whole tile (0 for a cache shorter than a tile); PAGED: of the last tile with a row of this
+    // range in it -- pages further on need not exist
+    const int last_tile = PAGED ? max(k1 - 1, 0) / kStreamTile * kStreamTile : max(p.cache_len - kStreamTile, 0);
     int t = k0 + wave * kStreamTile;
     if (t < k1) {
         load_tile(t, kA, vA, sA);
@@ -346,17 +368,31 @@ void attn_stream_plan(int B, int Hkv, int kv_len, int *slice, int *nsplit) {
     *nsplit = (kv_len + rows - 1) / rows;
 }
 
-template <typename T, int D, bool KVI8>
+template <typename T, int D, bool KVI8, bool PAGED>
 static int stream_g(const AttnParams &p, hipStream_t s) {
     dim3 grid(p.B * p.Hkv, p.nsplit), block(kStreamThreads);
     switch (p.Hq / p.Hkv) {
-    case 1: MYNN_LAUNCH((attn_stream_kernel<T, D, 1, KVI8>), grid, block, 0, s, p); break;
-    case 2: MYNN_LAUNCH((attn_stream_kernel<T, D, 2, KVI8>), grid, block, 0, s, p); break;
-    case 4: MYNN_LAUNCH((attn_stream_kernel<T, D, 4, KVI8>), grid, block, 0, s, p); break;
-    case 8: MYNN_LAUNCH((attn_stream_kernel<T, D, 8, KVI8>), grid, block, 0, s, p); break;
+    case 1: MYNN_LAUNCH((attn_stream_kernel<T, D, 1, KVI8, PAGED>), grid, block, 0, s, p); break;
+    case 2: MYNN_LAUNCH((attn_stream_kernel<T, D, 2, KVI8, PAGED>), grid, block, 0, s, p); break;
+    case 4: MYNN_LAUNCH((attn_stream_kernel<T, D, 4, KVI8, PAGED>), grid, block, 0, s, p); break;
+    case 8: MYNN_LAUNCH((attn_stream_kernel<T, D, 8, KVI8, PAGED>), grid, block, 0, s, p); break;
     default: return fail(MYNN_ERR_UNSUPPORTED, "streaming attention: %d query heads per kv head", p.Hq / p.Hkv);
     }
     return launch_status("attn_stream_kernel");
+}
+
+template <typename T, int D>
+static int stream_kv(const AttnParams &p, int kv_int8, hipStream_t s) {
+    if (p.page_table) return kv_int8 ? stream_g<T, D, true, true>(p, s) : stream_g<T, D, false, true>(p, s);
+    return kv_int8 ? stream_g<T, D, true, false>(p, s) : stream_g<T, D, false, false>(p, s);
+}
+
+// what the paged form needs whatever the sizes: one query row, a 16-bit type, head_dim 64 or 128, 1/2/4/8 query heads
+// per kv head, pages of a power of two >= 32 rows
+bool attn_stream_paged_supported(int Sq, int Hq, int Hkv, int D, int dtype, int page_rows) {
+    const int G = Hkv > 0 ? Hq / Hkv : 0;
+    return Sq == 1 && (dtype == MYNN_F16 || dtype == MYNN_BF16) && (D == 64 || D == 128) && (G == 1 || G == 2 || G == 4 || G == 8) &&
+           page_rows >= kStreamTile && (page_rows & (page_rows - 1)) == 0;
 }
 
 int attention_stream_launch(const AttnParams &p, int D, int dtype, int kv_int8, hipStream_t s) {
@@ -368,14 +404,19 @@ int attention_stream_launch(const AttnParams &p, int D, int dtype, int kv_int8, 
                  "streaming attention: no scratch for %d key ranges", p.nsplit);
     MYNN_REQUIRE(p.slice % (kStreamWaves * kStreamTile) == 0 && p.nsplit <= 65535, MYNN_ERR_INVALID,
                  "streaming attention: slice %d, %d ranges", p.slice, p.nsplit);
-    int rc;
-    if (kv_int8) {
-        if (dtype == MYNN_F16) rc = D == 64 ? stream_g<f16_t, 64, true>(p, s) : stream_g<f16_t, 128, true>(p, s);
-        else rc = D == 64 ? stream_g<bf16_t, 64, true>(p, s) : stream_g<bf16_t, 128, true>(p, s);
-    } else {
-        if (dtype == MYNN_F16) rc = D == 64 ? stream_g<f16_t, 64, false>(p, s) : stream_g<f16_t, 128, false>(p, s);
-        else rc = D == 64 ? stream_g<bf16_t, 64, false>(p, s) : stream_g<bf16_t, 128, false>(p, s);
+    if (p.page_table) {
+        MYNN_REQUIRE(attn_stream_paged_supported(p.Sq, p.Hq, p.Hkv, D, dtype, 1 << p.page_shift), MYNN_ERR_UNSUPPORTED,
+                     "paged attention: one query row, 16-bit type, head_dim 64/128, 1/2/4/8 heads per kv head, pages of 2^n >= %d rows",
+                     kStreamTile);
+        MYNN_REQUIRE(p.cache_len == p.pages_per_seq << p.page_shift, MYNN_ERR_INVALID,
+                     "paged attention: cache length %d is not %d pages of %d rows", p.cache_len, p.pages_per_seq, 1 << p.page_shift);
+        // a key range's pages travel in one register, a lane each
+        MYNN_REQUIRE((p.slice >> p.page_shift) + 2 <= 64, MYNN_ERR_UNSUPPORTED,
+                     "paged attention: a key range of %d rows spans more than 62 pages of %d rows", p.slice, 1 << p.page_shift);
     }
+    int rc;
+    if (dtype == MYNN_F16) rc = D == 64 ? stream_kv<f16_t, 64>(p, kv_int8, s) : stream_kv<f16_t, 128>(p, kv_int8, s);
+    else rc = D == 64 ? stream_kv<bf16_t, 64>(p, kv_int8, s) : stream_kv<bf16_t, 128>(p, kv_int8, s);
     if (rc || p.nsplit == 1) return rc;
     return attention_merge_launch(p, D, dtype, s);
 }

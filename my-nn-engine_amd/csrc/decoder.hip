@@ -19,6 +19,7 @@
 
 #include "attention.h"
 #include "kernels.h"
+#include "kv_pages.h"
 
 namespace mynn {
 
@@ -146,6 +147,8 @@ struct Model {
     void *q_ref = nullptr, *k_new = nullptr, *v_new = nullptr, *attn_ref = nullptr, *k_rot = nullptr;
     int last_status = 0;          // of the last model() call on this state
     void *warena = nullptr;       // weight_arena: every linear weight and scale of the model in one allocation, in execution order
+    mynn_kv_pages *pages = nullptr;  // kv_page_rows: the session's page table (the caller's); k_cache / v_cache then are pools
+    KvPaging paging;
     void *ws = nullptr;           // executors that dequantise a weight per call (M >= 16, no resident copy): their own workspace
     // per-launch record of the last enqueue (names + algorithmic bytes), events when profiling
     std::vector<Launch> record;
@@ -377,7 +380,7 @@ static int enqueue_step(Model &m) {
             nrm_ready = false;
             if (m.skinny) {
                 // (16-bit KV cache) RoPE and both cache appends ride on the launch that sums the projection's K ranges
-                const SkinnyRope rp{m.q, L.k_cache, L.v_cache, m.cos_t, m.sin_t, m.d_pos, m.d_past, S, Hq, Hkv, D, c.max_seq};
+                const SkinnyRope rp{m.q, L.k_cache, L.v_cache, m.cos_t, m.sin_t, m.d_pos, m.d_past, S, Hq, Hkv, D, c.max_seq, m.paging};
                 TRY(skinny_rows(m, m.qkv, m.nrm, L.qkv, L.pk_qkv, nullptr, rows, GEMM_PLAIN, "linear_qkv", nullptr, nullptr,
                                 kv8 || streaming ? nullptr : &rp, &roped));
             }
@@ -394,8 +397,9 @@ static int enqueue_step(Model &m) {
             p.is_causal = S > 1; p.B = B; p.Sq = S; p.Hq = Hq; p.Hkv = Hkv; p.cache_len = c.max_seq;
             p.d_active = m.d_active; p.nsplit = m.nsplit; p.slice = m.slice; p.heads_per_wg = m.heads_per_wg;
             attn_token_major_layout(p, D);
+            p.page_table = m.paging.table; p.page_shift = m.paging.shift; p.pages_per_seq = m.paging.pages_per_seq;
             // (an int8 cache: the form for a cache one workgroup covers quantises the new row itself)
-            const bool fuse_attn = (fused || qfused) &&
+            const bool fuse_attn = (fused || qfused) && !m.pages &&
                                    (kv8 ? attention_fused_kv8_supported(D, c.max_seq) : attention_fused_supported(D, Hq / Hkv));
             if (fuse_attn) {
                 // RoPE(q), RoPE(k), both cache appends and the attention in one launch
@@ -405,7 +409,9 @@ static int enqueue_step(Model &m) {
             } else {
                 // prefill on the matrix cores: the attention kernel rotates the queries itself, reading them from the
                 // projection's output; the RoPE launch is left with the keys and the values
-                const bool pf = S > 1 && !kv8 && !roped && attention_prefill_supported(p, D, c.dtype, kv8);
+                // (a paged cache: that kernel for every prefill shape -- the per-row kernel has no paged form)
+                const bool pf_kernel = S > 1 && (attention_prefill_supported(p, D, c.dtype, kv8) || m.pages);
+                const bool pf = pf_kernel && !kv8 && !roped;
                 const bool q_in_attn = pf && ((size_t)(QD + 2 * KD) * sizeof(T)) % 16 == 0 && aligned16(m.qkv);
                 if (!roped) note(m, kv8 ? "rope_quant_kv_append" : q_in_attn ? "rope_kv_append_k_v" : "rope_kv_append",
                                  q_in_attn ? (double)rows * 2 * KD * 2 * eb : (double)rows * (QD + 2 * KD) * 2 * eb);
@@ -415,7 +421,7 @@ static int enqueue_step(Model &m) {
                                                 m.cos_t, m.sin_t, m.d_pos, m.d_past, B, S, Hq, Hkv, D, c.max_seq, s));
                 else
                     TRY(rope_kv_append<T>(q_in_attn ? nullptr : m.q, L.k_cache, L.v_cache, m.qkv, m.cos_t, m.sin_t, m.d_pos, m.d_past, 0, B, S,
-                                          Hq, Hkv, D, c.max_seq, s));
+                                          Hq, Hkv, D, c.max_seq, s, m.paging));
                 if (q_in_attn) {
                     p.q = m.qkv; p.rope_q = 1; p.cos_t = m.cos_t; p.sin_t = m.sin_t; p.d_pos = m.d_pos;
                     p.q_bs = (long)S * (QD + 2 * KD); p.q_hs = D; p.q_rs = QD + 2 * KD;
@@ -424,7 +430,7 @@ static int enqueue_step(Model &m) {
                 // know under replay -- callers add 2*KD*eb per cached row when they report
                 // flops: the causal half of QK^T and PV over the new rows alone (exact when past_len is 0)
                 note(m, "attention", (double)rows * 2.0 * QD * eb, S > 1 ? 2.0 * B * Hq * D * (double)S * (S + 1) : 0.0);
-                if (S > 1 && attention_prefill_supported(p, D, c.dtype, kv8)) TRY(attention_prefill_launch(p, D, c.dtype, s));
+                if (pf_kernel) TRY(attention_prefill_launch(p, D, c.dtype, s));
                 else TRY(attention_decode_launch(p, D, c.dtype, kv8, m.attn_scratch, s));
             }
         }
@@ -614,6 +620,15 @@ static int build(Model &m, void **init, void **state) {
             MYNN_REQUIRE(L.k_scale && L.v_scale, MYNN_ERR_INVALID, "model_init: null KV scale buffer in layer %d", li);
         }
     }
+    if (c.kv_page_rows) {
+        m.pages = (mynn_kv_pages *)state[2 * c.n_layers];
+        MYNN_REQUIRE(m.pages, MYNN_ERR_INVALID, "model_init: kv_page_rows without a page set after the pools in session_state");
+        m.paging = kv_pages_paging(m.pages);
+        MYNN_REQUIRE((1 << m.paging.shift) == c.kv_page_rows && m.paging.pages_per_seq * c.kv_page_rows == c.max_seq &&
+                         kv_pages_batch(m.pages) == c.batch,
+                     MYNN_ERR_INVALID, "model_init: the page set (batch %d, %d pages of %d rows) does not fit batch %d, max_seq %d, kv_page_rows %d",
+                     kv_pages_batch(m.pages), m.paging.pages_per_seq, 1 << m.paging.shift, c.batch, c.max_seq, c.kv_page_rows);
+    }
     m.final_norm = init[i++];
     lin(m.lm_head, V, H);
     MYNN_REQUIRE(m.embed.w && m.final_norm && m.lm_head.w, MYNN_ERR_INVALID, "model_init: null embed/norm/lm_head");
@@ -723,10 +738,16 @@ static int build(Model &m, void **init, void **state) {
     // ---- arena: every activation of one step, the device scalars, attention split scratch
     const int rows = c.batch * c.seq_q;
     {
-        const bool fused_attn = m.quant && rows == 1 && !c.quantize_activations && !c.quant_kv_cache &&
+        const bool fused_attn = m.quant && rows == 1 && !c.quantize_activations && !c.quant_kv_cache && !m.pages &&
                                 attention_fused_supported(c.head_dim, c.n_heads / c.n_kv_heads);
         attn_plan(c.batch, c.seq_q, c.n_heads, c.n_kv_heads, c.head_dim, c.dtype, c.quant_kv_cache, c.max_seq, c.max_seq, fused_attn,
                   &m.slice, &m.nsplit, &m.heads_per_wg);
+        if (m.pages) {  // decode: the streaming kernel whatever the sizes; prefill: the matrix-core kernel, no key ranges
+            m.slice = 0;
+            m.nsplit = 1;
+            m.heads_per_wg = c.n_heads / c.n_kv_heads;
+            if (c.seq_q == 1) attn_stream_plan(c.batch, c.n_kv_heads, c.max_seq, &m.slice, &m.nsplit);
+        }
     }
     m.token_cap = c.max_seq + 8;
     ArenaPlan plan;
@@ -780,7 +801,7 @@ static int build(Model &m, void **init, void **state) {
 
     // ---- batch-1 decode: projection and attention in one launch when the shape allows
     m.spin_limit = c.handover_spin_limit > 0 ? c.handover_spin_limit : c.handover_spin_limit < 0 ? 0 : 400000;
-    if (m.quant && rows == 1 && !c.quantize_activations && !c.unfused_decode &&
+    if (m.quant && rows == 1 && !c.quantize_activations && !c.unfused_decode && !m.pages &&
         attention_fused_supported(c.head_dim, c.n_heads / c.n_kv_heads) &&
         (!c.quant_kv_cache || attention_fused_kv8_supported(c.head_dim, c.max_seq)) &&
         qkv_attention_supported(H, c.n_heads, c.n_kv_heads, c.head_dim, c.max_seq, c.dtype) && (QD + 2 * KD) * eb % 8 == 0) {
@@ -887,6 +908,8 @@ static int upload_inputs(Model &m, const int64_t *ids, const int64_t *pos, int64
     MYNN_REQUIRE(past >= 0 && past + c.seq_q <= c.max_seq, MYNN_ERR_TOO_LONG,
                  "past_len %lld + %d rows exceeds max_seq %d", (long long)past, c.seq_q, c.max_seq);
     MYNN_REQUIRE(active >= 1 && active <= c.max_seq, MYNN_ERR_INVALID, "active_seq_kv %lld out of range", (long long)active);
+    // paged cache: every row the step writes or may read has a page before anything is launched
+    if (m.pages) TRY(kv_pages_reserve(m.pages, std::max<long>(past + c.seq_q, active)));
     for (int s = 0; s < c.seq_q; s++)
         MYNN_REQUIRE(pos[s] >= 0 && pos[s] < c.max_seq, MYNN_ERR_INVALID, "position_id[%d]=%lld outside the RoPE table", s,
                      (long long)pos[s]);
@@ -956,6 +979,17 @@ static int check_config(const mynn_model_config *cfg) {
     MYNN_REQUIRE(cfg->gemm_tile >= 0 && cfg->gemm_tile <= 4, MYNN_ERR_INVALID, "model_configure: gemm_tile %d (0..4)", cfg->gemm_tile);
     MYNN_REQUIRE(!cfg->streaming_kv || (cfg->batch == 1 && cfg->head_dim % 2 == 0), MYNN_ERR_UNSUPPORTED,
                  "model_configure: streaming_kv is a batch-1 graph (crates/llm) with an even head_dim");
+    if (cfg->kv_page_rows) {
+        const int P = cfg->kv_page_rows;
+        MYNN_REQUIRE(P >= 64 && (P & (P - 1)) == 0 && cfg->max_seq % P == 0, MYNN_ERR_INVALID,
+                     "model_configure: kv_page_rows %d (a power of two >= 64 that divides max_seq %d)", P, cfg->max_seq);
+        MYNN_REQUIRE(!cfg->quant_kv_cache && !cfg->streaming_kv, MYNN_ERR_UNSUPPORTED,
+                     "model_configure: a paged KV cache is 16-bit and takes neither quant_kv_cache nor streaming_kv");
+        MYNN_REQUIRE(cfg->seq_q == 1 || cfg->max_seq / P <= 64, MYNN_ERR_UNSUPPORTED,
+                     "model_configure: a prefill model reads at most 64 pages per sequence (max_seq %d, %d rows per page)", cfg->max_seq, P);
+        MYNN_REQUIRE(attn_stream_paged_supported(1, cfg->n_heads, cfg->n_kv_heads, cfg->head_dim, cfg->dtype, P), MYNN_ERR_UNSUPPORTED,
+                     "model_configure: a paged KV cache needs head_dim 64 or 128 and 1, 2, 4 or 8 query heads per kv head");
+    }
     return 0;
 }
 
@@ -1136,6 +1170,7 @@ extern "C" int mynn_model_decode_loop(void *state, int32_t token, int64_t past_l
     MYNN_REQUIRE(c.batch * c.seq_q == 1 && !c.streaming_kv, MYNN_ERR_STATE, "decode_loop: needs a batch-1 decode model without streaming_kv");
     MYNN_REQUIRE(past_len + n_steps <= c.max_seq && n_steps <= m.token_cap, MYNN_ERR_TOO_LONG,
                  "decode_loop: past_len %lld + %d steps exceeds max_seq %d", (long long)past_len, n_steps, c.max_seq);
+    if (m.pages) TRY(kv_pages_reserve(m.pages, past_len + n_steps));
     for (int attempt = 0; attempt < 2; attempt++) {
         int64_t id = token, pos = past_len;
         TRY(upload_inputs(m, &id, &pos, past_len, past_len + 1));

@@ -26,6 +26,18 @@ size_t skinny_scratch_bytes(int M, int N, int K);
 // `packed`: wq is a tiled copy (skinny_packed_bytes, made by skinny_pack_weight) that a wave reads sequentially
 size_t skinny_packed_bytes(int N, int K);
 int skinny_pack_weight(void *dst, const int8_t *wq, int N, int K, hipStream_t s);
+// paging: the caches are pools [n_pages, Hkv, 1 << shift, D]; row r of sequence b goes to pool page
+// table[b * pages_per_seq + (r >> shift)] (a device array), row r % (1 << shift) of it.  table == nullptr: contiguous caches.
+struct KvPaging {
+    const int32_t *table = nullptr;
+    int shift = 0, pages_per_seq = 0;
+};
+// row index (in rows of D elements) of cache row `r` of kv head `hk` of sequence `b`
+__device__ inline size_t kv_cache_row(const KvPaging &pg, int b, int hk, int r, int Hkv, int max_seq) {
+    if (!pg.table) return ((size_t)b * Hkv + hk) * max_seq + r;
+    const int page = pg.table[(size_t)b * pg.pages_per_seq + (r >> pg.shift)];
+    return (((size_t)page * Hkv + hk) << pg.shift) + (size_t)(r & ((1 << pg.shift) - 1));
+}
 // rope (optional, plain store of a q|k|v projection): instead of storing the projection, rotate q and k by the
 // rows' positions and write q to q_out and k, v into the caches -- what rope_kv_append would do next
 struct SkinnyRope {
@@ -34,6 +46,7 @@ struct SkinnyRope {
     const int64_t *position;
     const int32_t *d_past;
     int S, Hq, Hkv, D, max_seq;
+    KvPaging paging;
 };
 int dequant_gemm_skinny(void *out, const void *act, const int8_t *wq, bool packed, const void *scale, const void *res, int M,
                         int N, int K, int dtype, int epi, float *scratch, hipStream_t s, const void *norm_w = nullptr,
@@ -138,7 +151,7 @@ int embed_dequant(void *out, const int8_t *table, const void *scale, const int64
 template <typename T>
 int rope_kv_append(void *q_out, void *k_cache, void *v_cache, const void *qkv, const void *cos_t, const void *sin_t,
                    const int64_t *position, const int32_t *d_past, int past_host, int B, int S, int Hq, int Hkv, int D,
-                   int max_seq, hipStream_t s);
+                   int max_seq, hipStream_t s, KvPaging paging = KvPaging());
 // the same for an int8 KV cache: k (after RoPE, rounded to T) and v are quantised per token row into
 // the caches and their scale rows [B,Hkv,max_seq] (QuantizingKVCacheUpdate, CPU backend rounding)
 template <typename T>

@@ -13,7 +13,7 @@ namespace mynn {
 template <typename T>
 __global__ void rope_kv_append_kernel(T *q_out, T *k_cache, T *v_cache, const T *qkv, const T *cos_t, const T *sin_t,
                                       const int64_t *position, const int32_t *d_past, int past_host, int S, int Hq,
-                                      int Hkv, int D, int max_seq) {
+                                      int Hkv, int D, int max_seq, KvPaging pg) {
     const int s = blockIdx.x, head = blockIdx.y, b = blockIdx.z;
     const int half = D / 2;
     const int past = d_past ? *d_past : past_host;
@@ -23,7 +23,7 @@ __global__ void rope_kv_append_kernel(T *q_out, T *k_cache, T *v_cache, const T 
     if (head < Hq && !q_out) return;
     if (head < Hq + Hkv) {
         T *dst = head < Hq ? q_out + row * (size_t)Hq * D + (size_t)head * D
-                           : k_cache + (((size_t)b * Hkv + (head - Hq)) * max_seq + past + s) * D;
+                           : k_cache + kv_cache_row(pg, b, head - Hq, past + s, Hkv, max_seq) * D;
         const size_t tab = (size_t)position[s] * D;
         for (int j = threadIdx.x; j < half; j += blockDim.x) {
             float xl = Elem<T>::ld(src, j), xh = Elem<T>::ld(src, j + half);
@@ -33,7 +33,7 @@ __global__ void rope_kv_append_kernel(T *q_out, T *k_cache, T *v_cache, const T 
             Elem<T>::st(dst, j + half, xh * ch + xl * sh);
         }
     } else {
-        T *dst = v_cache + (((size_t)b * Hkv + (head - Hq - Hkv)) * max_seq + past + s) * D;
+        T *dst = v_cache + kv_cache_row(pg, b, head - Hq - Hkv, past + s, Hkv, max_seq) * D;
         for (int j = threadIdx.x; j < D; j += blockDim.x) dst[j] = src[j];
     }
 }
@@ -45,7 +45,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void rope_kv_append_vec_kernel(T *q_out, T *k_cache, T *v_cache, const T *qkv,
                                                                  const T *cos_t, const T *sin_t, const int64_t *position,
                                                                  const int32_t *d_past, int past_host, int S, int Hq,
-                                                                 int Hkv, int D, int max_seq) {
+                                                                 int Hkv, int D, int max_seq, KvPaging pg) {
     const int s = blockIdx.x, b = blockIdx.y;
     const int half = D / 2, upc = half / 8;  // units per head
     const int past = d_past ? *d_past : past_host;
@@ -59,13 +59,13 @@ __global__ __launch_bounds__(256) void rope_kv_append_vec_kernel(T *q_out, T *k_
         const T *src = src_row + (size_t)head * D;
         const U4 lo = *(const U4 *)(src + j), hi = *(const U4 *)(src + j + half);
         if (head >= Hq + Hkv) {
-            T *dst = v_cache + (((size_t)b * Hkv + (head - Hq - Hkv)) * max_seq + past + s) * D;
+            T *dst = v_cache + kv_cache_row(pg, b, head - Hq - Hkv, past + s, Hkv, max_seq) * D;
             *(U4 *)(dst + j) = lo;
             *(U4 *)(dst + j + half) = hi;
             continue;
         }
         T *dst = head < Hq ? q_out + row * (size_t)Hq * D + (size_t)head * D
-                           : k_cache + (((size_t)b * Hkv + (head - Hq)) * max_seq + past + s) * D;
+                           : k_cache + kv_cache_row(pg, b, head - Hq, past + s, Hkv, max_seq) * D;
         float xl[8], xh[8], cl[8], ch[8], sl[8], sh[8], ol[8], oh[8];
         widen8<T>(lo, xl);
         widen8<T>(hi, xh);
@@ -157,26 +157,64 @@ template int rope_quant_kv_append<f16_t>(void *, int8_t *, int8_t *, void *, voi
 template <typename T>
 int rope_kv_append(void *q_out, void *k_cache, void *v_cache, const void *qkv, const void *cos_t, const void *sin_t,
                    const int64_t *position, const int32_t *d_past, int past_host, int B, int S, int Hq, int Hkv, int D,
-                   int max_seq, hipStream_t s) {
+                   int max_seq, hipStream_t s, KvPaging paging) {
     MYNN_REQUIRE(S <= 65535 * 32 && Hq + 2 * Hkv <= 65535 && B <= 65535, MYNN_ERR_UNSUPPORTED, "rope_kv_append: grid");
+    MYNN_REQUIRE(!paging.table || (paging.shift > 0 && paging.shift < 31 && max_seq == paging.pages_per_seq << paging.shift),
+                 MYNN_ERR_INVALID, "rope_kv_append: %d rows per sequence are not %d pages of %d rows", max_seq,
+                 paging.pages_per_seq, 1 << paging.shift);
     if (D % 16 == 0 && S <= 65535 * 32 && (!q_out || aligned16(q_out)) && aligned16(k_cache) && aligned16(v_cache) && aligned16(qkv) &&
         aligned16(cos_t) && aligned16(sin_t)) {
         const int units = (q_out ? Hq + 2 * Hkv : 2 * Hkv) * (D / 16);
         const int threads = units >= 256 ? 256 : (units + 63) / 64 * 64;
         MYNN_LAUNCH(rope_kv_append_vec_kernel<T>, dim3(S, B), dim3(threads), 0, s, (T *)q_out, (T *)k_cache,
                            (T *)v_cache, (const T *)qkv, (const T *)cos_t, (const T *)sin_t, position, d_past, past_host,
-                           S, Hq, Hkv, D, max_seq);
+                           S, Hq, Hkv, D, max_seq, paging);
         return launch_status("rope_kv_append_vec_kernel");
     }
     int threads = D / 2 >= 64 ? 64 : 32;
     MYNN_LAUNCH(rope_kv_append_kernel<T>, dim3(S, Hq + 2 * Hkv, B), dim3(threads), 0, s, (T *)q_out,
                        (T *)k_cache, (T *)v_cache, (const T *)qkv, (const T *)cos_t, (const T *)sin_t, position, d_past,
-                       past_host, S, Hq, Hkv, D, max_seq);
+                       past_host, S, Hq, Hkv, D, max_seq, paging);
     return launch_status("rope_kv_append_kernel");
 }
 template int rope_kv_append<bf16_t>(void *, void *, void *, const void *, const void *, const void *, const int64_t *,
-                                    const int32_t *, int, int, int, int, int, int, int, hipStream_t);
+                                    const int32_t *, int, int, int, int, int, int, int, hipStream_t, KvPaging);
 template int rope_kv_append<f16_t>(void *, void *, void *, const void *, const void *, const void *, const int64_t *,
-                                   const int32_t *, int, int, int, int, int, int, int, hipStream_t);
+                                   const int32_t *, int, int, int, int, int, int, int, hipStream_t, KvPaging);
+
+// KVCacheUpdate into a pool: pool row of (b, hk, offset + t) <- new[b, hk, t, :]; rows of `units` 4-byte units
+__global__ void kvcache_update_paged_kernel(uint32_t *pool, const uint32_t *src, int offset, int Hkv, int S_new, int units,
+                                            KvPaging pg, size_t total) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int u = (int)(i % units);
+    const size_t row = i / units;
+    const int t = (int)(row % S_new), hk = (int)((row / S_new) % Hkv), b = (int)(row / ((size_t)S_new * Hkv));
+    pool[kv_cache_row(pg, b, hk, offset + t, Hkv, 0) * units + u] = src[i];
+}
 
 }  // namespace mynn
+
+using namespace mynn;
+
+extern "C" int mynn_kvcache_update_paged(void *pool, const void *new_kv, int offset, int B, int Hkv, int S_new, int D, int dtype,
+                                         const int32_t *page_table, int pages_per_seq, int page_rows, mynn_stream s) {
+    MYNN_REQUIRE(pool && new_kv && page_table, MYNN_ERR_INVALID, "kvcache_update_paged: null operand");
+    MYNN_REQUIRE(page_rows >= 32 && page_rows <= (1 << 20) && (page_rows & (page_rows - 1)) == 0 && pages_per_seq > 0, MYNN_ERR_INVALID,
+                 "kvcache_update_paged: %d pages of %d rows (rows per page: a power of two, 32 or more)", pages_per_seq, page_rows);
+    MYNN_REQUIRE(B > 0 && Hkv > 0 && S_new > 0 && D > 0 && offset >= 0 && (long)offset + S_new <= (long)pages_per_seq * page_rows,
+                 MYNN_ERR_INVALID, "kvcache_update_paged: offset %d + %d rows exceeds %d pages of %d rows", offset, S_new, pages_per_seq,
+                 page_rows);
+    MYNN_REQUIRE(dtype_ok(dtype), MYNN_ERR_INVALID, "kvcache_update_paged: dtype %d", dtype);
+    const size_t row_bytes = (size_t)D * dtype_size(dtype);
+    MYNN_REQUIRE(row_bytes % 4 == 0, MYNN_ERR_UNSUPPORTED, "kvcache_update_paged: rows of %zu bytes", row_bytes);
+    KvPaging pg;
+    pg.table = page_table;
+    pg.pages_per_seq = pages_per_seq;
+    while ((1 << pg.shift) < page_rows) pg.shift++;
+    const int units = (int)(row_bytes / 4);
+    const size_t total = (size_t)B * Hkv * S_new * units;
+    MYNN_LAUNCH(kvcache_update_paged_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, as_stream(s), (uint32_t *)pool,
+                (const uint32_t *)new_kv, offset, Hkv, S_new, units, pg, total);
+    return launch_status("kvcache_update_paged_kernel");
+}

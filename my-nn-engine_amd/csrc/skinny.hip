@@ -281,7 +281,7 @@ __global__ __launch_bounds__(kReduceNormThreads) void skinny_reduce_rope_kernel(
                                                                               T *q_out, T *k_cache, T *v_cache, const T *cos_t,
                                                                               const T *sin_t, const int64_t *position,
                                                                               const int32_t *d_past, int S, int Hq, int Hkv, int D,
-                                                                              int max_seq) {
+                                                                              int max_seq, KvPaging pg) {
     const int m = blockIdx.x, b = m / S, sq = m % S;
     const int half = D / 2, upr = half / 4, upv = D / 4;  // units per rotated head / per v head
     const int rot_units = (Hq + Hkv) * upr, units = rot_units + Hkv * upv;
@@ -318,7 +318,7 @@ __global__ __launch_bounds__(kReduceNormThreads) void skinny_reduce_rope_kernel(
             const int hv = (u - rot_units) / upv, j = ((u - rot_units) % upv) * 4;
             float t[4];
             total4((Hq + Hkv + hv) * D + j, t);
-            T *dst = v_cache + (((size_t)b * Hkv + hv) * max_seq + past + sq) * D + j;
+            T *dst = v_cache + kv_cache_row(pg, b, hv, past + sq, Hkv, max_seq) * D + j;
             *(uint2 *)dst = uint2{pack2<T>(t[0], t[1]), pack2<T>(t[2], t[3])};
             continue;
         }
@@ -331,7 +331,7 @@ __global__ __launch_bounds__(kReduceNormThreads) void skinny_reduce_rope_kernel(
         ld4(sin_t + tab + j, sl);
         ld4(sin_t + tab + j + half, sh);
         T *dst = head < Hq ? q_out + (size_t)m * Hq * D + (size_t)head * D
-                           : k_cache + (((size_t)b * Hkv + (head - Hq)) * max_seq + past + sq) * D;
+                           : k_cache + kv_cache_row(pg, b, head - Hq, past + sq, Hkv, max_seq) * D;
         float ol[4], oh[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -408,7 +408,7 @@ int dequant_gemm_skinny(void *out, const void *act, const int8_t *wq, bool packe
             ((uintptr_t)rope->sin_t & 7) == 0) {
             MYNN_LAUNCH(skinny_reduce_rope_kernel<T>, dim3(M), dim3(kReduceNormThreads), 0, s, scratch, (const T *)scale, M, N, ks_used,
                         (T *)rope->q_out, (T *)rope->k_cache, (T *)rope->v_cache, (const T *)rope->cos_t, (const T *)rope->sin_t,
-                        rope->position, rope->d_past, rope->S, rope->Hq, rope->Hkv, rope->D, rope->max_seq);
+                        rope->position, rope->d_past, rope->S, rope->Hq, rope->Hkv, rope->D, rope->max_seq, rope->paging);
             *roped = true;
             return launch_status("skinny_reduce_rope_kernel");
         }
