@@ -420,7 +420,17 @@ def decode_batch_main(args, mynn):
     gen.manual_seed(args.seed + 1)
     shape = (B, cfg["n_kv_heads"], cfg["max_seq"], cfg["head_dim"])
     kv = []
-    for _ in range(cfg["n_layers"]):
+    pages = pool = None
+    if args.kv_pages:
+        # paged cache: one pool for the batch, pages of every sequence interleaved (page = slot * B + sequence)
+        assert not args.kv_int8 and cfg["max_seq"] % args.kv_pages == 0
+        pool = mynn.KvPool(B * cfg["max_seq"] // args.kv_pages, args.kv_pages)
+        pshape = (pool.n_pages, cfg["n_kv_heads"], args.kv_pages, cfg["head_dim"])
+        for _ in range(cfg["n_layers"]):
+            kv.append((torch.randn(pshape, generator=gen, device="cuda", dtype=tdt), torch.randn(pshape, generator=gen, device="cuda", dtype=tdt)))
+        pages = mynn.KvPages(pool, B, cfg["max_seq"])
+        pages.reserve(ctx)
+    for _ in range(0 if args.kv_pages else cfg["n_layers"]):
         if args.kv_int8:
             bufs = []
             for _ in range(2):
@@ -440,7 +450,7 @@ def decode_batch_main(args, mynn):
             v[:, :, :ctx] = torch.randn((B, shape[1], ctx, shape[3]), generator=gen, device="cuda", dtype=tdt)
             kv.append((k, v))
     torch.cuda.synchronize()
-    dec = mynn.Decoder(cfg, weights, batch=B, kv=kv, quant_kv_cache=args.kv_int8)
+    dec = mynn.Decoder(cfg, weights, batch=B, kv=kv, quant_kv_cache=args.kv_int8, kv_pages=pages)
     stats = dec.stats()
     rng = np.random.default_rng(args.seed)
     toks = rng.integers(0, cfg["vocab"], B).tolist()
@@ -484,8 +494,10 @@ def decode_batch_main(args, mynn):
         "dtype": "f32 accumulate over int8 weights, %s activations, %s KV" % (args.dtype, "int8" if args.kv_int8 else args.dtype),
         "data": "synthetic",
         "config": {"workload": "configs[4]: Llama-3-8B-shape int8 decoder, batch 32, context 2048 (caches filled with "
-                               "random rows%s), %d decode steps timed" % (", int8 KV cache" if args.kv_int8 else "", K),
+                               "random rows%s), %d decode steps timed" % (", int8 KV cache" if args.kv_int8 else ", paged KV cache" if args.kv_pages else "", K),
                    "batch": B, "context": ctx, "launches_per_step": stats["launches_per_step"], "hipgraph": stats["graph"],
+                   "kv_page_rows": args.kv_pages or None,
+                   "kv_pages_mapped": (pool.n_pages - pool.free_pages) if pool else None,
                    "seed": args.seed, "step_algorithmic_bytes": step_bytes,
                    "step_hbm_frac": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                    "per_kernel_ms": {k: round(v[1] / 2, 3) for k, v in sorted(agg.items(), key=lambda kv: -kv[1][1])}},
@@ -497,6 +509,8 @@ def decode_batch_main(args, mynn):
                      "avg_launch_us": round(ms_tot / calls * 1e3, 2)},
     }
     dec.close()
+    if pages:
+        pages.close(), pool.close()
     print(json.dumps(out))
 
 
@@ -552,6 +566,8 @@ def main():
                     help="prefill: quantise activations per row and run every linear as int8 x int8 (Options::quantize_activations)")
     ap.add_argument("--kv-int8", action="store_true",
                     help="decode / decode_batch: int8 KV cache with per-token scales (BuildOptions::quant_kv_cache)")
+    ap.add_argument("--kv-pages", type=int, default=0, metavar="ROWS",
+                    help="decode_batch: paged KV cache with this many rows per page (kv_page_rows), one pool for the batch")
     ap.add_argument("--weight-arena", action="store_true", help="decode: all weights in one allocation in execution order (weight_arena)")
     ap.add_argument("--unfused", action="store_true", help="decode: every op a launch of its own (unfused_decode)")
     ap.add_argument("--check-tokens", type=int, default=0,
