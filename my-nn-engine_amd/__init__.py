@@ -55,7 +55,7 @@ class ModelConfig(C.Structure):
                 ("ffn", _i), ("vocab", _i), ("max_seq", _i), ("eps", _f), ("rope_theta", _f), ("dtype", _i),
                 ("seq_q", _i), ("batch", _i), ("weights_int8", _i), ("quant_kv_cache", _i),
                 ("quantize_activations", _i), ("streaming_kv", _i), ("gemm_tile", _i), ("unfused_decode", _i),
-                ("handover_spin_limit", _i), ("weight_arena", _i), ("kv_page_rows", _i)]
+                ("handover_spin_limit", _i), ("weight_arena", _i), ("kv_page_rows", _i), ("qkv_bias", _i)]
 
 
 class KernelTime(C.Structure):
@@ -627,7 +627,7 @@ class Decoder:
 
     weights: dict of cuda tensors keyed like the oracle's Model:
       "embed", "lm_head", "layers.{i}.{q,k,v,o,gate,up,down}" -> (int8 [N,K], scale [N]) or a
-      single float tensor [N,K]; "final_norm", "layers.{i}.norm1|norm2".
+      single float tensor [N,K]; "final_norm", "layers.{i}.norm1|norm2"; optional "layers.{i}.{q,k,v}.bias" [N].
     kv: optional list of (k_cache, v_cache) cuda tensors [batch,Hkv,max_seq,D] per layer, so a
       prefill and a decode model can share them (PersistentBuffers in the reference).
     """
@@ -640,11 +640,13 @@ class Decoder:
         tdt = {F16: torch.float16, BF16: torch.bfloat16}[cfg["dtype"]]
         from_file = isinstance(weights, (str, os.PathLike, Weights))
         quant = True if from_file else isinstance(weights["embed"], tuple)
+        # q / k / v projection biases (qwen2): cfg["qkv_bias"], or "layers.{i}.{q,k,v}.bias" entries in a weight dict
+        qkv_bias = bool(cfg.get("qkv_bias")) or (not from_file and "layers.0.q.bias" in weights)
         self.cfg = ModelConfig(cfg["n_layers"], cfg["hidden"], cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"],
                                cfg["ffn"], cfg["vocab"], cfg["max_seq"], float(cfg["eps"]), float(cfg["rope_theta"]),
                                cfg["dtype"], seq_q, batch, int(quant), int(quant_kv_cache), int(quantize_activations),
                                int(streaming_kv), int(gemm_tile), int(unfused_decode), int(handover_spin_limit), int(weight_arena),
-                               kv_pages.pool.page_rows if kv_pages is not None else 0)
+                               kv_pages.pool.page_rows if kv_pages is not None else 0, int(qkv_bias))
         self.weights = weights  # keep the tensors alive
         self.kv_pages = kv_pages
         if kv_pages is not None:
@@ -686,6 +688,8 @@ class Decoder:
             init.append(_ptr(weights["layers.%d.norm1" % l]))
             for nm in ("q", "k", "v", "o"):
                 lin(weights["layers.%d.%s" % (l, nm)])
+                if self.cfg.qkv_bias and nm != "o":
+                    init.append(_ptr(weights["layers.%d.%s.bias" % (l, nm)]))
             init.append(_ptr(weights["layers.%d.norm2" % l]))
             for nm in ("gate", "up", "down"):
                 lin(weights["layers.%d.%s" % (l, nm)])

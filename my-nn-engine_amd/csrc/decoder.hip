@@ -86,6 +86,7 @@ struct Layer {
     void *k_cache = nullptr, *v_cache = nullptr;
     void *k_scale = nullptr, *v_scale = nullptr;  // int8 KV cache: per-token scales [B,Hkv,max_seq]
     void *own_qkv_w = nullptr, *own_qkv_s = nullptr, *own_gu_w = nullptr, *own_gu_s = nullptr;
+    void *qkv_b = nullptr;  // qkv_bias: the q, k, v projection biases concatenated [QD + 2 KD], T (owned)
     // prefill executors: weights dequantised once to the 16-bit type, [N, Kp] (wt_gu: gate/up in groups of 32)
     void *wt_qkv = nullptr, *wt_o = nullptr, *wt_gu = nullptr, *wt_down = nullptr;
     // few-row executors: int8 weights re-tiled so that a wave streams them sequentially
@@ -382,11 +383,16 @@ static int enqueue_step(Model &m) {
                 // (16-bit KV cache) RoPE and both cache appends ride on the launch that sums the projection's K ranges
                 const SkinnyRope rp{m.q, L.k_cache, L.v_cache, m.cos_t, m.sin_t, m.d_pos, m.d_past, S, Hq, Hkv, D, c.max_seq, m.paging};
                 TRY(skinny_rows(m, m.qkv, m.nrm, L.qkv, L.pk_qkv, nullptr, rows, GEMM_PLAIN, "linear_qkv", nullptr, nullptr,
-                                kv8 || streaming ? nullptr : &rp, &roped));
+                                kv8 || streaming || L.qkv_b ? nullptr : &rp, &roped));
             }
             else if (w8a8) TRY(linear_w8a8(m, m.qkv, m.nrm, L.qkv, rows, true, "qlinear_qkv"));
             else if (m.resident16) TRY(gemm_rows(m, m.qkv, m.nrm, L.wt_qkv, nullptr, rows, L.qkv.N, H, GEMM_PLAIN, "linear_qkv"));
             else TRY(linear_rows<T>(m, m.qkv, m.nrm, L.qkv, rows, "linear_qkv"));
+        }
+        if (L.qkv_b) {
+            // the `{node}_bias` Add behind each projection (decoder.rs:167-184): the stored projection plus the bias, rounded again
+            note(m, "add_qkv_bias", (double)rows * 2 * L.qkv.N * eb + (double)L.qkv.N * eb);
+            TRY(add_bias_rows(m.qkv, L.qkv_b, rows, L.qkv.N, c.dtype, s));
         }
         if (streaming) {
             TRY(streaming_attention<T>(m, L, softmax_scale));
@@ -589,8 +595,17 @@ static int build(Model &m, void **init, void **state) {
         Layer &L = m.layers[li];
         L.norm1 = init[i++];
         Lin q, k, v;
-        lin(q, QD, H); lin(k, KD, H); lin(v, KD, H);
+        const void *qb = nullptr, *kb = nullptr, *vb = nullptr;
+        lin(q, QD, H); if (c.qkv_bias) qb = init[i++];
+        lin(k, KD, H); if (c.qkv_bias) kb = init[i++];
+        lin(v, KD, H); if (c.qkv_bias) vb = init[i++];
         lin(L.o, H, QD);
+        if (c.qkv_bias) {
+            MYNN_REQUIRE(qb && kb && vb, MYNN_ERR_INVALID, "model_init: null projection bias in layer %d", li);
+            const void *bp[3] = {qb, kb, vb};
+            const size_t bb[3] = {(size_t)QD * eb, (size_t)KD * eb, (size_t)KD * eb};
+            TRY(concat_rows(&L.qkv_b, bp, bb, 3));
+        }
         L.norm2 = init[i++];
         lin(L.gate, F, H); lin(L.up, F, H); lin(L.down, H, F);
         MYNN_REQUIRE(L.norm1 && L.norm2 && q.w && k.w && v.w && L.o.w && L.gate.w && L.up.w && L.down.w,
@@ -801,7 +816,7 @@ static int build(Model &m, void **init, void **state) {
 
     // ---- batch-1 decode: projection and attention in one launch when the shape allows
     m.spin_limit = c.handover_spin_limit > 0 ? c.handover_spin_limit : c.handover_spin_limit < 0 ? 0 : 400000;
-    if (m.quant && rows == 1 && !c.quantize_activations && !c.unfused_decode && !m.pages &&
+    if (m.quant && rows == 1 && !c.quantize_activations && !c.unfused_decode && !m.pages && !c.qkv_bias &&
         attention_fused_supported(c.head_dim, c.n_heads / c.n_kv_heads) &&
         (!c.quant_kv_cache || attention_fused_kv8_supported(c.head_dim, c.max_seq)) &&
         qkv_attention_supported(H, c.n_heads, c.n_kv_heads, c.head_dim, c.max_seq, c.dtype) && (QD + 2 * KD) * eb % 8 == 0) {
@@ -876,6 +891,7 @@ static void destroy(Model *m) {
     for (Layer &L : m->layers) {
         if (L.own_qkv_w) hipFree(L.own_qkv_w);
         if (L.own_qkv_s) hipFree(L.own_qkv_s);
+        if (L.qkv_b) hipFree(L.qkv_b);
         if (L.own_gu_w) hipFree(L.own_gu_w);
         if (L.own_gu_s) hipFree(L.own_gu_s);
         if (L.wt_qkv) hipFree(L.wt_qkv);

@@ -572,6 +572,25 @@ extern "C" int mynn_add(void *out, const void *a, const void *b, size_t n, int d
     });
 }
 
+// x[r, n] = T(x[r, n] + bias[n]) in place: the broadcast Add behind a projection with a bias (crates/llm/src/decoder.rs:167-184)
+namespace mynn {
+template <typename T>
+__global__ void add_bias_rows_kernel(T *x, const T *bias, int N, size_t total) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    Elem<T>::st(x, i, Elem<T>::ld(x, i) + Elem<T>::ld(bias, i % N));
+}
+int add_bias_rows(void *x, const void *bias, int rows, int N, int dtype, hipStream_t s) {
+    MYNN_REQUIRE(x && bias && rows > 0 && N > 0, MYNN_ERR_INVALID, "add_bias_rows: bad operand");
+    const size_t total = (size_t)rows * N;
+    return dispatch_dtype(dtype, [&](auto *t) {
+        using T = std::remove_pointer_t<decltype(t)>;
+        MYNN_LAUNCH(add_bias_rows_kernel<T>, dim3(nblocks(total, 256)), dim3(256), 0, s, (T *)x, (const T *)bias, N, total);
+        return launch_status("add_bias_rows_kernel");
+    });
+}
+}  // namespace mynn
+
 extern "C" int mynn_dynamic_quantize_linear(void *y, void *y_scale, void *y_zero_point, const void *x, int axis_dim,
                                             int inner_size, int dtype, int symmetric, mynn_stream s) {
     MYNN_REQUIRE(y && y_scale && x && axis_dim > 0 && inner_size > 0, MYNN_ERR_INVALID,

@@ -26,6 +26,8 @@ size_t skinny_scratch_bytes(int M, int N, int K);
 // `packed`: wq is a tiled copy (skinny_packed_bytes, made by skinny_pack_weight) that a wave reads sequentially
 size_t skinny_packed_bytes(int N, int K);
 int skinny_pack_weight(void *dst, const int8_t *wq, int N, int K, hipStream_t s);
+// x[r, n] = T(x[r, n] + bias[n]) in place, x [rows, N] (elementwise.hip)
+int add_bias_rows(void *x, const void *bias, int rows, int N, int dtype, hipStream_t s);
 // paging: the caches are pools [n_pages, Hkv, 1 << shift, D]; row r of sequence b goes to pool page
 // table[b * pages_per_seq + (r >> shift)] (a device array), row r % (1 << shift) of it.  table == nullptr: contiguous caches.
 struct KvPaging {

@@ -514,9 +514,13 @@ static mynn_device_weights *weights_upload_impl(const mynn_weights *w, const myn
     for (int l = 0; l < c->n_layers && !rc; l++) {
         const std::string p = "model.layers." + std::to_string(l);
         rc = upload_float(*dw, *w, p + ".input_layernorm.weight", dt, H);
+        // (qkv_bias: `{base}.bias` behind each of the three, ModelSpec::from_hf, decoder.rs:557-569)
         if (!rc) rc = upload_linear(*dw, *w, p + ".self_attn.q_proj.weight", dt, QD, H);
+        if (!rc && c->qkv_bias) rc = upload_float(*dw, *w, p + ".self_attn.q_proj.bias", dt, QD);
         if (!rc) rc = upload_linear(*dw, *w, p + ".self_attn.k_proj.weight", dt, KD, H);
+        if (!rc && c->qkv_bias) rc = upload_float(*dw, *w, p + ".self_attn.k_proj.bias", dt, KD);
         if (!rc) rc = upload_linear(*dw, *w, p + ".self_attn.v_proj.weight", dt, KD, H);
+        if (!rc && c->qkv_bias) rc = upload_float(*dw, *w, p + ".self_attn.v_proj.bias", dt, KD);
         if (!rc) rc = upload_linear(*dw, *w, p + ".self_attn.o_proj.weight", dt, H, QD);
         if (!rc) rc = upload_float(*dw, *w, p + ".post_attention_layernorm.weight", dt, H);
         if (!rc) rc = upload_linear(*dw, *w, p + ".mlp.gate_proj.weight", dt, F, H);

@@ -91,6 +91,7 @@ _sig("orc_model_set_lm_head", None, _vp, Linear)
 _sig("orc_model_set_final_norm", None, _vp, _vp)
 _sig("orc_model_set_linear", None, _vp, _i, _i, Linear)
 _sig("orc_model_set_norm", None, _vp, _i, _i, _vp)
+_sig("orc_model_set_bias", None, _vp, _i, _i, _vp)
 _sig("orc_model_reset", None, _vp)
 _sig("orc_model_set_gemm_mode", None, _vp, _i)
 _sig("orc_model_set_options", None, _vp, _i, _i)
@@ -416,7 +417,8 @@ class Model:
     weights: dict with
       "embed", "lm_head", "layers.{i}.{q,k,v,o,gate,up,down}" -> (int8 [N,K], scale [N]) tuples for
       quantised tensors or a single storage array [N,K] for plain ones;
-      "final_norm", "layers.{i}.norm1", "layers.{i}.norm2" -> storage arrays.
+      "final_norm", "layers.{i}.norm1", "layers.{i}.norm2" -> storage arrays;
+      optional "layers.{i}.{q,k,v}.bias" -> storage arrays [N] (decoder.rs:167-184).
     """
 
     def __init__(self, cfg, weights):
@@ -430,6 +432,10 @@ class Model:
         for l in range(cfg["n_layers"]):
             for wi, nm in enumerate(LIN_NAMES):
                 _lib.orc_model_set_linear(self._h, l, wi, self._lin(weights["layers.%d.%s" % (l, nm)]))
+            for bi, nm in enumerate(("q", "k", "v")):  # optional projection bias (qwen2)
+                b = weights.get("layers.%d.%s.bias" % (l, nm))
+                if b is not None:
+                    _lib.orc_model_set_bias(self._h, l, bi, _p(self._hold(b)))
             _lib.orc_model_set_norm(self._h, l, 0, _p(self._hold(weights["layers.%d.norm1" % l])))
             _lib.orc_model_set_norm(self._h, l, 1, _p(self._hold(weights["layers.%d.norm2" % l])))
 

@@ -533,6 +533,7 @@ void orc_streaming_kv_position(int64_t *out, size_t sink, size_t window, size_t 
 /* ------------------------------------------------------------------ A12 / A13 decoder */
 struct orc_layer {
     orc_linear lin[7];
+    const void *bias[3]; /* q, k, v projection bias [N] in dtype, or NULL (decoder.rs:167-184, 542-600: qwen2) */
     const void *norm[2];
     void *k_cache, *v_cache; /* [Hkv, max_seq, D] dtype, or int8 with quant_kv_cache */
     void *k_scale, *v_scale; /* quant_kv_cache: [Hkv, max_seq] dtype */
@@ -582,6 +583,8 @@ void orc_model_set_lm_head(orc_model *m, orc_linear w) { m->lm_head = w; }
 void orc_model_set_final_norm(orc_model *m, const void *w) { m->final_norm = w; }
 void orc_model_set_linear(orc_model *m, int layer, int which, orc_linear w) { m->layers[layer].lin[which] = w; }
 void orc_model_set_norm(orc_model *m, int layer, int which, const void *w) { m->layers[layer].norm[which] = w; }
+/* which: 0 q, 1 k, 2 v */
+void orc_model_set_bias(orc_model *m, int layer, int which, const void *b) { m->layers[layer].bias[which] = b; }
 void orc_model_reset(orc_model *m) { m->past_len = 0; }
 void orc_model_set_gemm_mode(orc_model *m, int mode) { m->gemm_mode = mode; }
 /* must be called before the first forward: the caches change element type */
@@ -642,6 +645,14 @@ static void linear(const orc_model *m, void *out, const void *x, const orc_linea
     }
 }
 
+/* Add(matmul output [S,N], bias [N]) in place: the `{node}_bias` node of decoder.rs:167-184 -- the projection is
+ * stored in dtype first (it is the MatMul node's output), then the broadcast Add rounds once more */
+static void add_bias(void *y, const void *bias, size_t S, size_t N, int dt) {
+    if (!bias) return;
+    for (size_t s = 0; s < S; s++)
+        for (size_t n = 0; n < N; n++) st(y, s * N + n, ld(y, s * N + n, dt) + ld(bias, n, dt), dt);
+}
+
 /* [S, H, D] -> [H, S, D] (reshape + Transpose[0,2,1,3], decoder.rs:253-275) */
 static void to_heads(void *dst, const void *src, size_t S, size_t H, size_t D, size_t eb) {
     for (size_t s = 0; s < S; s++)
@@ -688,6 +699,9 @@ void orc_model_forward(orc_model *m, const int64_t *ids, const int64_t *position
         linear(m, qb, n1, &L->lin[0], S, QD, H);
         linear(m, kb, n1, &L->lin[1], S, KD, H);
         linear(m, vb, n1, &L->lin[2], S, KD, H);
+        add_bias(qb, L->bias[0], S, QD, dt);
+        add_bias(kb, L->bias[1], S, KD, dt);
+        add_bias(vb, L->bias[2], S, KD, dt);
         to_heads(qh, qb, S, Hq, D, eb);
         to_heads(kh, kb, S, Hkv, D, eb);
         to_heads(vh, vb, S, Hkv, D, eb);

@@ -30,6 +30,9 @@
  *   orc_model_* (decoder executor and generate loop)   the reference's exact ids on its tiny random Llama
  *                             (crates/llm/tests/tinyllama_random.rs:20-24) in f32/bf16/f16 and three summation orders;
  *                             mock_decode expectations (crates/llm/tests/mock_decode.rs:30-87)
+ *   orc_model_set_bias (q / k / v projection bias, decoder.rs:167-184)   no fixture in the reference (its only checkpoint is
+ *                             a Llama): an independent float64 textbook decoder with one bias at a time and all three,
+ *                             zero biases change no bit of the golden ids, token-by-token == prefill
  *   ring_phys_index, kv_cache_update_streaming, attention_streaming (numpy, oracle/__init__.py; sink + ring KV ops of the
  *                             reference's CUDA kernels)   brute-force ring simulation, reduction to the plain update /
  *                             attention when the ring has not wrapped, f64 attention over explicitly scattered rows
@@ -181,6 +184,9 @@ void orc_model_set_final_norm(orc_model *m, const void *w);
 void orc_model_set_linear(orc_model *m, int layer, int which, orc_linear w);
 /* which: 0 input_layernorm, 1 post_attention_layernorm */
 void orc_model_set_norm(orc_model *m, int layer, int which, const void *w);
+/* q / k / v projection bias (which 0 / 1 / 2), [N] in the model's dtype; NULL = none (llama, mistral).
+ * crates/llm/src/decoder.rs:167-184 (Add after the MatMul), 542-600 (model_type "qwen2") */
+void orc_model_set_bias(orc_model *m, int layer, int which, const void *b);
 void orc_model_reset(orc_model *m);                 /* past_len = 0 (session.rs:303-305) */
 /* which backend's DequantMatMul kernel choice the linears follow: -1 the CPU backend's (default),
  * 2 the CUDA backend's (rows >= 16: weight rounded to the 16-bit type before the product) */

@@ -64,3 +64,15 @@ def synthetic_int8(cfg, dt, seed=1234, std=0.02, quantize=None):
     c = dict(cfg)
     c["dtype"] = dt
     return c, w
+
+
+def add_qkv_bias(cfg, w, dt, seed=99, std=0.5):
+    """q / k / v projection biases (model_type "qwen2", crates/llm/src/decoder.rs:542-600) for a weight dict: [N] in the
+    model's type, seeded; large enough to move the logits."""
+    rng = np.random.default_rng(seed)
+    QD, KD = cfg["n_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
+    out = dict(w)
+    for l in range(cfg["n_layers"]):
+        for nm, n in (("q", QD), ("k", KD), ("v", KD)):
+            out["layers.%d.%s.bias" % (l, nm)] = orc.to_storage(rng.standard_normal(n).astype(np.float32) * np.float32(std), dt)
+    return out

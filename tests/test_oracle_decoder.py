@@ -108,3 +108,95 @@ def test_quant_kv_cache_and_quantize_activations_options_stay_close_to_the_plain
                     slack = 0.5 * 1.02 + (127 * 2.0 ** -8 if dt == orc.BF16 else 0.0)
                     assert np.all(np.abs(kd - orc.to_f32(kp, dt)[:, :10]) <= slack * step + 1e-6)
                 assert np.abs(kq[:, :10]).max() == 127 and not kq[:, 10:].any()
+
+
+# ------------------------------------------------------------------ q / k / v projection bias (qwen2)
+def decoder_f64(cfg, w, ids):
+    """Independent float64 statement of the decoder over a whole prompt (textbook form: y = x W^T + b, rotate-half
+    RoPE, causal softmax attention with grouped kv heads, SwiGLU), plain float weights; returns logits [S, vocab]."""
+    H, Hq, Hkv, D = cfg["hidden"], cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    S = len(ids)
+    f = lambda a: np.asarray(a, np.float64)
+    rms = lambda x, g: x / np.sqrt((x * x).mean(-1, keepdims=True) + cfg["eps"]) * f(g)
+    inv = cfg["rope_theta"] ** (-np.arange(0, D, 2, dtype=np.float64) / D)
+    ang = np.arange(S, dtype=np.float64)[:, None] * inv[None, :]
+    cos, sin = np.cos(np.concatenate([ang, ang], -1)), np.sin(np.concatenate([ang, ang], -1))
+    rot = lambda t: np.concatenate([-t[..., D // 2:], t[..., :D // 2]], -1)
+    x = f(w["embed"])[ids]
+    for l in range(cfg["n_layers"]):
+        g = lambda nm: f(w["layers.%d.%s" % (l, nm)])
+        b = lambda nm: f(w.get("layers.%d.%s.bias" % (l, nm), 0.0))
+        n = rms(x, w["layers.%d.norm1" % l])
+        q = (n @ g("q").T + b("q")).reshape(S, Hq, D)
+        k = (n @ g("k").T + b("k")).reshape(S, Hkv, D)
+        v = (n @ g("v").T + b("v")).reshape(S, Hkv, D)
+        q = q * cos[:, None] + rot(q) * sin[:, None]
+        k = k * cos[:, None] + rot(k) * sin[:, None]
+        o = np.zeros((S, Hq, D))
+        for h in range(Hq):
+            kh = h // (Hq // Hkv)
+            sc = q[:, h] @ k[:, kh].T / np.sqrt(D)
+            sc = np.where(np.tril(np.ones((S, S), bool)), sc, -np.inf)
+            p = np.exp(sc - sc.max(-1, keepdims=True))
+            o[:, h] = (p / p.sum(-1, keepdims=True)) @ v[:, kh]
+        x = x + o.reshape(S, Hq * D) @ g("o").T
+        n = rms(x, w["layers.%d.norm2" % l])
+        a, u = n @ g("gate").T, n @ g("up").T
+        x = x + (a / (1 + np.exp(-a)) * u) @ g("down").T
+    return rms(x, w["final_norm"]) @ f(w["lm_head"]).T
+
+
+BIAS_CFG = dict(n_layers=2, hidden=64, n_heads=4, n_kv_heads=2, head_dim=16, ffn=96, vocab=50, max_seq=16, eps=1e-5,
+                rope_theta=10000.0)
+
+
+def plain_f32_weights(cfg, seed):
+    rng = np.random.default_rng(seed)
+    H, F, V = cfg["hidden"], cfg["ffn"], cfg["vocab"]
+    QD, KD = cfg["n_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
+    r = lambda *s: (rng.standard_normal(s) * 0.2).astype(np.float32)
+    w = {"embed": r(V, H), "lm_head": r(V, H), "final_norm": (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)}
+    for l in range(cfg["n_layers"]):
+        for nm, (n, k) in {"q": (QD, H), "k": (KD, H), "v": (KD, H), "o": (H, QD), "gate": (F, H), "up": (F, H), "down": (H, F)}.items():
+            w["layers.%d.%s" % (l, nm)] = r(n, k)
+        w["layers.%d.norm1" % l] = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+        w["layers.%d.norm2" % l] = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    return w
+
+
+def test_qkv_bias_against_an_independent_f64_decoder():
+    """The bias path of decoder.rs:167-184 has no fixture in the reference (its only checkpoint is a Llama): the oracle's
+    f32 model with biases must follow a float64 textbook decoder, with one bias at a time and with all three -- a bias
+    added after RoPE, to the wrong projection, or scaled, would miss by the size of the bias's effect, which the test
+    shows to be orders of magnitude above the bound."""
+    cfg = dict(BIAS_CFG, dtype=orc.F32)
+    w = plain_f32_weights(cfg, 3)
+    wb = llm_weights.add_qkv_bias(cfg, w, orc.F32, seed=4)
+    ids = np.array([3, 41, 7, 7, 19, 0, 33], np.int64)
+    base = decoder_f64(cfg, w, ids)
+    assert np.max(np.abs(orc.Model(cfg, w).forward(ids, np.arange(len(ids)), 0, len(ids), True) - base)) <= 1e-4 * np.max(np.abs(base))
+    for which in (("q",), ("k",), ("v",), ("q", "k", "v")):
+        wsel = {k: v for k, v in wb.items() if not k.endswith(".bias") or k.split(".")[-2] in which}
+        want = decoder_f64(cfg, wsel, ids)
+        got = orc.Model(cfg, wsel).forward(ids, np.arange(len(ids)), 0, len(ids), True)
+        assert np.max(np.abs(got - want)) <= 1e-4 * np.max(np.abs(want)), which
+        if which != ("k",):  # (a k bias alone shifts every score of a query by nearly the same amount: its effect is small)
+            assert np.max(np.abs(want - base)) >= 1e-2 * np.max(np.abs(base)), which
+
+
+@pytest.mark.parametrize("dt", [orc.F32, orc.BF16, orc.F16])
+def test_zero_qkv_bias_changes_no_bit_and_decode_equals_prefill(dt):
+    cfg, w, golden = llm_weights.tiny_llama_random(dt)
+    zero = {k: orc.to_storage(np.zeros_like(orc.to_f32(v, dt)), dt) for k, v in llm_weights.add_qkv_bias(cfg, w, dt).items()
+            if k.endswith(".bias")}
+    m = orc.Model(cfg, dict(w, **zero))
+    assert m.generate(golden["prompt_ids"], 8) == golden["expected_new_ids"]
+    # with real biases: feeding a prompt token by token and as one prefill give the same rows (f32: to rounding)
+    wb = llm_weights.add_qkv_bias(cfg, w, dt, std=0.1)
+    a, b = orc.Model(cfg, wb), orc.Model(cfg, wb)
+    ids = np.array(golden["prompt_ids"] + [7, 99], np.int64)
+    full = a.forward(ids, np.arange(len(ids)), 0, len(ids), True)
+    for i, t in enumerate(ids):
+        row = b.forward([t], [i], i, i + 1, False)
+    fl, rl = orc.to_f32(full[-1], dt), orc.to_f32(row[0], dt)
+    assert np.max(np.abs(fl - rl)) <= (1e-5 if dt == orc.F32 else 3e-2) * np.max(np.abs(fl))
