@@ -42,6 +42,24 @@ def test_rejected_arguments_return_status_not_exit():
     assert lib.model_init(None, None) is None  # not configured / null arrays
 
 
+def test_kv_pool_is_host_side_bookkeeping():
+    """The free list of a paged KV cache lives in host memory: it can be made, asked and destroyed without a GPU;
+    bad sizes and the calls that would need the device with a null handle come back as errors."""
+    lib = mynn.lib()
+    for bad in ((0, 64), (4, 48), (4, 16), (-1, 256)):
+        assert lib.mynn_kv_pool_create(*bad) is None and b"power of two" in lib.mynn_last_error()
+    pool = mynn.KvPool(7, 128)
+    assert pool.free_pages == 7
+    assert lib.mynn_kv_pages_create(pool.handle, 0, 256) is None   # batch
+    assert lib.mynn_kv_pages_create(pool.handle, 2, 200) is None   # not a multiple of the page
+    assert lib.mynn_kv_pages_create(None, 2, 256) is None
+    assert lib.mynn_kv_pages_reserve(None, 10) == -1 and lib.mynn_kv_pages_release(None) == -1
+    assert lib.mynn_kv_pages_mapped_rows(None) == 0 and lib.mynn_kv_pages_table(None) is None
+    assert lib.mynn_kv_pool_free_pages(None) == -1
+    pool.close()
+    assert pool.handle is None
+
+
 def test_host_quantiser_known_answers_and_oracle_agreement():
     # crates/llm/tests/quantize.rs:106-159
     w = np.array([[127, -127, 0, 64], [2, -1, 0, 0.5], [0, 0, 0, 0]], np.float32)
