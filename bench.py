@@ -423,11 +423,15 @@ def decode_batch_main(args, mynn):
     pages = pool = None
     if args.kv_pages:
         # paged cache: one pool for the batch, pages of every sequence interleaved (page = slot * B + sequence)
-        assert not args.kv_int8 and cfg["max_seq"] % args.kv_pages == 0
+        assert cfg["max_seq"] % args.kv_pages == 0
         pool = mynn.KvPool(B * cfg["max_seq"] // args.kv_pages, args.kv_pages)
         pshape = (pool.n_pages, cfg["n_kv_heads"], args.kv_pages, cfg["head_dim"])
         for _ in range(cfg["n_layers"]):
-            kv.append((torch.randn(pshape, generator=gen, device="cuda", dtype=tdt), torch.randn(pshape, generator=gen, device="cuda", dtype=tdt)))
+            if args.kv_int8:
+                kv.append(tuple([torch.randint(-127, 128, pshape, generator=gen, device="cuda", dtype=torch.int8) for _ in range(2)] +
+                                [(torch.rand(pshape[:3], generator=gen, device="cuda") * 0.02 + 0.01).to(tdt) for _ in range(2)]))
+            else:
+                kv.append((torch.randn(pshape, generator=gen, device="cuda", dtype=tdt), torch.randn(pshape, generator=gen, device="cuda", dtype=tdt)))
         pages = mynn.KvPages(pool, B, cfg["max_seq"])
         pages.reserve(ctx)
     for _ in range(0 if args.kv_pages else cfg["n_layers"]):
@@ -494,7 +498,7 @@ def decode_batch_main(args, mynn):
         "dtype": "f32 accumulate over int8 weights, %s activations, %s KV" % (args.dtype, "int8" if args.kv_int8 else args.dtype),
         "data": "synthetic",
         "config": {"workload": "configs[4]: Llama-3-8B-shape int8 decoder, batch 32, context 2048 (caches filled with "
-                               "random rows%s), %d decode steps timed" % (", int8 KV cache" if args.kv_int8 else ", paged KV cache" if args.kv_pages else "", K),
+                               "random rows%s), %d decode steps timed" % ((", int8 KV cache" if args.kv_int8 else "") + (", paged KV cache" if args.kv_pages else ""), K),
                    "batch": B, "context": ctx, "launches_per_step": stats["launches_per_step"], "hipgraph": stats["graph"],
                    "kv_page_rows": args.kv_pages or None,
                    "kv_pages_mapped": (pool.n_pages - pool.free_pages) if pool else None,

@@ -375,13 +375,20 @@ class KvPool:
     def free_pages(self):
         return lib().mynn_kv_pool_free_pages(self.handle)
 
-    def buffers(self, n_layers, n_kv_heads, head_dim, dtype, fill=None):
+    def buffers(self, n_layers, n_kv_heads, head_dim, dtype, fill=None, kv_int8=False):
+        """One (K pool, V pool) per layer, [n_pages, Hkv, page_rows, D] in `dtype`; kv_int8: (K codes, V codes, K scales,
+        V scales) with int8 code pools and scale pools [n_pages, Hkv, page_rows] in `dtype`."""
         import torch
 
         shape = (self.n_pages, n_kv_heads, self.page_rows, head_dim)
-        make = (lambda: torch.zeros(shape, dtype=dtype, device="cuda")) if fill is None else \
-            (lambda: torch.full(shape, fill, dtype=dtype, device="cuda"))
-        return [(make(), make()) for _ in range(n_layers)]
+
+        def make(sh, dt):
+            return torch.zeros(sh, dtype=dt, device="cuda") if fill is None else torch.full(sh, fill, dtype=dt, device="cuda")
+
+        if kv_int8:
+            return [(torch.zeros(shape, dtype=torch.int8, device="cuda"), torch.zeros(shape, dtype=torch.int8, device="cuda"),
+                     make(shape[:3], dtype), make(shape[:3], dtype)) for _ in range(n_layers)]
+        return [(make(shape, dtype), make(shape, dtype)) for _ in range(n_layers)]
 
     def close(self):
         if getattr(self, "handle", None) and _lib is not None:

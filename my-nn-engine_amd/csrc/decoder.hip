@@ -424,7 +424,7 @@ static int enqueue_step(Model &m) {
                 if (roped) {
                 } else if (kv8)
                     TRY(rope_quant_kv_append<T>(m.q, (int8_t *)L.k_cache, (int8_t *)L.v_cache, L.k_scale, L.v_scale, m.qkv,
-                                                m.cos_t, m.sin_t, m.d_pos, m.d_past, B, S, Hq, Hkv, D, c.max_seq, s));
+                                                m.cos_t, m.sin_t, m.d_pos, m.d_past, B, S, Hq, Hkv, D, c.max_seq, s, m.paging));
                 else
                     TRY(rope_kv_append<T>(q_in_attn ? nullptr : m.q, L.k_cache, L.v_cache, m.qkv, m.cos_t, m.sin_t, m.d_pos, m.d_past, 0, B, S,
                                           Hq, Hkv, D, c.max_seq, s, m.paging));
@@ -636,7 +636,7 @@ static int build(Model &m, void **init, void **state) {
         }
     }
     if (c.kv_page_rows) {
-        m.pages = (mynn_kv_pages *)state[2 * c.n_layers];
+        m.pages = (mynn_kv_pages *)state[(c.quant_kv_cache ? 4 : 2) * c.n_layers];
         MYNN_REQUIRE(m.pages, MYNN_ERR_INVALID, "model_init: kv_page_rows without a page set after the pools in session_state");
         m.paging = kv_pages_paging(m.pages);
         MYNN_REQUIRE((1 << m.paging.shift) == c.kv_page_rows && m.paging.pages_per_seq * c.kv_page_rows == c.max_seq &&
@@ -999,8 +999,9 @@ static int check_config(const mynn_model_config *cfg) {
         const int P = cfg->kv_page_rows;
         MYNN_REQUIRE(P >= 64 && (P & (P - 1)) == 0 && cfg->max_seq % P == 0, MYNN_ERR_INVALID,
                      "model_configure: kv_page_rows %d (a power of two >= 64 that divides max_seq %d)", P, cfg->max_seq);
-        MYNN_REQUIRE(!cfg->quant_kv_cache && !cfg->streaming_kv, MYNN_ERR_UNSUPPORTED,
-                     "model_configure: a paged KV cache is 16-bit and takes neither quant_kv_cache nor streaming_kv");
+        MYNN_REQUIRE(!cfg->streaming_kv, MYNN_ERR_UNSUPPORTED, "model_configure: a paged KV cache does not take streaming_kv");
+        MYNN_REQUIRE(!cfg->quant_kv_cache || cfg->seq_q == 1, MYNN_ERR_UNSUPPORTED,
+                     "model_configure: a paged int8 KV cache serves decode models only (the prefill kernel reads 16-bit pages)");
         MYNN_REQUIRE(cfg->seq_q == 1 || cfg->max_seq / P <= 64, MYNN_ERR_UNSUPPORTED,
                      "model_configure: a prefill model reads at most 64 pages per sequence (max_seq %d, %d rows per page)", cfg->max_seq, P);
         MYNN_REQUIRE(attn_stream_paged_supported(1, cfg->n_heads, cfg->n_kv_heads, cfg->head_dim, cfg->dtype, P), MYNN_ERR_UNSUPPORTED,

@@ -159,6 +159,6 @@ int rope_kv_append(void *q_out, void *k_cache, void *v_cache, const void *qkv, c
 template <typename T>
 int rope_quant_kv_append(void *q_out, int8_t *k_cache, int8_t *v_cache, void *k_scale, void *v_scale, const void *qkv,
                          const void *cos_t, const void *sin_t, const int64_t *position, const int32_t *d_past, int B,
-                         int S, int Hq, int Hkv, int D, int max_seq, hipStream_t s);
+                         int S, int Hq, int Hkv, int D, int max_seq, hipStream_t s, KvPaging paging = KvPaging());
 
 }  // namespace mynn

@@ -91,7 +91,7 @@ template <typename T>
 __global__ __launch_bounds__(64) void rope_quant_kv_append_kernel(T *q_out, int8_t *k_cache, int8_t *v_cache, T *k_scale,
                                                                  T *v_scale, const T *qkv, const T *cos_t, const T *sin_t,
                                                                  const int64_t *position, const int32_t *d_past, int S,
-                                                                 int Hq, int Hkv, int D, int max_seq) {
+                                                                 int Hq, int Hkv, int D, int max_seq, KvPaging pg) {
     const int s = blockIdx.x, head = blockIdx.y, b = blockIdx.z, lane = threadIdx.x;
     const int half = D / 2;
     const int past = *d_past;
@@ -122,7 +122,7 @@ __global__ __launch_bounds__(64) void rope_quant_kv_append_kernel(T *q_out, int8
     }
     const bool is_k = head < Hq + Hkv;
     const int hk = is_k ? head - Hq : head - Hq - Hkv;
-    const size_t tok = ((size_t)b * Hkv + hk) * max_seq + past + s;
+    const size_t tok = kv_cache_row(pg, b, hk, past + s, Hkv, max_seq);  // (paged: the scale pools share the table)
     const float amax = wave_max(fmaxf(fabsf(lo), fabsf(hi)));
     const float inv = amax == 0.f ? 0.f : 127.0f / amax;
     if (lane == 0) Elem<T>::st(is_k ? k_scale : v_scale, tok, amax * (1.0f / 127.0f));
@@ -140,19 +140,22 @@ __global__ __launch_bounds__(64) void rope_quant_kv_append_kernel(T *q_out, int8
 template <typename T>
 int rope_quant_kv_append(void *q_out, int8_t *k_cache, int8_t *v_cache, void *k_scale, void *v_scale, const void *qkv,
                          const void *cos_t, const void *sin_t, const int64_t *position, const int32_t *d_past, int B,
-                         int S, int Hq, int Hkv, int D, int max_seq, hipStream_t s) {
+                         int S, int Hq, int Hkv, int D, int max_seq, hipStream_t s, KvPaging paging) {
     MYNN_REQUIRE(D % 2 == 0 && D <= 128, MYNN_ERR_UNSUPPORTED, "int8 KV append: head_dim %d", D);
+    MYNN_REQUIRE(!paging.table || (paging.shift > 0 && paging.shift < 31 && max_seq == paging.pages_per_seq << paging.shift),
+                 MYNN_ERR_INVALID, "int8 KV append: %d rows per sequence are not %d pages of %d rows", max_seq,
+                 paging.pages_per_seq, 1 << paging.shift);
     MYNN_REQUIRE(S <= 65535 * 32 && Hq + 2 * Hkv <= 65535 && B <= 65535, MYNN_ERR_UNSUPPORTED, "int8 KV append: grid");
     MYNN_REQUIRE(d_past, MYNN_ERR_INVALID, "int8 KV append: null past_len");
     MYNN_LAUNCH(rope_quant_kv_append_kernel<T>, dim3(S, Hq + 2 * Hkv, B), dim3(64), 0, s, (T *)q_out, k_cache, v_cache,
                 (T *)k_scale, (T *)v_scale, (const T *)qkv, (const T *)cos_t, (const T *)sin_t, position, d_past, S, Hq,
-                Hkv, D, max_seq);
+                Hkv, D, max_seq, paging);
     return launch_status("rope_quant_kv_append_kernel");
 }
 template int rope_quant_kv_append<bf16_t>(void *, int8_t *, int8_t *, void *, void *, const void *, const void *, const void *,
-                                          const int64_t *, const int32_t *, int, int, int, int, int, int, hipStream_t);
+                                          const int64_t *, const int32_t *, int, int, int, int, int, int, hipStream_t, KvPaging);
 template int rope_quant_kv_append<f16_t>(void *, int8_t *, int8_t *, void *, void *, const void *, const void *, const void *,
-                                         const int64_t *, const int32_t *, int, int, int, int, int, int, hipStream_t);
+                                         const int64_t *, const int32_t *, int, int, int, int, int, int, hipStream_t, KvPaging);
 
 template <typename T>
 int rope_kv_append(void *q_out, void *k_cache, void *v_cache, const void *qkv, const void *cos_t, const void *sin_t,

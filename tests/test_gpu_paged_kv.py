@@ -367,6 +367,37 @@ def test_paged_executor_batch1_decode_vs_oracle(g, dt):
     dec.close(), pages.close(), other.close(), pool.close()
 
 
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+def test_paged_int8_kv_decode_executor_equals_contiguous(g, dt):
+    """quant_kv_cache over pools (code pools + scale pools, decode models): 16 sequences fed token by token write and read
+    the same codes and scales as the executor with contiguous int8 caches, and return the same logits, bit for bit."""
+    cfg, w = llm_weights.synthetic_int8(dict(PAGED_D64, max_seq=1024), dt, seed=29)
+    dw = dev_weights(g, w, dt)
+    P, B = 64, 16
+    pool = g.mynn.KvPool(B * 3, P)
+    kvbufs = pool.buffers(cfg["n_layers"], cfg["n_kv_heads"], cfg["head_dim"], g.torch_dtype(dt), fill=float("nan"), kv_int8=True)
+    pages = g.mynn.KvPages(pool, B, cfg["max_seq"])
+    dec = g.mynn.Decoder(cfg, dw, batch=B, kv=kvbufs, kv_pages=pages, quant_kv_cache=True)
+    ref = g.mynn.Decoder(cfg, dw, batch=B, quant_kv_cache=True)
+    rng = np.random.default_rng(12)
+    n = 70
+    for i in range(n):
+        toks = rng.integers(0, cfg["vocab"], B)
+        a, la = dec.step(toks, [i], i, i + 1, want_logits=True)
+        b, lb = ref.step(toks, [i], i, i + 1, want_logits=True)
+        assert np.array_equal(la, lb) and a == b, i
+    assert pages.mapped_rows == 128 and pool.free_pages == B
+    table = pages.table()
+    for l in range(cfg["n_layers"]):
+        for j in range(4):
+            got = gather_cache(g, kvbufs[l][j], table, P)
+            want = g.to_host(ref.kv[l][j])
+            assert np.array_equal(got[:, :, :n], want[:, :, :n]), (l, j)
+    with pytest.raises(g.mynn.MynnError):  # a prefill model over int8 pages: no kernel
+        g.mynn.Decoder(cfg, dw, batch=B, seq_q=16, kv=kvbufs, kv_pages=pages, quant_kv_cache=True)
+    dec.close(), ref.close(), pages.close(), pool.close()
+
+
 def test_paged_executor_rejects_what_it_has_no_kernel_for(g):
     dt = orc.F16
     cfg, w = llm_weights.synthetic_int8(PAGED_D64, dt, seed=1)
@@ -374,7 +405,7 @@ def test_paged_executor_rejects_what_it_has_no_kernel_for(g):
     pool = g.mynn.KvPool(8, 64)
     kvbufs = pool.buffers(cfg["n_layers"], cfg["n_kv_heads"], cfg["head_dim"], g.torch_dtype(dt))
     pages = g.mynn.KvPages(pool, 1, cfg["max_seq"])
-    for kw in (dict(quant_kv_cache=True), dict(streaming_kv=True), dict(batch=2)):
+    for kw in (dict(streaming_kv=True), dict(batch=2)):
         with pytest.raises(g.mynn.MynnError):
             g.mynn.Decoder(cfg, dw, kv=kvbufs, kv_pages=pages, **kw)
     pool32 = g.mynn.KvPool(8, 32)  # pages smaller than a prefill tile
