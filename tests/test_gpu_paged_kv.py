@@ -398,6 +398,34 @@ def test_paged_int8_kv_decode_executor_equals_contiguous(g, dt):
     dec.close(), ref.close(), pages.close(), pool.close()
 
 
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+@pytest.mark.parametrize("opt", ["w8a8", "qkv_bias", "unfused", "kv_int8_w8a8"])
+def test_paged_batch1_decode_with_other_options_vs_oracle(g, dt, opt):
+    """The paged cache under the executor's other options (int8 activations, projection biases, one op per launch,
+    int8 cache + int8 activations): batch-1 decode across a page border against the oracle with the same options."""
+    cfg, w = llm_weights.synthetic_int8(PAGED_D64, dt, seed=37)
+    if opt == "qkv_bias":
+        w = llm_weights.add_qkv_bias(cfg, w, dt, seed=38, std=0.05)
+    w8a8, kv8 = "w8a8" in opt, "kv_int8" in opt
+    ref = orc.Model(cfg, w)
+    ref.set_options(quant_kv_cache=kv8, quantize_activations=w8a8)
+    P = 64
+    pool = g.mynn.KvPool(4, P)
+    kvbufs = pool.buffers(cfg["n_layers"], cfg["n_kv_heads"], cfg["head_dim"], g.torch_dtype(dt), fill=float("nan"), kv_int8=kv8)
+    pages = g.mynn.KvPages(pool, 1, cfg["max_seq"])
+    dec = g.mynn.Decoder(cfg, dev_weights(g, w, dt), kv=kvbufs, kv_pages=pages, quantize_activations=w8a8, quant_kv_cache=kv8,
+                         unfused_decode=opt == "unfused")
+    tol = 3e-2 if w8a8 else 1e-2
+    rng = np.random.default_rng(3)
+    for i, t in enumerate(rng.integers(0, cfg["vocab"], 68)):
+        want = ref.forward([t], [i], i, i + 1, False)
+        nxt, got = dec.step([t], [i], i, i + 1, want_logits=True)
+        assert max_err_rel_to_max(g.f32(got, dt), g.f32(want, dt)) <= tol, i
+        assert nxt[0] == orc.argmax_last(got[0], dt)
+    assert pages.mapped_rows == 128
+    dec.close(), pages.close(), pool.close()
+
+
 def test_paged_executor_rejects_what_it_has_no_kernel_for(g):
     dt = orc.F16
     cfg, w = llm_weights.synthetic_int8(PAGED_D64, dt, seed=1)
