@@ -121,6 +121,7 @@ SIGNATURES = {
     "mynn_model_step": (_i, [_vp, _vp, _vp, _i64, _i64, _vp, _vp]),
     "mynn_model_step_streaming": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp]),
     "mynn_model_handover_failures": (_i, [_vp]),
+    "mynn_model_release_kv_pages": (_i, [_vp]),
     "mynn_model_last_status": (_i, [_vp]),
     "mynn_model_argmax_row": (_i, [_vp, _i, C.POINTER(C.c_int32)]),
     "mynn_model_logits_device": (_vp, [_vp]),

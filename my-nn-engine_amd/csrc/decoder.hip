@@ -1131,6 +1131,11 @@ extern "C" int mynn_model_step_streaming(void *state, const int64_t *input_ids, 
     return step_once(m, input_ids, position_id, past_len, active_seq_kv, next_token, logits_host, &failed);
 }
 
+extern "C" int mynn_model_release_kv_pages(void *state) {
+    MYNN_REQUIRE(state, MYNN_ERR_INVALID, "model_release_kv_pages: null state");
+    Model &m = *(Model *)state;
+    return m.pages ? mynn_kv_pages_release(m.pages) : 0;
+}
 extern "C" int mynn_model_handover_failures(void *state) { return state ? ((Model *)state)->handover_failures : 0; }
 extern "C" int mynn_model_last_status(void *state) { return state ? ((Model *)state)->last_status : MYNN_ERR_INVALID; }
 

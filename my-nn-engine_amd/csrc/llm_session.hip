@@ -131,7 +131,13 @@ extern "C" mynn_llm *mynn_llm_create_with_step(mynn_step_fn step, void *user, in
     return l;
 }
 extern "C" void mynn_llm_destroy(mynn_llm *l) { delete l; }
-extern "C" void mynn_llm_reset(mynn_llm *l) { if (l) l->past_len = 0; }
+// reset (session.rs:303-305): past_len = 0; a paged cache also gives its pages back to the pool (the prefill model shares
+// the decode model's page set)
+extern "C" void mynn_llm_reset(mynn_llm *l) {
+    if (!l) return;
+    l->past_len = 0;
+    if (l->decode) (void)mynn_model_release_kv_pages(l->decode);
+}
 extern "C" int64_t mynn_llm_past_len(const mynn_llm *l) { return l ? l->past_len : -1; }
 extern "C" void mynn_llm_set_past_len(mynn_llm *l, int64_t p) { if (l) l->past_len = p < 0 ? 0 : p; }
 

@@ -426,6 +426,40 @@ def test_paged_batch1_decode_with_other_options_vs_oracle(g, dt, opt):
     dec.close(), pages.close(), pool.close()
 
 
+def test_generate_loop_over_a_paged_cache_and_reset_gives_the_pages_back(g):
+    """LlmSession (chunked zero-padded prefill, then greedy decode) over models with a paged cache produces the ids of the
+    same session over contiguous caches; reset returns the pages to the pool and a second run reproduces the first."""
+    dt = orc.F16
+    cfg, w = llm_weights.synthetic_int8(PAGED_D64, dt, seed=53)
+    dw = dev_weights(g, w, dt)
+    pool = g.mynn.KvPool(4, 64)
+    kvbufs = pool.buffers(cfg["n_layers"], cfg["n_kv_heads"], cfg["head_dim"], g.torch_dtype(dt), fill=float("nan"))
+    pages, dec, pre = _sessions(g, cfg, dw, dt, pool, kvbufs, 1, prefill_rows=16)
+    ref_dec = g.mynn.Decoder(cfg, dw, unfused_decode=True)
+    ref_pre = g.mynn.Decoder(cfg, dw, seq_q=16, kv=ref_dec.kv)
+    prompt = np.random.default_rng(9).integers(0, cfg["vocab"], 37).tolist()
+    a = g.mynn.LlmSession(dec, prefill=pre)
+    b = g.mynn.LlmSession(ref_dec, prefill=ref_pre)
+    ids = a.generate_ids(prompt, 40)
+    want = b.generate_ids(prompt, 40)
+    # the paged decode attention runs in another kernel than the contiguous executor's: equal ids up to ties the oracle confirms
+    if ids != want:
+        first = next(i for i in range(40) if ids[i] != want[i])
+        ref = orc.Model(cfg, w)
+        for i, t in enumerate(prompt + want[:first]):
+            logits = ref.forward([t], [i], i, i + 1, False)[0]
+        lf = orc.to_f32(logits, dt)
+        assert abs(float(lf[ids[first]] - lf[want[first]])) <= 8 * 2.0 ** -11 * float(np.max(np.abs(lf))), first
+    assert a.past_len == len(prompt) + 40 - 1 and pages.mapped_rows == 128 and pool.free_pages == 2
+    a.reset()
+    assert a.past_len == 0 and pages.mapped_rows == 0 and pool.free_pages == 4
+    assert a.generate_ids(prompt, 40) == ids
+    a.close(), b.close()
+    for d in (dec, pre, ref_dec, ref_pre):
+        d.close()
+    pages.close(), pool.close()
+
+
 def test_paged_executor_rejects_what_it_has_no_kernel_for(g):
     dt = orc.F16
     cfg, w = llm_weights.synthetic_int8(PAGED_D64, dt, seed=1)
