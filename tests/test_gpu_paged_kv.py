@@ -152,6 +152,45 @@ def test_paged_prefill_attention_vs_oracle_and_contiguous(g, dt, B, Hq, Hkv, D, 
         assert np.array_equal(got, plain)
 
 
+def test_paged_attention_rejects_bad_arguments_with_a_status(g):
+    """Shapes and page geometries the paged kernels have no form for come back as errors before anything is launched."""
+    import torch
+
+    q = torch.zeros((1, 8, 1, 64), dtype=torch.float16, device="cuda")
+    pool = torch.zeros((4, 2, 64, 64), dtype=torch.float16, device="cuda")
+    tab = torch.zeros((1, 2), dtype=torch.int32, device="cuda")
+    ok = g.mynn.attention_paged(q, pool, pool, tab, 64, 0.125, False, 100)
+    assert ok.shape == q.shape
+    lib = g.mynn.lib()
+
+    def call(**kw):
+        a = dict(out=ok, q=q, k=pool, v=pool, ks=None, vs=None, tab=tab, pps=2, P=64, scale=0.125, causal=0, B=1, Sq=1, active=100,
+                 d_active=None, qoff=0, Hq=8, Hkv=2, D=64, dt=g.mynn.F16, kv8=0)
+        a.update(kw)
+        p = lambda t: None if t is None else t.data_ptr()
+        return lib.mynn_attention_paged(p(a["out"]), p(a["q"]), p(a["k"]), p(a["v"]), p(a["ks"]), p(a["vs"]), p(a["tab"]), a["pps"], a["P"],
+                                        a["scale"], a["causal"], a["B"], a["Sq"], a["active"], p(a["d_active"]), a["qoff"], a["Hq"], a["Hkv"],
+                                        a["D"], a["dt"], a["kv8"], None, 0, None)
+
+    assert call() == 0
+    assert call(tab=None) == -1
+    assert call(P=48) == -1 and call(P=16) == -1          # not a power of two / below a tile
+    assert call(kv8=1) == -1                              # int8 pools without scale pools
+    assert call(active=0) == -1
+    assert call(dt=g.mynn.F32) == -2
+    assert call(Hq=7) == -1                               # not a multiple of the kv heads
+    assert call(Hq=6) == -2                               # 3 query heads per kv head: no form
+    assert call(D=32) == -2
+    q16 = torch.zeros((1, 8, 16, 64), dtype=torch.float16, device="cuda")
+    out16 = torch.zeros_like(q16)
+    assert call(out=out16, q=q16, Sq=16, causal=1, active=16) == 0
+    assert call(out=out16, q=q16, Sq=16, causal=1, active=16, P=32, pps=4) == -2   # a prefill tile is 64 keys
+    assert call(out=out16, q=q16, Sq=16, causal=1, active=16, kv8=1, ks=pool, vs=pool) == -2
+    big_tab = torch.zeros((1, 65), dtype=torch.int32, device="cuda")
+    assert call(out=out16, q=q16, Sq=16, causal=1, active=16, tab=big_tab, pps=65) == -2
+    torch.cuda.synchronize()
+
+
 def test_kvcache_update_paged_scatters_rows_through_the_table(g):
     import torch
 
