@@ -35,6 +35,23 @@ def test_library_exports_every_declared_symbol():
     assert lib.mynn_version() >= 1
 
 
+def test_model_config_mirror_matches_the_header_field_for_field():
+    text = open(os.path.join(ROOT, "include", "mynn_hip.h")).read()
+    body = text[:text.index("} mynn_model_config;")]
+    body = body[body.rindex("typedef struct {"):]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    fields = re.findall(r"\b(int|float)\s+([a-z_0-9, ]+);", body)
+    names, kinds = [], []
+    for kind, group in fields:
+        for n in group.split(","):
+            names.append(n.strip())
+            kinds.append(kind)
+    mirror = mynn.ModelConfig._fields_
+    assert names == [n for n, _ in mirror]
+    assert all((t is C.c_float) == (k == "float") for (_, t), k in zip(mirror, kinds))
+    assert C.sizeof(mynn.ModelConfig) == 4 * len(names)
+
+
 def test_rejected_arguments_return_status_not_exit():
     lib = mynn.lib()
     rc = lib.mynn_dequant_gemv(None, None, None, None, 8, 16, 2, 2, None)
