@@ -345,9 +345,11 @@ bool attn_stream_eligible(int B, int Sq, int Hq, int Hkv, int D, int dtype, int 
            (G == 1 || G == 2 || G == 4 || G == 8) && cache_len >= kStreamTile && (long)B * Hkv * kv_len >= 32768;
 }
 
-// key rows per workgroup and number of key ranges: as many workgroups as the device holds at once
-// (three per CU at the kernel's register count) and no more, so that there is no short second round;
-// ranges a multiple of the 128 keys a workgroup takes per step
+// key rows per workgroup and number of key ranges: ONE workgroup per CU (its four waves keep eight tiles in flight,
+// which is enough to stream; measured over batch x kv-head counts of 8 .. 384 and contexts of 512 .. 8192, two to
+// four workgroups per CU -- what the register count allows -- were 0-25 % slower: shorter sequential runs, more partial
+// results to write and to merge, and with at least one (sequence, kv head) per CU the merge launch disappears
+// altogether); ranges a multiple of the 128 keys a workgroup takes per step
 void attn_stream_plan(int B, int Hkv, int kv_len, int *slice, int *nsplit) {
     const int step = kStreamWaves * kStreamTile;
     static int slots = 0;
@@ -357,7 +359,7 @@ void attn_stream_plan(int B, int Hkv, int kv_len, int *slice, int *nsplit) {
             (void)hipGetLastError();
             cus = 256;
         }
-        slots = 3 * cus;
+        slots = cus;
     }
     int n = slots / (B * Hkv);
     const int nmax = (kv_len + 127) / 128;
