@@ -37,6 +37,10 @@ template <> struct Mfma16<bf16_t> {
 };
 
 constexpr int kStreamWaves = 4, kStreamThreads = kStreamWaves * 64, kStreamTile = 32;
+// (sequences x kv heads x keys) from which this kernel is taken instead of the latency kernel of attention_decode.hip:
+// measured cross-over (head_dim 64 and 128, 1 .. 32 sequences): below it that kernel's single launch of 9-11 us wins or
+// ties, above it this one (two launches, 11 us together, one of 9 us once every CU has a pair) is 25-50 % faster
+constexpr long kStreamMinKeys = 8192;
 
 // KVI8: int8 caches with one scale per token row (QuantizingKVCacheUpdate): K and V are widened exactly to
 // the 16-bit type in registers, the key's k scale multiplies its score and its v scale its p.
@@ -342,7 +346,7 @@ int attention_merge_launch(const AttnParams &p, int D, int dtype, hipStream_t s)
 bool attn_stream_eligible(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, int cache_len) {
     const int G = Hq / Hkv;
     return Sq == 1 && dtype != MYNN_F32 && (!kv_int8 || cache_len % kStreamTile == 0) && (D == 64 || D == 128) &&
-           (G == 1 || G == 2 || G == 4 || G == 8) && cache_len >= kStreamTile && (long)B * Hkv * kv_len >= 32768;
+           (G == 1 || G == 2 || G == 4 || G == 8) && cache_len >= kStreamTile && (long)B * Hkv * kv_len >= kStreamMinKeys;
 }
 
 // key rows per workgroup and number of key ranges: ONE workgroup per CU (its four waves keep eight tiles in flight,

@@ -91,7 +91,7 @@ def test_streaming_decode_attention_vs_oracle(g, dt, B, Hq, Hkv, D, L, active):
     device, and rows beyond it poisoned."""
     import torch
 
-    assert B * Hkv * min(active, L) >= 32768 or B * Hkv * L >= 32768
+    assert B * Hkv * min(active, L) >= 8192 or B * Hkv * L >= 8192
     rng = np.random.default_rng(B * 31 + D + active)
     q = orc.to_storage(rng.standard_normal((B, Hq, 1, D)), dt)
     k = orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt)
@@ -106,7 +106,7 @@ def test_streaming_decode_attention_vs_oracle(g, dt, B, Hq, Hkv, D, L, active):
         got = g.to_host(g.mynn.attention(dq, dk, dv, D ** -0.5, False, active=L, d_active=d_active))
         assert max_abs_rel(g.f32(got, dt), g.f32(want, dt)) <= 1e-2, rep
         assert max_abs_rel(g.f32(got, dt), exact) <= 1e-2, rep
-    if B * Hkv * active >= 32768:
+    if B * Hkv * active >= 8192:
         got = g.to_host(g.mynn.attention(dq, dk, dv, D ** -0.5, False, active))
         assert max_abs_rel(g.f32(got, dt), exact) <= 1e-2
 
