@@ -380,10 +380,11 @@ static int enqueue_step(Model &m) {
             }
             nrm_ready = false;
             if (m.skinny) {
-                // (16-bit KV cache) RoPE and both cache appends ride on the launch that sums the projection's K ranges
-                const SkinnyRope rp{m.q, L.k_cache, L.v_cache, m.cos_t, m.sin_t, m.d_pos, m.d_past, S, Hq, Hkv, D, c.max_seq, m.paging};
+                // RoPE and both cache appends (an int8 cache: with its quantiser) ride on the launch that sums the projection's K ranges
+                const SkinnyRope rp{m.q, L.k_cache, L.v_cache, m.cos_t, m.sin_t, m.d_pos, m.d_past, S, Hq, Hkv, D, c.max_seq, m.paging,
+                                    kv8 ? L.k_scale : nullptr, kv8 ? L.v_scale : nullptr};
                 TRY(skinny_rows(m, m.qkv, m.nrm, L.qkv, L.pk_qkv, nullptr, rows, GEMM_PLAIN, "linear_qkv", nullptr, nullptr,
-                                kv8 || streaming || L.qkv_b ? nullptr : &rp, &roped));
+                                (kv8 && D != 64 && D != 128) || streaming || L.qkv_b || c.unfused_decode ? nullptr : &rp, &roped));
             }
             else if (w8a8) TRY(linear_w8a8(m, m.qkv, m.nrm, L.qkv, rows, true, "qlinear_qkv"));
             else if (m.resident16) TRY(gemm_rows(m, m.qkv, m.nrm, L.wt_qkv, nullptr, rows, L.qkv.N, H, GEMM_PLAIN, "linear_qkv"));

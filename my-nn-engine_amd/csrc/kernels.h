@@ -49,6 +49,7 @@ struct SkinnyRope {
     const int32_t *d_past;
     int S, Hq, Hkv, D, max_seq;
     KvPaging paging;
+    void *k_scale = nullptr, *v_scale = nullptr;  // int8 caches: the per-row scale buffers (head_dim 64 or 128)
 };
 int dequant_gemm_skinny(void *out, const void *act, const int8_t *wq, bool packed, const void *scale, const void *res, int M,
                         int N, int K, int dtype, int epi, float *scratch, hipStream_t s, const void *norm_w = nullptr,

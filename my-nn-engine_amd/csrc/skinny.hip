@@ -276,14 +276,17 @@ __global__ __launch_bounds__(kReduceNormThreads) void skinny_reduce_norm_kernel(
 // The plain form of the reduction for a q|k|v projection, followed by what rope_kv_append_vec_kernel does with
 // the stored projection: one workgroup per token row, a thread per (head, 4 rotation pairs) or 4 values of v;
 // qkv values are rounded to the storage type before the rotation, exactly as if they had been stored.
-template <typename T>
+// KV8: the caches are int8 with one scale per token row (rope_quant_kv_append_kernel's arithmetic: k after RoPE rounded
+// to T, v as stored; s = amax / 127 stored as T, q = trunc(x * 127 / amax +- 0.5) clamped to [-128, 127]); every head
+// then takes D/8 threads (4 low + 4 high elements each), an aligned lane group, and the row maximum is a DPP reduction.
+template <typename T, bool KV8>
 __global__ __launch_bounds__(kReduceNormThreads) void skinny_reduce_rope_kernel(const float *part, const T *scale, int M, int N, int ksplit,
-                                                                              T *q_out, T *k_cache, T *v_cache, const T *cos_t,
-                                                                              const T *sin_t, const int64_t *position,
-                                                                              const int32_t *d_past, int S, int Hq, int Hkv, int D,
-                                                                              int max_seq, KvPaging pg) {
+                                                                              T *q_out, void *k_cache_v, void *v_cache_v, T *k_scale,
+                                                                              T *v_scale, const T *cos_t, const T *sin_t,
+                                                                              const int64_t *position, const int32_t *d_past, int S, int Hq,
+                                                                              int Hkv, int D, int max_seq, KvPaging pg) {
     const int m = blockIdx.x, b = m / S, sq = m % S;
-    const int half = D / 2, upr = half / 4, upv = D / 4;  // units per rotated head / per v head
+    const int half = D / 2, upr = half / 4, upv = KV8 ? upr : D / 4;  // units per rotated head / per v head
     const int rot_units = (Hq + Hkv) * upr, units = rot_units + Hkv * upv;
     const int past = *d_past;
     const size_t tab = (size_t)position[sq] * D;
@@ -313,13 +316,39 @@ __global__ __launch_bounds__(kReduceNormThreads) void skinny_reduce_rope_kernel(
 #pragma unroll
         for (int i = 0; i < 4; i++) f[i] = w[i];
     };
+    // KV8: the lane group's 8 x (D/8) values -> codes and the row's scale
+    auto quantise_store = [&](const float *lo, const float *hi, int8_t *cache, T *srow, size_t tok, int j) {
+        float amax = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) amax = fmaxf(amax, fmaxf(fabsf(lo[i]), fabsf(hi[i])));
+        amax = D == 128 ? group_max<16>(amax) : group_max<8>(amax);
+        const float inv = amax == 0.f ? 0.f : 127.0f / amax;
+        if (j == 0) Elem<T>::st(srow, tok, amax * (1.0f / 127.0f));
+        auto code = [&](float x) -> uint32_t {
+            const float a = x * inv;
+            int q = (int)(a + (a >= 0.f ? 0.5f : -0.5f));
+            q = q < -128 ? -128 : (q > 127 ? 127 : q);
+            return (uint32_t)(q & 0xFF);
+        };
+        int8_t *dst = cache + tok * D;
+        *(uint32_t *)(dst + j) = code(lo[0]) | (code(lo[1]) << 8) | (code(lo[2]) << 16) | (code(lo[3]) << 24);
+        *(uint32_t *)(dst + j + half) = code(hi[0]) | (code(hi[1]) << 8) | (code(hi[2]) << 16) | (code(hi[3]) << 24);
+    };
     for (int u = threadIdx.x; u < units; u += kReduceNormThreads) {
         if (u >= rot_units) {
-            const int hv = (u - rot_units) / upv, j = ((u - rot_units) % upv) * 4;
-            float t[4];
-            total4((Hq + Hkv + hv) * D + j, t);
-            T *dst = v_cache + kv_cache_row(pg, b, hv, past + sq, Hkv, max_seq) * D + j;
-            *(uint2 *)dst = uint2{pack2<T>(t[0], t[1]), pack2<T>(t[2], t[3])};
+            if constexpr (KV8) {
+                const int hv = (u - rot_units) / upr, j = ((u - rot_units) % upr) * 4;
+                float lo[4], hi[4];
+                total4((Hq + Hkv + hv) * D + j, lo);
+                total4((Hq + Hkv + hv) * D + j + half, hi);
+                quantise_store(lo, hi, (int8_t *)v_cache_v, v_scale, kv_cache_row(pg, b, hv, past + sq, Hkv, max_seq), j);
+            } else {
+                const int hv = (u - rot_units) / upv, j = ((u - rot_units) % upv) * 4;
+                float t[4];
+                total4((Hq + Hkv + hv) * D + j, t);
+                T *dst = (T *)v_cache_v + kv_cache_row(pg, b, hv, past + sq, Hkv, max_seq) * D + j;
+                *(uint2 *)dst = uint2{pack2<T>(t[0], t[1]), pack2<T>(t[2], t[3])};
+            }
             continue;
         }
         const int head = u / upr, j = (u % upr) * 4;
@@ -330,14 +359,25 @@ __global__ __launch_bounds__(kReduceNormThreads) void skinny_reduce_rope_kernel(
         ld4(cos_t + tab + j + half, ch);
         ld4(sin_t + tab + j, sl);
         ld4(sin_t + tab + j + half, sh);
-        T *dst = head < Hq ? q_out + (size_t)m * Hq * D + (size_t)head * D
-                           : k_cache + kv_cache_row(pg, b, head - Hq, past + sq, Hkv, max_seq) * D;
         float ol[4], oh[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             ol[i] = xl[i] * cl[i] - xh[i] * sl[i];
             oh[i] = xh[i] * ch[i] + xl[i] * sh[i];
         }
+        if constexpr (KV8) {
+            if (head >= Hq) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    ol[i] = Elem<T>::rnd(ol[i]);
+                    oh[i] = Elem<T>::rnd(oh[i]);
+                }
+                quantise_store(ol, oh, (int8_t *)k_cache_v, k_scale, kv_cache_row(pg, b, head - Hq, past + sq, Hkv, max_seq), j);
+                continue;
+            }
+        }
+        T *dst = head < Hq ? q_out + (size_t)m * Hq * D + (size_t)head * D
+                           : (T *)k_cache_v + kv_cache_row(pg, b, head - Hq, past + sq, Hkv, max_seq) * D;
         *(uint2 *)(dst + j) = uint2{pack2<T>(ol[0], ol[1]), pack2<T>(ol[2], ol[3])};
         *(uint2 *)(dst + j + half) = uint2{pack2<T>(oh[0], oh[1]), pack2<T>(oh[2], oh[3])};
     }
@@ -405,10 +445,17 @@ int dequant_gemm_skinny(void *out, const void *act, const int8_t *wq, bool packe
         if (epi == GEMM_PLAIN && rope && roped && rope->D % 8 == 0 && N == (rope->Hq + 2 * rope->Hkv) * rope->D &&
             ks_used <= kReduceNormMaxSplit && ((uintptr_t)scale & 7) == 0 && ((uintptr_t)rope->q_out & 7) == 0 &&
             ((uintptr_t)rope->k_cache & 7) == 0 && ((uintptr_t)rope->v_cache & 7) == 0 && ((uintptr_t)rope->cos_t & 7) == 0 &&
-            ((uintptr_t)rope->sin_t & 7) == 0) {
-            MYNN_LAUNCH(skinny_reduce_rope_kernel<T>, dim3(M), dim3(kReduceNormThreads), 0, s, scratch, (const T *)scale, M, N, ks_used,
-                        (T *)rope->q_out, (T *)rope->k_cache, (T *)rope->v_cache, (const T *)rope->cos_t, (const T *)rope->sin_t,
-                        rope->position, rope->d_past, rope->S, rope->Hq, rope->Hkv, rope->D, rope->max_seq, rope->paging);
+            ((uintptr_t)rope->sin_t & 7) == 0 && (!rope->k_scale || ((rope->D == 64 || rope->D == 128) && rope->v_scale))) {
+            if (rope->k_scale)
+                MYNN_LAUNCH((skinny_reduce_rope_kernel<T, true>), dim3(M), dim3(kReduceNormThreads), 0, s, scratch, (const T *)scale, M, N,
+                            ks_used, (T *)rope->q_out, rope->k_cache, rope->v_cache, (T *)rope->k_scale, (T *)rope->v_scale,
+                            (const T *)rope->cos_t, (const T *)rope->sin_t, rope->position, rope->d_past, rope->S, rope->Hq, rope->Hkv,
+                            rope->D, rope->max_seq, rope->paging);
+            else
+                MYNN_LAUNCH((skinny_reduce_rope_kernel<T, false>), dim3(M), dim3(kReduceNormThreads), 0, s, scratch, (const T *)scale, M, N,
+                            ks_used, (T *)rope->q_out, rope->k_cache, rope->v_cache, (T *)nullptr, (T *)nullptr, (const T *)rope->cos_t,
+                            (const T *)rope->sin_t, rope->position, rope->d_past, rope->S, rope->Hq, rope->Hkv, rope->D, rope->max_seq,
+                            rope->paging);
             *roped = true;
             return launch_status("skinny_reduce_rope_kernel");
         }

@@ -472,3 +472,36 @@ def test_full_size_tinyllama_shape_greedy_tokens_match_oracle(g):
     assert all(abs(gap) <= 8 for _, gap in near), near
     assert sum(a == b for a, b in zip(gpu_ids, ref_ids)) >= 22
     dec.close()
+
+
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("kv8", [False, True], ids=["kv16", "kv_int8"])
+def test_batched_decode_rope_and_append_in_the_reduce_launch_vs_separate_launches(g, dt, D, kv8):
+    """16 sequences: the launch that sums the q|k|v projection's K ranges also rotates q and k and appends k and v (an
+    int8 cache: quantises them) -- logits, cache rows and scales are those of the executor that keeps these as launches
+    of their own (unfused_decode), bit for bit, and the logits follow the per-sequence oracles."""
+    B = 16
+    # (hidden 1536: the projection's K range is split, so there is a launch that sums the ranges)
+    shape = dict(FEWROWS, n_layers=2, hidden=1536, n_heads=1536 // D, n_kv_heads=768 // D, head_dim=D)
+    cfg, w = llm_weights.synthetic_int8(shape, dt, seed=77)
+    dw = dev_weights(g, w, dt)
+    a = g.mynn.Decoder(cfg, dw, batch=B, quant_kv_cache=kv8)
+    b = g.mynn.Decoder(cfg, dw, batch=B, quant_kv_cache=kv8, unfused_decode=True)
+    assert a.stats()["launches_per_step"] < b.stats()["launches_per_step"]
+    refs = [orc.Model(cfg, w) for _ in range(3)]
+    for r in refs:
+        r.set_options(quant_kv_cache=kv8)
+    rng = np.random.default_rng(8)
+    for step in range(6):
+        toks = rng.integers(0, cfg["vocab"], B)
+        na, la = a.step(toks, [step], step, step + 1, want_logits=True)
+        nb, lb = b.step(toks, [step], step, step + 1, want_logits=True)
+        assert np.array_equal(la, lb) and na == nb, step
+        for i, r in enumerate(refs):
+            want = r.forward([toks[i]], [step], step, step + 1, False)
+            assert max_err_rel_to_max(g.f32(la[i:i + 1], dt), g.f32(want, dt)) <= 2e-2 if kv8 else 1e-2, (step, i)
+    for l in range(cfg["n_layers"]):
+        for j in range(len(a.kv[l])):
+            assert np.array_equal(g.to_host(a.kv[l][j]), g.to_host(b.kv[l][j])), (l, j)
+    a.close(), b.close()
