@@ -10,8 +10,8 @@
 // 32 activation rows (B operand, columns m).  The reduction index of an MFMA is free to permute as long
 // as both operands agree, so a lane takes 64 CONTIGUOUS bytes of its weight row per step of 128 k
 // (a full 128-byte line per row and step across the two lane halves) and the matching activation
-// elements (staged through LDS once per workgroup and step).  Four steps' loads are in flight per wave
-// (HBM latency under load is microseconds); when the matrix has too few rows to fill the device the K range is split over gridDim.y.  Partial sums [ksplit][M][N] (f32) are summed,
+// elements (staged through LDS once per workgroup and step).  Two steps' loads are in flight per wave behind the
+// one in use; when the matrix has too few rows to fill the device the K range is split over gridDim.y.  Partial sums [ksplit][M][N] (f32) are summed,
 // scaled and stored by a second launch that also applies the residual or SwiGLU.
 #include <type_traits>
 
@@ -20,7 +20,10 @@
 
 namespace mynn {
 
-constexpr int kSkinnyWaves = 4, kSkinnyThreads = kSkinnyWaves * 64, kSkinnyK = 128, kSkinnyStages = 5;
+// (stages: two steps of loads in flight behind the one in use.  Measured over a batch-32 decode step of the 8B shape: 3
+// stages 4.18 ms, 4 stages 4.20, 5 stages 4.24-4.26, 6 and 7 stages 4.27-4.31, 2 stages 4.59 -- the weight stream alone,
+// taken out of the kernel, also runs faster with fewer requests outstanding: 21.4 us at 3 stages, 22.8 at 5, 24.4 at 8)
+constexpr int kSkinnyWaves = 4, kSkinnyThreads = kSkinnyWaves * 64, kSkinnyK = 128, kSkinnyStages = 3;
 
 constexpr int kSkinnyLd = kSkinnyK + 8;  // LDS row stride of the activation chunk (272 bytes: conflict-free 128-bit reads)
 
