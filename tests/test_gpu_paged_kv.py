@@ -152,6 +152,49 @@ def test_paged_prefill_attention_vs_oracle_and_contiguous(g, dt, B, Hq, Hkv, D, 
         assert np.array_equal(got, plain)
 
 
+def test_paged_attention_seeded_shape_sweep(g):
+    """60 seeded shapes: 1..40 sequences, 1 / 2 / 4 / 8 query heads per kv head, head_dim 64 / 128, pages of 32..512 rows, 1..12
+    pages per sequence in a shuffled pool, ragged active lengths (first row of a page, last row, one row), one query row
+    (streaming kernel, with and without key ranges to merge) or a causal block of query rows behind a prefix (prefill
+    kernel), fp16 and bf16 -- against the f64 formula on the gathered rows; unused pages and rows hold NaN."""
+    import torch
+
+    rng = np.random.default_rng(2024)
+    for case in range(60):
+        dt = orc.F16 if case % 2 == 0 else orc.BF16
+        D = int(rng.choice([64, 128]))
+        G = int(rng.choice([1, 2, 4, 8]))
+        Hkv = int(rng.choice([1, 2, 4, 8]))
+        prefill = case % 5 == 4
+        P = int(rng.choice([64, 128, 256] if prefill else [32, 64, 128, 256, 512]))
+        pps = int(rng.integers(1, 7 if prefill else 13))
+        B = int(rng.integers(1, 4 if prefill else 41))
+        L = P * pps
+        while B * Hkv * L * D > 24e6:  # keep the host-side f64 loop short
+            B = max(1, B // 2)
+        Sq = int(rng.integers(2, min(L, 96) + 1)) if prefill else 1
+        kind = case % 4
+        active = L if kind == 0 else max(Sq, (L - 1) // P * P + 1) if kind == 1 else Sq if kind == 2 else int(rng.integers(Sq, L + 1))
+        Hq = G * Hkv
+        q = orc.to_storage(rng.standard_normal((B, Hq, Sq, D)), dt)
+        k = orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt)
+        v = orc.to_storage(rng.standard_normal((B, Hkv, L, D)), dt)
+        k[:, :, active:] = 0xFFFF
+        v[:, :, active:] = 0xFFFF
+        exact = orc.attention_f64(q, np.ascontiguousarray(k[:, :, :active]), np.ascontiguousarray(v[:, :, :active]), dt, D ** -0.5, prefill)
+        kp, table = scatter_to_pool(k, P, rng, spare=int(rng.integers(0, 5)))
+        vp = np.full_like(kp, 0xFFFF)
+        for b in range(B):
+            for s_ in range(pps):
+                vp[table[b, s_]] = v[b, :, s_ * P:(s_ + 1) * P]
+        tab = table.copy()
+        tab[:, (active + P - 1) // P:] = -1
+        got = g.to_host(g.mynn.attention_paged(g.to_dev(q, dt), g.to_dev(kp, dt), g.to_dev(vp, dt), torch.from_numpy(tab).cuda(), P,
+                                               D ** -0.5, prefill, active, q_pos_offset=active - Sq))
+        err = max_err_rel_to_max(g.f32(got, dt), exact) if prefill else max_abs_rel(g.f32(got, dt), exact)
+        assert err <= 1e-2, (case, dt, B, Hq, Hkv, D, Sq, L, active, P, err)
+
+
 def test_paged_attention_rejects_bad_arguments_with_a_status(g):
     """Shapes and page geometries the paged kernels have no form for come back as errors before anything is launched."""
     import torch
