@@ -102,6 +102,9 @@ SIGNATURES = {
     "mynn_kvcache_update_streaming": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "mynn_quantizing_kvcache_update_streaming": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "mynn_attention_streaming": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
+    "mynn_attention_streaming_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i, _i, _i, _i]),
+    "mynn_attention_streaming_ws": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp,
+                                         _vp, _sz, _vp]),
     "mynn_quantizing_kvcache_update": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "mynn_rms_norm": (_i, [_vp, _vp, _vp, _i, _i, _f, _i, _vp]),
     "mynn_rope": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
@@ -484,9 +487,10 @@ def quantizing_kvcache_update_streaming(cache, scale, new_kv, offset, ring_sink,
 
 
 def attention_streaming(q, k, v, scale, is_causal, active, ring_sink, ring_window, ring_start, q_pos_offset=None,
-                        k_scale=None, v_scale=None, rope=None):
+                        k_scale=None, v_scale=None, rope=None, workspace=None):
     """Attention over the sink + ring layout: keys by recency rank, rank -> cache row by the ring map.
-    rope = (cos_table, sin_table, kv_position int64): rotate K inside the operator."""
+    rope = (cos_table, sin_table, kv_position int64): rotate K inside the operator.
+    workspace (uint8 tensor of mynn_attention_streaming_workspace_bytes): the caller's scratch memory."""
     import torch
 
     B, Hq, Sq, D = q.shape
@@ -494,6 +498,13 @@ def attention_streaming(q, k, v, scale, is_causal, active, ring_sink, ring_windo
     if q_pos_offset is None:
         q_pos_offset = active - Sq
     out = torch.empty_like(q)
+    if workspace is not None:
+        check(lib().mynn_attention_streaming_ws(_ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(k_scale), _ptr(v_scale), float(scale),
+                                                int(is_causal), B, Sq, int(active), cache_len, int(q_pos_offset), Hq, Hkv, D,
+                                                _dt(q), int(k.dtype == torch.int8), int(ring_sink), int(ring_window),
+                                                int(ring_start), _ptr(rope[0]) if rope else None, _ptr(rope[1]) if rope else None,
+                                                _ptr(rope[2]) if rope else None, _ptr(workspace), workspace.numel(), _stream()))
+        return out
     check(lib().mynn_attention_streaming(_ptr(out), _ptr(q), _ptr(k), _ptr(v), _ptr(k_scale), _ptr(v_scale), float(scale),
                                          int(is_causal), B, Sq, int(active), cache_len, int(q_pos_offset), Hq, Hkv, D,
                                          _dt(q), int(k.dtype == torch.int8), int(ring_sink), int(ring_window),

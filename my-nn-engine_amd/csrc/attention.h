@@ -60,6 +60,12 @@ bool attention_prefill_supported(const AttnParams &p, int D, int dtype, int kv_i
 // streaming decode kernel (attention_stream.hip): taken when eligible; attn_plan then returns its plan
 bool attn_stream_eligible(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, int cache_len);
 void attn_stream_plan(int B, int Hkv, int kv_len, int *slice, int *nsplit);
+int attn_stream_max_ranges(int B, int Hkv, int kv_len_max);  // most key ranges any length <= kv_len_max is planned with
+void attn_stream_plan_paged(int B, int Hkv, int kv_len, int page_shift, int *slice, int *nsplit);
+int attn_stream_max_ranges_paged(int B, int Hkv, int kv_len_max, int page_shift);
+bool attn_stream_possible(int B, int Sq, int Hq, int Hkv, int D, int dtype, int cache_len);
+// bytes of partial results that hold for EVERY call with this shape and an active length / cache length up to cache_len
+size_t attn_max_scratch_bytes(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int cache_len);
 int attention_stream_launch(const AttnParams &p, int D, int dtype, int kv_int8, hipStream_t s);
 // paged K/V: the streaming kernel takes every decode shape it has a form for, whatever the sizes
 bool attn_stream_paged_supported(int Sq, int Hq, int Hkv, int D, int dtype, int page_rows);

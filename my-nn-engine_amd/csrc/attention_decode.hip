@@ -413,6 +413,20 @@ size_t attn_scratch_bytes(int B, int Hq, int Sq, int D, int nsplit) {
     size_t bytes = rows * nsplit * (D + 2) * sizeof(float);
     return (bytes + 255) / 256 * 256;
 }
+// The plan of a call depends on its active length and the number of key ranges is not monotonic in it, so a
+// caller-owned workspace is sized for the most ranges any length up to cache_len can get: the per-slice kernel's
+// count grows with the length, the streaming kernel's is bounded by the CUs per (sequence, kv head).
+size_t attn_max_scratch_bytes(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int cache_len) {
+    const int Gt = Hq / Hkv;
+    const size_t kv_elem = kv_int8 ? 1 : dtype_size(dtype);
+    const int rows = slice_rows(D, Gt, kv_elem);
+    int n = (cache_len + rows - 1) / rows;
+    if (attn_stream_possible(B, Sq, Hq, Hkv, D, dtype, cache_len)) {
+        const int ns = attn_stream_max_ranges(B, Hkv, cache_len);
+        if (ns > n) n = ns;
+    }
+    return n > 1 ? attn_scratch_bytes(B, Hq, Sq, D, n) : 0;
+}
 // scratch = [part_o | part_ml] of attn_scratch_bytes (contents need not survive the call)
 int attention_decode_launch(AttnParams p, int D, int dtype, int kv_int8, void *scratch, hipStream_t s) {
     if (p.nsplit > 1) {
@@ -505,13 +519,6 @@ static int static_scratch(void **out) {
 
 enum { WS_LIBRARY = 0, WS_CALLER = 1, WS_STATIC = 2 };
 
-// bytes of partial results the launch plan of this call needs (0: no key range is split)
-static size_t plan_scratch_bytes(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, int kv_len, int cache_len, bool masked) {
-    int slice = 0, nsplit = 1, hpw = 1;
-    attn_plan(B, Sq, Hq, Hkv, D, dtype, kv_int8, kv_len, cache_len, masked, &slice, &nsplit, &hpw);
-    return nsplit > 1 ? attn_scratch_bytes(B, Hq, Sq, D, nsplit) : 0;
-}
-
 static int attention_entry(void *out, const void *Q, const void *K, const void *V, const void *mask, long mask_os, long mask_rs,
                            const void *k_scale, const void *v_scale, float scale, int is_causal, int B, int Sq, int active_seq_kv,
                            const int32_t *d_active, int cache_seq_len, int q_pos_offset, int num_q_heads, int num_kv_heads,
@@ -579,10 +586,8 @@ extern "C" int mynn_attention(void *out, const void *Q, const void *K, const voi
 extern "C" size_t mynn_attention_workspace_bytes(int B, int Sq, int cache_seq_len, int num_q_heads, int num_kv_heads, int head_dim,
                                                  int dtype, int kv_int8) {
     if (B <= 0 || Sq <= 0 || cache_seq_len <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads) return 0;
-    // the longest key range a call can have, with and without a mask (a mask keeps the call off the streaming kernel)
-    const size_t a = plan_scratch_bytes(B, Sq, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, cache_seq_len, cache_seq_len, false);
-    const size_t b = plan_scratch_bytes(B, Sq, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, cache_seq_len, cache_seq_len, true);
-    return a > b ? a : b;
+    // enough for every active length up to the cache length, with and without a mask
+    return attn_max_scratch_bytes(B, Sq, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, cache_seq_len);
 }
 
 extern "C" int mynn_attention_ws(void *out, const void *Q, const void *K, const void *V, const void *mask, long mask_outer_stride,
@@ -605,17 +610,19 @@ extern "C" int mynn_attention_noalloc(void *out, const void *Q, const void *K, c
 }
 
 // ---- paged K/V: the same operator over pools and a page table
-static void paged_plan(int B, int Sq, int Hkv, int kv_len, int *slice, int *nsplit) {
+static void paged_plan(int B, int Sq, int Hkv, int kv_len, int page_shift, int *slice, int *nsplit) {
     *slice = 0;
     *nsplit = 1;
-    if (Sq == 1) attn_stream_plan(B, Hkv, kv_len, slice, nsplit);
+    if (Sq == 1) attn_stream_plan_paged(B, Hkv, kv_len, page_shift, slice, nsplit);
 }
 
 extern "C" size_t mynn_attention_paged_workspace_bytes(int B, int Sq, int pages_per_seq, int page_rows, int num_q_heads,
                                                        int num_kv_heads, int head_dim) {
     if (B <= 0 || Sq <= 0 || pages_per_seq <= 0 || page_rows <= 0 || num_q_heads <= 0 || num_kv_heads <= 0) return 0;
-    int slice, nsplit;
-    paged_plan(B, Sq, num_kv_heads, pages_per_seq * page_rows, &slice, &nsplit);
+    if (Sq != 1) return 0;
+    int shift = 0;
+    while ((1 << shift) < page_rows) shift++;
+    const int nsplit = attn_stream_max_ranges_paged(B, num_kv_heads, pages_per_seq * page_rows, shift);
     return nsplit > 1 ? attn_scratch_bytes(B, num_q_heads, Sq, head_dim, nsplit) : 0;
 }
 
@@ -647,7 +654,7 @@ extern "C" int mynn_attention_paged(void *out, const void *Q, const void *K_pool
         return attention_prefill_launch(p, head_dim, dtype, as_stream(s));
     }
     const int kv_len = d_active ? p.cache_len : (active_seq_kv < p.cache_len ? active_seq_kv : p.cache_len);
-    paged_plan(B, Sq, num_kv_heads, kv_len, &p.slice, &p.nsplit);
+    paged_plan(B, Sq, num_kv_heads, kv_len, p.page_shift, &p.slice, &p.nsplit);
     p.heads_per_wg = num_q_heads / num_kv_heads;
     if (p.nsplit > 1) {
         const size_t need = attn_scratch_bytes(B, num_q_heads, Sq, head_dim, p.nsplit);
@@ -684,7 +691,6 @@ __global__ void ring_rows_kernel(uint16_t *dst, const uint16_t *src, size_t unit
     }
 }
 
-static Grown g_ring_k, g_ring_v, g_ring_ks, g_ring_vs, g_ring_q, g_ring_o;
 
 // K rotated inside the operator (reference attention.cuh:407-420, 559-570): the key of rank r, dequantised,
 // is rotated by table row kv_position[r], everything in f32; V is dequantised.  Both land in rank order as f32.
@@ -751,23 +757,64 @@ extern "C" int mynn_kvcache_update_streaming(void *cache, const void *new_kv, in
     return launch_status("ring_rows_kernel");
 }
 
-extern "C" int mynn_attention_streaming(void *out, const void *Q, const void *K, const void *V, const void *k_scale,
-                                        const void *v_scale, float scale, int is_causal, int B, int Sq, int active_seq_kv,
-                                        int cache_seq_len, int q_pos_offset, int num_q_heads, int num_kv_heads, int head_dim,
-                                        int dtype, int kv_int8, int ring_sink, int ring_window, int ring_start,
-                                        const void *cos_t, const void *sin_t, const int64_t *kv_position, mynn_stream s) {
+// ---- mynn_attention_streaming: one workspace, carved into the rank-ordered K / V rows (and scales), the widened
+// queries and f32 output of the rotating form, and the partial results of the attention kernels behind it
+namespace mynn {
+struct RingCarve {
+    size_t k, v, ks, vs, q, o, attn, attn_bytes, total;
+};
+static RingCarve ring_carve(int B, int Sq, int Hq, int Hkv, int D, int dtype, int kv_int8, bool rope_on, int rows_max) {
+    RingCarve c{};
+    size_t off = 0;
+    auto take = [&](size_t bytes) { size_t o = off; off = (off + bytes + 255) / 256 * 256; return o; };
+    const size_t BH = (size_t)B * Hkv, eb = dtype_size(dtype), q_n = (size_t)B * Hq * Sq * D;
+    if (rope_on) {
+        c.k = take(BH * rows_max * D * 4);
+        c.v = take(BH * rows_max * D * 4);
+        c.q = take(dtype != MYNN_F32 ? q_n * 4 : 0);
+        c.o = take(dtype != MYNN_F32 ? q_n * 4 : 0);
+        c.attn_bytes = attn_max_scratch_bytes(B, Sq, Hq, Hkv, D, MYNN_F32, 0, rows_max);
+    } else {
+        const size_t rb = (size_t)D * (kv_int8 ? 1 : eb);
+        c.k = take(BH * rows_max * rb);
+        c.v = take(BH * rows_max * rb);
+        c.ks = take(kv_int8 ? BH * rows_max * eb : 0);
+        c.vs = take(kv_int8 ? BH * rows_max * eb : 0);
+        c.attn_bytes = attn_max_scratch_bytes(B, Sq, Hq, Hkv, D, dtype, kv_int8, rows_max);
+    }
+    c.attn = take(c.attn_bytes);
+    c.total = off;
+    return c;
+}
+static std::mutex g_ring_mu;
+static std::map<hipStream_t, Grown> g_ring;  // mynn_attention_streaming: one block per stream
+}  // namespace mynn
+
+extern "C" size_t mynn_attention_streaming_workspace_bytes(int B, int Sq, int cache_seq_len, int num_q_heads, int num_kv_heads,
+                                                           int head_dim, int dtype, int kv_int8, int rope_on) {
+    if (B <= 0 || Sq <= 0 || cache_seq_len <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads ||
+        head_dim <= 0 || !mynn::dtype_ok(dtype))
+        return 0;
+    return mynn::ring_carve(B, Sq, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, rope_on != 0, cache_seq_len).total;
+}
+
+extern "C" int mynn_attention_streaming_ws(void *out, const void *Q, const void *K, const void *V, const void *k_scale,
+                                           const void *v_scale, float scale, int is_causal, int B, int Sq, int active_seq_kv,
+                                           int cache_seq_len, int q_pos_offset, int num_q_heads, int num_kv_heads, int head_dim,
+                                           int dtype, int kv_int8, int ring_sink, int ring_window, int ring_start,
+                                           const void *cos_t, const void *sin_t, const int64_t *kv_position, void *workspace,
+                                           size_t workspace_bytes, mynn_stream s) {
     using namespace mynn;
     MYNN_REQUIRE(ring_sink >= 0 && ring_window >= 0 && ring_start >= 0 && (ring_window == 0 || ring_start < ring_window),
                  MYNN_ERR_INVALID, "attention: ring sink=%d window=%d start=%d", ring_sink, ring_window, ring_start);
     const bool rope_on = cos_t || sin_t || kv_position;
     MYNN_REQUIRE(!rope_on || (cos_t && sin_t && kv_position), MYNN_ERR_INVALID,
                  "attention: the K rotation needs cos, sin and kv_position together");
-    if (ring_window == 0 && !rope_on)
-        return mynn_attention(out, Q, K, V, k_scale, v_scale, scale, is_causal, B, Sq, active_seq_kv, nullptr, cache_seq_len,
-                              q_pos_offset, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, s);
     MYNN_REQUIRE(out && Q && K && V, MYNN_ERR_INVALID, "attention: null operand");
-    MYNN_REQUIRE(B > 0 && Sq > 0 && cache_seq_len > 0 && num_q_heads > 0 && num_kv_heads > 0 && head_dim > 0, MYNN_ERR_INVALID,
-                 "attention: B=%d Sq=%d cache=%d Hq=%d Hkv=%d D=%d", B, Sq, cache_seq_len, num_q_heads, num_kv_heads, head_dim);
+    MYNN_REQUIRE(B > 0 && Sq > 0 && cache_seq_len > 0 && num_q_heads > 0 && num_kv_heads > 0 && head_dim > 0 &&
+                     num_q_heads % num_kv_heads == 0,
+                 MYNN_ERR_INVALID, "attention: B=%d Sq=%d cache=%d Hq=%d Hkv=%d D=%d", B, Sq, cache_seq_len, num_q_heads, num_kv_heads,
+                 head_dim);
     MYNN_REQUIRE(active_seq_kv >= 1, MYNN_ERR_INVALID, "attention: active_seq_kv=%d", active_seq_kv);
     MYNN_REQUIRE(ring_sink + ring_window <= cache_seq_len, MYNN_ERR_INVALID, "attention: sink %d + window %d exceeds the cache of %d rows",
                  ring_sink, ring_window, cache_seq_len);
@@ -777,6 +824,10 @@ extern "C" int mynn_attention_streaming(void *out, const void *Q, const void *K,
     // never asks for them, and the plain kernels clamp the same way
     int rows = active_seq_kv < ring_sink + ring_window ? active_seq_kv : ring_sink + ring_window;
     if (ring_window == 0) rows = active_seq_kv < cache_seq_len ? active_seq_kv : cache_seq_len;
+    const RingCarve c = ring_carve(B, Sq, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, rope_on, rows);
+    MYNN_REQUIRE(workspace && ((uintptr_t)workspace & 255) == 0 && workspace_bytes >= c.total, MYNN_ERR_INVALID,
+                 "attention: the workspace must hold %zu bytes (mynn_attention_streaming_workspace_bytes), 256-byte aligned", c.total);
+    char *ws = (char *)workspace;
     const int BH = B * num_kv_heads;
     hipStream_t st = as_stream(s);
     if (rope_on) {
@@ -784,60 +835,82 @@ extern "C" int mynn_attention_streaming(void *out, const void *Q, const void *K,
         // queries widened, the f32 attention over them, one rounding of the result
         MYNN_REQUIRE(head_dim % 2 == 0, MYNN_ERR_INVALID, "attention: head_dim %d", head_dim);
         const size_t kv_n = (size_t)BH * rows * head_dim, q_n = (size_t)B * num_q_heads * Sq * head_dim;
-        int rc = ensure(g_ring_k, kv_n * 4, false, st);
-        if (!rc) rc = ensure(g_ring_v, kv_n * 4, false, st);
-        if (rc) return rc;
+        float *kf = (float *)(ws + c.k), *vf = (float *)(ws + c.v);
         const void *qf = Q;
         void *of = out;
         if (dtype != MYNN_F32) {
-            rc = ensure(g_ring_q, q_n * 4, false, st);
-            if (!rc) rc = ensure(g_ring_o, q_n * 4, false, st);
-            if (rc) return rc;
-            qf = g_ring_q.ptr;
-            of = g_ring_o.ptr;
+            qf = ws + c.q;
+            of = ws + c.o;
         }
-        rc = dispatch_dtype(dtype, [&](auto *t) {
+        int rc = dispatch_dtype(dtype, [&](auto *t) {
             using T = std::remove_pointer_t<decltype(t)>;
             const dim3 grid((unsigned)((kv_n + 255) / 256));
             if (kv_int8)
-                MYNN_LAUNCH((ring_rope_rows_kernel<T, true>), grid, dim3(256), 0, st, (float *)g_ring_k.ptr, (float *)g_ring_v.ptr, K, V,
-                            (const T *)k_scale, (const T *)v_scale, (const T *)cos_t, (const T *)sin_t, kv_position, head_dim, rows,
-                            cache_seq_len, ring_sink, ring_window, ring_start, kv_n);
+                MYNN_LAUNCH((ring_rope_rows_kernel<T, true>), grid, dim3(256), 0, st, kf, vf, K, V, (const T *)k_scale, (const T *)v_scale,
+                            (const T *)cos_t, (const T *)sin_t, kv_position, head_dim, rows, cache_seq_len, ring_sink, ring_window,
+                            ring_start, kv_n);
             else
-                MYNN_LAUNCH((ring_rope_rows_kernel<T, false>), grid, dim3(256), 0, st, (float *)g_ring_k.ptr, (float *)g_ring_v.ptr, K, V,
-                            (const T *)nullptr, (const T *)nullptr, (const T *)cos_t, (const T *)sin_t, kv_position, head_dim, rows,
-                            cache_seq_len, ring_sink, ring_window, ring_start, kv_n);
+                MYNN_LAUNCH((ring_rope_rows_kernel<T, false>), grid, dim3(256), 0, st, kf, vf, K, V, (const T *)nullptr, (const T *)nullptr,
+                            (const T *)cos_t, (const T *)sin_t, kv_position, head_dim, rows, cache_seq_len, ring_sink, ring_window,
+                            ring_start, kv_n);
             if (dtype != MYNN_F32)
-                MYNN_LAUNCH(widen_rows_kernel<T>, dim3((unsigned)((q_n + 255) / 256)), dim3(256), 0, st, (float *)g_ring_q.ptr, (const T *)Q, q_n);
+                MYNN_LAUNCH(widen_rows_kernel<T>, dim3((unsigned)((q_n + 255) / 256)), dim3(256), 0, st, (float *)(ws + c.q), (const T *)Q, q_n);
             return launch_status("ring_rope_rows_kernel");
         });
         if (rc) return rc;
-        rc = mynn_attention(of, qf, g_ring_k.ptr, g_ring_v.ptr, nullptr, nullptr, scale, is_causal, B, Sq, rows, nullptr, rows, q_pos_offset,
-                            num_q_heads, num_kv_heads, head_dim, MYNN_F32, 0, s);
+        rc = attention_entry(of, qf, kf, vf, nullptr, 0, 0, nullptr, nullptr, scale, is_causal, B, Sq, rows, nullptr, rows, q_pos_offset,
+                             num_q_heads, num_kv_heads, head_dim, MYNN_F32, 0, WS_CALLER, ws + c.attn, c.attn_bytes, st);
         if (rc || dtype == MYNN_F32) return rc;
         return dispatch_dtype16(dtype, [&](auto *t) {
             using T = std::remove_pointer_t<decltype(t)>;
-            MYNN_LAUNCH(narrow_rows_kernel<T>, dim3((unsigned)((q_n + 255) / 256)), dim3(256), 0, st, (T *)out, (const float *)g_ring_o.ptr, q_n);
+            MYNN_LAUNCH(narrow_rows_kernel<T>, dim3((unsigned)((q_n + 255) / 256)), dim3(256), 0, st, (T *)out, (const float *)(ws + c.o), q_n);
             return launch_status("narrow_rows_kernel");
         });
     }
     const size_t eb = dtype_size(dtype), row_bytes = (size_t)head_dim * (kv_int8 ? 1 : eb);
     MYNN_REQUIRE(row_bytes % 2 == 0 && eb % 2 == 0, MYNN_ERR_UNSUPPORTED, "attention: rows of %zu bytes", row_bytes);
-    auto gather = [&](Grown &gbuf, const void *src, size_t rb) -> int {
-        // (16 bytes of slack: the attention kernels want 16-byte aligned K / V, which hipMalloc gives)
-        int rc = ensure(gbuf, (size_t)BH * rows * rb + 16, false, st);
-        if (rc) return rc;
+    auto gather = [&](void *dst, const void *src, size_t rb) -> int {
         const size_t units = rb / 2, total = (size_t)BH * rows * units;
-        MYNN_LAUNCH((ring_rows_kernel<false>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, (uint16_t *)gbuf.ptr,
+        MYNN_LAUNCH((ring_rows_kernel<false>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, (uint16_t *)dst,
                     (const uint16_t *)src, units, rows, cache_seq_len, 0, ring_sink, ring_window, ring_start, total);
         return launch_status("ring_rows_kernel");
     };
-    int rc = gather(g_ring_k, K, row_bytes);
-    if (!rc) rc = gather(g_ring_v, V, row_bytes);
-    if (!rc && kv_int8) rc = gather(g_ring_ks, k_scale, eb);
-    if (!rc && kv_int8) rc = gather(g_ring_vs, v_scale, eb);
+    int rc = gather(ws + c.k, K, row_bytes);
+    if (!rc) rc = gather(ws + c.v, V, row_bytes);
+    if (!rc && kv_int8) rc = gather(ws + c.ks, k_scale, eb);
+    if (!rc && kv_int8) rc = gather(ws + c.vs, v_scale, eb);
     if (rc) return rc;
-    return mynn_attention(out, Q, g_ring_k.ptr, g_ring_v.ptr, kv_int8 ? g_ring_ks.ptr : nullptr, kv_int8 ? g_ring_vs.ptr : nullptr, scale,
-                          is_causal, B, Sq, rows, nullptr, rows, q_pos_offset, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, s);
+    return attention_entry(out, Q, ws + c.k, ws + c.v, nullptr, 0, 0, kv_int8 ? ws + c.ks : nullptr, kv_int8 ? ws + c.vs : nullptr, scale,
+                           is_causal, B, Sq, rows, nullptr, rows, q_pos_offset, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8,
+                           WS_CALLER, ws + c.attn, c.attn_bytes, st);
 }
 
+extern "C" int mynn_attention_streaming(void *out, const void *Q, const void *K, const void *V, const void *k_scale,
+                                        const void *v_scale, float scale, int is_causal, int B, int Sq, int active_seq_kv,
+                                        int cache_seq_len, int q_pos_offset, int num_q_heads, int num_kv_heads, int head_dim,
+                                        int dtype, int kv_int8, int ring_sink, int ring_window, int ring_start,
+                                        const void *cos_t, const void *sin_t, const int64_t *kv_position, mynn_stream s) {
+    using namespace mynn;
+    const bool rope_on = cos_t || sin_t || kv_position;
+    if (ring_window == 0 && !rope_on && ring_sink >= 0 && ring_start >= 0)
+        return mynn_attention(out, Q, K, V, k_scale, v_scale, scale, is_causal, B, Sq, active_seq_kv, nullptr, cache_seq_len,
+                              q_pos_offset, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, s);
+    MYNN_REQUIRE(B > 0 && Sq > 0 && cache_seq_len > 0 && num_q_heads > 0 && num_kv_heads > 0 && head_dim > 0 &&
+                     num_q_heads % num_kv_heads == 0 && dtype_ok(dtype),
+                 MYNN_ERR_INVALID, "attention: B=%d Sq=%d cache=%d Hq=%d Hkv=%d D=%d dtype=%d", B, Sq, cache_seq_len, num_q_heads,
+                 num_kv_heads, head_dim, dtype);
+    // the library's block of this stream, sized once for the whole cache (it then never grows for this shape)
+    const size_t need = ring_carve(B, Sq, num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, rope_on, cache_seq_len).total;
+    hipStream_t st = as_stream(s);
+    void *ws = nullptr;
+    {
+        std::lock_guard<std::mutex> lk(g_ring_mu);
+        Grown &g = g_ring[st];
+        int rc = ensure(g, need, false, st);
+        if (rc) return rc;
+        ws = g.ptr;
+    }
+    return mynn_attention_streaming_ws(out, Q, K, V, k_scale, v_scale, scale, is_causal, B, Sq, active_seq_kv, cache_seq_len, q_pos_offset,
+                                       num_q_heads, num_kv_heads, head_dim, dtype, kv_int8, ring_sink, ring_window, ring_start, cos_t,
+                                       sin_t, kv_position, ws, need, s);
+}

@@ -354,8 +354,7 @@ bool attn_stream_eligible(int B, int Sq, int Hq, int Hkv, int D, int dtype, int 
 // four workgroups per CU -- what the register count allows -- were 0-25 % slower: shorter sequential runs, more partial
 // results to write and to merge, and with at least one (sequence, kv head) per CU the merge launch disappears
 // altogether); ranges a multiple of the 128 keys a workgroup takes per step
-void attn_stream_plan(int B, int Hkv, int kv_len, int *slice, int *nsplit) {
-    const int step = kStreamWaves * kStreamTile;
+static int stream_slots() {
     static int slots = 0;
     if (!slots) {
         int dev = 0, cus = 0;
@@ -365,13 +364,50 @@ void attn_stream_plan(int B, int Hkv, int kv_len, int *slice, int *nsplit) {
         }
         slots = cus;
     }
-    int n = slots / (B * Hkv);
+    return slots;
+}
+void attn_stream_plan(int B, int Hkv, int kv_len, int *slice, int *nsplit) {
+    const int step = kStreamWaves * kStreamTile;
+    int n = stream_slots() / (B * Hkv);
     const int nmax = (kv_len + 127) / 128;
     if (n > nmax) n = nmax;
     if (n < 1) n = 1;
     int rows = ((kv_len + n - 1) / n + step - 1) / step * step;
     *slice = rows;
     *nsplit = (kv_len + rows - 1) / rows;
+}
+// The number of key ranges is not monotonic in the length (a longer cache can round to fewer, longer ranges), so a
+// workspace is sized for the most ranges ANY length up to kv_len_max can be planned with.
+int attn_stream_max_ranges(int B, int Hkv, int kv_len_max) {
+    int n = stream_slots() / (B * Hkv);
+    const int nmax = (kv_len_max + 127) / 128;
+    if (n > nmax) n = nmax;
+    return n < 1 ? 1 : n;
+}
+// Paged caches: the pages of a key range travel in one vector register, a lane each, so a range spans at most 62
+// pages (one more at either end for ranges that start inside a page); longer ranges are cut into more of them.
+static int paged_slice_cap(int page_shift) {
+    const int step = kStreamWaves * kStreamTile;
+    return ((62 << page_shift) / step) * step;
+}
+void attn_stream_plan_paged(int B, int Hkv, int kv_len, int page_shift, int *slice, int *nsplit) {
+    attn_stream_plan(B, Hkv, kv_len, slice, nsplit);
+    const int cap = paged_slice_cap(page_shift);
+    if (*slice > cap) {
+        *slice = cap;
+        *nsplit = (kv_len + cap - 1) / cap;
+    }
+}
+int attn_stream_max_ranges_paged(int B, int Hkv, int kv_len_max, int page_shift) {
+    const int a = attn_stream_max_ranges(B, Hkv, kv_len_max), cap = paged_slice_cap(page_shift);
+    const int b = (kv_len_max + cap - 1) / cap;
+    return a > b ? a : b;
+}
+// the conditions of attn_stream_eligible that do not depend on the length of one call
+bool attn_stream_possible(int B, int Sq, int Hq, int Hkv, int D, int dtype, int cache_len) {
+    const int G = Hq / Hkv;
+    return Sq == 1 && dtype != MYNN_F32 && (D == 64 || D == 128) && (G == 1 || G == 2 || G == 4 || G == 8) &&
+           cache_len >= kStreamTile && (long)B * Hkv * cache_len >= kStreamMinKeys;
 }
 
 template <typename T, int D, bool KVI8, bool PAGED>

@@ -146,6 +146,8 @@ struct Model {
     int ring_sink = 0, ring_window = 0, ring_start = 0, h_past = 0, h_active = 0;
     int64_t *d_kvpos = nullptr;
     void *q_ref = nullptr, *k_new = nullptr, *v_new = nullptr, *attn_ref = nullptr, *k_rot = nullptr;
+    void *ring_ws = nullptr;      // ... and the scratch memory of the ring attention (rank-ordered rows, partial results)
+    size_t ring_ws_bytes = 0;
     int last_status = 0;          // of the last model() call on this state
     void *warena = nullptr;       // weight_arena: every linear weight and scale of the model in one allocation, in execution order
     mynn_kv_pages *pages = nullptr;  // kv_page_rows: the session's page table (the caller's); k_cache / v_cache then are pools
@@ -285,9 +287,9 @@ static int streaming_attention(Model &m, Layer &L, float softmax_scale) {
         TRY(mynn_quantizing_kvcache_update_streaming((int8_t *)L.v_cache, L.v_scale, m.v_new, m.h_past, Hkv, S, c.max_seq, D,
                                                      m.ring_sink, m.ring_window, m.ring_start, c.dtype, s));
         note(m, "attention_streaming_rope", (double)S * 2.0 * Hq * D * eb);
-        TRY(mynn_attention_streaming(attn_out, m.q_ref, L.k_cache, L.v_cache, L.k_scale, L.v_scale, softmax_scale, S > 1, 1, S,
-                                     m.h_active, c.max_seq, m.h_active - S, Hq, Hkv, D, c.dtype, 1, m.ring_sink, m.ring_window,
-                                     m.ring_start, m.cos_t, m.sin_t, m.d_kvpos, s));
+        TRY(mynn_attention_streaming_ws(attn_out, m.q_ref, L.k_cache, L.v_cache, L.k_scale, L.v_scale, softmax_scale, S > 1, 1, S,
+                                        m.h_active, c.max_seq, m.h_active - S, Hq, Hkv, D, c.dtype, 1, m.ring_sink, m.ring_window,
+                                        m.ring_start, m.cos_t, m.sin_t, m.d_kvpos, m.ring_ws, m.ring_ws_bytes, s));
     } else {
         note(m, "kvcache_update_streaming", (double)S * 4 * Hkv * D * eb);
         TRY(mynn_kvcache_update_streaming(L.k_cache, m.k_new, m.h_past, Hkv, S, c.max_seq, D, m.ring_sink, m.ring_window,
@@ -297,9 +299,9 @@ static int streaming_attention(Model &m, Layer &L, float softmax_scale) {
         note(m, "rope_k_cache", 2.0 * Hkv * c.max_seq * D * eb);
         TRY(mynn_rope(m.k_rot, L.k_cache, m.cos_t, m.sin_t, m.d_kvpos, Hkv, c.max_seq, D, c.dtype, s));
         note(m, "attention_streaming", (double)S * 2.0 * Hq * D * eb);
-        TRY(mynn_attention_streaming(attn_out, m.q_ref, m.k_rot, L.v_cache, nullptr, nullptr, softmax_scale, S > 1, 1, S,
-                                     m.h_active, c.max_seq, m.h_active - S, Hq, Hkv, D, c.dtype, 0, m.ring_sink, m.ring_window,
-                                     m.ring_start, nullptr, nullptr, nullptr, s));
+        TRY(mynn_attention_streaming_ws(attn_out, m.q_ref, m.k_rot, L.v_cache, nullptr, nullptr, softmax_scale, S > 1, 1, S,
+                                        m.h_active, c.max_seq, m.h_active - S, Hq, Hkv, D, c.dtype, 0, m.ring_sink, m.ring_window,
+                                        m.ring_start, nullptr, nullptr, nullptr, m.ring_ws, m.ring_ws_bytes, s));
     }
     if (S > 1) {
         const size_t n = (size_t)Hq * S * D;
@@ -762,7 +764,7 @@ static int build(Model &m, void **init, void **state) {
             m.slice = 0;
             m.nsplit = 1;
             m.heads_per_wg = c.n_heads / c.n_kv_heads;
-            if (c.seq_q == 1) attn_stream_plan(c.batch, c.n_kv_heads, c.max_seq, &m.slice, &m.nsplit);
+            if (c.seq_q == 1) attn_stream_plan_paged(c.batch, c.n_kv_heads, c.max_seq, m.paging.shift, &m.slice, &m.nsplit);
         }
     }
     m.token_cap = c.max_seq + 8;
@@ -792,6 +794,10 @@ static int build(Model &m, void **init, void **state) {
     size_t o_qref = plan.take(strm ? (size_t)rows * QD * eb : 0), o_knew = plan.take(strm ? (size_t)rows * KD * eb : 0);
     size_t o_vnew = plan.take(strm ? (size_t)rows * KD * eb : 0), o_aref = plan.take(strm ? (size_t)rows * QD * eb : 0);
     size_t o_krot = plan.take(strm && !c.quant_kv_cache ? (size_t)KD * c.max_seq * eb : 0);
+    m.ring_ws_bytes = strm ? mynn_attention_streaming_workspace_bytes(1, c.seq_q, c.max_seq, c.n_heads, c.n_kv_heads, c.head_dim, c.dtype,
+                                                                      c.quant_kv_cache, c.quant_kv_cache)
+                           : 0;
+    size_t o_ring = plan.take(m.ring_ws_bytes);
     m.arena_bytes = plan.off;
     MYNN_HIP(hipMalloc((void **)&m.arena, m.arena_bytes));
     MYNN_HIP(hipMemset(m.arena, 0, m.arena_bytes));
@@ -809,6 +815,7 @@ static int build(Model &m, void **init, void **state) {
     m.d_kvpos = (int64_t *)(m.arena + o_kvpos);
     m.q_ref = m.arena + o_qref; m.k_new = m.arena + o_knew; m.v_new = m.arena + o_vnew; m.attn_ref = m.arena + o_aref;
     m.k_rot = m.arena + o_krot;
+    m.ring_ws = m.arena + o_ring;
     m.next_stage = align_up((size_t)c.batch * 4, 256);  // the sequences' next tokens live in the tail of the staging buffer
     m.stage_bytes = align_up((size_t)rows * 8 + (size_t)c.seq_q * 8 + 64 + (size_t)m.token_cap * 4 + (strm ? (size_t)c.max_seq * 8 : 0), 256) +
                     256 + m.next_stage;
@@ -817,7 +824,7 @@ static int build(Model &m, void **init, void **state) {
 
     // ---- batch-1 decode: projection and attention in one launch when the shape allows
     m.spin_limit = c.handover_spin_limit > 0 ? c.handover_spin_limit : c.handover_spin_limit < 0 ? 0 : 400000;
-    if (m.quant && rows == 1 && !c.quantize_activations && !c.unfused_decode && !m.pages && !c.qkv_bias &&
+    if (m.quant && rows == 1 && !c.quantize_activations && !c.unfused_decode && !m.pages && !c.qkv_bias && !c.streaming_kv &&
         attention_fused_supported(c.head_dim, c.n_heads / c.n_kv_heads) &&
         (!c.quant_kv_cache || attention_fused_kv8_supported(c.head_dim, c.max_seq)) &&
         qkv_attention_supported(H, c.n_heads, c.n_kv_heads, c.head_dim, c.max_seq, c.dtype) && (QD + 2 * KD) * eb % 8 == 0) {
@@ -922,7 +929,8 @@ static void destroy(Model *m) {
 static int upload_inputs(Model &m, const int64_t *ids, const int64_t *pos, int64_t past, int64_t active) {
     const mynn_model_config &c = m.cfg;
     const int rows = c.batch * c.seq_q;
-    MYNN_REQUIRE(past >= 0 && past + c.seq_q <= c.max_seq, MYNN_ERR_TOO_LONG,
+    // (streaming_kv: past_len is the session's unbounded stream position; the ring map folds it into the cache)
+    MYNN_REQUIRE(past >= 0 && (c.streaming_kv ? past + c.seq_q <= INT32_MAX : past + c.seq_q <= c.max_seq), MYNN_ERR_TOO_LONG,
                  "past_len %lld + %d rows exceeds max_seq %d", (long long)past, c.seq_q, c.max_seq);
     MYNN_REQUIRE(active >= 1 && active <= c.max_seq, MYNN_ERR_INVALID, "active_seq_kv %lld out of range", (long long)active);
     // paged cache: every row the step writes or may read has a page before anything is launched
@@ -1112,13 +1120,12 @@ extern "C" int mynn_model_step_streaming(void *state, const int64_t *input_ids, 
     MYNN_REQUIRE(ring_sink >= 0 && ring_window > 0 && ring_sink + ring_window <= c.max_seq && ring_start >= 0 && ring_start < ring_window,
                  MYNN_ERR_INVALID, "model_step_streaming: ring sink=%lld window=%lld start=%lld (max_seq %d)", (long long)ring_sink,
                  (long long)ring_window, (long long)ring_start, c.max_seq);
-    // Past sink + window the reference's session (session.rs:572-597) and its kernels' slot map (kvcache_update.cuh:21,
-    // common.cuh:55-60) disagree: the update maps the unbounded position through ring_start a second time, so every
-    // second ring slot is never overwritten again and the rank order the attention enumerates is not the token order.
-    // No fixture pins a value there; nothing is invented here.
-    MYNN_REQUIRE(past_len + c.seq_q <= ring_sink + ring_window, MYNN_ERR_UNSUPPORTED,
-                 "streaming_kv: past_len %lld + %d rows goes past sink + window = %lld, where the reference's session inputs and "
-                 "slot map are not consistent with each other", (long long)past_len, c.seq_q, (long long)(ring_sink + ring_window));
+    // past_len may lie past sink + window: the operators then apply the reference's own formulas to the session's
+    // inputs (kvcache_update.cuh:21 maps past_len + t through ring_phys_index with the session's ring_start;
+    // attention.cuh:397, 549 enumerate ranks through the same map), whatever slot that names.
+    MYNN_REQUIRE(active_seq_kv >= c.seq_q && active_seq_kv <= ring_sink + ring_window, MYNN_ERR_INVALID,
+                 "model_step_streaming: active_seq_kv %lld outside [%d, sink + window = %lld]", (long long)active_seq_kv, c.seq_q,
+                 (long long)(ring_sink + ring_window));
     for (int r = 0; r < c.max_seq; r++)
         MYNN_REQUIRE(kv_position[r] >= 0 && kv_position[r] < c.max_seq, MYNN_ERR_INVALID, "kv_position[%d]=%lld outside the RoPE table",
                      r, (long long)kv_position[r]);

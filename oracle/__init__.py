@@ -100,6 +100,12 @@ _sig("orc_model_v_scale", _vp, _vp, _i)
 _sig("orc_model_past_len", _ll, _vp)
 _sig("orc_model_set_past_len", None, _vp, _ll)
 _sig("orc_model_forward", None, _vp, _vp, _vp, _sz, _ll, _ll, _i, _vp)
+_sig("orc_model_forward_streaming", None, _vp, _vp, _vp, _sz, _ll, _ll, _i, _i, _i, _i, _vp, _vp)
+_sig("orc_model_set_streaming", None, _vp, _i, _i)
+_sig("orc_kv_cache_update_ring", None, _vp, _vp, _ll, _sz, _sz, _sz, _sz, _sz, _i, _i, _i)
+_sig("orc_quantizing_kv_cache_update_ring", None, _vp, _vp, _vp, _ll, _sz, _sz, _sz, _sz, _i, _i, _i, _i)
+_sig("orc_attention_ring", None, _vp, _vp, _vp, _vp, _vp, _vp, _ll, _sz, _sz, _sz, _sz, _sz, _sz, _i, _f, _i, _i, _i, _i, _i,
+     _vp, _vp, _vp)
 _sig("orc_model_decode_step", C.c_int64, _vp, C.c_int64)
 _sig("orc_model_prefill", C.c_int64, _vp, _vp, _sz, _sz)
 _sig("orc_model_generate", _ll, _vp, _vp, _sz, _sz, _sz, C.c_int64, _vp)
@@ -319,6 +325,28 @@ def attention_streaming(q, k, v, dt, scale, is_causal, active, ring_sink, ring_w
     return to_storage(out, dt)
 
 
+def attention_ring(q, k, v, dt, scale, is_causal, active, ring_sink, ring_window, ring_start, k_scale=None, v_scale=None,
+                   rope=None):
+    """The C restatement of the same operator (orc_attention_ring): one loop nest that follows the CUDA decode
+    kernel key by key instead of gathering rows first; used by the streaming decoder of this module."""
+    kv_int8 = k.dtype == np.int8
+    q = _c(q, np_dtype(dt))
+    k = _c(k, np.int8 if kv_int8 else np_dtype(dt))
+    v = _c(v, np.int8 if kv_int8 else np_dtype(dt))
+    B, Hq, Sq, D = q.shape
+    Hkv, Sk = k.shape[1], k.shape[2]
+    out = np.empty(q.shape, np_dtype(dt))
+    ks = _c(k_scale, np_dtype(dt)) if kv_int8 else None
+    vs = _c(v_scale, np_dtype(dt)) if kv_int8 else None
+    cos_t = sin_t = kvp = None
+    if rope is not None:
+        cos_t, sin_t, kvp = _c(rope[0], np_dtype(dt)), _c(rope[1], np_dtype(dt)), _c(np.asarray(rope[2], np.int64))
+    _lib.orc_attention_ring(_p(out), _p(q), _p(k), _p(v), _p(ks), _p(vs), int(active), B, Hq, Hkv, Sq, Sk, D, int(is_causal),
+                            float(scale), dt, int(kv_int8), int(ring_sink), int(ring_window), int(ring_start), _p(cos_t),
+                            _p(sin_t), _p(kvp))
+    return out
+
+
 def quantizing_kv_cache_update(cache, scale, new_kv, offset, dt):
     assert cache.flags.c_contiguous and cache.dtype == np.int8 and scale.flags.c_contiguous
     new_kv = _c(new_kv, np_dtype(dt))
@@ -487,6 +515,22 @@ class Model:
         logits = np.empty((S, self.cfg.vocab), np_dtype(self.dt))
         _lib.orc_model_forward(self._h, _p(ids), _p(positions), S, int(past_len), int(active),
                                int(is_causal), _p(logits))
+        return logits
+
+    def set_streaming(self, sink, window):
+        """DecodeKind::LlamaStreaming { sink, window } over the BuildOptions::streaming_kv graph: decode_step,
+        prefill and generate then build the session's ring inputs themselves (session.rs:539-635)."""
+        _lib.orc_model_set_streaming(self._h, int(sink), int(window))
+
+    def forward_streaming(self, ids, positions, past_len, active, is_causal, sink, window, ring_start, kv_position):
+        ids = _c(np.asarray(ids, np.int64))
+        positions = _c(np.asarray(positions, np.int64))
+        kv_position = _c(np.asarray(kv_position, np.int64))
+        assert kv_position.size == self.cfg.max_seq
+        S = ids.size
+        logits = np.empty((S, self.cfg.vocab), np_dtype(self.dt))
+        _lib.orc_model_forward_streaming(self._h, _p(ids), _p(positions), S, int(past_len), int(active), int(is_causal),
+                                         int(sink), int(window), int(ring_start), _p(kv_position), _p(logits))
         return logits
 
     def decode_step(self, token):

@@ -530,6 +530,91 @@ void orc_streaming_kv_position(int64_t *out, size_t sink, size_t window, size_t 
     }
 }
 
+/* KVCacheUpdate / QuantizingKVCacheUpdate with the ring inputs (cuda kvcache_update.cuh:12-26,
+ * quantizing_kvcache_update.cuh:24-36): row t of new_kv goes to cache row ring_phys_index(offset + t), rows in
+ * increasing t, so a later row wins a shared slot.  `offset` is the session's unbounded stream position
+ * (session.rs:541, 573), which the map folds into the ring with the session's ring_start -- past sink + window
+ * that is slot sink + (ring_start + offset + t - sink) % window, whatever that slot holds.  The quantiser is the
+ * one of orc_quantizing_kv_cache_update (the CPU backend's rounding, which the library follows everywhere; the
+ * CUDA kernel's roundf(x * (1/s)) differs from it in the last code of some values). */
+void orc_kv_cache_update_ring(void *cache, const void *new_kv, long long offset, size_t BH, size_t S_new,
+                              size_t max_seq, size_t D, size_t eb, int sink, int window, int start) {
+    for (size_t bh = 0; bh < BH; bh++)
+        for (size_t t = 0; t < S_new; t++) {
+            size_t slot = (size_t)orc_ring_phys_index((int)(offset + (long long)t), sink, window, start);
+            memcpy((char *)cache + ((bh * max_seq + slot) * D) * eb,
+                   (const char *)new_kv + ((bh * S_new + t) * D) * eb, D * eb);
+        }
+}
+void orc_quantizing_kv_cache_update_ring(int8_t *cache, void *scale, const void *new_kv, long long offset,
+                                         size_t BH, size_t S_new, size_t max_seq, size_t D, int dtype,
+                                         int sink, int window, int start) {
+    size_t eb = esize(dtype);
+    int8_t *row = (int8_t *)malloc(D);
+    char sc[4];
+    for (size_t bh = 0; bh < BH; bh++)
+        for (size_t t = 0; t < S_new; t++) {
+            size_t slot = (size_t)orc_ring_phys_index((int)(offset + (long long)t), sink, window, start);
+            /* one row through the plain quantiser into a one-row cache, then placed */
+            orc_quantizing_kv_cache_update(row, sc, (const char *)new_kv + ((bh * S_new + t) * D) * eb, 0, 1, 1, 1, D, dtype);
+            memcpy(cache + (bh * max_seq + slot) * D, row, D);
+            memcpy((char *)scale + (bh * max_seq + slot) * eb, sc, eb);
+        }
+    free(row);
+}
+
+/* Attention over the sink + ring layout, as the CUDA kernels enumerate it (attention.cuh:495-606 decode,
+ * 100-200 / 386-420 tiled): keys by recency rank r = 0 .. bound-1, the key of rank r is cache row
+ * ring_phys_index(r); causal rule in ranks, r <= (active - Sq) + query row (cuda.rs:1360-1364).
+ * kv_position != NULL: the dequantised key is rotated (half-split) by table row kv_position[r] -- indexed by
+ * RANK, as the kernels do (attention.cuh:163, 416, 560), although the session fills the table by slot
+ * (session.rs:604-635); everything in f32.  int8 K/V: score = (q . (code * k_scale rotated)) * scale,
+ * weight * v_scale before it meets the V codes (attention.cuh:549-598). */
+void orc_attention_ring(void *out, const void *q, const void *k, const void *v, const void *k_scale,
+                        const void *v_scale, long long active, size_t B, size_t Hq, size_t Hkv, size_t Sq,
+                        size_t Sk, size_t D, int is_causal, float scale, int dtype, int kv_int8, int sink,
+                        int window, int start, const void *cos_t, const void *sin_t, const int64_t *kv_position) {
+    long long past = active - (long long)Sq;
+    size_t group = Hq / Hkv, half = D / 2;
+    float *o = (float *)malloc(D * sizeof(float)), *kr = (float *)malloc(D * sizeof(float));
+    for (size_t bh = 0; bh < B * Hq; bh++)
+        for (size_t sq = 0; sq < Sq; sq++) {
+            size_t b = bh / Hq, h = bh % Hq, bhkv = b * Hkv + h / group;
+            size_t qo = (bh * Sq + sq) * D;
+            long long bound = active;
+            if (is_causal && past + (long long)sq + 1 < bound) bound = past + (long long)sq + 1;
+            for (size_t d = 0; d < D; d++) o[d] = 0.0f;
+            float m = -INFINITY, s = 0.0f;
+            for (long long r = 0; r < bound; r++) {
+                size_t tok = bhkv * Sk + (size_t)orc_ring_phys_index((int)r, sink, window, start);
+                float ks = kv_int8 ? ld(k_scale, tok, dtype) : 1.0f;
+                for (size_t d = 0; d < D; d++) kr[d] = kv_ld(k, tok * D + d, dtype, kv_int8) * ks;
+                float sum = 0.0f;
+                if (kv_position) {
+                    size_t tab = (size_t)kv_position[r] * D;
+                    for (size_t d = 0; d < D; d++) {
+                        float kp = d < half ? kr[d + half] : kr[d - half];
+                        float sign = d < half ? -1.0f : 1.0f;
+                        float rot = kr[d] * ld(cos_t, tab + d, dtype) + (sign * kp) * ld(sin_t, tab + d, dtype);
+                        sum = sum + ld(q, qo + d, dtype) * rot;
+                    }
+                } else {
+                    for (size_t d = 0; d < D; d++) sum = sum + ld(q, qo + d, dtype) * kr[d];
+                }
+                float qk = sum * scale;
+                float m_new = fmaxf(m, qk);
+                float factor = expf(m - m_new);
+                float e = expf(qk - m_new);
+                s = s * factor + e;
+                float e_eff = kv_int8 ? e * ld(v_scale, tok, dtype) : e;
+                for (size_t d = 0; d < D; d++) o[d] = o[d] * factor + e_eff * kv_ld(v, tok * D + d, dtype, kv_int8);
+                m = m_new;
+            }
+            for (size_t d = 0; d < D; d++) st(out, qo + d, o[d] / s, dtype);
+        }
+    free(o); free(kr);
+}
+
 /* ------------------------------------------------------------------ A12 / A13 decoder */
 struct orc_layer {
     orc_linear lin[7];
@@ -548,6 +633,7 @@ struct orc_model {
     int gemm_mode; /* -1: CPU backend's dispatch; 2: CUDA backend's (M >= 16 -> W rounded first) */
     int quant_kv_cache;       /* BuildOptions::quant_kv_cache (decoder.rs:672, 405-470) */
     int quantize_activations; /* Options::quantize_activations (transform/optimize/quantize_activations.rs) */
+    int streaming, sink, window; /* BuildOptions::streaming_kv + DecodeKind::LlamaStreaming { sink, window } */
     void *last_hidden;
     size_t last_S;
 };
@@ -665,8 +751,13 @@ static void from_heads(void *dst, const void *src, size_t S, size_t H, size_t D,
             memcpy((char *)dst + ((s * H + h) * D) * eb, (const char *)src + ((h * S + s) * D) * eb, D * eb);
 }
 
-void orc_model_forward(orc_model *m, const int64_t *ids, const int64_t *positions, size_t S,
-                       long long past_len, long long active, int is_causal, void *logits) {
+/* ring != NULL: the streaming graph (decoder.rs:281-347, 472-487) -- RoPE(q) by `positions`; k and v go
+ * UN-ROTATED into the caches through the slot map; 16-bit KV: Rope over the whole K cache by kv_position (one
+ * table row per cache SLOT, result rounded to dtype: it is a graph value), then Attention with the ring inputs;
+ * int8 KV: Attention rotates the dequantised keys itself, by kv_position[rank]. */
+typedef struct { int sink, window, start; const int64_t *kv_position; } orc_ring;
+static void forward_impl(orc_model *m, const int64_t *ids, const int64_t *positions, size_t S,
+                         long long past_len, long long active, int is_causal, const orc_ring *ring, void *logits) {
     const orc_model_cfg *c = &m->cfg;
     const int dt = c->dtype;
     const size_t eb = esize(dt);
@@ -706,6 +797,26 @@ void orc_model_forward(orc_model *m, const int64_t *ids, const int64_t *position
         to_heads(kh, kb, S, Hkv, D, eb);
         to_heads(vh, vb, S, Hkv, D, eb);
         orc_rope(qr, qh, m->cos_t, m->sin_t, positions, Hq, S, D, dt);
+        if (ring) {
+            const size_t MS = (size_t)c->max_seq;
+            if (m->quant_kv_cache) {
+                orc_quantizing_kv_cache_update_ring((int8_t *)L->k_cache, L->k_scale, kh, past_len, Hkv, S, MS, D, dt,
+                                                    ring->sink, ring->window, ring->start);
+                orc_quantizing_kv_cache_update_ring((int8_t *)L->v_cache, L->v_scale, vh, past_len, Hkv, S, MS, D, dt,
+                                                    ring->sink, ring->window, ring->start);
+                orc_attention_ring(ao, qr, L->k_cache, L->v_cache, L->k_scale, L->v_scale, active, 1, Hq, Hkv, S, MS, D,
+                                   is_causal, scale, dt, 1, ring->sink, ring->window, ring->start, m->cos_t, m->sin_t,
+                                   ring->kv_position);
+            } else {
+                orc_kv_cache_update_ring(L->k_cache, kh, past_len, Hkv, S, MS, D, eb, ring->sink, ring->window, ring->start);
+                orc_kv_cache_update_ring(L->v_cache, vh, past_len, Hkv, S, MS, D, eb, ring->sink, ring->window, ring->start);
+                void *krot = malloc(Hkv * MS * D * eb);
+                orc_rope(krot, L->k_cache, m->cos_t, m->sin_t, ring->kv_position, Hkv, MS, D, dt);
+                orc_attention_ring(ao, qr, krot, L->v_cache, NULL, NULL, active, 1, Hq, Hkv, S, MS, D, is_causal, scale,
+                                   dt, 0, ring->sink, ring->window, ring->start, NULL, NULL, NULL);
+                free(krot);
+            }
+        } else {
         orc_rope(kr, kh, m->cos_t, m->sin_t, positions, Hkv, S, D, dt);
         if (m->quant_kv_cache) {
             orc_quantizing_kv_cache_update((int8_t *)L->k_cache, L->k_scale, kr, past_len, Hkv, S, (size_t)c->max_seq, D, dt);
@@ -717,6 +828,7 @@ void orc_model_forward(orc_model *m, const int64_t *ids, const int64_t *position
             orc_kv_cache_update(L->v_cache, vh, past_len, Hkv, S, (size_t)c->max_seq, D, eb);
             orc_attention(ao, qr, L->k_cache, L->v_cache, NULL, NULL, active, 1, Hq, Hkv, S,
                           (size_t)c->max_seq, D, is_causal, scale, dt, 0);
+        }
         }
         from_heads(ab, ao, S, Hq, D, eb);
         linear(m, ob, ab, &L->lin[3], S, H, QD);
@@ -738,10 +850,40 @@ void orc_model_forward(orc_model *m, const int64_t *ids, const int64_t *position
     free(qr); free(kr); free(ao); free(ab); free(ob); free(g); free(u); free(hmid); free(dn);
 }
 
+void orc_model_forward(orc_model *m, const int64_t *ids, const int64_t *positions, size_t S,
+                       long long past_len, long long active, int is_causal, void *logits) {
+    forward_impl(m, ids, positions, S, past_len, active, is_causal, NULL, logits);
+}
+void orc_model_forward_streaming(orc_model *m, const int64_t *ids, const int64_t *positions, size_t S,
+                                 long long past_len, long long active, int is_causal, int sink, int window,
+                                 int ring_start, const int64_t *kv_position, void *logits) {
+    orc_ring ring = {sink, window, ring_start, kv_position};
+    forward_impl(m, ids, positions, S, past_len, active, is_causal, &ring, logits);
+}
+void orc_model_set_streaming(orc_model *m, int sink, int window) {
+    m->streaming = window > 0;
+    m->sink = sink;
+    m->window = window;
+}
+
+/* streaming_decode_inputs (session.rs:571-597) */
+static void streaming_decode(orc_model *m, int64_t token, void *logits) {
+    long long max_active = m->sink + m->window, sp = m->past_len;
+    int64_t qpos = sp < max_active - 1 ? sp : max_active - 1;
+    long long active = sp + 1 < max_active ? sp + 1 : max_active;
+    int ring_start = sp < max_active ? 0 : (int)((sp - m->sink) % m->window);
+    int64_t *kvpos = (int64_t *)malloc((size_t)m->cfg.max_seq * sizeof(int64_t));
+    orc_streaming_kv_position(kvpos, (size_t)m->sink, (size_t)m->window, (size_t)sp, (size_t)m->cfg.max_seq);
+    orc_model_forward_streaming(m, &token, &qpos, 1, sp, active, 0, m->sink, m->window, ring_start, kvpos, logits);
+    free(kvpos);
+}
+
 int64_t orc_model_decode_step(orc_model *m, int64_t token) {
     size_t V = (size_t)m->cfg.vocab;
     void *logits = malloc(V * esize(m->cfg.dtype));
     int64_t pos = m->past_len;
+    if (m->streaming) streaming_decode(m, token, logits);
+    else
     orc_model_forward(m, &token, &pos, 1, m->past_len, m->past_len + 1, 0, logits);
     int64_t next = orc_argmax_last(logits, V, m->cfg.dtype);
     free(logits);
@@ -757,6 +899,17 @@ int64_t orc_model_prefill(orc_model *m, const int64_t *ids, size_t n, size_t P) 
     while (n > 0) {
         size_t chunk = n < P ? n : P;
         for (size_t i = 0; i < P; i++) { padded[i] = i < chunk ? ids[i] : 0; pos[i] = m->past_len + (int64_t)i; }
+        if (m->streaming) {
+            /* streaming_prefill_inputs (session.rs:539-569) */
+            long long max_active = m->sink + m->window, sp = m->past_len, after = sp + (long long)P;
+            for (size_t i = 0; i < P; i++) pos[i] = sp + (long long)i < max_active - 1 ? sp + (long long)i : max_active - 1;
+            int ring_start = after <= max_active ? 0 : (int)((after - m->sink) % m->window);
+            int64_t *kvpos = (int64_t *)malloc((size_t)m->cfg.max_seq * sizeof(int64_t));
+            orc_streaming_kv_position(kvpos, (size_t)m->sink, (size_t)m->window, (size_t)after, (size_t)m->cfg.max_seq);
+            orc_model_forward_streaming(m, padded, pos, P, sp, after < max_active ? after : max_active, 1, m->sink,
+                                        m->window, ring_start, kvpos, logits);
+            free(kvpos);
+        } else
         orc_model_forward(m, padded, pos, P, m->past_len, m->past_len + (long long)P, 1, logits);
         m->past_len += (long long)chunk;
         if (chunk == n) result = orc_argmax_last((const char *)logits + (chunk - 1) * V * eb, V, m->cfg.dtype);
@@ -774,10 +927,10 @@ long long orc_model_generate(orc_model *m, const int64_t *prompt, size_t n_promp
     long long needed = prefill_len
         ? m->past_len + (long long)(((n_prompt + prefill_len - 1) / prefill_len) * prefill_len)
         : m->past_len + (long long)n_prompt;
-    if (max_seq < needed) return -1; /* PromptTooLong */
+    if (!m->streaming && max_seq < needed) return -1; /* PromptTooLong (not checked in streaming mode, session.rs:357) */
     long long n_new = 0;
     for (size_t i = 0; i < max_new; i++) {
-        if (max_seq < m->past_len + 1) break;
+        if (!m->streaming && max_seq < m->past_len + 1) break;
         int64_t tok;
         if (i == 0) {
             if (prefill_len) tok = orc_model_prefill(m, prompt, n_prompt, prefill_len);

@@ -155,6 +155,20 @@ int  orc_ring_phys_index(int rank, int sink, int window, int start);
 void orc_streaming_kv_position(int64_t *out, size_t sink, size_t window, size_t stream_pos,
                                size_t max_seq);
 
+/* The two cache updates and the attention with the ring inputs, as the reference's CUDA kernels apply them
+ * (kvcache_update.cuh:12-26, quantizing_kvcache_update.cuh:24-36, attention.cuh:100-200, 386-420, 495-606):
+ * the only backend that has the mechanism.  `offset` may lie past sink + window (the session passes the
+ * unbounded stream position); kv_position (NULL = keys are used as stored) is indexed by rank. */
+void orc_kv_cache_update_ring(void *cache, const void *new_kv, long long offset, size_t BH, size_t S_new,
+                              size_t max_seq, size_t D, size_t eb, int sink, int window, int start);
+void orc_quantizing_kv_cache_update_ring(int8_t *cache, void *scale, const void *new_kv, long long offset,
+                                         size_t BH, size_t S_new, size_t max_seq, size_t D, int dtype,
+                                         int sink, int window, int start);
+void orc_attention_ring(void *out, const void *q, const void *k, const void *v, const void *k_scale,
+                        const void *v_scale, long long active, size_t B, size_t Hq, size_t Hkv, size_t Sq,
+                        size_t Sk, size_t D, int is_causal, float scale, int dtype, int kv_int8, int sink,
+                        int window, int start, const void *cos_t, const void *sin_t, const int64_t *kv_position);
+
 /* ---- A12/A13: whole decoder + generate loop (crates/llm/src/decoder.rs:222-865,
  * session.rs:311-537).  Weights are int8 [N,K] + scale[N] (dtype) when quantised, or plain
  * dtype matrices when `wq` is NULL for a tensor (un-quantised checkpoints such as the tiny
@@ -204,6 +218,15 @@ void orc_model_set_past_len(orc_model *m, long long p);
  * keys [0, min(active, causal cap)); logits [S,vocab] in cfg.dtype.  Does not move past_len. */
 void orc_model_forward(orc_model *m, const int64_t *ids, const int64_t *positions, size_t S,
                        long long past_len, long long active, int is_causal, void *logits);
+/* The same run of the streaming graph (BuildOptions::streaming_kv, decoder.rs:281-347, 472-487) with the
+ * session's eight inputs (session.rs:539-597): positions = clamped query positions, past_len = the unbounded
+ * stream position, active = min(.., sink + window), ring_start, kv_position [max_seq]. */
+void orc_model_forward_streaming(orc_model *m, const int64_t *ids, const int64_t *positions, size_t S,
+                                 long long past_len, long long active, int is_causal, int sink, int window,
+                                 int ring_start, const int64_t *kv_position, void *logits);
+/* DecodeKind::LlamaStreaming { sink, window }: decode_step / prefill / generate then build the streaming
+ * inputs themselves and never report PromptTooLong (session.rs:350-366); window 0 switches it off */
+void orc_model_set_streaming(orc_model *m, int sink, int window);
 /* decode_step (session.rs:508-537): forward one token at past_len, argmax, past_len += 1 */
 int64_t orc_model_decode_step(orc_model *m, int64_t token);
 /* chunked, zero-padded prefill (session.rs:426-485); returns argmax of the last real row */

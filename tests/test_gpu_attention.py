@@ -446,3 +446,29 @@ def test_attention_streaming_with_k_rotation_inside_the_operator(g, dt, kv8, Sq,
                 w = np.exp(sc - sc.max())
                 out[b, h, 0] = (w / w.sum()) @ np.array(vv)
         assert max_err_rel_to_max(g.f32(got, dt), out) <= (4e-3 if dt == orc.BF16 else 1e-3 if dt == orc.F16 else 1e-5)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,D,L", [(2, 32, 8, 64, 2176), (4, 16, 4, 128, 1664), (1, 8, 8, 64, 4096)])
+def test_workspace_size_holds_for_every_active_length(g, B, Hq, Hkv, D, L):
+    """mynn_attention_workspace_bytes is asked once, for the cache; the number of key ranges a call is planned with
+    is not monotonic in its active length (2176 rows over 16 (sequence, kv head) pairs: 9 ranges, 2048 rows: 16), so
+    the reported size must cover every length: a workspace of exactly that size serves active = 1 .. L."""
+    import torch
+
+    dt = orc.F16
+    rng = np.random.default_rng(L)
+    q = g.to_dev(orc.to_storage(rng.standard_normal((B, Hq, 1, D)), dt), dt)
+    k = g.to_dev(orc.to_storage(rng.standard_normal((B, Hkv, L, D), dtype=np.float32), dt), dt)
+    v = g.to_dev(orc.to_storage(rng.standard_normal((B, Hkv, L, D), dtype=np.float32), dt), dt)
+    lib = g.mynn.lib()
+    need = lib.mynn_attention_workspace_bytes(B, 1, L, Hq, Hkv, D, dt, 0)
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+    out = torch.empty_like(q)
+    lengths = sorted(set(list(range(1, L + 1, 97)) + list(range(128, L + 1, 128)) + [L - 1, L]))
+    for active in lengths:
+        g.mynn.check(lib.mynn_attention_ws(out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), None, 0, 0, None, None,
+                                           D ** -0.5, 0, B, 1, active, None, L, active - 1, Hq, Hkv, D, dt, 0, ws.data_ptr(), need,
+                                           torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    # the last call (the full cache) against the library-scratch entry point
+    assert torch.equal(out, g.mynn.attention(q, k, v, D ** -0.5, False, L))

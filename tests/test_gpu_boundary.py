@@ -1,6 +1,6 @@
 """The boundary's own contracts on the GPU: the KV row a decode step writes, recovery when a shared launch's
 hand-over gives up, the additive attention mask (operator slot 3), caller-owned workspaces and prepared weights,
-the executor's own weight workspace, the streaming-KV graph up to sink + window."""
+the executor's own weight workspace, the streaming-KV graph up to sink + window (past it: test_gpu_streaming.py)."""
 import os
 
 import numpy as np
@@ -275,10 +275,6 @@ def test_streaming_kv_executor_reproduces_the_reference_ids(g, dt, prefill_len):
     ids = llm.generate_ids(golden["prompt_ids"], len(golden["expected_new_ids"]))
     assert ids == golden["expected_new_ids"]
     assert not dec.stats()["graph"]  # the ring inputs are read at launch time, as the reference's kernels do
-    # past sink + window the step is refused, with the reason
-    with pytest.raises(g.mynn.MynnError, match="sink \\+ window"):
-        llm.generate_ids([5], 64)
-    assert llm.past_len == 32
     llm.close(), dec.close()
     if pre:
         pre.close()
@@ -329,7 +325,5 @@ def test_streaming_kv_executor_steps_vs_oracle(g, dt, kv8):
     # a plain step on a streaming model, and ring inputs on a plain model, are refused
     with pytest.raises(g.mynn.MynnError):
         dec.step([1], [past], past, past + 1)
-    # past the window: refused
-    with pytest.raises(g.mynn.MynnError, match="sink \\+ window"):
-        dec.step_streaming([1], [43], 44, 44, sink, window, 0, orc.streaming_kv_position(sink, window, 44, cfg["max_seq"]))
+    # (steps past sink + window: tests/test_gpu_streaming.py)
     dec.close(), pre.close()

@@ -557,3 +557,31 @@ def test_paged_executor_rejects_what_it_has_no_kernel_for(g):
     with pytest.raises(g.mynn.MynnError):
         g.mynn.Decoder(cfg, dw, kv=kvbufs, kv_pages=pages32)
     pages32.close(), pool32.close(), pages.close(), pool.close()
+
+
+def test_paged_decode_key_range_longer_than_62_pages_is_cut(g):
+    """Batch 32 x 8 kv heads fills the CUs with one key range per (sequence, kv head); at 4096 rows in pages of 64 that
+    range would span 64 pages, more than the one register of page numbers a workgroup carries (62): the plan cuts it
+    into two ranges and merges them.  Result against the oracle and the contiguous call."""
+    import torch
+
+    dt = orc.F16
+    B, Hq, Hkv, D, L, active, P = 32, 32, 8, 64, 4096, 4001, 64
+    rng = np.random.default_rng(77)
+    q = orc.to_storage(rng.standard_normal((B, Hq, 1, D)), dt)
+    k = orc.to_storage(rng.standard_normal((B, Hkv, L, D), dtype=np.float32), dt)
+    v = orc.to_storage(rng.standard_normal((B, Hkv, L, D), dtype=np.float32), dt)
+    k[:, :, active:] = 0xFFFF
+    v[:, :, active:] = 0xFFFF
+    kp, table = scatter_to_pool(k, P, rng)
+    vp = np.full_like(kp, 0xFFFF)
+    for b in range(B):
+        for s in range(L // P):
+            vp[table[b, s]] = v[b, :, s * P:(s + 1) * P]
+    dq, dtab = g.to_dev(q, dt), torch.from_numpy(table).cuda()
+    got = g.to_host(g.mynn.attention_paged(dq, g.to_dev(kp, dt), g.to_dev(vp, dt), dtab, P, D ** -0.5, False, active))
+    del kp, vp
+    plain = g.to_host(g.mynn.attention(dq, g.to_dev(k, dt), g.to_dev(v, dt), D ** -0.5, False, active))
+    assert max_abs_rel(g.f32(got, dt), g.f32(plain, dt)) <= 1e-2
+    want = orc.attention(q[:2], k[:2], v[:2], dt, D ** -0.5, False, active)
+    assert max_abs_rel(g.f32(got[:2], dt), g.f32(want, dt)) <= 1e-2
