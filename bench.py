@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Headline benchmark: batch-1 greedy decode of a TinyLlama-1.1B-shape int8 model on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode|prefill]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode|prefill|attention|decode_batch|gemv]
 
 `--workload prefill` times the matrix-core side of the same path instead: one step = one prefill
 pass of 8 prompts x 1024 tokens through the decoder executor (roofline bound: MFMA).
@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 PROFILE_JSON = {"decode": "decode_tinyllama_int8_bs1.json", "prefill": "prefill_tinyllama_int8_8x1024.json",
                 "prefill_w8a8": "prefill_w8a8_tinyllama_8x1024.json", "decode_batch": "decode_llama3_8b_int8_bs32_ctx2048.json",
                 "decode_batch_kv8": "decode_llama3_8b_int8_bs32_ctx2048_kv_int8.json",
-                "attention": "attention_decode_b16_l4096.json"}
+                "attention": "attention_decode_b16_l4096.json", "gemv": "gemv_rotating_weight_sets.json"}
 # launch role (the executor's name for a launch) -> pattern of the mangled kernel name
 ROLE_PATTERNS = {
     "gemv_norm_gateup_swiglu": r"dequant_gemv1_kernelI\w+?Li\d+ELi\d+ELi2ELb1ELb0EE",
@@ -41,6 +41,12 @@ ROLE_PATTERNS = {
     "linear_gateup_swiglu": r"(gemm_nt_dma_kernelI\w+?Li2ELb0EE|skinny_gemm_kernel)",
     "qlinear_gateup_swiglu": r"gemm_nt_dma_kernelI\w+?Li2ELb1EE",
     "attention": r"(attn_stream_kernel|attn_prefill_kernel)",
+    # --workload gemv: the stand-alone GEMV launches and the read probe of the same geometry
+    "gemv_configs0_f32": r"dequant_gemv_kernelIffLi\d+ELi1ELi0ELb0EE",
+    "gemv_gate_up": r"dequant_gemv1_kernelI\w+?Li4ELi2ELi0ELb0ELb0EE",
+    "gemv_down": r"dequant_gemv1_kernelI\w+?Li2ELi6ELi0ELb0ELb0EE",
+    "read_probe_gate_up": r"gemv_read_probe_kernelILi4ELi2EE",
+    "read_probe_down": r"gemv_read_probe_kernelILi2ELi6EE",
 }
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16/fp16 matrix rate
 INT8_PEAK_TOPS = 5000.0    # MI355X published dense int8 matrix rate
@@ -397,6 +403,159 @@ def attention_main(args, mynn):
     print(json.dumps(out))
 
 
+def time_launches(fn, n_sets, steps, warmup):
+    """Average device time of launches fn(i) that follow one another on one stream (each waits for the one before it,
+    as the launches of a decode step do), rotating over n_sets operand sets.  fn allocates nothing and launches on the
+    current stream; the launches are captured into a hipGraph in chunks of up to 200 and the graph is replayed, so the
+    host's per-call cost is not in the figure.  Returns (us per launch, launches timed, wall seconds)."""
+    import torch
+
+    for i in range(max(warmup, 1)):  # eager first: function attributes are set outside the capture
+        fn(i % n_sets)
+    torch.cuda.synchronize()
+    chunk = max(1, min(steps, 200))
+    reps = max(1, steps // chunk)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for i in range(chunk):
+            fn((i * 7) % n_sets)
+    graph.replay()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(reps):
+        graph.replay()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return start.elapsed_time(stop) * 1e3 / (reps * chunk), reps * chunk, wall
+
+
+def read_floor(mynn, shapes, steps=400, warmup=40, pool_bytes=1 << 30):
+    """The pure-read floor of a dependent GEMV launch: mynn_gemv_read_probe (the decode GEMV's grid and loads, nothing
+    else) over matrices rotating through a 1 GiB pool, so that no launch finds its bytes in the 256 MB Infinity Cache.
+    shapes: {name: (N, K)}.  Returns {name: {bytes, us, GBs, frac}, "empty_launch_us": ..}."""
+    import torch
+
+    pool = torch.empty(pool_bytes, dtype=torch.uint8, device="cuda")
+    pool.fill_(1)
+    sink = torch.zeros(4, dtype=torch.uint8, device="cuda")
+    lib = mynn.lib()
+    cur = lambda: torch.cuda.current_stream().cuda_stream
+    out = {}
+    for name, (N, K) in shapes.items():
+        nbytes = N * K
+        stride = (nbytes + 255) // 256 * 256
+        n_sets = pool_bytes // stride
+        us, _, _ = time_launches(lambda i: mynn.check(lib.mynn_gemv_read_probe(pool.data_ptr() + i * stride, sink.data_ptr(), N, K, 0, cur())),
+                                 n_sets, steps, warmup)
+        out[name] = {"bytes": nbytes, "us": round(us, 3), "GBs": round(nbytes / us / 1e3, 1),
+                     "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "rotating_sets": n_sets}
+        if "empty_launch_us" not in out:
+            e_us, _, _ = time_launches(lambda i: mynn.check(lib.mynn_gemv_read_probe(pool.data_ptr(), sink.data_ptr(), N, K, 1, cur())), 1, steps, warmup)
+            out["empty_launch_us"] = round(e_us, 3)
+    del pool
+    torch.cuda.empty_cache()
+    return out
+
+
+def gemv_main(args, mynn):
+    """The dequant GEMV on its own (configs[0] and the metric's second clause): one step = one launch of
+    mynn_dequant_gemv, launched back to back on one stream over weight matrices that rotate through more than 256 MB
+    (the Infinity Cache), so every launch streams its int8 weights from HBM.  The headline shape is configs[0] exactly
+    (f32 x [1,2048], int8 W [5632,2048], f32 per-channel scales, f32 out); the 16-bit shapes of the TinyLlama decode
+    step and a 537 MB matrix are timed beside it, each next to the pure-read floor of the same launch geometry."""
+    import numpy as np
+    import torch
+
+    K_steps = 2000 if args.steps is None else args.steps
+    W = 100 if args.warmup is None else args.warmup
+    tdt = {"f16": torch.float16, "bf16": torch.bfloat16}[args.dtype]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(args.seed)
+    shapes = [("configs[0] f32", 5632, 2048, torch.float32), ("gate_up %s" % args.dtype, 11264, 2048, tdt),
+              ("down %s" % args.dtype, 2048, 5632, tdt), ("lm_head %s" % args.dtype, 32000, 2048, tdt),
+              ("537 MB matrix %s" % args.dtype, 262144, 2048, tdt)]
+    rows = {}
+    head = None
+    for name, N, Kd, t in shapes:
+        nbytes = N * Kd
+        n_sets = max(2, -(-(320 << 20) // nbytes))
+        Ws = [torch.randint(-127, 128, (N, Kd), generator=gen, device="cuda", dtype=torch.int8) for _ in range(n_sets)]
+        sc = (torch.rand((N,), generator=gen, device="cuda") * 9e-3 + 1e-3).to(t)
+        x = torch.randn((Kd,), generator=gen, device="cuda", dtype=torch.float32).to(t)
+        y = torch.empty((N,), dtype=t, device="cuda")
+        code = {torch.float32: mynn.F32, torch.float16: mynn.F16, torch.bfloat16: mynn.BF16}[t]
+        lib = mynn.lib()
+
+        def launch(i):
+            mynn.check(lib.mynn_dequant_gemv(y.data_ptr(), x.data_ptr(), Ws[i].data_ptr(), sc.data_ptr(), N, Kd, code, code,
+                                             torch.cuda.current_stream().cuda_stream))
+
+        us, timed, wall = time_launches(launch, n_sets, K_steps, W)
+        eb = 4 if t == torch.float32 else 2
+        alg = nbytes + N * eb + Kd * eb + N * eb  # int8 W + scales + activation + output
+        row = {"N": N, "K": Kd, "bytes_per_launch": alg, "avg_launch_us": round(us, 3), "GBs": round(alg / us / 1e3, 1),
+               "frac": round(alg / us / 1e3 / HBM_PEAK_GBS, 4), "rotating_sets": n_sets, "rotating_MB": round(n_sets * nbytes / 1e6)}
+        if head is None:
+            launch(0)
+            torch.cuda.synchronize()
+            head = (name, N, Kd, alg, us, wall, Ws[0], sc, x, y.clone(), timed)
+        rows[name] = row
+        del Ws
+        torch.cuda.empty_cache()
+    floor = read_floor(mynn, {n: (N, Kd) for n, N, Kd, _ in shapes[:4]})
+    for n in list(rows)[:4]:
+        rows[n]["read_floor_us"] = floor[n]["us"]
+        rows[n]["read_floor_frac"] = floor[n]["frac"]
+    name, N, Kd, alg, us, wall, W0, sc0, x0, y0, timed = head
+    prof = load_profile("gemv") if args.dtype == "f16" else None
+    entry = profile_entry(prof, "gemv_configs0_f32")
+    achieved = alg / us / 1e3
+    out = {
+        "metric": "dequant-GEMV HBM GB/s vs peak (configs[0]: f32 [1,2048] x int8 [5632,2048], per-channel f32 scales)",
+        "value": round(achieved, 1), "unit": "GB/s", "n_gpus": 1, "steps": timed, "warmup": W,
+        "ms_per_step": round(wall * 1e3 / timed, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32 accumulate over int8 weights (f32 activation and scales for configs[0]; %s for the decode shapes)" % args.dtype,
+        "data": "synthetic",
+        "config": {"workload": "configs[0]: DequantizeLinear->MatMul as the fused DequantMatMul, M=1, K=2048, N=5632, f32; launched "
+                               "back to back over %d weight matrices (%d MB) so each launch reads HBM" % (rows[name]["rotating_sets"], rows[name]["rotating_MB"]),
+                   "seed": args.seed, "shapes": rows, "empty_launch_us": floor["empty_launch_us"],
+                   "read_floor": "mynn_gemv_read_probe: the decode GEMV's grid and 16-byte loads with no arithmetic, same launch pattern"},
+        "roofline": {"bound": "hbm", "kernel": "dequant_gemv_kernel<f32> (configs[0])", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic_bytes(entry),
+                     "avg_launch_us_rocprof": entry["avg_us"] if entry else None,
+                     "profile": {"file": prof["file"], "commit": prof.get("commit"), "stale": prof["stale"]} if prof and entry else None,
+                     "bytes_per_launch": alg, "avg_launch_us": round(us, 3),
+                     "floor": {"bytes": floor[name]["bytes"], "us": floor[name]["us"], "frac": floor[name]["frac"]},
+                     "gate_up": rows["gate_up %s" % args.dtype], "largest_matrix": rows["537 MB matrix %s" % args.dtype]},
+    }
+    if not args.no_cpu_baseline:
+        import oracle as orc
+
+        hx, hs = x0.cpu().numpy(), sc0.cpu().numpy()
+        hW = W0.cpu().numpy()
+        want = orc.dequant_matmul(hx[None, :], hW, hs, orc.F32, orc.F32)[0]
+        got = y0.cpu().numpy()
+        exact = (hW.astype(np.float64) @ hx.astype(np.float64)) * hs.astype(np.float64)
+        out["config"]["max_rel_err_vs_f64_closed_form"] = float(np.max(np.abs(got - exact)) / np.max(np.abs(exact)))
+        out["config"]["max_rel_err_vs_oracle"] = float(np.max(np.abs(got - want)) / np.max(np.abs(want)))
+        # the C port on the same shape, rotating over host copies of > 256 MB as well; about 10 s of CPU work
+        copies = [hW] + [np.ascontiguousarray(np.roll(hW, i + 1, axis=0)) for i in range(31)]
+        orc.dequant_matmul(hx[None, :], copies[1], hs, orc.F32, orc.F32)
+        n, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < 10.0:
+            orc.dequant_matmul(hx[None, :], copies[n % len(copies)], hs, orc.F32, orc.F32)
+            n += 1
+        cpu = (time.perf_counter() - t0) / n
+        out["cpu_baseline"] = {"value": round(alg / cpu / 1e9, 2), "unit": "GB/s", "cores": orc.get_threads(), "kind": "port",
+                               "sample": "%d calls of the same configs[0] GEMV (10 s), C port of the reference CPU backend "
+                                         "(OpenMP over N, f32), rotating over 32 host copies of W" % n}
+    print(json.dumps(out))
+
+
+
 LLAMA3_8B = dict(n_layers=32, hidden=4096, n_heads=32, n_kv_heads=8, head_dim=128, ffn=14336, vocab=128256,
                  max_seq=2304, eps=1e-5, rope_theta=500000.0)
 
@@ -556,7 +715,7 @@ def short_prefill(mynn, cfg, weights, seed):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--workload", choices=["decode", "prefill", "attention", "decode_batch"], default="decode")
+    ap.add_argument("--workload", choices=["decode", "prefill", "attention", "decode_batch", "gemv"], default="decode")
     ap.add_argument("--steps", type=int, default=None, help="default 256 (decode) / 5 (prefill)")
     ap.add_argument("--warmup", type=int, default=None, help="default 16 (decode) / 2 (prefill)")
     ap.add_argument("--dtype", choices=["f16", "bf16"], default="f16")
@@ -614,6 +773,8 @@ def main():
         return attention_main(args, mynn)
     if args.workload == "decode_batch":
         return decode_batch_main(args, mynn)
+    if args.workload == "gemv":
+        return gemv_main(args, mynn)
     K = 256 if args.steps is None else args.steps
     W = 16 if args.warmup is None else args.warmup
     assert PROMPT_LEN + max(K, W) <= cfg["max_seq"], "steps/warmup do not fit max_seq %d" % cfg["max_seq"]
@@ -721,6 +882,14 @@ def main():
         "roofline": roof,
     }
     dec.close()
+    # the pure-read floor of the two dequant-GEMV launches (same grid and loads, no arithmetic, dependent launches over
+    # rotating matrices): what a launch of that geometry needs just to pull its weight bytes in
+    H, F = cfg["hidden"], cfg["ffn"]
+    fl = read_floor(mynn, {"gateup": (2 * F, H), "down": (H, F)})
+    roof["floor"] = {"gateup": {k: fl["gateup"][k] for k in ("bytes", "us", "frac")},
+                     "down": {k: fl["down"][k] for k in ("bytes", "us", "frac")}, "empty_launch_us": fl["empty_launch_us"],
+                     "what": "mynn_gemv_read_probe: weight bytes of one launch / its average duration, 400 dependent launches "
+                             "over matrices rotating through 1 GiB"}
     if not args.no_prefill and not (args.kv_int8 or args.w8a8 or args.unfused):
         out["config"]["prefill"] = short_prefill(mynn, cfg, weights, args.seed)
 

@@ -494,6 +494,44 @@ static int gemv1_dispatch(const GemvParams &p, hipStream_t s) {
     return launch_gemv<T, T, 2, 1, EPI, NORM>(p, s);
 }
 
+// ---- measurement aid: the weight stream of dequant_gemv1_kernel and nothing else.  Same grid, same row groups per
+// wave, the same R x NC non-temporal 16-byte loads per lane and group, no activation, no arithmetic beyond an xor
+// that keeps the loads alive, no store.  Launched like the GEMV (dependent launches on one stream, a different
+// matrix each time) it gives the time a launch of this geometry needs just to pull its bytes in: the floor the
+// GEMV's duration is judged against.
+template <int R, int NC>
+__global__ __launch_bounds__(kGemvThreads) void gemv_read_probe_kernel(const int8_t *wq, uint32_t *sink, int N, int K, int groups,
+                                                                         int total_waves) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nchunks = K >> 4;
+    uint32_t acc = 0;
+    for (int g = blockIdx.x * kGemvWaves + wave; g < groups; g += total_waves) {
+        U4 w[R][NC];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int row = g * R + r < N ? g * R + r : N - 1;
+            const U4 *wrow = (const U4 *)(wq + (size_t)row * K);
+#pragma unroll
+            for (int j = 0; j < NC; j++) w[r][j] = __builtin_nontemporal_load(&wrow[min(lane + j * kWave, nchunks - 1)]);
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int j = 0; j < NC; j++) acc ^= w[r][j].x ^ w[r][j].y ^ w[r][j].z ^ w[r][j].w;
+    }
+    if (acc == 0x9E3779B9u && sink) sink[0] = acc;  // (never true for the patterns the benchmark fills in; keeps the loads)
+}
+template <int R, int NC>
+static int launch_read_probe(const int8_t *wq, uint32_t *sink, int N, int K, bool empty, hipStream_t s) {
+    const int groups = (N + R - 1) / R;
+    const int max_waves = 256 * 16;
+    const int passes = (groups + max_waves - 1) / max_waves;
+    int waves = (groups + passes - 1) / passes;
+    const int blocks = (waves + kGemvWaves - 1) / kGemvWaves;
+    waves = blocks * kGemvWaves;
+    MYNN_LAUNCH((gemv_read_probe_kernel<R, NC>), dim3(blocks), dim3(kGemvThreads), 0, s, wq, sink, N, K, empty ? 0 : groups, waves);
+    return launch_status("gemv_read_probe_kernel");
+}
+
 template <typename T>
 int gemv_norm(void *out, const void *x, const void *norm_w, float eps, const int8_t *wq, const void *scale,
               int N, int K, hipStream_t s) {
@@ -573,4 +611,19 @@ extern "C" int mynn_dequant_gemv(void *out, const void *act, const int8_t *wq, c
     MYNN_REQUIRE(mynn::aligned16(wq), MYNN_ERR_INVALID, "dequant_gemv: wq must be 16-byte aligned");
     MYNN_REQUIRE((size_t)K * sizeof(float) <= 64 * 1024, MYNN_ERR_UNSUPPORTED, "dequant_gemv: K=%d exceeds the LDS stage", K);
     return mynn::dequant_gemv_dispatch(out, act, wq, scale, 1, N, K, act_dtype, out_dtype, mynn::as_stream(s));
+}
+
+extern "C" int mynn_gemv_read_probe(const int8_t *wq, void *sink, int N, int K, int empty, mynn_stream s) {
+    using namespace mynn;
+    MYNN_REQUIRE(wq && N > 0 && K > 0 && K % 16 == 0 && aligned16(wq), MYNN_ERR_INVALID, "gemv_read_probe: N=%d K=%d", N, K);
+    const int nc = (K + 1023) / 1024;
+    MYNN_REQUIRE(nc <= 14, MYNN_ERR_UNSUPPORTED, "gemv_read_probe: K=%d (the decode GEMV's row limit is 14336)", K);
+    hipStream_t st = as_stream(s);
+    // the geometry of gemv1_dispatch: four rows per wave for K <= 2048, two beyond
+    if (nc <= 1) return launch_read_probe<4, 1>(wq, (uint32_t *)sink, N, K, empty != 0, st);
+    if (nc <= 2) return launch_read_probe<4, 2>(wq, (uint32_t *)sink, N, K, empty != 0, st);
+    if (nc <= 4) return launch_read_probe<2, 4>(wq, (uint32_t *)sink, N, K, empty != 0, st);
+    if (nc <= 6) return launch_read_probe<2, 6>(wq, (uint32_t *)sink, N, K, empty != 0, st);
+    if (nc <= 8) return launch_read_probe<2, 8>(wq, (uint32_t *)sink, N, K, empty != 0, st);
+    return launch_read_probe<2, 14>(wq, (uint32_t *)sink, N, K, empty != 0, st);
 }

@@ -5,12 +5,14 @@
 // bf16 (and any other T): the row as f32 [K]; a weight byte is converted to f32 and multiplied with an FMA (two
 // vector operations per weight).
 // fp16: the row as fp16, the first and the second 8 elements of every 16-element chunk in two separate arrays (so that
-// the lanes of a wave read consecutive 16-byte words), followed by the f32 sum of every 8-element piece.  A weight
-// byte b, as b ^ 0x80 under an 0x64 high byte, IS the fp16 number 1152 + b: one byte permute makes two of them, and
-// v_dot2_f32_f16 multiplies two by two activations with f32 accumulation -- one vector operation per weight.  Every
-// product is exact in f32; the sum carries 1152 * (sum of the lane's activations), which is subtracted once per row
-// before the lanes meet (the f32 rounding of the sum grows with that term: about 1e-6 of the result for normalised
-// activations, two orders below the fp16 rounding of the stored output).
+// the lanes of a wave read consecutive 16-byte words), followed by one f32 bias term for every 8-element piece.  A
+// weight byte b, as b ^ 0x80 under an 0x64 high byte, IS the fp16 number 1152 + b, and as b ^ 0x7F under an 0xE4 high
+// byte the fp16 number b - 1151: one xor per four weights and one byte permute per two make an (even, odd) pair
+// (1152 + b0, b1 - 1151), and v_dot2_f32_f16 multiplies it with two activations with f32 accumulation -- one vector
+// operation per weight.  Every product is exact in f32.  The sums carry 1152 * (even activations) - 1151 * (odd
+// activations), which is subtracted once per row before the lanes meet; the opposite signs matter: for activations
+// with a non-zero mean (SwiGLU outputs, attention outputs) the two halves cancel inside every dot2, so the running
+// sum stays near the size of the result instead of growing to 1152 * K/64 * mean and rounding at that magnitude.
 // Semantics either way: out[n] = T(scale[n] * sum_k act[k] * wq[n,k]), scale after the f32 sum
 // (dequant_gemv.cuh:12-59).
 #pragma once
@@ -34,7 +36,9 @@ template <typename T> __device__ inline void gemv_stage_piece(float *lds, int K,
         const U4 v = U4{pack2<T>(f[0], f[1]), pack2<T>(f[2], f[3]), pack2<T>(f[4], f[5]), pack2<T>(f[6], f[7])};
         U4 *half = (U4 *)lds + (pc & 1) * (K >> 4);  // [2][K / 16] words of 16 bytes
         half[pc >> 1] = v;
-        lds[(K >> 1) + pc] = ((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7]));
+        // 1152 * (f0 + f2 + f4 + f6) - 1151 * (f1 + f3 + f5 + f7), as 1152 * (even - odd) + odd
+        const float ev = (f[0] + f[2]) + (f[4] + f[6]), od = (f[1] + f[3]) + (f[5] + f[7]);
+        lds[(K >> 1) + pc] = fmaf(1152.f, ev - od, od);
     } else {
         float4 *dst = (float4 *)(lds + pc * 8);
         dst[0] = float4{f[0], f[1], f[2], f[3]};
@@ -42,14 +46,16 @@ template <typename T> __device__ inline void gemv_stage_piece(float *lds, int K,
     }
 }
 
-// acc += sum over 16 weights of (1152 + w) * a   (w: 16 int8 of one 128-bit load, a0 / a1: the 16 fp16 activations)
+// acc += sum over 16 weights of (1152 + w) * a (even elements) and (w - 1151) * a (odd elements)
+// (w: 16 int8 of one 128-bit load, a0 / a1: the 16 fp16 activations)
 __device__ inline float gemv_dot16_biased(const U4 &w, const U4 &a0, const U4 &a1, float acc) {
-    const uint32_t x[4] = {w.x ^ 0x80808080u, w.y ^ 0x80808080u, w.z ^ 0x80808080u, w.w ^ 0x80808080u};
+    const uint32_t x[4] = {w.x ^ 0x7F807F80u, w.y ^ 0x7F807F80u, w.z ^ 0x7F807F80u, w.w ^ 0x7F807F80u};
     const uint32_t a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const uint32_t lo = __builtin_amdgcn_perm(0x64646464u, x[i], 0x04010400u);
-        const uint32_t hi = __builtin_amdgcn_perm(0x64646464u, x[i], 0x04030402u);
+        // high bytes: 0x64 for the even element of a pair, 0xE4 for the odd one (bytes 0 and 1 of the constant)
+        const uint32_t lo = __builtin_amdgcn_perm(0x6464E464u, x[i], 0x05010400u);
+        const uint32_t hi = __builtin_amdgcn_perm(0x6464E464u, x[i], 0x05030402u);
         acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, a[2 * i]), __builtin_bit_cast(h2_t, lo), acc, false);
         acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, a[2 * i + 1]), __builtin_bit_cast(h2_t, hi), acc, false);
     }
@@ -65,14 +71,14 @@ __device__ __forceinline__ void gemv_rows_dot(const float *lds, int K, int lane,
     if constexpr (kGemvDot2<T>) {
         const U4 *lo = (const U4 *)lds, *hi = lo + nchunks;
         const float2 *psum = (const float2 *)(lds + (K >> 1));
-        float asum = 0.f;
+        float bias = 0.f;
 #pragma unroll
         for (int j = 0; j < NC; j++) {
             const int c = lane + j * kWave;
             if (c < nchunks) {
                 const U4 a0 = lo[c], a1 = hi[c];
                 const float2 s = psum[c];
-                asum += s.x + s.y;
+                bias += s.x + s.y;
 #pragma unroll
                 for (int r = 0; r < R; r++) {
                     pin(w[r][j]);
@@ -81,7 +87,7 @@ __device__ __forceinline__ void gemv_rows_dot(const float *lds, int K, int lane,
             }
         }
 #pragma unroll
-        for (int r = 0; r < R; r++) acc[r] = fmaf(-1152.f, asum, acc[r]);
+        for (int r = 0; r < R; r++) acc[r] -= bias;
     } else {
 #pragma unroll
         for (int j = 0; j < NC; j++) {

@@ -51,6 +51,33 @@ def test_dequant_gemv_vs_oracle(g, dt, N, K):
         assert np.mean(got == want) > 0.95
 
 
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+@pytest.mark.parametrize("N,K", [(2048, 5632), (4096, 14336), (11264, 2048)])
+@pytest.mark.parametrize("mean", [0.0, 0.5, 1.0, 3.0])
+def test_dequant_gemv_accumulation_noise_with_non_zero_mean_activations(g, dt, N, K, mean):
+    """The fp16 decode GEMV multiplies biased weights (1152 + w for even elements, w - 1151 for odd ones) and takes the
+    bias back out of the f32 sums; activations with a non-zero mean (SwiGLU outputs into down_proj, attention outputs
+    into o_proj, long rows) must not turn that into cancellation error.  With a power-of-two scale the stored value is
+    the f32 sum rounded once, so the distance to the exact sum is the accumulation noise plus one 16-bit rounding: the
+    noise stays below 1/16 of half a 16-bit spacing of the row's largest output, for every mean (the plain
+    convert-and-FMA path of bf16 models is held to the same bound)."""
+    rng = np.random.default_rng(K + int(mean * 10))
+    W = rng.integers(-127, 128, (N, K)).astype(np.int8)
+    x = orc.to_storage(rng.standard_normal(K) * 0.5 + mean, dt)
+    sc = orc.to_storage(np.full(N, 2.0 ** -7), dt)
+    exact = (W.astype(np.float64) @ g.f32(x, dt).astype(np.float64)) * 2.0 ** -7
+    got = g.f32(g.to_host(g.mynn.dequant_gemv(g.to_dev(x, dt), g.to_dev(W), g.to_dev(sc, dt))), dt).astype(np.float64)
+    mant = 10 if dt == orc.F16 else 7
+    half_ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(exact), 1e-30))) - mant - 1)
+    noise = np.maximum(np.abs(got - exact) - half_ulp, 0.0)  # what is left after one correct rounding
+    top = float(np.max(np.abs(exact)))
+    assert noise.max() <= 2.0 ** -(mant + 2 + 4) * top, (noise.max() / top, mean)
+    # the large outputs (the ones a greedy choice is made among) are the correctly rounded sums
+    big = np.abs(exact) >= top / 4
+    ideal = g.f32(orc.to_storage(exact.astype(np.float32), dt), dt)
+    assert np.mean(got[big] == ideal[big]) >= 0.98
+
+
 def test_dequant_gemv_mixed_types_cfg1(g):
     """First benchmark config: f32 x, int8 W [5632,2048], f32 scale, f32 out."""
     rng = np.random.default_rng(1)
