@@ -722,7 +722,7 @@ def main():
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-prefill", action="store_true", help="decode: leave the short prefill run (config.prefill) out")
-    ap.add_argument("--cpu-steps", type=int, default=96)
+    ap.add_argument("--cpu-steps", type=int, default=96, help="decode: generated positions the CPU port is timed (and tokens checked) on")
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="first run one 256 MiB device-to-device copy (a kernel of known traffic, for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
@@ -897,43 +897,51 @@ def main():
         import oracle as orc
 
         hw = to_host_weights(weights)
-        ref = orc.Model(dict(cfg), hw)
-        ref.set_options(quant_kv_cache=args.kv_int8, quantize_activations=args.w8a8)
-        n_cpu = args.cpu_steps
-        ref.past_len = 0
+        # The oracle under three f32 summation orders (the reference leaves the order open), each with its own KV
+        # cache, on the GPU's token stream: the prompt, then the first n_cpu generated positions -- the same contexts
+        # the timed GPU steps start with.  The first order's forward calls at those contexts are the timed CPU sample.
+        n_cpu = min(args.cpu_steps, K)
+        ref = orc.SummationOrders(dict(cfg), hw, quant_kv_cache=args.kv_int8, quantize_activations=args.w8a8)
         stream = prompt + generated
-        # bounded sample: the first n_cpu decode steps of the same token stream
-        t0 = time.perf_counter()
-        cpu_choice, cpu_logits = [], []
-        for i in range(n_cpu):
-            logits = ref.forward([stream[i]], [i], i, i + 1, False)[0]
-            cpu_choice.append(orc.argmax_last(logits, dt))
-            cpu_logits.append(logits)
-        cpu_elapsed = time.perf_counter() - t0
+        gpu_choice = prompt_choice + generated[1:]  # the GPU's greedy token after each position of the stream
+        counts = {"identical": 0, "order_dependent": 0, "within_order_noise": 0, "different": 0}
+        notes = []
+        for i in range(PROMPT_LEN + n_cpu):
+            if i == PROMPT_LEN:
+                ref.seconds_first = 0.0
+            rows = [l[0] for l in ref.forward([stream[i]], [i], i, i + 1, False)]
+            if i >= len(gpu_choice):
+                continue
+            verdict, choices = ref.judge(rows, gpu_choice[i])
+            if verdict != "identical":
+                lf = orc.to_f32(rows[0], dt)
+                gap, noise = float(lf[choices[0]] - lf[gpu_choice[i]]), ref.order_noise(rows)
+                spacing = 2.0 ** (-11 if dt == orc.F16 else -8) * abs(float(lf[choices[0]]))
+                notes.append({"step": i, "oracle_by_order": sorted(set(choices)), "orders_tried": len(choices), "gpu": gpu_choice[i],
+                              "verdict": verdict, "oracle_gap_in_16bit_spacings": round(gap / spacing, 2),
+                              "largest_logit_shift_between_orders_in_16bit_spacings": round(noise / spacing, 2)})
+            counts[verdict] += 1
+        cpu_elapsed = ref.seconds_first
+        ref.close()
         out["cpu_baseline"] = {"value": round(n_cpu / cpu_elapsed, 3), "unit": "tok/s", "cores": orc.get_threads(),
                                "kind": "port",
-                               "sample": "first %d decode steps (contexts 0..%d) of the same model and token stream, "
-                                         "C port of the reference CPU backend, OpenMP over N" % (n_cpu, n_cpu - 1)}
-        # the same steps ran on the GPU: the greedy choice after each of them, both sides on the same context
-        gpu_choice = (prompt_choice + generated[1:])[:n_cpu]
-        same = sum(int(a == b) for a, b in zip(cpu_choice, gpu_choice))
-        # a disagreement is a tie when the oracle's own logits of the two tokens are a few fp16 spacings apart (two
-        # correct f32 summation orders round such a pair differently)
-        ties = []
-        for i, (a, b) in enumerate(zip(cpu_choice, gpu_choice)):
-            if a != b:
-                lf = orc.to_f32(cpu_logits[i], dt)
-                ties.append({"step": i, "oracle": a, "gpu": b,
-                             "oracle_gap_in_16bit_spacings": round(float(lf[a] - lf[b]) / (2.0 ** (-11 if dt == orc.F16 else -8) * abs(float(lf[a]))), 2)})
-        out["config"]["tokens_identical_to_oracle"] = same == n_cpu
-        # (with int8 activations a one-spacing difference of an activation becomes another int8 code: the bound is the
-        # 2e-2 of the top logit that the parity tests allow that path, in spacings)
-        tie_bound = 41.0 if args.w8a8 else 8.0
-        out["config"]["tokens_identical_or_tied"] = all(0 <= t["oracle_gap_in_16bit_spacings"] <= tie_bound for t in ties)
-        out["config"]["tokens_checked"] = {"steps": n_cpu, "identical": same, "disagreements": ties,
-                                           "what": "greedy choice after each of the first %d positions of the stream, oracle and "
-                                                   "GPU on the same context; a disagreement counts as a tie when the oracle's own "
-                                                   "logits of the two tokens are at most %g spacings of the 16-bit type apart" % (n_cpu, tie_bound)}
+                               "sample": "%d decode steps at contexts %d..%d (the contexts the timed GPU steps start with) of the same "
+                                         "model and token stream, C port of the reference CPU backend, OpenMP over N"
+                                         % (n_cpu, PROMPT_LEN, PROMPT_LEN + n_cpu - 1)}
+        checked = sum(counts.values())
+        out["config"]["tokens_identical_to_oracle"] = counts["identical"] == checked
+        out["config"]["tokens_identical_or_order_dependent"] = counts["different"] + counts["within_order_noise"] == 0
+        out["config"]["tokens_checked"] = {"steps": checked, "identical": counts["identical"], "order_dependent": counts["order_dependent"],
+                                           "within_order_noise": counts["within_order_noise"], "different": counts["different"], "summation_orders": {"whole_stream": list(ref.lanes), "disputed_steps": list(ref.step_lanes)},
+                                           "disagreements": notes,
+                                           "what": "greedy choice after each of the first %d positions of the stream (prompt and generated), "
+                                                   "oracle and GPU on the same context; the oracle follows the stream under four f32 summation "
+                                                   "orders (16 / 8 / 32 / 64 partial sums, a KV cache each) and repeats a disputed step under "
+                                                   "1 / 2 / 4; a GPU token that is not the first order's choice counts as order_dependent only "
+                                                   "if it is the choice under another order or the orders disagree among themselves; of the rest, "
+                                                   "within_order_noise where the oracle's own gap between the two tokens is below twice the "
+                                                   "largest shift any logit of that step shows between the oracle's orders, different "
+                                                   "otherwise" % checked}
         if args.check_tokens:
             n = min(args.check_tokens, K)
             ref2 = orc.Model(dict(cfg), hw)

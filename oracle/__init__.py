@@ -566,3 +566,88 @@ class Model:
         vs = np.ctypeslib.as_array(C.cast(_lib.orc_model_v_scale(self._h, layer), C.POINTER(typ)), (n,))
         shape = (self.cfg.n_kv_heads, self.cfg.max_seq)
         return ks.reshape(shape).copy(), vs.reshape(shape).copy()
+
+
+class SummationOrders:
+    """The same decoder under several f32 summation orders (orc_set_lanes: n interleaved partial sums + a pairwise
+    tree; 16 is the default, 1 = sequential), stepped together on one token stream.  The reference leaves the order of
+    its f32 sums open (LLVM fast-math vectorisation, BLAS), so where two orders pick different greedy tokens the
+    reference's own choice is not determined either; that is the only kind of disagreement a checked implementation
+    may show.  `lanes`: orders that run the whole stream, one Model with its own KV cache each (the effect of an order
+    on earlier cache rows is then part of the sample); `step_lanes`: further orders tried only at a disputed position,
+    as a re-evaluation of that one step over each of those caches."""
+
+    def __init__(self, cfg, weights, lanes=(16, 8, 32, 64), step_lanes=(1, 2, 4), quant_kv_cache=False,
+                 quantize_activations=False, gemm_mode=None):
+        self.lanes = tuple(lanes)
+        self.step_lanes = tuple(step_lanes)
+        self.models = []
+        for _ in self.lanes:
+            m = Model(dict(cfg), weights)
+            if quant_kv_cache or quantize_activations:
+                m.set_options(quant_kv_cache=quant_kv_cache, quantize_activations=quantize_activations)
+            if gemm_mode is not None:
+                m.set_gemm_mode(gemm_mode)
+            self.models.append(m)
+        self.dt = cfg["dtype"]
+        self.seconds_first = 0.0  # wall time of the first order's forward calls (the CPU baseline times that one)
+        self._last = None
+
+    def forward(self, ids, positions, past_len, active, is_causal):
+        """[logits of order 0, logits of order 1, ...] for the orders that follow the whole stream"""
+        import time
+
+        self._last = (ids, positions, past_len, active, is_causal)
+        out = []
+        try:
+            for i, (n, m) in enumerate(zip(self.lanes, self.models)):
+                set_lanes(n)
+                t0 = time.perf_counter()
+                out.append(m.forward(ids, positions, past_len, active, is_causal))
+                if i == 0:
+                    self.seconds_first += time.perf_counter() - t0
+        finally:
+            set_lanes(16)
+        return out
+
+    def judge(self, logits_rows, token):
+        """logits_rows: the last row of each order's logits of the forward call just made.  Returns (verdict, choices):
+        "identical" -- `token` is the first order's greedy choice;
+        "order_dependent" -- it is the choice under another order, or the orders disagree among themselves (the
+            oracle is undecided at this position), the step orders included;
+        "within_order_noise" -- no order tried flips the choice, but the first order's own gap between its choice and
+            `token` is below twice the largest shift any single logit of this step shows between the oracle's orders
+            (order_noise): the oracle's arithmetic does not separate the two tokens;
+        "different" otherwise.  choices: the greedy token of every order tried."""
+        choices = [argmax_last(r, self.dt) for r in logits_rows]
+        if token == choices[0]:
+            return "identical", choices
+        if token in choices or len(set(choices)) > 1:
+            return "order_dependent", choices
+        # undisputed so far: this one step again under the remaining orders, over each cache (the cache row the step
+        # writes is put back by repeating the step under the cache's own order)
+        try:
+            for n_own, m in zip(self.lanes, self.models):
+                for n in self.step_lanes:
+                    set_lanes(n)
+                    choices.append(argmax_last(m.forward(*self._last)[-1], self.dt))
+                set_lanes(n_own)
+                m.forward(*self._last)
+        finally:
+            set_lanes(16)
+        if token in choices or len(set(choices)) > 1:
+            return "order_dependent", choices
+        lf = to_f32(logits_rows[0], self.dt)
+        if float(lf[choices[0]] - lf[token]) <= 2.0 * self.order_noise(logits_rows):
+            return "within_order_noise", choices
+        return "different", choices
+
+    def order_noise(self, logits_rows):
+        """The largest shift any single logit shows between the first order and another whole-stream order at this
+        step (f32): two logits closer than twice that are not separated by the oracle's own arithmetic."""
+        base = to_f32(logits_rows[0], self.dt)
+        return max(float(np.max(np.abs(to_f32(r, self.dt) - base))) for r in logits_rows[1:])
+
+    def close(self):
+        for m in self.models:
+            m.close()

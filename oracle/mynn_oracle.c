@@ -139,6 +139,15 @@ static float dot_f32_i8(const float *a, const int8_t *w, size_t K) {
     if (L == 16) {
         for (; k + 16 <= K; k += 16)
             for (int j = 0; j < 16; j++) acc[j] = acc[j] + a[k + j] * (float)w[k + j];
+    } else if (L == 8) {  /* (constant trip counts: the compiler vectorises these; the sums are those of the generic loop) */
+        for (; k + 8 <= K; k += 8)
+            for (int j = 0; j < 8; j++) acc[j] = acc[j] + a[k + j] * (float)w[k + j];
+    } else if (L == 32) {
+        for (; k + 32 <= K; k += 32)
+            for (int j = 0; j < 32; j++) acc[j] = acc[j] + a[k + j] * (float)w[k + j];
+    } else if (L == 64) {
+        for (; k + 64 <= K; k += 64)
+            for (int j = 0; j < 64; j++) acc[j] = acc[j] + a[k + j] * (float)w[k + j];
     } else {
         for (; k + (size_t)L <= K; k += (size_t)L)
             for (int j = 0; j < L; j++) acc[j] = acc[j] + a[k + j] * (float)w[k + j];
@@ -154,6 +163,15 @@ static float dot_f32_f32(const float *a, const float *b, size_t K) {
     if (L == 16) {
         for (; k + 16 <= K; k += 16)
             for (int j = 0; j < 16; j++) acc[j] = acc[j] + a[k + j] * b[k + j];
+    } else if (L == 8) {
+        for (; k + 8 <= K; k += 8)
+            for (int j = 0; j < 8; j++) acc[j] = acc[j] + a[k + j] * b[k + j];
+    } else if (L == 32) {
+        for (; k + 32 <= K; k += 32)
+            for (int j = 0; j < 32; j++) acc[j] = acc[j] + a[k + j] * b[k + j];
+    } else if (L == 64) {
+        for (; k + 64 <= K; k += 64)
+            for (int j = 0; j < 64; j++) acc[j] = acc[j] + a[k + j] * b[k + j];
     } else {
         for (; k + (size_t)L <= K; k += (size_t)L)
             for (int j = 0; j < L; j++) acc[j] = acc[j] + a[k + j] * b[k + j];

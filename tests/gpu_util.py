@@ -44,30 +44,45 @@ def f32(a, dt):
     return orc.to_f32(a, dt)
 
 
-def greedy_compare(ref, dec, prompt, n_new, dt):
+def greedy_compare(cfg, weights, dec, prompt, n_new, dt, **oracle_options):
     """Runs the GPU decoder greedily (prompt fed token by token, as LlmSession does without a
     prefill session) and the oracle on the SAME token stream (teacher-forced with the GPU's
-    choices, so both always see the same context).  Returns (gpu_ids, oracle_ids, near_ties):
-    oracle_ids[i] is the oracle's greedy choice at step i; near_ties lists the steps where the two
-    differ together with the oracle's logit gap between its choice and the GPU's, in units of the
-    16-bit spacing at the top logit."""
-    ulp = {orc.F32: 2.0 ** -23, orc.BF16: 2.0 ** -8, orc.F16: 2.0 ** -11}[dt]
-    gpu_ids, ref_ids, near = [], [], []
+    choices, so both always see the same context), the oracle under three f32 summation orders
+    (oracle.SummationOrders).  Returns (gpu_ids, oracle_ids, undecided, different):
+    oracle_ids[i] is the first order's greedy choice at step i; the two lists hold the steps where
+    the GPU's token is not that choice -- undecided where the oracle's own arithmetic does not
+    separate the two tokens (the choice flips under another summation order, or the gap is inside
+    the shifts the orders show among themselves: SummationOrders.judge), different otherwise (a
+    failure)."""
+    ref = orc.SummationOrders(cfg, weights, **oracle_options)
+    gpu_ids, ref_ids, undecided, different = [], [], [], []
     stream = list(prompt)
     pos = 0
-    tok_gpu = None
     while len(gpu_ids) < n_new:
         t = stream[pos]
-        logits = ref.forward([t], [pos], pos, pos + 1, False)[0]
+        rows = [l[0] for l in ref.forward([t], [pos], pos, pos + 1, False)]
         nxt, _ = dec.step([t], [pos], pos, pos + 1)
         pos += 1
         if pos >= len(prompt):
-            lf = orc.to_f32(logits, dt)
-            r = orc.argmax_last(logits, dt)
+            verdict, choices = ref.judge(rows, nxt[0])
             gpu_ids.append(nxt[0])
-            ref_ids.append(r)
-            if r != nxt[0]:
-                gap = float(lf[r] - lf[nxt[0]])
-                near.append((len(gpu_ids) - 1, gap / (ulp * max(abs(float(lf[r])), 1e-30))))
+            ref_ids.append(choices[0])
+            if verdict in ("order_dependent", "within_order_noise"):
+                undecided.append((len(gpu_ids) - 1, verdict, sorted(set(choices)), nxt[0]))
+            elif verdict == "different":
+                different.append((len(gpu_ids) - 1, sorted(set(choices)), nxt[0]))
             stream.append(nxt[0])
-    return gpu_ids, ref_ids, near
+    ref.close()
+    return gpu_ids, ref_ids, undecided, different
+
+
+def both_acceptable(cfg, weights, stream, candidates, dt, **oracle_options):
+    """Two library paths part at the token after `stream`: every candidate must be a choice the oracle can make there
+    -- its greedy token under one of the summation orders, or the orders disagree among themselves."""
+    ref = orc.SummationOrders(cfg, weights, **oracle_options)
+    rows = None
+    for i, t in enumerate(stream):
+        rows = [l[0] for l in ref.forward([t], [i], i, i + 1, False)]
+    verdicts = [ref.judge(rows, c) for c in candidates]
+    ref.close()
+    return all(v != "different" for v, _ in verdicts), verdicts

@@ -45,11 +45,13 @@ def test_config2_full_greedy_decode_128_prompt_256_generated_vs_oracle(g, bench,
     """configs[2] at full length: 128 prompt tokens through the decode path, then 256 greedy tokens, through
     LlmSession and through the device-resident loop the benchmark times (the same ids).  The oracle follows the
     GPU's token stream step by step (so both always see the same context) and its own greedy choice is compared at
-    each of the 256 generated positions.  Two correct f32 summation orders differ in the last bit of a logit now
-    and then, and with random-init weights the two best logits are sometimes closer than that: every disagreement
-    must be such a tie (the oracle's own gap between the two tokens at most 8 fp16 spacings of its top logit), and
-    there may be at most 3 of them in 256 (measured on MI355X, seed 1234: 2 of 256, at generated positions 149 and
-    186, gaps of 3.5 and 1.2 spacings).  Up to the first one the ids are those of the oracle generating freely."""
+    each of the 256 generated positions.  The reference leaves the order of its f32 sums open, and with random-init
+    weights the two best logits are sometimes closer than two orders differ: the oracle therefore runs under three
+    summation orders (16 lanes + tree, sequential, 64 lanes; one KV cache each), and a token that is not the first
+    order's choice is accepted only where the oracle's own arithmetic does not separate the two tokens: the GPU's
+    token is the choice under another order, the orders disagree among themselves, or the oracle's gap between the
+    two is inside the shifts its orders show among themselves at that step (oracle.SummationOrders.judge) -- anything
+    else fails.  Measured on MI355X, seed 1234: 2 of 256 (positions 149 and 186), both flipped by another order."""
     cfg, weights, host = tinyllama
     dt = cfg["dtype"]
     prompt = np.random.default_rng(1234).integers(0, cfg["vocab"], bench.PROMPT_LEN).tolist()
@@ -66,21 +68,24 @@ def test_config2_full_greedy_decode_128_prompt_256_generated_vs_oracle(g, bench,
         first_tok, _ = dec.step([t], [i], i, i + 1)
     assert [first_tok[0]] + dec.decode_loop(first_tok[0], len(prompt), n_new - 1) == got
     dec.close()
-    ref = orc.Model(dict(cfg), host)
+    ref = orc.SummationOrders(cfg, host)
     stream = prompt + got[:-1]
-    ties = []
+    undecided, wrong = [], []
     for i, t in enumerate(stream):
-        logits = ref.forward([t], [i], i, i + 1, False)[0]
+        rows = [l[0] for l in ref.forward([t], [i], i, i + 1, False)]
         j = i - (len(prompt) - 1)
         if j < 0:
             continue
-        want = orc.argmax_last(logits, dt)
-        if want != got[j]:
-            lf = orc.to_f32(logits, dt)
-            ties.append((j, want, got[j], float(lf[want] - lf[got[j]]) / (2.0 ** -11 * abs(float(lf[want])))))
-    print("config2: %d of %d generated tokens differ from the oracle's choice: %s" % (len(ties), n_new, ties))
-    assert all(0 <= gap <= 8.0 for _, _, _, gap in ties), ties
-    assert len(ties) <= 3, ties
+        verdict, choices = ref.judge(rows, got[j])
+        if verdict != "identical":
+            lf = orc.to_f32(rows[0], dt)
+            gap = float(lf[choices[0]] - lf[got[j]]) / (2.0 ** -11 * abs(float(lf[choices[0]])))
+            (wrong if verdict == "different" else undecided).append((j, verdict, sorted(set(choices)), got[j], round(gap, 2)))
+    ref.close()
+    print("config2: %d of %d generated tokens are not the first summation order's choice; undecided by the oracle: %s; different: %s"
+          % (len(undecided) + len(wrong), n_new, undecided, wrong))
+    assert not wrong, wrong
+    assert len(undecided) <= 8, undecided
 
 
 def test_config3_prefill_8x1024_executor_vs_oracle(g, bench, tinyllama):

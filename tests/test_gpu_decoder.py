@@ -114,17 +114,17 @@ def test_decode_attention_short_cache_every_pass_vs_oracle(g, dt, D, rounds):
 @pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
 def test_int8_greedy_tokens_vs_oracle_small(g, dt):
     """Greedy ids of the HIP path against the oracle on a small int8 model.  The oracle is
-    teacher-forced with the GPU's tokens; any step where the two disagree must be a tie at
-    16-bit resolution in the ORACLE's own logits (a few spacings of the storage type), which is
-    the only way two f32-summation orders can pick different tokens."""
+    teacher-forced with the GPU's tokens and runs under several f32 summation orders; a step where
+    the GPU's token is not the first order's choice must be one where the oracle's own arithmetic
+    does not separate the two tokens (oracle.SummationOrders.judge; the reference leaves the order
+    of its sums open)."""
     cfg, w = llm_weights.synthetic_int8(SMALL, dt, seed=11)
-    ref = orc.Model(cfg, w)
     rng = np.random.default_rng(5)
     prompt = rng.integers(0, cfg["vocab"], 24).tolist()
     dec = g.mynn.Decoder(cfg, dev_weights(g, w, dt))
-    got, want, near = g.greedy_compare(ref, dec, prompt, 48, dt)
-    assert all(abs(gap) <= 8.0 for _, gap in near), near
-    assert len(near) <= 4, near
+    got, want, undecided, different = g.greedy_compare(cfg, w, dec, prompt, 48, dt)
+    assert not different, different
+    assert len(undecided) <= 4, undecided
     # LlmSession drives the same steps; the device-resident decode loop repeats them
     llm = g.mynn.LlmSession(dec)
     assert llm.generate_ids(prompt, 48) == got
@@ -211,14 +211,9 @@ def test_prefill_then_decode_shares_kv_and_matches_decode_only(g, dt):
     # the two paths use different kernels for the prompt (GEMM vs GEMV numerics), so compare
     # through the oracle when they part
     if ids_prefill != ids_decode:
-        ref = orc.Model(cfg, w)
         first = next(i for i in range(20) if ids_prefill[i] != ids_decode[i])
-        stream = prompt + ids_decode[:first]
-        for i, t in enumerate(stream):
-            logits = ref.forward([t], [i], i, i + 1, False)[0]
-        lf = orc.to_f32(logits, dt)
-        gap = abs(float(lf[ids_prefill[first]] - lf[ids_decode[first]]))
-        assert gap <= 8 * 2.0 ** -11 * float(np.max(np.abs(lf))), (first, gap)
+        ok, verdicts = g.both_acceptable(cfg, w, prompt + ids_decode[:first], [ids_prefill[first], ids_decode[first]], dt)
+        assert ok, (first, verdicts)
     with pytest.raises(g.mynn.MynnError):  # padded prompt does not fit: PromptTooLong
         c = g.mynn.LlmSession(dec2, prefill=pre)
         c.generate_ids(list(range(100)), 1)
@@ -451,8 +446,8 @@ def test_batched_decode_equals_independent_sequences(g, dt):
 def test_full_size_tinyllama_shape_greedy_tokens_match_oracle(g):
     """The benchmark's own model (TinyLlama-1.1B shape, int8, fp16 activations, seed 1234, GPU-generated
     weights): a 16-token prompt and 24 greedy tokens through the captured decode step, against the oracle
-    on the same weights, teacher-forced with the GPU's tokens; a disagreement must be a tie within 8
-    spacings of fp16 in the oracle's own logits."""
+    on the same weights under three summation orders, teacher-forced with the GPU's tokens; a disagreement must
+    be one the oracle's own orders disagree on."""
     import os
     import sys
     import torch
@@ -466,10 +461,9 @@ def test_full_size_tinyllama_shape_greedy_tokens_match_oracle(g):
     torch.cuda.synchronize()
     dec = g.mynn.Decoder(cfg, weights)
     assert dec.stats()["graph"] and dec.stats()["launches_per_step"] == 67
-    ref = orc.Model(dict(cfg), bench.to_host_weights(weights))
     prompt = np.random.default_rng(1234).integers(0, cfg["vocab"], 16).tolist()
-    gpu_ids, ref_ids, near = g.greedy_compare(ref, dec, prompt, 24, dt)
-    assert all(abs(gap) <= 8 for _, gap in near), near
+    gpu_ids, ref_ids, undecided, different = g.greedy_compare(dict(cfg), bench.to_host_weights(weights), dec, prompt, 24, dt)
+    assert not different, different
     assert sum(a == b for a, b in zip(gpu_ids, ref_ids)) >= 22
     dec.close()
 

@@ -200,3 +200,34 @@ def test_zero_qkv_bias_changes_no_bit_and_decode_equals_prefill(dt):
         row = b.forward([t], [i], i, i + 1, False)
     fl, rl = orc.to_f32(full[-1], dt), orc.to_f32(row[0], dt)
     assert np.max(np.abs(fl - rl)) <= (1e-5 if dt == orc.F32 else 3e-2) * np.max(np.abs(fl))
+
+
+@pytest.mark.parametrize("dt", [orc.F32, orc.BF16, orc.F16])
+@pytest.mark.parametrize("kv8,w8a8", [(False, False), (True, False), (False, True), (True, True)])
+def test_decoder_options_equal_the_composition_of_the_pinned_operators(dt, kv8, w8a8):
+    """BuildOptions::quant_kv_cache and Options::quantize_activations in the C decoder against the same graph composed
+    in numpy from the operator-level functions (DynamicQuantizeLinear + QuantizedMatMul for every int8 linear with
+    K % 32 == 0, RoPE before the quantising cache update, scales into the attention): bit-equal logits and caches over
+    a 12-token causal prefill chunk and 10 decode steps of a 2-layer model."""
+    from oracle_compose import compose_step, empty_caches
+
+    shape = dict(n_layers=2, hidden=64, n_heads=4, n_kv_heads=2, head_dim=16, ffn=96, vocab=97, max_seq=32, eps=1e-5,
+                 rope_theta=10000.0)
+    cfg, w = llm_weights.synthetic_int8(shape, dt, seed=21)
+    m = orc.Model(cfg, w)
+    m.set_options(quant_kv_cache=kv8, quantize_activations=w8a8)
+    caches = empty_caches(cfg, dt, kv8)
+    rng = np.random.default_rng(3)
+    ids = [int(t) for t in rng.integers(0, cfg["vocab"], 12)]
+    want = compose_step(cfg, w, caches, ids, list(range(12)), 0, 12, True, dt, kv8=kv8, w8a8=w8a8)
+    assert np.array_equal(m.forward(ids, np.arange(12), 0, 12, True), want)
+    for p in range(12, 22):
+        t = int(rng.integers(0, cfg["vocab"]))
+        want = compose_step(cfg, w, caches, [t], [p], p, p + 1, False, dt, kv8=kv8, w8a8=w8a8)
+        assert np.array_equal(m.forward([t], [p], p, p + 1, False), want), p
+    for l in range(cfg["n_layers"]):
+        k, v = m.kv_cache(l)
+        assert np.array_equal(k, caches[l][0][0]) and np.array_equal(v, caches[l][1][0])
+        if kv8:
+            ks, vs = m.kv_scales(l)
+            assert np.array_equal(ks, caches[l][2][0]) and np.array_equal(vs, caches[l][3][0])

@@ -15,6 +15,7 @@ import pytest
 import oracle as orc
 import llm_weights
 from conftest import max_err_rel_to_max
+from oracle_compose import compose_step
 
 TINY = dict(n_layers=2, hidden=64, n_heads=4, n_kv_heads=2, head_dim=16, ffn=96, vocab=97, max_seq=32,
             eps=1e-5, rope_theta=10000.0)
@@ -165,41 +166,8 @@ def test_ring_attention_vs_f64_over_hand_listed_rows(dt, kv8, rope_on, Sq):
         assert np.array_equal(got, other)  # same loop order over the same rows
 
 
-def heads(x, S, H, D):
-    return np.ascontiguousarray(x.reshape(S, H, D).transpose(1, 0, 2))[None]
-
-
 def numpy_streaming_step(cfg, w, caches, ids, positions, past, active, causal, ring_start, kvp, dt, kv8):
-    """One run of the streaming graph composed from the operator-level functions of the oracle module (each pinned
-    on its own), op for op as decoder.rs:222-347, 472-487 builds it.  caches: per layer [k, v] (+ [ks, vs])."""
-    H, Hq, Hkv, D = cfg["hidden"], cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
-    S = len(ids)
-    lin = lambda x, name: orc.dequant_matmul(x, w[name][0], w[name][1], dt, dt)
-    x = orc.gather_rows(orc.dequantize_linear(w["embed"][0], w["embed"][1], dt), ids)
-    cos, sin = orc.rope_table(cfg["max_seq"], D, cfg["rope_theta"], dt)
-    for l in range(cfg["n_layers"]):
-        n1 = orc.rms_norm(x, w["layers.%d.norm1" % l], cfg["eps"], dt)
-        q = orc.rope(heads(lin(n1, "layers.%d.q" % l), S, Hq, D), cos, sin, positions, dt)
-        k = heads(lin(n1, "layers.%d.k" % l), S, Hkv, D)
-        v = heads(lin(n1, "layers.%d.v" % l), S, Hkv, D)
-        c = caches[l]
-        scale = np.float32(1.0) / np.sqrt(np.float32(D))
-        if kv8:
-            orc.quantizing_kv_cache_update_streaming(c[0], c[2], k, past, SINK, WINDOW, ring_start, dt)
-            orc.quantizing_kv_cache_update_streaming(c[1], c[3], v, past, SINK, WINDOW, ring_start, dt)
-            a = orc.attention_streaming(q, c[0], c[1], dt, scale, causal, active, SINK, WINDOW, ring_start, c[2], c[3],
-                                        (cos, sin, kvp))
-        else:
-            orc.kv_cache_update_streaming(c[0], k, past, SINK, WINDOW, ring_start)
-            orc.kv_cache_update_streaming(c[1], v, past, SINK, WINDOW, ring_start)
-            k_rot = orc.rope(c[0], cos, sin, kvp, dt)  # Rope over the whole cache: one table row per SLOT
-            a = orc.attention_streaming(q, k_rot, c[1], dt, scale, causal, active, SINK, WINDOW, ring_start)
-        a = np.ascontiguousarray(a[0].transpose(1, 0, 2)).reshape(S, Hq * D)
-        x2 = orc.add(x, lin(a, "layers.%d.o" % l), dt)
-        n2 = orc.rms_norm(x2, w["layers.%d.norm2" % l], cfg["eps"], dt)
-        hm = orc.swiglu(lin(n2, "layers.%d.gate" % l), lin(n2, "layers.%d.up" % l), dt)
-        x = orc.add(x2, lin(hm, "layers.%d.down" % l), dt)
-    return orc.dequant_matmul(orc.rms_norm(x, w["final_norm"], cfg["eps"], dt), w["lm_head"][0], w["lm_head"][1], dt, dt)
+    return compose_step(cfg, w, caches, ids, positions, past, active, causal, dt, kv8=kv8, ring=(SINK, WINDOW, ring_start, kvp))
 
 
 @pytest.mark.parametrize("dt", [orc.F32, orc.F16])
