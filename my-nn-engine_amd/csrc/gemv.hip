@@ -206,19 +206,33 @@ __global__ __launch_bounds__(kGemvThreads) void dequant_gemv1_kernel(const int8_
                 st_past = *p.adv.past;
                 st_active = *p.adv.active;
             }
-            for (int i = tid; i < nb; i += kGemvThreads) {
-                uint64_t w = __hip_atomic_load(p.cand + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                for (int spins = 0; w == ~0ull; spins++) {
-                    if (spins > p.spin_limit) {
-                        __hip_atomic_store(p.err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        break;
-                    }
-                    __builtin_amdgcn_s_sleep(1);
-                    w = __hip_atomic_load(p.cand + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // a thread's candidate words are asked for together every round: one round trip per round, not per word
+            constexpr int CW = (kGemvArgmaxWords + kGemvThreads - 1) / kGemvThreads;
+            uint64_t w[CW];
+            for (int spins = 0;; spins++) {
+                bool empty = false;
+#pragma unroll
+                for (int k = 0; k < CW; k++) {
+                    const int i = tid + k * kGemvThreads;
+                    w[k] = i < nb ? __hip_atomic_load(p.cand + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0ull;
                 }
-                const int oi = (int)(uint32_t)w;
-                if (w != ~0ull && oi >= 0) argmax_take(bv, bi, __builtin_bit_cast(float, (uint32_t)(w >> 32)), oi);
-                p.cand[i] = ~0ull;  // empty again for the next launch
+#pragma unroll
+                for (int k = 0; k < CW; k++) empty = empty || w[k] == ~0ull;
+                if (!empty) break;
+                if (spins > p.spin_limit) {
+                    __hip_atomic_store(p.err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
+#pragma unroll
+            for (int k = 0; k < CW; k++) {
+                const int i = tid + k * kGemvThreads;
+                if (i < nb) {
+                    const int oi = (int)(uint32_t)w[k];
+                    if (w[k] != ~0ull && oi >= 0) argmax_take(bv, bi, __builtin_bit_cast(float, (uint32_t)(w[k] >> 32)), oi);
+                    p.cand[i] = ~0ull;  // empty again for the next launch
+                }
             }
             meet();
             if (tid == 0) {
