@@ -568,6 +568,10 @@ def decode_batch_main(args, mynn):
     import torch
 
     B, ctx = 32, 2048
+    if args.kv_pages is None:
+        args.kv_pages = 256  # configs[4] names a paged cache
+    if args.skinny_ablation:
+        mynn.lib().mynn_skinny_set_ablation({"loads": 1, "nomfma": 2}[args.skinny_ablation])
     K = 32 if args.steps is None else args.steps
     W = 4 if args.warmup is None else args.warmup
     dt = {"f16": mynn.F16, "bf16": mynn.BF16}[args.dtype]
@@ -659,7 +663,7 @@ def decode_batch_main(args, mynn):
         "config": {"workload": "configs[4]: Llama-3-8B-shape int8 decoder, batch 32, context 2048 (caches filled with "
                                "random rows%s), %d decode steps timed" % ((", int8 KV cache" if args.kv_int8 else "") + (", paged KV cache" if args.kv_pages else ""), K),
                    "batch": B, "context": ctx, "launches_per_step": stats["launches_per_step"], "hipgraph": stats["graph"],
-                   "kv_page_rows": args.kv_pages or None,
+                   "kv_page_rows": args.kv_pages or None, "skinny_ablation": args.skinny_ablation,
                    "kv_pages_mapped": (pool.n_pages - pool.free_pages) if pool else None,
                    "seed": args.seed, "step_algorithmic_bytes": step_bytes,
                    "step_hbm_frac": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
@@ -730,8 +734,12 @@ def main():
                     help="prefill: quantise activations per row and run every linear as int8 x int8 (Options::quantize_activations)")
     ap.add_argument("--kv-int8", action="store_true",
                     help="decode / decode_batch: int8 KV cache with per-token scales (BuildOptions::quant_kv_cache)")
-    ap.add_argument("--kv-pages", type=int, default=0, metavar="ROWS",
-                    help="decode_batch: paged KV cache with this many rows per page (kv_page_rows), one pool for the batch")
+    ap.add_argument("--kv-pages", type=int, default=None, metavar="ROWS",
+                    help="decode_batch: rows per page of the paged KV cache (kv_page_rows), one pool for the batch; default 256, "
+                         "0 = contiguous caches")
+    ap.add_argument("--skinny-ablation", choices=["loads", "nomfma"], default=None,
+                    help="decode_batch: run the gate/up few-row GEMM as its loads alone / without its MFMAs (garbage results: "
+                         "only the launch duration is meaningful)")
     ap.add_argument("--weight-arena", action="store_true", help="decode: all weights in one allocation in execution order (weight_arena)")
     ap.add_argument("--unfused", action="store_true", help="decode: every op a launch of its own (unfused_decode)")
     ap.add_argument("--check-tokens", type=int, default=0,

@@ -72,6 +72,7 @@ SIGNATURES = {
     "mynn_dequantize_linear": (_i, [_vp, _vp, _vp, _sz, _sz, _i, _vp]),
     "mynn_dequant_gemv": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mynn_gemv_read_probe": (_i, [_vp, _vp, _i, _i, _i, _vp]),
+    "mynn_skinny_set_ablation": (None, [_i]),
     "mynn_dequant_matmul": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "mynn_dequant_matmul_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "mynn_dequant_matmul_ws": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _sz, _i, _vp]),

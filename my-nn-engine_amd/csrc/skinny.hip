@@ -29,11 +29,16 @@ constexpr int kSkinnyLd = kSkinnyK + 8;  // LDS row stride of the activation chu
 
 // PACKED: wq is the tiled copy made by skinny_pack_kernel -- for every (32 rows, 128 k) tile the 4 KB a
 // wave needs, in the order its four load instructions want them (instruction j, lane l -> 16 bytes at
-// j*1024 + l*16): one sequential stream per wave instead of 128-byte pieces of 32 rows a row pitch apart
-// (measured 2.3 TB/s for the row-major form: DRAM pages are opened for 128 bytes each).
+// j*1024 + l*16) instead of 128-byte pieces of 32 rows a row pitch apart (measured 2.3 TB/s for the row-major
+// form: DRAM pages are opened for 128 bytes each).  Tiles are ordered K STEP FIRST, [step][row block]: the waves
+// of a launch walk their K ranges in step, so what is in flight at any moment is one contiguous stretch of the
+// copy (the row blocks of a few consecutive steps) and the launch as a whole sweeps it front to back -- the access
+// pattern of the batch-1 GEMV, which streams at 7 TB/s -- and not some 900 separate streams 128 KB apart.
 // FEPI < 0: partial sums to `part` (several K ranges, summed by skinny_reduce_kernel).  FEPI = GEMM_*: the
 // workgroup covers the whole K range and stores the finished output itself (scale, residual or SwiGLU).
-template <typename T, int MT, bool PACKED, int FEPI>
+// ABL (measurement aid, mynn_skinny_set_ablation): 1 = the loads alone -- no LDS, no conversion, no MFMA, no barrier; the
+// loaded words are folded into the accumulator so that they stay; 2 = everything but the MFMAs.  Results are garbage.
+template <typename T, int MT, bool PACKED, int FEPI, int ABL = 0>
 __global__ __launch_bounds__(kSkinnyThreads) void skinny_gemm_kernel(float *part, const T *act, const int8_t *wq, int M,
                                                                     int N, int K, int iters_per_split, T *out,
                                                                     const T *scale, const T *res) {
@@ -46,7 +51,8 @@ __global__ __launch_bounds__(kSkinnyThreads) void skinny_gemm_kernel(float *part
     const int it0 = blockIdx.y * iters_per_split, it1 = min(it0 + iters_per_split, iters);
     if (it0 >= it1) return;  // whole workgroup
     // waves past N recompute the last rows (row-major) or read the zero-padded last tile (packed), store nothing
-    const int8_t *wrow = PACKED ? wq + (size_t)min(n0 / 32, (N - 1) / 32) * iters * 4096 + lane * 16
+    const size_t step_pitch = (size_t)((N + 31) / 32) * 4096;  // PACKED: bytes of one K step over all row blocks
+    const int8_t *wrow = PACKED ? wq + (size_t)min(n0 / 32, (N - 1) / 32) * 4096 + lane * 16
                                 : wq + (size_t)min(n0 + r, N - 1) * K + 64 * h;
 
     f16x_t acc[MT];
@@ -71,30 +77,44 @@ __global__ __launch_bounds__(kSkinnyThreads) void skinny_gemm_kernel(float *part
     // Workgroups walk their K range from different starting steps: all rows of the matrix are a multiple of
     // 128 bytes apart, so in lockstep every request in flight would carry the same low address bits and
     // land on the same few memory channels.
-    const int len = it1 - it0, rot = (int)((blockIdx.x * 7u + blockIdx.y * 3u) % (unsigned)len);
+    // (the packed copy is read in step by every workgroup on purpose: see PACKED above)
+    const int len = it1 - it0, rot = PACKED ? 0 : (int)((blockIdx.x * 7u + blockIdx.y * 3u) % (unsigned)len);
     auto load = [&](int it, Stage &st) {
         int step = min(it, it1 - 1) - it0 + rot;
         if (step >= len) step -= len;
         const size_t k = (size_t)(it0 + step) * kSkinnyK;
-        const U4 *src = (const U4 *)(wrow + (PACKED ? (size_t)(it0 + step) * 4096 : k));
-#pragma unroll
-        for (int j = 0; j < 4; j++) st.w[j] = __builtin_nontemporal_load(src + (PACKED ? j * 64 : j));
+        const U4 *src = (const U4 *)(wrow + (PACKED ? (size_t)(it0 + step) * step_pitch : k));
+        // the activation share FIRST: loads return in order, and the chunk of step it+1 is wanted (for LDS) one step
+        // before that step's weights are -- asked for behind them, the wait for it would drain the weight loads too
+        // and leave a single step in flight
 #pragma unroll
         for (int q = 0; q < AP; q++) st.a[q] = *(const U4 *)(ap[q] + k);
+#pragma unroll
+        for (int j = 0; j < 4; j++) st.w[j] = __builtin_nontemporal_load(src + (PACKED ? j * 64 : j));
     };
     auto store_act = [&](int buf, const Stage &st) {
 #pragma unroll
         for (int q = 0; q < AP; q++) *(U4 *)&a_s[buf][(arow + 16 * q) * kSkinnyLd + acol] = st.a[q];
     };
     auto compute = [&](int buf, const Stage &st) {
+        // all activation operands of the step first (one LDS latency for the step, not one in front of every MFMA;
+        // the scheduling barrier keeps the compiler from sinking each read back to its use)
+        U4 b[MT][8];
+#pragma unroll
+        for (int s = 0; s < 8; s++)
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) b[mt][s] = *(const U4 *)&a_s[buf][(mt * 32 + r) * kSkinnyLd + 64 * h + 8 * s];
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int s = 0; s < 8; s++) {
             const U4 &q = st.w[s >> 1];
             const U4 a = (s & 1) ? i8x8_to_operand<T>(q.z, q.w) : i8x8_to_operand<T>(q.x, q.y);
 #pragma unroll
             for (int mt = 0; mt < MT; mt++) {
-                const U4 b = *(const U4 *)&a_s[buf][(mt * 32 + r) * kSkinnyLd + 64 * h + 8 * s];
-                acc[mt] = Mfma<T>::run(a, b, acc[mt]);
+                if constexpr (ABL == 2)
+                    acc[mt][s] += __builtin_bit_cast(float, (a.x ^ b[mt][s].x ^ a.y ^ b[mt][s].y ^ a.z ^ b[mt][s].z ^ a.w ^ b[mt][s].w) & 0x3fffffffu);
+                else
+                    acc[mt] = Mfma<T>::run(a, b[mt][s], acc[mt]);
             }
         }
     };
@@ -107,20 +127,36 @@ __global__ __launch_bounds__(kSkinnyThreads) void skinny_gemm_kernel(float *part
     store_act(0, st[0]);
     __syncthreads();
     int buf = 0;
-    bool more = true;
-    while (more) {
+    auto step = [&](Stage &cur, Stage &next, Stage &refill) {
+        load(it + S - 1, refill);
+        if constexpr (ABL == 1) {
+            uint32_t x = 0;
 #pragma unroll
-        for (int j = 0; j < S; j++) {  // fully unrolled: every stage index is a constant
-            if (more) {
-                load(it + S - 1, st[(j + S - 1) % S]);
-                compute(buf, st[j]);
-                store_act(buf ^ 1, st[(j + 1) % S]);  // the chunk of step it+1 for the other buffer
-                __syncthreads();
-                buf ^= 1;
-                more = ++it < it1;
-            }
+            for (int j = 0; j < 4; j++) x ^= cur.w[j].x ^ cur.w[j].y ^ cur.w[j].z ^ cur.w[j].w;
+#pragma unroll
+            for (int q = 0; q < AP; q++) x ^= cur.a[q].x;
+            acc[0][0] += __builtin_bit_cast(float, x & 0x3fffffffu);
+        } else {
+            compute(buf, cur);
+            store_act(buf ^ 1, next);  // the chunk of step it+1 for the other buffer
+            __syncthreads();
         }
+        buf ^= 1;
+        ++it;
+    };
+    // Whole groups of S steps in a loop body without branches: every stage index is a constant and the loads that are
+    // still in flight at the loop's end sit in the registers they sit in at its start, so the waits inside the body
+    // are counted waits.  (With an exit test after every step the compiler could not count across the back edge and
+    // drained every load once per group: the stream restarted from empty every S steps.)
+    while (it + S <= it1) {
+#pragma unroll
+        for (int j = 0; j < S; j++) step(st[j], st[(j + 1) % S], st[(j + S - 1) % S]);
     }
+    // the remaining steps (fewer than S); the stage indices continue from 0
+    const int rest = it1 - it;
+#pragma unroll
+    for (int j = 0; j < S - 1; j++)
+        if (j < rest) step(st[j], st[(j + 1) % S], st[(j + S - 1) % S]);
 
     // D[n][m]: lane holds column m = lane%32 and rows n = 8*(e/4) + 4*(lane/32) + e%4: four consecutive n
     if (n0 >= N) return;
@@ -174,15 +210,14 @@ __global__ __launch_bounds__(kSkinnyThreads) void skinny_gemm_kernel(float *part
     }
 }
 
-// tile[(nb * iters + it)][j][l] (16 bytes) = W[nb*32 + l%32][it*128 + 64*(l/32) + 16*j ..]; rows past N are zero
+// tile[(it * row_blocks + nb)][j][l] (16 bytes) = W[nb*32 + l%32][it*128 + 64*(l/32) + 16*j ..]; rows past N are zero
 __global__ __launch_bounds__(256) void skinny_pack_kernel(U4 *dst, const int8_t *wq, int N, int K, size_t chunks) {
     const size_t c = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (c >= chunks) return;
-    const int iters = K / kSkinnyK;
     const int l = (int)(c & 63), j = (int)((c >> 6) & 3);
-    const size_t tile = c >> 8;
-    const int it = (int)(tile % iters);
-    const size_t row = (tile / iters) * 32 + (l & 31);
+    const size_t tile = c >> 8, row_blocks = (size_t)(N + 31) / 32;
+    const int it = (int)(tile / row_blocks);
+    const size_t row = (tile % row_blocks) * 32 + (l & 31);
     U4 v = U4{0u, 0u, 0u, 0u};
     if (row < (size_t)N) v = *(const U4 *)(wq + row * K + (size_t)it * kSkinnyK + 64 * (l >> 5) + 16 * j);
     dst[c] = v;
@@ -386,6 +421,10 @@ __global__ __launch_bounds__(kReduceNormThreads) void skinny_reduce_rope_kernel(
     }
 }
 
+// 0 = the product kernel; 1 / 2 = the ablations of skinny_gemm_kernel for the one-launch SwiGLU form (packed weights,
+// M <= 32): what bench.py --workload decode_batch --skinny-ablation times
+static int g_skinny_ablation = 0;
+
 bool skinny_gemm_supported(int M, int N, int K) { return M >= 16 && M <= 64 && K % kSkinnyK == 0 && K >= 2 * kSkinnyK && N >= 1; }
 
 // K ranges: enough waves to keep ~1000 in flight, each with at least as many steps as it has stages
@@ -433,6 +472,16 @@ int dequant_gemm_skinny(void *out, const void *act, const int8_t *wq, bool packe
         };
         // the whole K range in one workgroup: no partial sums, no second launch (the wide shapes: gate/up and
         // lm_head; a residual store never meets this width, it keeps the two-launch form)
+        if (ks_used == 1 && epi == GEMM_SWIGLU && g_skinny_ablation && M <= 32 && packed) {
+            T *o = (T *)out;
+            if (g_skinny_ablation == 1)
+                MYNN_LAUNCH((skinny_gemm_kernel<T, 1, true, GEMM_SWIGLU, 1>), grid, dim3(kSkinnyThreads), 0, s, scratch, (const T *)act, wq, M, N, K, ips, o,
+                            (const T *)scale, (const T *)res);
+            else
+                MYNN_LAUNCH((skinny_gemm_kernel<T, 1, true, GEMM_SWIGLU, 2>), grid, dim3(kSkinnyThreads), 0, s, scratch, (const T *)act, wq, M, N, K, ips, o,
+                            (const T *)scale, (const T *)res);
+            return launch_status("skinny_gemm_kernel (ablation)");
+        }
         if (ks_used == 1 && epi == GEMM_SWIGLU) return gemm(std::integral_constant<int, GEMM_SWIGLU>{});
         if (ks_used == 1 && epi == GEMM_PLAIN) return gemm(std::integral_constant<int, GEMM_PLAIN>{});
         int rc = gemm(std::integral_constant<int, -1>{});
@@ -477,3 +526,5 @@ int dequant_gemm_skinny(void *out, const void *act, const int8_t *wq, bool packe
 }
 
 }  // namespace mynn
+
+extern "C" void mynn_skinny_set_ablation(int mode) { mynn::g_skinny_ablation = mode == 1 || mode == 2 ? mode : 0; }
