@@ -681,15 +681,16 @@ def decode_batch_main(args, mynn):
     print(json.dumps(out))
 
 
-def short_prefill(mynn, cfg, weights, seed):
-    """Three timed passes (after three untimed ones) of the 8 x 1024 prefill (configs[3]) over the same weights, outside
-    any timed decode region: the matrix-core side of the path, for the same JSON line."""
+def short_prefill(mynn, cfg, weights, seed, weight_set=None):
+    """Three timed passes (after three untimed ones) of the 8 x 1024 prefill (configs[3]) over the same weights (and, as in
+    a session, the same weight set as the decode executor), outside any timed decode region: the matrix-core side of the
+    path, for the same JSON line."""
     import numpy as np
     import torch
 
     B, S = PREFILL_BATCH, PREFILL_LEN
     pcfg = dict(cfg, max_seq=S)
-    pre = mynn.Decoder(pcfg, weights, seq_q=S, batch=B)
+    pre = mynn.Decoder(pcfg, weights, seq_q=S, batch=B, weight_set=weight_set)
     ids = np.random.default_rng(seed).integers(0, cfg["vocab"], B * S)
     pos = np.arange(S)
     for _ in range(3):  # (the matrix pipes' clock settles over the first passes)
@@ -789,8 +790,9 @@ def main():
 
     weights = make_weights(cfg, dt, args.seed)
     torch.cuda.synchronize()
+    wset = mynn.WeightSet(cfg, weights)  # one set of derived weight copies for the decode and the prefill executor
     dec = mynn.Decoder(cfg, weights, quant_kv_cache=args.kv_int8, quantize_activations=args.w8a8, unfused_decode=args.unfused,
-                       weight_arena=args.weight_arena)
+                       weight_arena=args.weight_arena, weight_set=wset)
     stats = dec.stats()
     rng = np.random.default_rng(args.seed)
     prompt = rng.integers(0, cfg["vocab"], PROMPT_LEN).tolist()
@@ -899,7 +901,8 @@ def main():
                      "what": "mynn_gemv_read_probe: weight bytes of one launch / its average duration, 400 dependent launches "
                              "over matrices rotating through 1 GiB"}
     if not args.no_prefill and not (args.kv_int8 or args.w8a8 or args.unfused):
-        out["config"]["prefill"] = short_prefill(mynn, cfg, weights, args.seed)
+        out["config"]["prefill"] = short_prefill(mynn, cfg, weights, args.seed, wset)
+        out["config"]["weight_set"] = wset.stats()
 
     if not args.no_cpu_baseline:
         import oracle as orc

@@ -116,6 +116,10 @@ SIGNATURES = {
     "mynn_argmax_last": (_i, [_vp, _vp, _i, _i, _vp]),
     "mynn_model_configure": (_i, [C.POINTER(ModelConfig)]),
     "mynn_model_create": (_vp, [C.POINTER(ModelConfig), C.POINTER(_vp), C.POINTER(_vp)]),
+    "mynn_weight_set_create": (_vp, [C.POINTER(ModelConfig), C.POINTER(_vp)]),
+    "mynn_model_create_shared": (_vp, [C.POINTER(ModelConfig), _vp, C.POINTER(_vp)]),
+    "mynn_weight_set_stats": (_i, [_vp, C.POINTER(_sz), C.POINTER(_i)]),
+    "mynn_weight_set_destroy": (None, [_vp]),
     "model_init": (_vp, [C.POINTER(_vp), C.POINTER(_vp)]),
     "model": (None, [_vp, C.POINTER(_vp), C.POINTER(_vp)]),
     "model_destroy": (None, [_vp]),
@@ -643,6 +647,69 @@ class DeviceWeights:
             pass
 
 
+def _initializer_array(cfg, weights, quant):
+    """The `initializer` array of model_init for a weight dict (order of the reference's graph initializers)."""
+    init = []
+
+    def lin(w):
+        if quant:
+            init.extend([_ptr(w[0]), _ptr(w[1])])
+        else:
+            init.extend([_ptr(w), None])
+
+    lin(weights["embed"])
+    for l in range(cfg.n_layers):
+        init.append(_ptr(weights["layers.%d.norm1" % l]))
+        for nm in ("q", "k", "v", "o"):
+            lin(weights["layers.%d.%s" % (l, nm)])
+            if cfg.qkv_bias and nm != "o":
+                init.append(_ptr(weights["layers.%d.%s.bias" % (l, nm)]))
+        init.append(_ptr(weights["layers.%d.norm2" % l]))
+        for nm in ("gate", "up", "down"):
+            lin(weights["layers.%d.%s" % (l, nm)])
+    init.append(_ptr(weights["final_norm"]))
+    lin(weights["lm_head"])
+    return (_vp * len(init))(*init)
+
+
+class WeightSet:
+    """mynn_weight_set: the library's derived copies of one checkpoint's weights (decode repacks, 16-bit resident copy,
+    tiled int8 copy, W8A8 interleave), each made once and shared by every Decoder built with weight_set=this."""
+
+    def __init__(self, cfg, weights):
+        import torch
+
+        quant = isinstance(weights["embed"], tuple)
+        qkv_bias = bool(cfg.get("qkv_bias")) or "layers.0.q.bias" in weights
+        self.cfg = ModelConfig(cfg["n_layers"], cfg["hidden"], cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"], cfg["ffn"],
+                               cfg["vocab"], cfg["max_seq"], float(cfg["eps"]), float(cfg["rope_theta"]), cfg["dtype"], 1, 1,
+                               int(quant), 0, 0, 0, 0, 0, 0, 0, 0, int(qkv_bias))
+        self.weights = weights
+        self._init = _initializer_array(self.cfg, weights, quant)
+        torch.cuda.synchronize()
+        self.handle = lib().mynn_weight_set_create(C.byref(self.cfg), self._init)
+        if not self.handle:
+            raise MynnError("weight_set_create failed: %s" % lib().mynn_last_error().decode())
+
+    def stats(self):
+        b = (_sz * 4)()
+        n = _i(0)
+        check(lib().mynn_weight_set_stats(self.handle, b, C.byref(n)))
+        return {"repack_bytes": b[0], "resident16_bytes": b[1], "tiled_int8_bytes": b[2], "w8a8_interleave_bytes": b[3],
+                "holders": n.value}
+
+    def close(self):
+        if getattr(self, "handle", None) and _lib is not None:
+            _lib.mynn_weight_set_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 class Decoder:
     """Thin holder around model_init / model_step / model_destroy.
 
@@ -655,7 +722,9 @@ class Decoder:
 
     def __init__(self, cfg, weights, seq_q=1, batch=1, kv=None, quant_kv_cache=False, quantize_activations=False,
                  streaming_kv=False, gemm_tile=0, unfused_decode=False, handover_spin_limit=0, weight_arena=False,
-                 reference_abi=False, kv_pages=None):
+                 reference_abi=False, kv_pages=None, weight_set=None):
+        """weight_set: a WeightSet made from the same cfg shapes and weights -- the executor then shares the library's
+        derived weight copies with the other executors built on it (mynn_model_create_shared)."""
         import torch
 
         tdt = {F16: torch.float16, BF16: torch.bfloat16}[cfg["dtype"]]
@@ -670,6 +739,7 @@ class Decoder:
                                kv_pages.pool.page_rows if kv_pages is not None else 0, int(qkv_bias))
         self.weights = weights  # keep the tensors alive
         self.kv_pages = kv_pages
+        self.weight_set = weight_set
         if kv_pages is not None:
             # paged cache: kv = the pool buffers (KvPool.buffers), one (K pool, V pool) per layer, shared by every session of the pool
             assert kv is not None, "a paged decoder takes the pool's buffers as kv"
@@ -696,27 +766,13 @@ class Decoder:
             self.cfg.weights_int8 = int(self.weights.int8)
             self.handle = self._create(self.weights.initializer, reference_abi)
             return
-        init = []
-
-        def lin(w):
-            if quant:
-                init.extend([_ptr(w[0]), _ptr(w[1])])
-            else:
-                init.extend([_ptr(w), None])
-
-        lin(weights["embed"])
-        for l in range(cfg["n_layers"]):
-            init.append(_ptr(weights["layers.%d.norm1" % l]))
-            for nm in ("q", "k", "v", "o"):
-                lin(weights["layers.%d.%s" % (l, nm)])
-                if self.cfg.qkv_bias and nm != "o":
-                    init.append(_ptr(weights["layers.%d.%s.bias" % (l, nm)]))
-            init.append(_ptr(weights["layers.%d.norm2" % l]))
-            for nm in ("gate", "up", "down"):
-                lin(weights["layers.%d.%s" % (l, nm)])
-        init.append(_ptr(weights["final_norm"]))
-        lin(weights["lm_head"])
-        self._init = (_vp * len(init))(*init)
+        if weight_set is not None:
+            handle = lib().mynn_model_create_shared(C.byref(self.cfg), weight_set.handle, self._state)
+            if not handle:
+                raise MynnError("model_create_shared failed: %s" % lib().mynn_last_error().decode())
+            self.handle = handle
+            return
+        self._init = _initializer_array(self.cfg, weights, quant)
         torch.cuda.synchronize()
         self.handle = self._create(self._init, reference_abi)
 

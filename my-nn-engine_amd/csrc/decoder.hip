@@ -85,8 +85,8 @@ struct Layer {
     Lin qkv, o, gate, up, gu, down;  // qkv = rows of q,k,v concatenated; gu = gate/up rows interleaved
     void *k_cache = nullptr, *v_cache = nullptr;
     void *k_scale = nullptr, *v_scale = nullptr;  // int8 KV cache: per-token scales [B,Hkv,max_seq]
-    void *own_qkv_w = nullptr, *own_qkv_s = nullptr, *own_gu_w = nullptr, *own_gu_s = nullptr;
-    void *qkv_b = nullptr;  // qkv_bias: the q, k, v projection biases concatenated [QD + 2 KD], T (owned)
+    // (everything below points into the model's WeightSet)
+    void *qkv_b = nullptr;  // qkv_bias: the q, k, v projection biases concatenated [QD + 2 KD], T
     // prefill executors: weights dequantised once to the 16-bit type, [N, Kp] (wt_gu: gate/up in groups of 32)
     void *wt_qkv = nullptr, *wt_o = nullptr, *wt_gu = nullptr, *wt_down = nullptr;
     // few-row executors: int8 weights re-tiled so that a wave streams them sequentially
@@ -94,6 +94,58 @@ struct Layer {
     // W8A8 prefill executors: int8 gate/up rows and their scales interleaved in groups of 32 (SwiGLU store)
     void *q8_gu = nullptr, *q8_gu_scale = nullptr;
 };
+
+// Every copy the library derives from a checkpoint's weights, made at most once and shared by the executors of a
+// session (prefill, decode, few-row): the q|k|v and gate/up repacks, the 16-bit resident copy of the matrix-core path,
+// the tiled int8 copy of the few-row path, the W8A8 gate/up interleave.  A copy is made by the first executor that
+// needs it (under the set's mutex) and lives until the last holder -- the caller's handle or a model -- lets go.
+struct WeightLayer {
+    void *qkv_w = nullptr, *qkv_s = nullptr, *gu_w = nullptr, *gu_s = nullptr, *qkv_b = nullptr;
+    void *wt_qkv = nullptr, *wt_o = nullptr, *wt_gu = nullptr, *wt_down = nullptr;
+    void *pk_qkv = nullptr, *pk_o = nullptr, *pk_gu = nullptr, *pk_down = nullptr;
+    void *q8_gu = nullptr, *q8_gu_scale = nullptr;
+};
+struct WeightSet {
+    std::mutex mu;
+    int refs = 1;
+    // what the copies depend on: the shapes, the storage type, the caller's buffers
+    int n_layers = 0, hidden = 0, n_heads = 0, n_kv_heads = 0, head_dim = 0, ffn = 0, vocab = 0, dtype = 0, int8_weights = 0, qkv_bias = 0;
+    std::vector<void *> initializer;
+    std::vector<WeightLayer> layers;
+    void *wt_lm_head = nullptr, *pk_lm_head = nullptr;
+    bool repacked = false, resident16 = false, packed8 = false, q8 = false;
+    size_t bytes_repack = 0, bytes_resident16 = 0, bytes_packed8 = 0, bytes_q8 = 0;
+};
+static size_t initializer_count(const mynn_model_config &c) {
+    return 2 + (size_t)c.n_layers * (2 + 14 + (c.qkv_bias ? 3 : 0)) + 1 + 2;
+}
+static WeightSet *weight_set_new(const mynn_model_config &c, void **init) {
+    WeightSet *w = new WeightSet;
+    w->n_layers = c.n_layers; w->hidden = c.hidden; w->n_heads = c.n_heads; w->n_kv_heads = c.n_kv_heads; w->head_dim = c.head_dim;
+    w->ffn = c.ffn; w->vocab = c.vocab; w->dtype = c.dtype; w->int8_weights = c.weights_int8; w->qkv_bias = c.qkv_bias;
+    w->initializer.assign(init, init + initializer_count(c));
+    w->layers.resize(c.n_layers);
+    return w;
+}
+static bool weight_set_fits(const WeightSet &w, const mynn_model_config &c) {
+    return w.n_layers == c.n_layers && w.hidden == c.hidden && w.n_heads == c.n_heads && w.n_kv_heads == c.n_kv_heads &&
+           w.head_dim == c.head_dim && w.ffn == c.ffn && w.vocab == c.vocab && w.dtype == c.dtype && w.int8_weights == c.weights_int8 &&
+           w.qkv_bias == c.qkv_bias;
+}
+static void weight_set_release(WeightSet *w) {
+    if (!w) return;
+    {
+        std::lock_guard<std::mutex> lk(w->mu);
+        if (--w->refs > 0) return;
+    }
+    for (WeightLayer &L : w->layers)
+        for (void *p : {L.qkv_w, L.qkv_s, L.gu_w, L.gu_s, L.qkv_b, L.wt_qkv, L.wt_o, L.wt_gu, L.wt_down, L.pk_qkv, L.pk_o, L.pk_gu, L.pk_down,
+                        L.q8_gu, L.q8_gu_scale})
+            if (p) (void)hipFree(p);
+    if (w->wt_lm_head) (void)hipFree(w->wt_lm_head);
+    if (w->pk_lm_head) (void)hipFree(w->pk_lm_head);
+    delete w;
+}
 
 struct Launch {
     const char *name;
@@ -108,6 +160,7 @@ struct Model {
     const void *final_norm = nullptr;
     std::vector<Layer> layers;
     void *wt_lm_head = nullptr, *pk_lm_head = nullptr;
+    WeightSet *wset = nullptr;  // the derived weight copies (shared with the session's other executors)
     bool w8a8_fused = false;  // W8A8 with the large int8 tiles: norm+quantise, residual and SwiGLU ride on the launches
     bool qgemv1 = false;      // W8A8 at batch 1: norm, quantiser, int8 GEMV and residual / SwiGLU of a linear in one launch
     bool resident16 = false;  // the wt_* copies exist and the matrix-core path with fused stores is used
@@ -592,6 +645,15 @@ static int build(Model &m, void **init, void **state) {
         l.N = N;
         l.K = K;
     };
+    WeightSet &ws = *m.wset;
+    std::lock_guard<std::mutex> ws_lock(ws.mu);  // derived copies are made once per set, by whichever executor comes first
+    // a stage that failed half-way (out of memory) left its flag unset: the next builder makes the stage again, over
+    // whatever the failed one had allocated
+    auto renew = [](void **p) {
+        if (*p) (void)hipFree(*p);
+        *p = nullptr;
+    };
+    if (!ws.repacked) ws.bytes_repack = 0;
     lin(m.embed, V, H);
     m.layers.resize(c.n_layers);
     for (int li = 0; li < c.n_layers; li++) {
@@ -603,11 +665,17 @@ static int build(Model &m, void **init, void **state) {
         lin(k, KD, H); if (c.qkv_bias) kb = init[i++];
         lin(v, KD, H); if (c.qkv_bias) vb = init[i++];
         lin(L.o, H, QD);
+        WeightLayer &W = ws.layers[li];
         if (c.qkv_bias) {
             MYNN_REQUIRE(qb && kb && vb, MYNN_ERR_INVALID, "model_init: null projection bias in layer %d", li);
             const void *bp[3] = {qb, kb, vb};
             const size_t bb[3] = {(size_t)QD * eb, (size_t)KD * eb, (size_t)KD * eb};
-            TRY(concat_rows(&L.qkv_b, bp, bb, 3));
+            if (!ws.repacked) {
+                renew(&W.qkv_b);
+                TRY(concat_rows(&W.qkv_b, bp, bb, 3));
+                ws.bytes_repack += bb[0] + bb[1] + bb[2];
+            }
+            L.qkv_b = W.qkv_b;
         }
         L.norm2 = init[i++];
         lin(L.gate, F, H); lin(L.up, F, H); lin(L.down, H, F);
@@ -617,16 +685,24 @@ static int build(Model &m, void **init, void **state) {
                      MYNN_ERR_INVALID, "model_init: null scale in layer %d", li);
         const void *parts[3] = {q.w, k.w, v.w};
         const size_t pb[3] = {(size_t)QD * H * wb, (size_t)KD * H * wb, (size_t)KD * H * wb};
-        TRY(concat_rows(&L.own_qkv_w, parts, pb, 3));
-        L.qkv.w = L.own_qkv_w; L.qkv.N = QD + 2 * KD; L.qkv.K = H;
+        if (!ws.repacked) {
+            renew(&W.qkv_w);
+            TRY(concat_rows(&W.qkv_w, parts, pb, 3));
+            ws.bytes_repack += pb[0] + pb[1] + pb[2];
+        }
+        L.qkv.w = W.qkv_w; L.qkv.N = QD + 2 * KD; L.qkv.K = H;
         if (m.quant) {
             const void *sp[3] = {q.scale, k.scale, v.scale};
             const size_t sb[3] = {(size_t)QD * eb, (size_t)KD * eb, (size_t)KD * eb};
-            TRY(concat_rows(&L.own_qkv_s, sp, sb, 3));
-            L.qkv.scale = L.own_qkv_s;
-            TRY(interleave_rows(&L.own_gu_w, L.gate.w, L.up.w, F, (size_t)H));
-            TRY(interleave_rows(&L.own_gu_s, L.gate.scale, L.up.scale, F, eb));
-            L.gu.w = L.own_gu_w; L.gu.scale = L.own_gu_s; L.gu.N = 2 * F; L.gu.K = H;
+            if (!ws.repacked) {
+                renew(&W.qkv_s); renew(&W.gu_w); renew(&W.gu_s);
+                TRY(concat_rows(&W.qkv_s, sp, sb, 3));
+                TRY(interleave_rows(&W.gu_w, L.gate.w, L.up.w, F, (size_t)H));
+                TRY(interleave_rows(&W.gu_s, L.gate.scale, L.up.scale, F, eb));
+                ws.bytes_repack += sb[0] + sb[1] + sb[2] + 2 * (size_t)F * H + 2 * (size_t)F * eb;
+            }
+            L.qkv.scale = W.qkv_s;
+            L.gu.w = W.gu_w; L.gu.scale = W.gu_s; L.gu.N = 2 * F; L.gu.K = H;
         }
         const int per_layer = c.quant_kv_cache ? 4 : 2;
         L.k_cache = state[per_layer * li];
@@ -647,6 +723,7 @@ static int build(Model &m, void **init, void **state) {
                      MYNN_ERR_INVALID, "model_init: the page set (batch %d, %d pages of %d rows) does not fit batch %d, max_seq %d, kv_page_rows %d",
                      kv_pages_batch(m.pages), m.paging.pages_per_seq, 1 << m.paging.shift, c.batch, c.max_seq, c.kv_page_rows);
     }
+    ws.repacked = true;
     m.final_norm = init[i++];
     lin(m.lm_head, V, H);
     MYNN_REQUIRE(m.embed.w && m.final_norm && m.lm_head.w, MYNN_ERR_INVALID, "model_init: null embed/norm/lm_head");
@@ -674,10 +751,7 @@ static int build(Model &m, void **init, void **state) {
             *pc.slot = (char *)m.warena + off;
             off += align_up(pc.bytes, 256);
         }
-        for (Layer &L : m.layers) {  // the separate repacked copies are not needed any more
-            (void)hipFree(L.own_qkv_w); (void)hipFree(L.own_qkv_s); (void)hipFree(L.own_gu_w); (void)hipFree(L.own_gu_s);
-            L.own_qkv_w = L.own_qkv_s = L.own_gu_w = L.own_gu_s = nullptr;
-        }
+        // (the set keeps its repacked copies: other executors of the session may use them)
     }
 
     // ---- prefill executors keep every linear weight dequantised to the 16-bit type (2 bytes per weight
@@ -691,34 +765,64 @@ static int build(Model &m, void **init, void **state) {
     }
     if (m.skinny) {
         // one more int8 copy of every linear weight, tiled for sequential streaming (1 byte per weight)
-        auto pack = [&](void **dst, const Lin &l) {
-            MYNN_HIP(hipMalloc(dst, skinny_packed_bytes(l.N, l.K)));
-            return skinny_pack_weight(*dst, (const int8_t *)l.w, l.N, l.K, m.stream);
-        };
-        for (Layer &L : m.layers) {
-            TRY(pack(&L.pk_qkv, L.qkv));
-            TRY(pack(&L.pk_o, L.o));
-            TRY(pack(&L.pk_gu, L.gu));
-            TRY(pack(&L.pk_down, L.down));
+        if (!ws.packed8) {
+            ws.bytes_packed8 = 0;
+            auto pack = [&](void **dst, const Lin &l) {
+                renew(dst);
+                MYNN_HIP(hipMalloc(dst, skinny_packed_bytes(l.N, l.K)));
+                ws.bytes_packed8 += skinny_packed_bytes(l.N, l.K);
+                return skinny_pack_weight(*dst, (const int8_t *)l.w, l.N, l.K, m.stream);
+            };
+            for (size_t li = 0; li < m.layers.size(); li++) {
+                Layer &L = m.layers[li];
+                WeightLayer &W = ws.layers[li];
+                TRY(pack(&W.pk_qkv, L.qkv));
+                TRY(pack(&W.pk_o, L.o));
+                TRY(pack(&W.pk_gu, L.gu));
+                TRY(pack(&W.pk_down, L.down));
+            }
+            TRY(pack(&ws.pk_lm_head, m.lm_head));
+            MYNN_HIP(hipStreamSynchronize(m.stream));
+            ws.packed8 = true;
         }
-        TRY(pack(&m.pk_lm_head, m.lm_head));
-        MYNN_HIP(hipStreamSynchronize(m.stream));
+        for (size_t li = 0; li < m.layers.size(); li++) {
+            Layer &L = m.layers[li];
+            const WeightLayer &W = ws.layers[li];
+            L.pk_qkv = W.pk_qkv; L.pk_o = W.pk_o; L.pk_gu = W.pk_gu; L.pk_down = W.pk_down;
+        }
+        m.pk_lm_head = ws.pk_lm_head;
     }
     if (m.quant && !m.skinny && !c.quantize_activations && c.batch * c.seq_q >= 16 && H % 8 == 0 && QD % 8 == 0 && F % 32 == 0) {
-        auto resident = [&](void **dst, const Lin &l) {
-            MYNN_HIP(hipMalloc(dst, gemm_weight_bytes(l.N, l.K)));
-            return dequant_weight_rows(*dst, (const int8_t *)l.w, l.scale, l.N, l.K, c.dtype, 0, 0, m.stream);
-        };
-        for (Layer &L : m.layers) {
-            TRY(resident(&L.wt_qkv, L.qkv));
-            TRY(resident(&L.wt_o, L.o));
-            TRY(resident(&L.wt_down, L.down));
-            MYNN_HIP(hipMalloc(&L.wt_gu, gemm_weight_bytes(2 * F, H)));
-            TRY(dequant_weight_rows(L.wt_gu, (const int8_t *)L.gate.w, L.gate.scale, F, H, c.dtype, 32, 0, m.stream));
-            TRY(dequant_weight_rows(L.wt_gu, (const int8_t *)L.up.w, L.up.scale, F, H, c.dtype, 32, 1, m.stream));
+        if (!ws.resident16) {
+            ws.bytes_resident16 = 0;
+            auto resident = [&](void **dst, const Lin &l) {
+                renew(dst);
+                MYNN_HIP(hipMalloc(dst, gemm_weight_bytes(l.N, l.K)));
+                ws.bytes_resident16 += gemm_weight_bytes(l.N, l.K);
+                return dequant_weight_rows(*dst, (const int8_t *)l.w, l.scale, l.N, l.K, c.dtype, 0, 0, m.stream);
+            };
+            for (size_t li = 0; li < m.layers.size(); li++) {
+                Layer &L = m.layers[li];
+                WeightLayer &W = ws.layers[li];
+                TRY(resident(&W.wt_qkv, L.qkv));
+                TRY(resident(&W.wt_o, L.o));
+                TRY(resident(&W.wt_down, L.down));
+                renew(&W.wt_gu);
+                MYNN_HIP(hipMalloc(&W.wt_gu, gemm_weight_bytes(2 * F, H)));
+                ws.bytes_resident16 += gemm_weight_bytes(2 * F, H);
+                TRY(dequant_weight_rows(W.wt_gu, (const int8_t *)L.gate.w, L.gate.scale, F, H, c.dtype, 32, 0, m.stream));
+                TRY(dequant_weight_rows(W.wt_gu, (const int8_t *)L.up.w, L.up.scale, F, H, c.dtype, 32, 1, m.stream));
+            }
+            TRY(resident(&ws.wt_lm_head, m.lm_head));
+            MYNN_HIP(hipStreamSynchronize(m.stream));
+            ws.resident16 = true;
         }
-        TRY(resident(&m.wt_lm_head, m.lm_head));
-        MYNN_HIP(hipStreamSynchronize(m.stream));
+        for (size_t li = 0; li < m.layers.size(); li++) {
+            Layer &L = m.layers[li];
+            const WeightLayer &W = ws.layers[li];
+            L.wt_qkv = W.wt_qkv; L.wt_o = W.wt_o; L.wt_gu = W.wt_gu; L.wt_down = W.wt_down;
+        }
+        m.wt_lm_head = ws.wt_lm_head;
         m.resident16 = true;
     }
 
@@ -740,15 +844,25 @@ static int build(Model &m, void **init, void **state) {
             qgemm_dma_supported(rows_, H, QD) && qgemm_dma_supported(rows_, 2 * F, H) && qgemm_dma_supported(rows_, H, F) &&
             qgemm_dma_supported(rows_, V, H)) {
             const size_t seb = dtype_size(c.dtype);
-            for (Layer &L : m.layers) {
-                MYNN_HIP(hipMalloc(&L.q8_gu, (size_t)2 * F * H));
-                MYNN_HIP(hipMalloc(&L.q8_gu_scale, (size_t)2 * F * seb));
-                TRY(interleave_row_groups(L.q8_gu, L.gate.w, F, (size_t)H, 32, 0, m.stream));
-                TRY(interleave_row_groups(L.q8_gu, L.up.w, F, (size_t)H, 32, 1, m.stream));
-                TRY(interleave_row_groups(L.q8_gu_scale, L.gate.scale, F, seb, 32, 0, m.stream));
-                TRY(interleave_row_groups(L.q8_gu_scale, L.up.scale, F, seb, 32, 1, m.stream));
+            if (!ws.q8) ws.bytes_q8 = 0;
+            for (size_t li = 0; li < m.layers.size() && !ws.q8; li++) {
+                Layer &L = m.layers[li];
+                WeightLayer &W = ws.layers[li];
+                renew(&W.q8_gu); renew(&W.q8_gu_scale);
+                MYNN_HIP(hipMalloc(&W.q8_gu, (size_t)2 * F * H));
+                MYNN_HIP(hipMalloc(&W.q8_gu_scale, (size_t)2 * F * seb));
+                ws.bytes_q8 += (size_t)2 * F * H + (size_t)2 * F * seb;
+                TRY(interleave_row_groups(W.q8_gu, L.gate.w, F, (size_t)H, 32, 0, m.stream));
+                TRY(interleave_row_groups(W.q8_gu, L.up.w, F, (size_t)H, 32, 1, m.stream));
+                TRY(interleave_row_groups(W.q8_gu_scale, L.gate.scale, F, seb, 32, 0, m.stream));
+                TRY(interleave_row_groups(W.q8_gu_scale, L.up.scale, F, seb, 32, 1, m.stream));
             }
             MYNN_HIP(hipStreamSynchronize(m.stream));
+            ws.q8 = true;
+            for (size_t li = 0; li < m.layers.size(); li++) {
+                m.layers[li].q8_gu = ws.layers[li].q8_gu;
+                m.layers[li].q8_gu_scale = ws.layers[li].q8_gu_scale;
+            }
             m.w8a8_fused = true;
         }
     }
@@ -896,27 +1010,9 @@ static void destroy(Model *m) {
     for (hipEvent_t e : m->events) hipEventDestroy(e);
     if (m->graph_exec) hipGraphExecDestroy(m->graph_exec);
     if (m->graph) hipGraphDestroy(m->graph);
-    for (Layer &L : m->layers) {
-        if (L.own_qkv_w) hipFree(L.own_qkv_w);
-        if (L.own_qkv_s) hipFree(L.own_qkv_s);
-        if (L.qkv_b) hipFree(L.qkv_b);
-        if (L.own_gu_w) hipFree(L.own_gu_w);
-        if (L.own_gu_s) hipFree(L.own_gu_s);
-        if (L.wt_qkv) hipFree(L.wt_qkv);
-        if (L.wt_o) hipFree(L.wt_o);
-        if (L.wt_gu) hipFree(L.wt_gu);
-        if (L.q8_gu) hipFree(L.q8_gu);
-        if (L.q8_gu_scale) hipFree(L.q8_gu_scale);
-        if (L.wt_down) hipFree(L.wt_down);
-        if (L.pk_qkv) hipFree(L.pk_qkv);
-        if (L.pk_o) hipFree(L.pk_o);
-        if (L.pk_gu) hipFree(L.pk_gu);
-        if (L.pk_down) hipFree(L.pk_down);
-    }
+    weight_set_release(m->wset);
     if (m->ws) hipFree(m->ws);
     if (m->warena) hipFree(m->warena);
-    if (m->wt_lm_head) hipFree(m->wt_lm_head);
-    if (m->pk_lm_head) hipFree(m->pk_lm_head);
     if (m->cos_t) hipFree(m->cos_t);
     if (m->sin_t) hipFree(m->sin_t);
     if (m->arena) hipFree(m->arena);
@@ -1027,20 +1123,62 @@ extern "C" int mynn_model_configure(const mynn_model_config *cfg) {
     return 0;
 }
 
+static void *model_create_with(const mynn_model_config *cfg, WeightSet *wset, void **session_state) {
+    Model *m = new Model;
+    m->cfg = *cfg;
+    m->quant = cfg->weights_int8 != 0;
+    m->wset = wset;  // (one reference is the model's from here on: destroy() lets it go)
+    if (build(*m, wset->initializer.data(), session_state)) {
+        destroy(m);
+        return nullptr;
+    }
+    return m;
+}
+
 extern "C" void *mynn_model_create(const mynn_model_config *cfg, void **initializer, void **session_state) {
     if (check_config(cfg)) return nullptr;
     if (!initializer || !session_state) {
         fail(MYNN_ERR_INVALID, "model_create: null initializer / session_state array");
         return nullptr;
     }
-    Model *m = new Model;
-    m->cfg = *cfg;
-    m->quant = cfg->weights_int8 != 0;
-    if (build(*m, initializer, session_state)) {
-        destroy(m);
+    return model_create_with(cfg, weight_set_new(*cfg, initializer), session_state);  // a set of its own
+}
+
+extern "C" mynn_weight_set *mynn_weight_set_create(const mynn_model_config *cfg, void **initializer) {
+    if (check_config(cfg)) return nullptr;
+    if (!initializer) {
+        fail(MYNN_ERR_INVALID, "weight_set_create: null initializer array");
         return nullptr;
     }
-    return m;
+    return (mynn_weight_set *)weight_set_new(*cfg, initializer);
+}
+extern "C" void mynn_weight_set_destroy(mynn_weight_set *set) { weight_set_release((WeightSet *)set); }
+extern "C" int mynn_weight_set_stats(mynn_weight_set *set, size_t *bytes /*[4]*/, int *holders) {
+    MYNN_REQUIRE(set, MYNN_ERR_INVALID, "weight_set_stats: null set");
+    WeightSet &w = *(WeightSet *)set;
+    std::lock_guard<std::mutex> lk(w.mu);
+    if (bytes) {
+        bytes[0] = w.bytes_repack; bytes[1] = w.bytes_resident16; bytes[2] = w.bytes_packed8; bytes[3] = w.bytes_q8;
+    }
+    if (holders) *holders = w.refs;
+    return 0;
+}
+extern "C" void *mynn_model_create_shared(const mynn_model_config *cfg, mynn_weight_set *set, void **session_state) {
+    if (check_config(cfg)) return nullptr;
+    if (!set || !session_state) {
+        fail(MYNN_ERR_INVALID, "model_create_shared: null weight set / session_state array");
+        return nullptr;
+    }
+    WeightSet *w = (WeightSet *)set;
+    {
+        std::lock_guard<std::mutex> lk(w->mu);
+        if (!weight_set_fits(*w, *cfg)) {
+            fail(MYNN_ERR_INVALID, "model_create_shared: the weight set was made for other shapes, another storage type or other weight options");
+            return nullptr;
+        }
+        w->refs++;
+    }
+    return model_create_with(cfg, w, session_state);
 }
 
 extern "C" void *model_init(void **initializer, void **session_state) {
