@@ -717,6 +717,56 @@ def short_prefill(mynn, cfg, weights, seed, weight_set=None):
     return out
 
 
+def decode_variants(mynn, cfg, weights, wset, prompt, K, tdt):
+    """The same batch-1 decode through the two other cache forms of the executor, on the same weights (and weight
+    set), outside the timed region of the main figure: a paged KV cache (device-resident loop, as the main figure) and
+    the streaming (sink + ring) cache, whose steps are host round trips because the ring inputs change per step."""
+    import torch
+
+    out = {}
+    P = 128
+    pool = mynn.KvPool(cfg["max_seq"] // P, P)
+    pages = mynn.KvPages(pool, 1, cfg["max_seq"])
+    kv = pool.buffers(cfg["n_layers"], cfg["n_kv_heads"], cfg["head_dim"], tdt)
+    dec = mynn.Decoder(cfg, weights, kv=kv, kv_pages=pages, weight_set=wset)
+    pages.reserve(cfg["max_seq"])
+    first = None
+    for i, t in enumerate(prompt):
+        first, _ = dec.step([t], [i], i, i + 1)
+    dec.decode_loop(first[0], len(prompt), 16)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    dec.decode_loop(first[0], len(prompt), K)
+    torch.cuda.synchronize()
+    el = time.perf_counter() - t0
+    out["paged_kv_bs1"] = {"tok_s": round(K / el, 1), "ms_per_step": round(el * 1e3 / K, 4), "kv_page_rows": P,
+                           "launches_per_step": dec.stats()["launches_per_step"]}
+    dec.close(), pages.close(), pool.close()
+    del kv
+
+    sink, window = 4, 252
+    sdec = mynn.Decoder(cfg, weights, streaming_kv=True, weight_set=wset)
+    llm = mynn.LlmSession(sdec, eos=-1, streaming=(sink, window))
+    n1 = sink + window - len(prompt) - 8  # stays inside the window
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ids = llm.generate_ids(prompt, n1)
+    t1 = time.perf_counter()
+    n2 = 256  # second turn: every step past the window
+    llm.generate_ids(ids[-1:] + prompt[:7], 8)  # (walks over the edge)
+    t2 = time.perf_counter()
+    llm.generate_ids(prompt[:1], n2)
+    t3 = time.perf_counter()
+    out["streaming_kv_bs1"] = {"sink": sink, "window": window,
+                               "tok_s_inside_window": round((len(prompt) + n1 - 1) / (t1 - t0), 1),
+                               "tok_s_past_window": round(n2 / (t3 - t2), 1), "past_len": llm.past_len,
+                               "launches_per_step": sdec.stats()["launches_per_step"],
+                               "what": "LlmSession.generate_ids: one host round trip per token (ring inputs per step)"}
+    llm.close(), sdec.close()
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -903,6 +953,7 @@ def main():
     if not args.no_prefill and not (args.kv_int8 or args.w8a8 or args.unfused):
         out["config"]["prefill"] = short_prefill(mynn, cfg, weights, args.seed, wset)
         out["config"]["weight_set"] = wset.stats()
+        out["config"]["variants"] = decode_variants(mynn, cfg, weights, wset, prompt, K, torch.float16 if args.dtype == "f16" else torch.bfloat16)
 
     if not args.no_cpu_baseline:
         import oracle as orc

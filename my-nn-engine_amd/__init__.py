@@ -130,6 +130,7 @@ SIGNATURES = {
     "mynn_model_step": (_i, [_vp, _vp, _vp, _i64, _i64, _vp, _vp]),
     "mynn_model_step_streaming": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp]),
     "mynn_model_handover_failures": (_i, [_vp]),
+    "mynn_model_set_handover_rearm": (_i, [_vp, _i]),
     "mynn_model_release_kv_pages": (_i, [_vp]),
     "mynn_model_last_status": (_i, [_vp]),
     "mynn_model_argmax_row": (_i, [_vp, _i, C.POINTER(C.c_int32)]),
@@ -859,6 +860,11 @@ class Decoder:
     @property
     def handover_failures(self):
         return lib().mynn_model_handover_failures(self.handle)
+
+    def set_handover_rearm(self, clean_steps):
+        """Steps without a give-up after which a model that fell back to one op per launch tries the shared launches
+        again (0: never)."""
+        check(lib().mynn_model_set_handover_rearm(self.handle, int(clean_steps)))
 
     def decode_loop(self, token, past_len, n_steps):
         out = (C.c_int32 * n_steps)()

@@ -29,10 +29,19 @@ constexpr int kShortWaves = 8;
 // 127 stored as T, codes rounded half away from zero), appended as codes, and met by the query as the codes times the
 // stored scale -- exactly what a later step reads back; a score is (q . codes) * k_scale * scale and a weight
 // exp(..) * v_scale, as the int8-KV attention operator computes them (attention.cuh:495-513 with its scale slots).
-template <typename T, int D, bool KV8 = false, typename Ready>
+// PAGED: Kcache / Vcache (and the scales) are page pools [n_pages, Hkv, 1 << shift rows, ..] and cache row r of this
+// kv head is row ((page(r >> shift) * Hkv + hkv) << shift) + r % (1 << shift) of them; `pages` holds the sequence's
+// page table with entry j in lane j (at most 64 pages; a wave-wide shuffle picks a key's entry, so the table costs
+// one load per wave before the cache loads and nothing per key).  Same keys, same order: the same bits as the
+// contiguous form.
+struct ShortPaging {
+    int pages = 0;  // lane j: page number of the sequence's j-th page
+    int shift = 0, Hkv = 1, hkv = 0;
+};
+template <typename T, int D, bool KV8 = false, bool PAGED = false, typename Ready>
 __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, const T *vsrc, void *Kcache_v, void *Vcache_v, T *Kscale,
                                                 T *Vscale, int bound, int new_row, bool append, const T *cs, const T *snp, float scale,
-                                                float (*part_s)[D + 2], int tid, float &result, Ready ready) {
+                                                float (*part_s)[D + 2], int tid, float &result, Ready ready, const ShortPaging pg = ShortPaging{}) {
     constexpr int LPK = D / 8, GPW = 64 / LPK, KPP = kShortWaves * GPW;  // lanes per key, keys per wave / workgroup and pass
     const int lane = tid & 63, wave = tid >> 6;
     const int dc = lane % LPK, grp = lane / LPK;
@@ -41,6 +50,16 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
     TKV *Kcache = (TKV *)Kcache_v, *Vcache = (TKV *)Vcache_v;
     const TKV *Kc = Kcache + dc * 8, *Vc = Vcache + dc * 8;
 
+    // row of the cache buffers that holds cache row `key` (every lane of the wave calls it: the page entry comes
+    // from another lane)
+    auto row_of = [&](int key) -> size_t {
+        if constexpr (PAGED) {
+            const int page = __shfl(pg.pages, min(max(key, 0), max(bound - 1, 0)) >> pg.shift, 64);
+            return (((size_t)page * pg.Hkv + pg.hkv) << pg.shift) + (size_t)(key & ((1 << pg.shift) - 1));
+        } else {
+            return (size_t)key;
+        }
+    };
     // ---- all K / V loads of this lane for a round of kShortPasses passes (the first round before anything else)
     Chunk kreg[kShortPasses], vreg[kShortPasses];
     T ksc[KV8 ? kShortPasses : 1], vsc[KV8 ? kShortPasses : 1];  // as loaded
@@ -48,14 +67,15 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
 #pragma unroll
         for (int i = 0; i < kShortPasses; i++) {
             const int key = base + i * KPP + wave * GPW + grp;
+            const size_t row = row_of(key);
             kreg[i] = vreg[i] = Chunk{};
             if constexpr (KV8) ksc[i] = vsc[i] = T{};
             if (key < bound && key != new_row) {
-                kreg[i] = *(const Chunk *)(Kc + (size_t)key * D);
-                vreg[i] = *(const Chunk *)(Vc + (size_t)key * D);
+                kreg[i] = *(const Chunk *)(Kc + row * D);
+                vreg[i] = *(const Chunk *)(Vc + row * D);
                 if constexpr (KV8) {
-                    ksc[i] = Kscale[key];
-                    vsc[i] = Vscale[key];
+                    ksc[i] = Kscale[row];
+                    vsc[i] = Vscale[row];
                 }
             }
         }
@@ -118,18 +138,20 @@ __device__ __forceinline__ bool attn_short_body(const T *qsrc, const T *ksrc, co
         };
         quantise(kn, kn_q, kn_sc);
         quantise(vn, vn_q, vn_sc);
+        const size_t new_at = row_of(new_row);
         if (append && wave == 0 && grp == 0) {
-            *(Chunk *)(Kcache + (size_t)new_row * D + d0) = kn_q;
-            *(Chunk *)(Vcache + (size_t)new_row * D + d0) = vn_q;
+            *(Chunk *)(Kcache + new_at * D + d0) = kn_q;
+            *(Chunk *)(Vcache + new_at * D + d0) = vn_q;
             if (dc == 0) {
-                Elem<T>::st(Kscale, new_row, kn_sc);
-                Elem<T>::st(Vscale, new_row, vn_sc);
+                Elem<T>::st(Kscale, new_at, kn_sc);
+                Elem<T>::st(Vscale, new_at, vn_sc);
             }
         }
     } else {
+        const size_t new_at = row_of(new_row);
         if (append && wave == 0 && grp == 0) {  // one lane group appends the new row
-            *(U4 *)(Kcache + (size_t)new_row * D + d0) = kn_packed;
-            *(U4 *)(Vcache + (size_t)new_row * D + d0) = v_new;
+            *(U4 *)(Kcache + new_at * D + d0) = kn_packed;
+            *(U4 *)(Vcache + new_at * D + d0) = v_new;
         }
     }
 

@@ -194,6 +194,11 @@ struct Model {
     uint64_t *lm_cand = nullptr;  // its candidate words (all ~0 between launches)
     int spin_limit = 400000;      // polls a consumer role makes before it gives up and raises the error word
     int handover_failures = 0;    // steps whose hand-over gave up; the executor then rebuilt itself with one op per launch
+    // what build() had chosen before a give-up switched the shared launches off, and when they are tried again: after
+    // rearm_after clean steps (doubled by every further give-up; 0 = never)
+    bool shared_qkv_attn = false, shared_lm_argmax = false, fell_back = false;
+    int rearm_after = 256;
+    long clean_steps = 0;
     // streaming_kv: the ring inputs of the step in flight (host copies: the operators take them at launch time, as the
     // reference's kernels do), kv_position on the device, and the operators' [heads, S, D] tensors
     int ring_sink = 0, ring_window = 0, ring_start = 0, h_past = 0, h_active = 0;
@@ -415,6 +420,7 @@ static int enqueue_step(Model &m) {
             p.k_scale = kv8 ? L.k_scale : nullptr; p.v_scale = kv8 ? L.v_scale : nullptr;
             p.cos_t = m.cos_t; p.sin_t = m.sin_t; p.d_pos = m.d_pos; p.d_active = m.d_active; p.d_past = m.d_past; p.Hq = Hq; p.Hkv = Hkv;
             p.max_seq = c.max_seq; p.softmax_scale = softmax_scale; p.err = m.d_past + 3; p.spin_limit = m.spin_limit;
+            p.paging = m.paging;
             if (li == 0) {  // the input row of the first layer: the token's embedding
                 p.embed_w = (const int8_t *)m.embed.w; p.embed_s = m.embed.scale; p.d_ids = m.d_ids; p.vocab = V;
             }
@@ -938,8 +944,8 @@ static int build(Model &m, void **init, void **state) {
 
     // ---- batch-1 decode: projection and attention in one launch when the shape allows
     m.spin_limit = c.handover_spin_limit > 0 ? c.handover_spin_limit : c.handover_spin_limit < 0 ? 0 : 400000;
-    if (m.quant && rows == 1 && !c.quantize_activations && !c.unfused_decode && !m.pages && !c.qkv_bias && !c.streaming_kv &&
-        attention_fused_supported(c.head_dim, c.n_heads / c.n_kv_heads) &&
+    if (m.quant && rows == 1 && !c.quantize_activations && !c.unfused_decode && (!m.pages || m.paging.pages_per_seq <= 64) && !c.qkv_bias &&
+        !c.streaming_kv && attention_fused_supported(c.head_dim, c.n_heads / c.n_kv_heads) &&
         (!c.quant_kv_cache || attention_fused_kv8_supported(c.head_dim, c.max_seq)) &&
         qkv_attention_supported(H, c.n_heads, c.n_kv_heads, c.head_dim, c.max_seq, c.dtype) && (QD + 2 * KD) * eb % 8 == 0) {
         bool ok = aligned16(m.qkv) && aligned16(m.x) && aligned16(m.attn) && aligned16(m.embed.w);
@@ -1061,11 +1067,39 @@ static int handover_recover(Model &m) {
     MYNN_HIP(hipMemset(m.qkv, 0xFF, (size_t)((char *)m.attn + (size_t)c.n_heads * c.head_dim * dtype_size(c.dtype) - (char *)m.qkv)));
     MYNN_HIP(hipMemset(m.lm_cand, 0xFF, (size_t)kGemvArgmaxWords * 8));
     MYNN_HIP(hipMemset(m.d_past + 3, 0, 4));
+    if (!m.fell_back && m.handover_failures == 0) {
+        m.shared_qkv_attn = m.qkv_attn;
+        m.shared_lm_argmax = m.lm_argmax;
+    } else if (m.rearm_after > 0 && m.rearm_after < (1 << 20)) {
+        m.rearm_after *= 2;  // it happened again after a re-arm: wait twice as long before the next try
+    }
     m.handover_failures++;
+    m.fell_back = true;
+    m.clean_steps = 0;
     m.qkv_attn = false;
     m.lm_argmax = false;
     set_error("decode step: a stage of a fused launch waited too long for the stage before it (is the device shared?); "
               "the executor now runs one op per launch");
+    return capture_step(m);
+}
+
+// `steps` more steps went through without a give-up (the stream is drained).  A model that fell back goes back to the
+// shared launches once enough of them have: what made a producer late (another process on the device, a debugger, a
+// serialising tool) is usually gone by then, and staying with one op per launch for the rest of a long-lived
+// executor's life would cost it a third of its speed.  The hand-over vectors are emptied first: as ordinary
+// activation buffers of the one-op-per-launch step they hold data.
+static int handover_clean_steps(Model &m, long steps) {
+    if (!m.fell_back || m.rearm_after <= 0) return 0;
+    m.clean_steps += steps;
+    if (m.clean_steps < m.rearm_after) return 0;
+    const mynn_model_config &c = m.cfg;
+    MYNN_HIP(hipMemset(m.qkv, 0xFF, (size_t)((char *)m.attn + (size_t)c.n_heads * c.head_dim * dtype_size(c.dtype) - (char *)m.qkv)));
+    MYNN_HIP(hipMemset(m.lm_cand, 0xFF, (size_t)kGemvArgmaxWords * 8));
+    MYNN_HIP(hipMemset(m.d_past + 3, 0, 4));
+    m.qkv_attn = m.shared_qkv_attn;
+    m.lm_argmax = m.shared_lm_argmax;
+    m.fell_back = false;
+    m.clean_steps = 0;
     return capture_step(m);
 }
 
@@ -1242,7 +1276,7 @@ extern "C" int mynn_model_step(void *state, const int64_t *input_ids, const int6
     MYNN_REQUIRE(!m.cfg.streaming_kv, MYNN_ERR_STATE, "model_step: a streaming_kv model takes the ring inputs (mynn_model_step_streaming)");
     bool failed = false;
     TRY(step_once(m, input_ids, position_id, past_len, active_seq_kv, next_token, logits_host, &failed));
-    if (!failed) return 0;
+    if (!failed) return handover_clean_steps(m, 1);
     TRY(handover_recover(m));
     TRY(step_once(m, input_ids, position_id, past_len, active_seq_kv, next_token, logits_host, &failed));
     return failed ? fail(MYNN_ERR_STATE, "decode step: hand-over failure after recovery") : 0;
@@ -1283,6 +1317,11 @@ extern "C" int mynn_model_release_kv_pages(void *state) {
     return m.pages ? mynn_kv_pages_release(m.pages) : 0;
 }
 extern "C" int mynn_model_handover_failures(void *state) { return state ? ((Model *)state)->handover_failures : 0; }
+extern "C" int mynn_model_set_handover_rearm(void *state, int clean_steps) {
+    MYNN_REQUIRE(state && clean_steps >= 0, MYNN_ERR_INVALID, "model_set_handover_rearm: bad argument");
+    ((Model *)state)->rearm_after = clean_steps;
+    return 0;
+}
 extern "C" int mynn_model_last_status(void *state) { return state ? ((Model *)state)->last_status : MYNN_ERR_INVALID; }
 
 // Reference ABI: void, host pointers, synchronous.  A failure is reported on stderr, through mynn_last_error()
@@ -1354,7 +1393,7 @@ extern "C" int mynn_model_decode_loop(void *state, int32_t token, int64_t past_l
             continue;
         }
         memcpy(out_tokens, m.h_stage, (size_t)n_steps * 4);
-        return 0;
+        return handover_clean_steps(m, n_steps);
     }
     return fail(MYNN_ERR_STATE, "decode loop: hand-over failure after recovery");
 }

@@ -93,8 +93,9 @@ struct QkvAttnParams {
     uint64_t *qkv;           // hand-over vector of N 16-bit elements: all 0xFFFF ("empty") on entry
     int gemv_blocks, groups; // filled in by the launcher
     void *out;               // [Hq * D]
-    void *k_cache, *v_cache; // [Hkv, max_seq, D]
+    void *k_cache, *v_cache; // [Hkv, max_seq, D]; paging.table set: page pools [n_pages, Hkv, page rows, D]
     void *k_scale, *v_scale; // int8 cache (BuildOptions::quant_kv_cache): [Hkv, max_seq] row scales; null: 16-bit cache
+    KvPaging paging;         // paged cache: the sequence's page table (at most 64 pages)
     const void *cos_t, *sin_t;
     const int64_t *d_pos;
     const int32_t *d_active;

@@ -212,7 +212,7 @@ __device__ __forceinline__ void qa_gemv(const QaGemv &a, float *act_lds, float *
 // EMBED: the layer's input row is the embedding row of token *p.d_ids (first layer of a step)
 // What a workgroup's first loads need are leading scalar arguments (copies of the fields of p): they arrive
 // preloaded in SGPRs with the wave instead of through a scalar load from the kernarg segment.
-template <typename T, int D, int NC, bool EMBED, bool KV8>
+template <typename T, int D, int NC, bool EMBED, bool KV8, bool PAGED>
 __global__ __launch_bounds__(kQaThreads, 2) void qkv_attention_kernel(const void *x, const void *norm_w, const int8_t *wq,
                                                                           const int32_t *d_active, const int64_t *d_pos,
                                                                           int gemv_blocks, int N, int K, int Hq, QkvAttnParams p) {
@@ -250,7 +250,15 @@ __global__ __launch_bounds__(kQaThreads, 2) void qkv_attention_kernel(const void
     const int h = blockIdx.x - gemv_blocks, Gt = Hq / p.Hkv, hkv = h / Gt;
     const int active = *d_active;
     const int64_t pos = *d_pos;
-    const size_t kv_base = (size_t)hkv * p.max_seq * D;  // in elements of the cache's type
+    // contiguous caches [Hkv, max_seq, D]; PAGED: pools, rows found through the sequence's page table (one entry per lane)
+    const size_t kv_rows = PAGED ? 0 : (size_t)hkv * p.max_seq;
+    const size_t kv_base = kv_rows * D;  // in elements of the cache's type
+    ShortPaging sp{};
+    if constexpr (PAGED) {
+        const int lane = tid & 63;
+        sp.pages = lane < p.paging.pages_per_seq ? p.paging.table[lane] : 0;
+        sp.shift = p.paging.shift; sp.Hkv = p.Hkv; sp.hkv = hkv;
+    }
     using TKV = typename std::conditional<KV8, int8_t, T>::type;
     constexpr int WPH = D / 4;  // 8-byte words per head slice
     auto ready = [&] {
@@ -262,10 +270,10 @@ __global__ __launch_bounds__(kQaThreads, 2) void qkv_attention_kernel(const void
         __syncthreads();
     };
     float r = 0.f;
-    if (attn_short_body<T, D, KV8>(qkv_l, qkv_l + D, qkv_l + 2 * D, (TKV *)p.k_cache + kv_base, (TKV *)p.v_cache + kv_base,
-                              KV8 ? (T *)p.k_scale + (size_t)hkv * p.max_seq : nullptr, KV8 ? (T *)p.v_scale + (size_t)hkv * p.max_seq : nullptr,
-                              min(active, p.max_seq), *p.d_past, h % Gt == 0, (const T *)p.cos_t + pos * D,
-                              (const T *)p.sin_t + pos * D, p.softmax_scale, part_s, tid, r, ready)) {
+    if (attn_short_body<T, D, KV8, PAGED>(qkv_l, qkv_l + D, qkv_l + 2 * D, (TKV *)p.k_cache + kv_base, (TKV *)p.v_cache + kv_base,
+                                          KV8 ? (T *)p.k_scale + kv_rows : nullptr, KV8 ? (T *)p.v_scale + kv_rows : nullptr,
+                                          min(active, p.max_seq), *p.d_past, h % Gt == 0, (const T *)p.cos_t + pos * D,
+                                          (const T *)p.sin_t + pos * D, p.softmax_scale, part_s, tid, r, ready, sp)) {
         if (p.o_blocks) qa_put16(p.attn_words, h * D + tid, qa_bits<T>(r));
         else Elem<T>::st((T *)p.out, (size_t)h * D + tid, r);
     }
@@ -301,7 +309,10 @@ int qkv_attention_launch(QkvAttnParams p, int D, int dtype, hipStream_t s) {
     const int nc = (p.K + 1023) / 1024;
     const size_t lds = (size_t)p.K * sizeof(float);
     const dim3 grid(p.gemv_blocks + p.Hq + p.o_blocks), block(kQaThreads);
-    const bool embed = p.embed_w != nullptr, kv8 = p.k_scale != nullptr;
+    const bool embed = p.embed_w != nullptr, kv8 = p.k_scale != nullptr, paged = p.paging.table != nullptr;
+    MYNN_REQUIRE(!paged || (p.paging.pages_per_seq <= 64 && (p.paging.pages_per_seq << p.paging.shift) == p.max_seq), MYNN_ERR_UNSUPPORTED,
+                 "qkv + attention: a paged cache of %d pages of %d rows (at most 64 pages, covering max_seq %d)", p.paging.pages_per_seq,
+                 1 << p.paging.shift, p.max_seq);
     MYNN_REQUIRE(!kv8 || p.v_scale, MYNN_ERR_INVALID, "qkv + attention: int8 KV needs both scale buffers");
     MYNN_REQUIRE(!embed || (p.embed_s && p.d_ids && p.vocab > 0 && p.o_wq && ((uintptr_t)p.embed_w & 7) == 0 && p.K % 8 == 0),
                  MYNN_ERR_INVALID, "qkv + attention + o: bad embedding operand");
@@ -310,10 +321,15 @@ int qkv_attention_launch(QkvAttnParams p, int D, int dtype, hipStream_t s) {
 #define MYNN_QA_LAUNCH(...) MYNN_LAUNCH((qkv_attention_kernel<T, __VA_ARGS__>), grid, block, lds, s, p.x, p.norm_w, p.wq, p.d_active, p.d_pos, p.gemv_blocks, p.N, p.K, p.Hq, p)
 #define MYNN_QA(D_, NC_)                                                                          \
     do {                                                                                          \
-        if (embed && kv8) MYNN_QA_LAUNCH(D_, NC_, true, true);                                    \
-        else if (embed) MYNN_QA_LAUNCH(D_, NC_, true, false);                                     \
-        else if (kv8) MYNN_QA_LAUNCH(D_, NC_, false, true);                                       \
-        else MYNN_QA_LAUNCH(D_, NC_, false, false);                                               \
+        if (paged) {                                                                              \
+            if (embed && kv8) MYNN_QA_LAUNCH(D_, NC_, true, true, true);                          \
+            else if (embed) MYNN_QA_LAUNCH(D_, NC_, true, false, true);                           \
+            else if (kv8) MYNN_QA_LAUNCH(D_, NC_, false, true, true);                             \
+            else MYNN_QA_LAUNCH(D_, NC_, false, false, true);                                     \
+        } else if (embed && kv8) MYNN_QA_LAUNCH(D_, NC_, true, true, false);                      \
+        else if (embed) MYNN_QA_LAUNCH(D_, NC_, true, false, false);                              \
+        else if (kv8) MYNN_QA_LAUNCH(D_, NC_, false, true, false);                                \
+        else MYNN_QA_LAUNCH(D_, NC_, false, false, false);                                        \
         return launch_status("qkv_attention_kernel");                                             \
     } while (0)
         if (D == 64) {

@@ -91,6 +91,37 @@ def test_handover_give_up_falls_back_to_one_op_per_launch(g, dt, kv8):
     loop.close(), plain.close()
 
 
+@pytest.mark.parametrize("dt", [orc.F16])
+def test_handover_fallback_rearms_after_clean_steps(g, dt):
+    """A model that fell back goes back to the shared launches after the given number of clean steps.  With a consumer
+    that always gives up at once the first shared step after the re-arm fails again (and doubles the wait), so the
+    failure count shows where the re-arms happened; every step's results stay those of the un-fused executor."""
+    cfg, w = llm_weights.synthetic_int8(SHORT_CACHE[64], dt, seed=72)
+    dw = dev_weights(g, w, dt)
+    plain = g.mynn.Decoder(cfg, dw, unfused_decode=True)
+    quick = g.mynn.Decoder(cfg, dw, handover_spin_limit=-1)
+    quick.set_handover_rearm(3)
+    shared, single = quick.stats()["launches_per_step"], plain.stats()["launches_per_step"]
+    toks = np.random.default_rng(2).integers(0, cfg["vocab"], 14)
+    failures, launches = [], []
+    for i, t in enumerate(toks):
+        a, la = quick.step([t], [i], i, i + 1, want_logits=True)
+        b, lb = plain.step([t], [i], i, i + 1, want_logits=True)
+        assert np.array_equal(la, lb) and a == b, i
+        failures.append(quick.handover_failures)
+        launches.append(quick.stats()["launches_per_step"])
+    # step 0 gives up (1); clean steps 1-3 re-arm; step 4 gives up (2) and the wait doubles to 6: clean steps
+    # 5-10 re-arm; step 11 gives up (3); the wait is 12 from there
+    assert failures == [1, 1, 1, 1, 2, 2, 2, 2, 2, 2, 2, 3, 3, 3]
+    assert launches == [single] * 3 + [shared] + [single] * 6 + [shared] + [single] * 3
+    # never again once switched off
+    quick.set_handover_rearm(0)
+    for i in range(14, 40):
+        quick.step([int(toks[i % 14])], [i], i, i + 1)
+    assert quick.handover_failures == 3 and quick.stats()["launches_per_step"] == single
+    quick.close(), plain.close()
+
+
 # ------------------------------------------------------------------ additive mask (operator slot 3)
 def test_attention_causal_golden_as_explicit_mask(g):
     """The reference's `attention_causal` fixture with the causal rule written as an additive mask (0 on and below

@@ -398,8 +398,9 @@ def test_paged_executor_prefill_then_batched_decode_equals_contiguous(g, dt):
 
 @pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
 def test_paged_executor_batch1_decode_vs_oracle(g, dt):
-    """Batch-1 decode over a paged cache (hipGraph replay, the device-resident loop included) against the oracle: the
-    attention runs in the streaming kernel here, in the single-launch block with a contiguous cache."""
+    """Batch-1 decode over a paged cache (hipGraph replay, the device-resident loop included) against the oracle: as
+    with a contiguous cache, projection, attention and o projection of a layer are one launch that finds its rows
+    through the page table."""
     cfg, w = llm_weights.synthetic_int8(PAGED_D64, dt, seed=23)
     dw = dev_weights(g, w, dt)
     ref = orc.Model(cfg, w)
@@ -411,7 +412,7 @@ def test_paged_executor_batch1_decode_vs_oracle(g, dt):
     other.reserve(1)
     pages, dec, _ = _sessions(g, cfg, dw, dt, pool, kvbufs, 1)
     st = dec.stats()
-    assert st["graph"] and st["launches_per_step"] == 6 * cfg["n_layers"] + 3
+    assert st["graph"] and st["launches_per_step"] == 3 * cfg["n_layers"] + 1
     rng = np.random.default_rng(2)
     n = 70  # crosses the first page border
     toks = rng.integers(0, cfg["vocab"], n)
@@ -447,6 +448,59 @@ def test_paged_executor_batch1_decode_vs_oracle(g, dt):
         dec.step([1], [200], 200, 201)
     assert "mynn error -5" in str(e.value)
     dec.close(), pages.close(), other.close(), pool.close()
+
+
+@pytest.mark.parametrize("kv8", [False, True], ids=["kv16", "kv_int8"])
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
+def test_paged_batch1_single_launch_layer_equals_contiguous(g, dt, D, kv8):
+    """The single-launch layer (q|k|v projection, RoPE + append + attention, o projection) over a paged cache reads and
+    writes the same rows in the same order as over a contiguous one: logits, tokens and cached rows bit for bit, step
+    by step across page borders and inside the device-resident loop; one op per launch (unfused_decode: the streaming
+    attention kernel) agrees with it within the 16-bit tolerance."""
+    from test_gpu_decoder import SHORT_CACHE
+
+    cfg, w = llm_weights.synthetic_int8(SHORT_CACHE[D], dt, seed=37)
+    dw = dev_weights(g, w, dt)
+    P = 64
+    pool = g.mynn.KvPool(2 * cfg["max_seq"] // P + 3, P)
+    tdt = g.torch_dtype(dt)
+    other = g.mynn.KvPages(pool, 1, cfg["max_seq"])
+    other.reserve(P + 1)  # (the session's pages then are not 0, 1, 2 ...)
+    plain = g.mynn.Decoder(cfg, dw, quant_kv_cache=kv8)
+    kv_a = pool.buffers(cfg["n_layers"], cfg["n_kv_heads"], cfg["head_dim"], tdt, fill=float("nan"), kv_int8=kv8)
+    pages_a = g.mynn.KvPages(pool, 1, cfg["max_seq"])
+    paged = g.mynn.Decoder(cfg, dw, kv=kv_a, kv_pages=pages_a, quant_kv_cache=kv8)
+    pages_b = g.mynn.KvPages(pool, 1, cfg["max_seq"])
+    single = g.mynn.Decoder(cfg, dw, kv=kv_a, kv_pages=pages_b, quant_kv_cache=kv8, unfused_decode=True)
+    L = cfg["n_layers"]
+    assert plain.stats()["launches_per_step"] == paged.stats()["launches_per_step"] == 3 * L + 1
+    assert single.stats()["launches_per_step"] > 3 * L + 1
+    rng = np.random.default_rng(D)
+    n = 2 * P + 7
+    toks = rng.integers(0, cfg["vocab"], n)
+    for i, t in enumerate(toks):
+        a, la = plain.step([t], [i], i, i + 1, want_logits=True)
+        b, lb = paged.step([t], [i], i, i + 1, want_logits=True)
+        assert a == b and np.array_equal(la, lb), i
+        if i % 16 == 5 or i >= n - 3:
+            _, lc = single.step([t], [i], i, i + 1, want_logits=True)
+            assert max_err_rel_to_max(g.f32(lc, dt), g.f32(la, dt)) <= (3e-2 if kv8 else 1e-2), i
+        else:
+            single.step([t], [i], i, i + 1)
+    table = pages_a.table()
+    assert table[0, 0] >= 2 and pages_a.mapped_rows == 3 * P
+    for l in range(L):
+        for j in range(len(plain.kv[l])):  # (int8 KV: codes, then per-row scales)
+            got = gather_cache(g, kv_a[l][j] if kv_a[l][j].dim() == 4 else kv_a[l][j].unsqueeze(-1), table, P)[0]
+            want = g.to_host(plain.kv[l][j])[0]
+            want = want if want.ndim == 3 else want[..., None]
+            assert np.array_equal(got[:, :n], want[:, :n]), (l, j)
+    # the device-resident loop
+    assert paged.decode_loop(int(toks[-1]), n - 1, 40) == plain.decode_loop(int(toks[-1]), n - 1, 40)
+    for d in (plain, paged, single):
+        d.close()
+    pages_a.close(), pages_b.close(), other.close(), pool.close()
 
 
 @pytest.mark.parametrize("dt", [orc.F16, orc.BF16])
