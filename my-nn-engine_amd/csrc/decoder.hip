@@ -189,6 +189,10 @@ struct Model {
     int launches = 0;
     // batch-1 decode: projection and attention share a launch; m.qkv is then the hand-over vector between them
     // (all 0xFFFF between uses) and d_past[3] the error word of its bounded waits
+    // the device-resident loop replays kLoopSteps steps per graph launch where it can (a graph launch costs the device a
+    // few microseconds of its own, a tenth of a batch-1 step's launches)
+    hipGraph_t graph_loop = nullptr;
+    hipGraphExec_t graph_loop_exec = nullptr;
     bool qkv_attn = false;
     bool lm_argmax = false;       // ... and the lm_head launch finds the greedy token and moves the loop state on
     uint64_t *lm_cand = nullptr;  // its candidate words (all ~0 between launches)
@@ -977,11 +981,14 @@ static int build(Model &m, void **init, void **state) {
 
 // Captures the decode step once (one new token per sequence, any batch: every launch reads its positions and
 // lengths from device memory).  Called again when the executor changes its launch plan.
+constexpr int kLoopSteps = 32;
 static int capture_step(Model &m) {
     if (m.graph_exec) (void)hipGraphExecDestroy(m.graph_exec);
     if (m.graph) (void)hipGraphDestroy(m.graph);
-    m.graph_exec = nullptr;
-    m.graph = nullptr;
+    if (m.graph_loop_exec) (void)hipGraphExecDestroy(m.graph_loop_exec);
+    if (m.graph_loop) (void)hipGraphDestroy(m.graph_loop);
+    m.graph_exec = m.graph_loop_exec = nullptr;
+    m.graph = m.graph_loop = nullptr;
     m.use_graph = false;
     if (m.cfg.seq_q != 1 || m.cfg.streaming_kv) return 0;  // (the streaming operators take host scalars at launch time)
     hipError_t e = hipStreamBeginCapture(m.stream, hipStreamCaptureModeThreadLocal);
@@ -992,6 +999,20 @@ static int capture_step(Model &m) {
             m.use_graph = true;
         else {
             (void)hipGetLastError();
+            if (rc) return rc;
+        }
+    } else (void)hipGetLastError();
+    // batch-1 decode: several steps in one graph for the device-resident loop (every step leaves the next one's token,
+    // position and lengths on the device, so the steps of a graph chain like separate launches of the one-step graph)
+    if (m.use_graph && m.cfg.batch == 1 && hipStreamBeginCapture(m.stream, hipStreamCaptureModeThreadLocal) == hipSuccess) {
+        int rc = 0;
+        for (int i = 0; i < kLoopSteps && rc == 0; i++) rc = enqueue(m);
+        hipError_t e2 = hipStreamEndCapture(m.stream, &m.graph_loop);
+        if (rc != 0 || e2 != hipSuccess || hipGraphInstantiate(&m.graph_loop_exec, m.graph_loop, nullptr, nullptr, 0) != hipSuccess) {
+            (void)hipGetLastError();
+            if (m.graph_loop) (void)hipGraphDestroy(m.graph_loop);
+            m.graph_loop = nullptr;
+            m.graph_loop_exec = nullptr;
             if (rc) return rc;
         }
     } else (void)hipGetLastError();
@@ -1016,6 +1037,8 @@ static void destroy(Model *m) {
     for (hipEvent_t e : m->events) hipEventDestroy(e);
     if (m->graph_exec) hipGraphExecDestroy(m->graph_exec);
     if (m->graph) hipGraphDestroy(m->graph);
+    if (m->graph_loop_exec) hipGraphExecDestroy(m->graph_loop_exec);
+    if (m->graph_loop) hipGraphDestroy(m->graph_loop);
     weight_set_release(m->wset);
     if (m->ws) hipFree(m->ws);
     if (m->warena) hipFree(m->warena);
@@ -1381,7 +1404,10 @@ extern "C" int mynn_model_decode_loop(void *state, int32_t token, int64_t past_l
     for (int attempt = 0; attempt < 2; attempt++) {
         int64_t id = token, pos = past_len;
         TRY(upload_inputs(m, &id, &pos, past_len, past_len + 1));
-        for (int i = 0; i < n_steps; i++) TRY(run_once(m));
+        int done = 0;
+        if (m.use_graph && !m.profiling && m.graph_loop_exec)
+            for (; done + kLoopSteps <= n_steps; done += kLoopSteps) MYNN_HIP(hipGraphLaunch(m.graph_loop_exec, m.stream));
+        for (; done < n_steps; done++) TRY(run_once(m));
         MYNN_HIP(hipMemcpyAsync(m.h_stage, m.d_tokens, (size_t)n_steps * 4, hipMemcpyDeviceToHost, m.stream));
         char *h_err = m.h_stage + m.stage_bytes - m.next_stage;
         if (m.qkv_attn) MYNN_HIP(hipMemcpyAsync(h_err, m.d_past + 3, 4, hipMemcpyDeviceToHost, m.stream));
