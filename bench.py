@@ -744,6 +744,23 @@ def decode_variants(mynn, cfg, weights, wset, prompt, K, tdt):
     dec.close(), pages.close(), pool.close()
     del kv
 
+    # the session call a user of the reference makes (LlmSession::generate_ids): prompt token by token, then runs of the
+    # device-resident loop
+    gdec = mynn.Decoder(cfg, weights, weight_set=wset)
+    llm = mynn.LlmSession(gdec, eos=-1)
+    llm.generate_ids(prompt, 1)
+    llm.reset()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    llm.generate_ids(prompt, 1)
+    t1 = time.perf_counter()
+    llm.reset()
+    llm.generate_ids(prompt, 1 + K)
+    t2 = time.perf_counter()
+    out["llm_session_generate_ids"] = {"new_tokens": K, "tok_s_after_the_prompt": round(K / ((t2 - t1) - (t1 - t0)), 1),
+                                       "prompt_tok_s": round(len(prompt) / (t1 - t0), 1)}
+    llm.close(), gdec.close()
+
     sink, window = 4, 252
     sdec = mynn.Decoder(cfg, weights, streaming_kv=True, weight_set=wset)
     llm = mynn.LlmSession(sdec, eos=-1, streaming=(sink, window))

@@ -224,7 +224,12 @@ extern "C" int mynn_llm_generate_ids(mynn_llm *l, const int64_t *prompt_ids, siz
     MYNN_REQUIRE(l->streaming || l->max_seq >= needed, MYNN_ERR_TOO_LONG, "prompt needs %lld cache rows, max_seq_len is %d (past_len %lld)",
                  (long long)needed, l->max_seq, (long long)l->past_len);
     int n_new = 0;
-    for (size_t i = 0; i < max_new_tokens; i++) {
+    // the executor's device-resident loop (mynn_model_decode_loop) serves runs of decode steps without a host round
+    // trip per token; with an end-of-sequence id the runs are short, and what a run computed past that id is dropped
+    // (its cache rows lie beyond past_len, where the next turn overwrites them)
+    bool loop_ok = !l->step && !l->streaming && l->decode != nullptr;
+    std::vector<int32_t> run;
+    for (size_t i = 0; i < max_new_tokens;) {
         if (!l->streaming && l->max_seq < l->past_len + 1) break;
         int64_t tok = 0;
         int rc;
@@ -234,9 +239,29 @@ extern "C" int mynn_llm_generate_ids(mynn_llm *l, const int64_t *prompt_ids, siz
                 rc = 0;
                 for (size_t j = 0; j < n_prompt && rc == 0; j++) rc = decode_step(l, prompt_ids[j], &tok);
             }
-        } else rc = decode_step(l, out[n_new - 1], &tok);
+        } else {
+            const int64_t room = l->max_seq - l->past_len;
+            const size_t want = std::min<size_t>(std::min<size_t>(max_new_tokens - i, l->eos >= 0 ? 32 : 256), (size_t)room);
+            if (loop_ok && want >= 4) {
+                run.resize(want);
+                if (mynn_model_decode_loop(l->decode, out[n_new - 1], l->past_len, (int)want, run.data()) == 0) {
+                    size_t used = 0;
+                    while (used < want) {
+                        out[n_new++] = run[used++];
+                        if (out[n_new - 1] == l->eos) break;
+                    }
+                    l->past_len += (int64_t)used;
+                    i += used;
+                    if (out[n_new - 1] == l->eos) break;
+                    continue;
+                }
+                loop_ok = false;  // (a model without the loop, or no pages for the whole run: step by step from here)
+            }
+            rc = decode_step(l, out[n_new - 1], &tok);
+        }
         if (rc) return rc > 0 ? -1000 - rc : rc;
         out[n_new++] = tok;
+        i++;
         if (tok == l->eos) break;
     }
     return n_new;

@@ -156,6 +156,44 @@ def test_generate_bookkeeping_and_errors(g):
     llm.close(), dec.close()
 
 
+@pytest.mark.parametrize("shape", ["generic_head_dim_32", "single_launch_layer"])
+def test_generate_runs_of_steps_on_the_device_equal_step_by_step(g, shape):
+    """LlmSession.generate_ids serves decode steps in runs of the executor's device-resident loop.  Ids, the stop at
+    the end-of-sequence id in the middle of a run, past_len and a following turn (which overwrites the rows the run
+    computed past the stop) are those of feeding one token per call (session.rs:508-537, 612-640)."""
+    dt = orc.F16
+    cfg, w = llm_weights.synthetic_int8(SMALL if shape == "generic_head_dim_32" else SHORT_CACHE[64], dt, seed=13)
+    dw = dev_weights(g, w, dt)
+    prompt = [7, 8, 9, 10, 11]
+
+    def by_steps(dec, past, feed, n_new, eos):
+        out, nxt = [], None
+        for t in feed:
+            nxt, _ = dec.step([t], [past], past, past + 1)
+            past += 1
+        out.append(nxt[0])
+        while len(out) < n_new and out[-1] != eos:
+            nxt, _ = dec.step([out[-1]], [past], past, past + 1)
+            past += 1
+            out.append(nxt[0])
+        return out, past
+
+    dec, ref = g.mynn.Decoder(cfg, dw), g.mynn.Decoder(cfg, dw)
+    free, _ = by_steps(ref, 0, prompt, 60, -1)
+    llm = g.mynn.LlmSession(dec, eos=-1)
+    assert llm.generate_ids(prompt, 60) == free and llm.past_len == len(prompt) + 59
+    llm.close()
+    # an end-of-sequence id that first shows up inside a run
+    j0 = next(j for j in range(10, 60) if free[j] not in free[:j])
+    eos = free[j0]
+    llm = g.mynn.LlmSession(dec, eos=eos)
+    assert llm.generate_ids(prompt, 60) == free[:j0 + 1]
+    assert llm.past_len == len(prompt) + j0
+    want2, past2 = by_steps(ref, len(prompt) + j0, [3, 4], 12, eos)
+    assert llm.generate_ids([3, 4], 12) == want2 and llm.past_len == past2
+    llm.close(), dec.close(), ref.close()
+
+
 @pytest.fixture(params=[0, 1, 2, 3, 4], ids=["tile_auto", "tile_256x128", "tile_256x256", "tile_256x256_direct_lds", "tile_256x320_direct_lds"])
 def gemm_tile(request):
     return request.param
