@@ -36,8 +36,8 @@ ROLE_PATTERNS = {
     "gemv_norm_gateup_swiglu": r"dequant_gemv1_kernelI\w+?Li\d+ELi\d+ELi2ELb1ELb0EE",
     "gemv_down_residual": r"dequant_gemv1_kernelI\w+?Li\d+ELi\d+ELi1ELb0ELb0EE",
     "gemv_norm_lm_head_argmax": r"dequant_gemv1_kernelI\w+?Li\d+ELi\d+ELi0ELb1ELb1EE",
-    "qkv_attention_o": r"qkv_attention_kernelI\w+?Li\d+ELi\d+ELb0ELb0EE",        # <T, D, NC, EMBED = false, KV8 = false>
-    "embed_qkv_attention_o": r"qkv_attention_kernelI\w+?Li\d+ELi\d+ELb1ELb0EE",
+    "qkv_attention_o": r"qkv_attention_kernelI\w+?Li\d+ELi\d+ELb0ELb0ELb0EE",   # <T, D, NC, EMBED = false, KV8 = false, PAGED = false>
+    "embed_qkv_attention_o": r"qkv_attention_kernelI\w+?Li\d+ELi\d+ELb1ELb0ELb0EE",
     "linear_gateup_swiglu": r"(gemm_nt_dma_kernelI\w+?Li2ELb0EE|skinny_gemm_kernel)",
     "qlinear_gateup_swiglu": r"gemm_nt_dma_kernelI\w+?Li2ELb1EE",
     "attention": r"(attn_stream_kernel|attn_prefill_kernel)",
@@ -136,11 +136,14 @@ def summarize_rocprof(args):
         if "mynn" not in name:
             continue
         d = (int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e3
-        k = kern.setdefault(name, {"mangled": name, "calls": 0, "total_us": 0.0, "min_us": 1e30, "max_us": 0.0})
+        k = kern.setdefault(name, {"mangled": name, "calls": 0, "total_us": 0.0, "min_us": 1e30, "max_us": 0.0, "by_grid": {}})
         k["calls"] += 1
         k["total_us"] += d
         k["min_us"] = min(k["min_us"], d)
         k["max_us"] = max(k["max_us"], d)
+        g = k["by_grid"].setdefault("%sx%sx%s" % (r.get("Grid_Size_X"), r.get("Grid_Size_Y"), r.get("Grid_Size_Z")), [0, 0.0])
+        g[0] += 1
+        g[1] += d
     copy = {}
     for which, d in (("fetch", args.pmc_fetch), ("write", args.pmc_write)):
         if not d:
@@ -183,6 +186,10 @@ def summarize_rocprof(args):
         k["avg_us"] = round(k["total_us"] / k["calls"], 3)
         k["total_ms"] = round(k.pop("total_us") / 1e3, 3)
         k["min_us"], k["max_us"] = round(k["min_us"], 3), round(k["max_us"], 3)
+        # one instantiation launched over several shapes (grids, in work-items): the average per grid beside the mixed one
+        grids = k.pop("by_grid")
+        if len(grids) > 1:
+            k["by_grid"] = [{"grid": g, "calls": v[0], "avg_us": round(v[1] / v[0], 3)} for g, v in sorted(grids.items(), key=lambda kv: -kv[1][1])]
         for f in ("fetch_kib", "write_kib"):
             if f in k:
                 k[f] = round(k[f], 1)
@@ -197,6 +204,11 @@ def summarize_rocprof(args):
         lines.append("| `%s` | %d | %.2f | %.2f | %.2f | %.2f | %s | %s | %s |" % (
             k["mangled"], k["calls"], k["avg_us"], k["min_us"], k["max_us"], k["total_ms"], k.get("fetch_kib", "-"),
             k.get("write_kib", "-"), tb if tb is not None else "-"))
+    for k in out["kernels"]:
+        if k.get("by_grid"):
+            lines.append("")
+            lines.append("`%s` by grid (work-items): " % k["mangled"][:60] +
+                         "; ".join("%s: %d launches, %.2f us" % (g["grid"], g["calls"], g["avg_us"]) for g in k["by_grid"]))
     print("\n".join(lines))
 
 
