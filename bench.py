@@ -38,7 +38,7 @@ ROLE_PATTERNS = {
     "gemv_norm_lm_head_argmax": r"dequant_gemv1_kernelI\w+?Li\d+ELi\d+ELi0ELb1ELb1EE",
     "qkv_attention_o": r"qkv_attention_kernelI\w+?Li\d+ELi\d+ELb0ELb0ELb0EE",   # <T, D, NC, EMBED = false, KV8 = false, PAGED = false>
     "embed_qkv_attention_o": r"qkv_attention_kernelI\w+?Li\d+ELi\d+ELb1ELb0ELb0EE",
-    "linear_gateup_swiglu": r"(gemm_nt_dma_kernelI\w+?Li2ELb0EE|skinny_gemm_kernel)",
+    "linear_gateup_swiglu": r"(gemm_nt_dma_kernelI\w+?Li2ELb0EE|skinny_gemm_kernelI\w+?Li\d+ELb\dELi2ELi0EE)",  # (skinny: <T, MT, PACKED, FEPI = SwiGLU, ABL = 0>)
     "qlinear_gateup_swiglu": r"gemm_nt_dma_kernelI\w+?Li2ELb1EE",
     "attention": r"(attn_stream_kernel|attn_prefill_kernel)",
     # --workload gemv: the stand-alone GEMV launches and the read probe of the same geometry
@@ -687,6 +687,14 @@ def decode_batch_main(args, mynn):
                      "bytes_per_launch": bytes_tot / calls,
                      "avg_launch_us": round(ms_tot / calls * 1e3, 2)},
     }
+    if "attention" in agg:  # the launch with the most time in the step: K and V rows of every sequence at this context
+        a_calls, a_ms, _ = agg["attention"]
+        a_bytes = float(B) * 2 * kv_row * past
+        a_entry = profile_entry(prof, "attention")
+        out["roofline"]["attention"] = {"bytes_per_launch": a_bytes, "avg_launch_us": round(a_ms / a_calls * 1e3, 2),
+                                        "frac": round(a_bytes / (a_ms / a_calls * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                                        "avg_launch_us_rocprof": a_entry["avg_us"] if a_entry else None,
+                                        "traffic": traffic_bytes(a_entry)}
     dec.close()
     if pages:
         pages.close(), pool.close()
