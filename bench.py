@@ -777,7 +777,8 @@ def decode_variants(mynn, cfg, weights, wset, prompt, K, tdt):
     llm.reset()
     llm.generate_ids(prompt, 1 + K)
     t2 = time.perf_counter()
-    out["llm_session_generate_ids"] = {"new_tokens": K, "tok_s_after_the_prompt": round(K / ((t2 - t1) - (t1 - t0)), 1),
+    gen_s = (t2 - t1) - (t1 - t0)
+    out["llm_session_generate_ids"] = {"new_tokens": K, "tok_s_after_the_prompt": round(K / gen_s, 1) if gen_s > 0 else None,
                                        "prompt_tok_s": round(len(prompt) / (t1 - t0), 1)}
     llm.close(), gdec.close()
 
@@ -873,7 +874,14 @@ def main():
         return gemv_main(args, mynn)
     K = 256 if args.steps is None else args.steps
     W = 16 if args.warmup is None else args.warmup
-    assert PROMPT_LEN + max(K, W) <= cfg["max_seq"], "steps/warmup do not fit max_seq %d" % cfg["max_seq"]
+    # the cache of configs[2] holds 128 + 256 rows; longer runs get a longer cache (whole 128-row pages, up to the 2048 rows
+    # the single-launch layer covers at head_dim 64: the workload stays the same kernels)
+    need = PROMPT_LEN + max(K, W)
+    if need > cfg["max_seq"]:
+        cfg["max_seq"] = (need + 127) // 128 * 128
+    if cfg["max_seq"] > 2048:
+        raise SystemExit("bench.py: --steps / --warmup of at most %d fit this workload (128 prompt rows + the generated ones <= 2048)"
+                         % (2048 - PROMPT_LEN))
 
     weights = make_weights(cfg, dt, args.seed)
     torch.cuda.synchronize()
