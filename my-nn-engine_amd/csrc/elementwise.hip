@@ -393,11 +393,21 @@ __global__ __launch_bounds__(1024) void argmax_last_kernel(int32_t *out, const T
     int bi = -1;
     if constexpr (sizeof(T) == 2) {
         const int nvec = (((uintptr_t)row & 15) == 0) ? n / 8 : 0;
-        for (int c = threadIdx.x; c < nvec; c += 1024) {
-            float f[8];
-            widen8<T>(((const U4 *)row)[c], f);
+        // eight loads in flight per thread (one at a time, a 128256-entry row was sixteen dependent round trips: 17 us)
+        constexpr int kAhead = 8;
+        for (int c0 = threadIdx.x; c0 < nvec; c0 += 1024 * kAhead) {
+            U4 v[kAhead];
 #pragma unroll
-            for (int e = 0; e < 8; e++) argmax_take(bv, bi, f[e], c * 8 + e);
+            for (int j = 0; j < kAhead; j++) v[j] = ((const U4 *)row)[min(c0 + j * 1024, nvec - 1)];
+#pragma unroll
+            for (int j = 0; j < kAhead; j++) {
+                const int c = c0 + j * 1024;
+                if (c >= nvec) break;
+                float f[8];
+                widen8<T>(v[j], f);
+#pragma unroll
+                for (int e = 0; e < 8; e++) argmax_take(bv, bi, f[e], c * 8 + e);
+            }
         }
         for (int i = nvec * 8 + threadIdx.x; i < n; i += 1024) argmax_take(bv, bi, Elem<T>::ld(row, i), i);
     } else {

@@ -312,7 +312,8 @@ __global__ __launch_bounds__(kReduceNormThreads) void skinny_reduce_norm_kernel(
 }
 
 // The plain form of the reduction for a q|k|v projection, followed by what rope_kv_append_vec_kernel does with
-// the stored projection: one workgroup per token row, a thread per (head, 4 rotation pairs) or 4 values of v;
+// the stored projection: a thread per (head, 4 rotation pairs) or 4 values of v, a token row's threads spread over
+// several two-wave workgroups;
 // qkv values are rounded to the storage type before the rotation, exactly as if they had been stored.
 // KV8: the caches are int8 with one scale per token row (rope_quant_kv_append_kernel's arithmetic: k after RoPE rounded
 // to T, v as stored; s = amax / 127 stored as T, q = trunc(x * 127 / amax +- 0.5) clamped to [-128, 127]); every head
@@ -373,8 +374,11 @@ __global__ __launch_bounds__(kReduceRopeThreads) void skinny_reduce_rope_kernel(
         *(uint32_t *)(dst + j) = code(lo[0]) | (code(lo[1]) << 8) | (code(lo[2]) << 16) | (code(lo[3]) << 24);
         *(uint32_t *)(dst + j + half) = code(hi[0]) | (code(hi[1]) << 8) | (code(hi[2]) << 16) | (code(hi[3]) << 24);
     };
-    // (one workgroup per row read its 150 KB of partial sums on one CU: 5.7 us; spread over the device 3.6 us)
-    for (int u = blockIdx.y * kReduceRopeThreads + threadIdx.x; u < units; u = units) {
+    // one unit per thread, a row's units over gridDim.y workgroups (as one workgroup per row, which pulled the row's
+    // 150 KB of partial sums through a single CU, the launch took 5.7 us at batch 32; 4.7 us spread over the device)
+    const int u = blockIdx.y * kReduceRopeThreads + threadIdx.x;
+    if (u >= units) return;
+    {
         if (u >= rot_units) {
             if constexpr (KV8) {
                 const int hv = (u - rot_units) / upr, j = ((u - rot_units) % upr) * 4;
@@ -389,7 +393,7 @@ __global__ __launch_bounds__(kReduceRopeThreads) void skinny_reduce_rope_kernel(
                 T *dst = (T *)v_cache_v + kv_cache_row(pg, b, hv, past + sq, Hkv, max_seq) * D + j;
                 *(uint2 *)dst = uint2{pack2<T>(t[0], t[1]), pack2<T>(t[2], t[3])};
             }
-            continue;
+            return;
         }
         const int head = u / upr, j = (u % upr) * 4;
         float xl[4], xh[4], cl[4], ch[4], sl[4], sh[4];
@@ -413,7 +417,7 @@ __global__ __launch_bounds__(kReduceRopeThreads) void skinny_reduce_rope_kernel(
                     oh[i] = Elem<T>::rnd(oh[i]);
                 }
                 quantise_store(ol, oh, (int8_t *)k_cache_v, k_scale, kv_cache_row(pg, b, head - Hq, past + sq, Hkv, max_seq), j);
-                continue;
+                return;
             }
         }
         T *dst = head < Hq ? q_out + (size_t)m * Hq * D + (size_t)head * D
