@@ -46,9 +46,9 @@ def test_config2_full_greedy_decode_128_prompt_256_generated_vs_oracle(g, bench,
     LlmSession and through the device-resident loop the benchmark times (the same ids).  The oracle follows the
     GPU's token stream step by step (so both always see the same context) and its own greedy choice is compared at
     each of the 256 generated positions.  The reference leaves the order of its f32 sums open, and with random-init
-    weights the two best logits are sometimes closer than two orders differ: the oracle therefore runs under three
-    summation orders (16 lanes + tree, sequential, 64 lanes; one KV cache each), and a token that is not the first
-    order's choice is accepted only where the oracle's own arithmetic does not separate the two tokens: the GPU's
+    weights the two best logits are sometimes closer than two orders differ: the oracle therefore runs under four
+    summation orders (16, 8, 32, 64 lanes + tree; one KV cache each; a disputed step again under 1, 2 and 4), and a token
+    that is not the first order's choice is accepted only where the oracle's own arithmetic does not separate the two tokens: the GPU's
     token is the choice under another order, the orders disagree among themselves, or the oracle's gap between the
     two is inside the shifts its orders show among themselves at that step (oracle.SummationOrders.judge) -- anything
     else fails.  Measured on MI355X, seed 1234: 2 of 256 (positions 149 and 186), both flipped by another order."""
@@ -68,6 +68,22 @@ def test_config2_full_greedy_decode_128_prompt_256_generated_vs_oracle(g, bench,
         first_tok, _ = dec.step([t], [i], i, i + 1)
     assert [first_tok[0]] + dec.decode_loop(first_tok[0], len(prompt), n_new - 1) == got
     dec.close()
+    # ... and so does the same model over a paged cache (the single-launch layer finds its rows through the page
+    # table), built on a weight set it shares with a second executor
+    wset = g.mynn.WeightSet(cfg, weights)
+    pool = g.mynn.KvPool(cfg["max_seq"] // 128 + 2, 128)
+    other = g.mynn.KvPages(pool, 1, cfg["max_seq"])
+    other.reserve(129)  # (two pages gone: the session's pages are not 0, 1, 2)
+    pages = g.mynn.KvPages(pool, 1, cfg["max_seq"])
+    kv = pool.buffers(cfg["n_layers"], cfg["n_kv_heads"], cfg["head_dim"], g.torch_dtype(dt))
+    paged = g.mynn.Decoder(cfg, weights, kv=kv, kv_pages=pages, weight_set=wset)
+    twin = g.mynn.Decoder(cfg, weights, weight_set=wset)
+    assert paged.stats()["launches_per_step"] == 3 * cfg["n_layers"] + 1 and wset.stats()["holders"] == 3
+    for d in (paged, twin):
+        for i, t in enumerate(prompt):
+            first_tok, _ = d.step([t], [i], i, i + 1)
+        assert [first_tok[0]] + d.decode_loop(first_tok[0], len(prompt), n_new - 1) == got
+    paged.close(), twin.close(), wset.close(), pages.close(), other.close(), pool.close()
     ref = orc.SummationOrders(cfg, host)
     stream = prompt + got[:-1]
     undecided, wrong = [], []
